@@ -1,0 +1,133 @@
+"""Pins oracle/mesh_oracle.c's block formats by means independent of it: numpy's IEEE binary16,
+the exact-rational golden vectors of tests/golden/make_golden.py, natural-domain closed forms and
+invariants.  (ggml itself is not reachable offline, so this is what "parity" rests on.)"""
+import numpy as np
+import pytest
+
+import oracle
+
+
+def test_fp16_decode_exhaustive_vs_numpy():
+    h = np.arange(65536, dtype=np.uint16)
+    got = oracle.fp16_to_fp32(h)
+    ref = h.view(np.float16).astype(np.float32)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+
+
+def test_fp16_encode_vs_numpy_random_bits():
+    rng = np.random.Generator(np.random.PCG64(5))
+    bits = rng.integers(0, 2**32, size=4_000_000, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        ref = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.fp32_to_fp16(x), ref)
+
+
+def test_fp16_encode_all_ties_and_neighbours():
+    # every midpoint between adjacent finite halves, and the binary32 values just below/above it
+    h = np.arange(0, 0x7C00, dtype=np.uint16)
+    lo = h.view(np.float16).astype(np.float64)
+    hi = (h + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    hi[-1] = 65536.0  # the value "after" 65504 for rounding purposes
+    mid = ((lo + hi) / 2).astype(np.float32)  # exactly representable in binary32
+    for x in (mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)), -mid):
+        with np.errstate(over="ignore"):
+            ref = x.astype(np.float16).view(np.uint16)
+        assert np.array_equal(oracle.fp32_to_fp16(x), ref)
+
+
+def test_fp16_encode_nan_inf():
+    x = np.array([np.inf, -np.inf, np.nan, -np.nan], dtype=np.float32)
+    got = oracle.fp32_to_fp16(x)
+    assert got[0] == 0x7C00 and got[1] == 0xFC00
+    assert got[2] & 0x7FFF == 0x7E00 and got[3] & 0x7FFF == 0x7E00
+
+
+def test_fp16_golden(golden):
+    assert np.array_equal(oracle.fp32_to_fp16(golden["f16_x"]), golden["f16_bits"])
+
+
+def test_q8_0_golden(golden):
+    x, y = golden["q8_0_x"], golden["q8_0_blocks"]
+    got = oracle.quantize_q8_0(x.reshape(-1)).reshape(-1, 34)
+    assert np.array_equal(got, y)
+    # rounding mode spelled out: block 0 has d = 1
+    q = got[0, 2:].view(np.int8)
+    assert list(q[:14]) == [127, -127, 64, 1, -1, 2, 3, -3, 4, -4, 127, -127, 0, 0]
+
+
+def _c2_like(T, h=4096, seed=None):
+    rng = np.random.Generator(np.random.PCG64(1234 + T if seed is None else seed))
+    x = rng.standard_normal((T, h)).astype(np.float32)
+    ch = np.random.Generator(np.random.PCG64(1234)).choice(h, size=5, replace=False)
+    x[:, ch] *= 50
+    return x
+
+
+def test_q8_0_invariants():
+    x = _c2_like(16)
+    blk = oracle.quantize_q8_0(x.reshape(-1)).reshape(-1, 34)
+    q = blk[:, 2:].view(np.int8).astype(np.int32)
+    d = blk[:, :2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    xb = x.reshape(-1, 32)
+    am = np.argmax(np.abs(xb), axis=1)
+    rows = np.arange(xb.shape[0])
+    assert np.array_equal(q[rows, am], np.where(xb[rows, am] > 0, 127, -127))
+    assert np.abs(q).max() <= 127
+    # reconstruction bound: half a step plus the fp16 rounding of the scale
+    err = np.abs(xb - q * d[:, None])
+    dtrue = np.abs(xb).max(axis=1) / 127
+    assert np.all(err <= dtrue[:, None] * 0.5 * 1.0001 + np.abs(xb) * 2.0**-10)
+    # dequantize is q * fp16(d)
+    deq = oracle.dequantize(oracle.Q8_0, blk.reshape(-1), x.size).reshape(-1, 32)
+    assert np.array_equal(deq, (q * d[:, None]).astype(np.float32))
+
+
+def test_q8_0_matches_float32_numpy_restatement():
+    # same definition evaluated by numpy's IEEE float32 ops (vectorised), half-away rounding done in float64
+    x = _c2_like(64, seed=9).reshape(-1, 32)
+    amax = np.abs(x).max(axis=1)
+    d = (amax / np.float32(127)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(d != 0, np.float32(1) / d, np.float32(0)).astype(np.float32)
+    v = (x * inv[:, None]).astype(np.float32).astype(np.float64)
+    q = (np.sign(v) * np.floor(np.abs(v) + 0.5)).astype(np.int8)
+    blk = oracle.quantize_q8_0(x.reshape(-1)).reshape(-1, 34)
+    assert np.array_equal(blk[:, 2:].view(np.int8), q)
+    assert np.array_equal(blk[:, :2].copy().view(np.uint16).reshape(-1), d.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("name,type_,k", [("q4_K", oracle.Q4_K, 256), ("q6_K", oracle.Q6_K, 256), ("q5_0", oracle.Q5_0, 32)])
+def test_kquant_golden(golden, name, type_, k):
+    blocks, y = golden[name + "_blocks"], golden[name + "_y"]
+    got = oracle.dequantize(type_, blocks.reshape(-1), k * blocks.shape[0]).reshape(-1, k)
+    assert np.array_equal(got.view(np.uint32), y.view(np.uint32))
+
+
+def test_q4_K_plain_affine_special_case():
+    # all sub-scales equal and dmin = 0 reduces to y = (d*s) * nibble, nibble l of byte b at 64c+l / 64c+32+l
+    rng = np.random.Generator(np.random.PCG64(3))
+    qs = rng.integers(0, 256, 128, dtype=np.uint8)
+    s = 21
+    scales = bytes([s] * 4 + [0] * 4 + [s & 0xF] * 4)  # j<4: sc=s,m=0 ; j>=4: low nibble sc, high bits from q[j-4]>>6 = 0
+    d = np.float16(0.0123)
+    blk = np.frombuffer(d.tobytes() + np.float16(0).tobytes() + scales + qs.tobytes(), dtype=np.uint8)
+    y = oracle.dequantize(oracle.Q4_K, blk, 256)
+    ds_lo = np.float32(d) * np.float32(s)
+    ds_hi = np.float32(d) * np.float32(s & 0xF)
+    for c in range(4):
+        ds = ds_lo if c < 2 else ds_hi
+        assert np.array_equal(y[64 * c:64 * c + 32], ds * (qs[32 * c:32 * c + 32] & 0xF).astype(np.float32) - np.float32(0))
+        assert np.array_equal(y[64 * c + 32:64 * c + 64], ds * (qs[32 * c:32 * c + 32] >> 4).astype(np.float32))
+
+
+def test_row_bytes():
+    assert oracle.row_bytes(oracle.Q4_K, 4096) == 16 * 144
+    assert oracle.row_bytes(oracle.Q6_K, 14336) == 56 * 210
+    assert oracle.row_bytes(oracle.Q8_0, 896) == 28 * 34
+    assert oracle.row_bytes(oracle.Q5_0, 896) == 28 * 22
+    assert oracle.row_bytes(oracle.Q4_K, 896) == -1
+    assert oracle.row_bytes(oracle.F16, 7) == 14 and oracle.row_bytes(oracle.F32, 7) == 28
