@@ -83,6 +83,104 @@ int mesh_act_unpack_dev(int fmt, const void *d_src, float *d_dst, int64_t n, voi
  * dequantize_row_* (what to_float does for a weight tensor).  Device pointers, queued on `stream`. */
 int mesh_dequantize_dev(int type, const void *d_src, float *d_dst, int64_t n, void *stream);
 
+/* ---- weights and mul_mat -------------------------------------------------------------------------
+ * One weight matrix resident in HBM, as ggml_backend_tensor_set leaves it after SET_TENSOR /
+ * SET_TENSOR_GGUF (patches/0001:261), and the mul_mat node of the worker's graph
+ * (patches/0002:443-451 -> ggml_backend_graph_compute). */
+typedef struct mesh_weight mesh_weight;
+
+/* host_data: n_rows rows of row_len elements in GGUF block layout of `type` (F32, F16, Q8_0, Q5_0, Q4_K, Q6_K). */
+int mesh_weight_upload(int type, const void *host_data, int64_t n_rows, int64_t row_len, mesh_weight **out);
+void mesh_weight_free(mesh_weight *w);
+/* GGUF bytes of the matrix (what one mul_mat must read from HBM). */
+size_t mesh_weight_nbytes(const mesh_weight *w);
+/* d_y[t][m] = sum_k W[m][k] * d_x[t][k], t < n_tokens; f32 activations on the device, queued on `stream`. */
+int mesh_mul_mat_dev(const mesh_weight *w, const float *d_x, int64_t n_tokens, float *d_y, void *stream);
+/* Round trip for tests: the matrix back in GGUF block layout (host buffer of mesh_weight_nbytes bytes). */
+int mesh_weight_download(const mesh_weight *w, void *host_data);
+
+/* ---- GGUF --------------------------------------------------------------------------------------- */
+typedef struct mesh_model_info {
+    char arch[32];
+    uint32_t n_layer, n_embd, n_head, n_head_kv, head_dim, n_ff, n_vocab;
+    uint32_t n_rot, rope_mode;            /* rope_mode: 0 = NORM (llama), 2 = NEOX (qwen2/qwen3) */
+    uint32_t n_expert, n_expert_used, n_ff_exp;
+    float rms_eps, rope_freq_base;
+    uint32_t gguf_version, alignment;
+    uint64_t n_tensors, data_offset, file_size;
+} mesh_model_info;
+
+typedef struct mesh_tensor_info {
+    uint32_t type, n_dims;
+    uint64_t ne[4];
+    uint64_t file_offset;                 /* data section offset + tensor offset (patches/0001:209) */
+    uint64_t nbytes;
+} mesh_tensor_info;
+
+/* Header-only scan of a GGUF file: hyper-parameters and container facts, no tensor data touched.
+ * The bounded parse of mesh-client/src/models/gguf.rs:318-420 (scan_gguf_compact_meta). */
+int mesh_gguf_probe(const char *gguf_path, mesh_model_info *out);
+/* Directory entry of one tensor by name -- the lookup rpc_server::set_tensor_gguf does (patches/0001:203-209).
+ * MESH_ERR_INVALID if the tensor is absent, MESH_ERR_FORMAT if its bytes would leave the file. */
+int mesh_gguf_tensor(const char *gguf_path, const char *name, mesh_tensor_info *out);
+
+/* ---- stage -------------------------------------------------------------------------------------- */
+typedef struct mesh_stage mesh_stage;
+typedef struct mesh_session mesh_session;
+
+/* Pseudo-formats for the two ends of the pipeline. */
+#define MESH_TOKENS 100   /* input: int32 token ids (stage must start at layer 0 and the file hold token_embd) */
+#define MESH_LOGITS 101   /* output: f32 [n_tokens][n_vocab] after output_norm and the output projection */
+
+typedef struct mesh_stage_opts {
+    const char *device;     /* "ROCm0" / "HIP0" / "0"; NULL = current device               (-d, launch.rs:920-952) */
+    int32_t n_ctx;          /* KV positions per sequence; 0 = 4096                          (-c, launch.rs:474-504) */
+    int32_t n_seq_max;      /* sequences the KV cache holds; 0 = 1                          (--parallel, launch.rs:1338-1390) */
+    int32_t n_batch_max;    /* most tokens one decode call may carry; 0 = 512 */
+    int32_t kv_type;        /* 0 or MESH_F16 (f16 K and V, the tier of launch.rs:585-589) */
+} mesh_stage_opts;
+
+typedef struct mesh_batch {
+    int32_t n_tokens;
+    const int32_t *pos;     /* [n_tokens] cache position of each token */
+    const int32_t *seq_id;  /* [n_tokens] sequence of each token; NULL = all 0 */
+} mesh_batch;
+
+/* Load layers [layer_begin, layer_end) of the GGUF model at gguf_path into HBM (layer_end < 0 = to the last
+ * layer).  What `rpc-server --gguf PATH` plus the SET_TENSOR_GGUF traffic of start-up amount to
+ * (mesh-llm/src/inference/launch.rs:887-1030; patches/0001:179-266). */
+int mesh_stage_open(const char *gguf_path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out);
+void mesh_stage_close(mesh_stage *stage);
+int mesh_stage_info(const mesh_stage *stage, mesh_model_info *out);
+/* GGUF bytes of everything this stage keeps resident (the weight traffic of one decode step). */
+size_t mesh_stage_weight_bytes(const mesh_stage *stage);
+
+/* A session owns the KV cache of n_seq_max sequences and the activation buffers. */
+int mesh_stage_session_new(mesh_stage *stage, mesh_session **out);
+void mesh_stage_session_free(mesh_session *session);
+
+/* Run the stage over a batch: `in` holds n_tokens rows of n_embd in in_fmt (MESH_F32 / MESH_F16 / MESH_Q8_0, the
+ * boundary tensor of the previous stage) or int32 token ids (MESH_TOKENS); each token's K/V is stored at
+ * (seq_id, pos) and it attends to positions [0, pos] of its sequence.  `out` receives the boundary hidden state
+ * packed in out_fmt, or logits (MESH_LOGITS).  *out_len = bytes written (set even when out_cap is too small).
+ * Host pointers; blocks until done.  The GRAPH_COMPUTE + tensor push of one step (patches/0002:443-451,544-622). */
+int mesh_stage_decode(mesh_session *session, const mesh_batch *batch, const void *in, int in_fmt,
+                      void *out, int out_fmt, size_t out_cap, size_t *out_len);
+/* Same with device pointers for in/out; queued on the session's stream, returns without waiting. */
+int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const void *d_in, int in_fmt,
+                          void *d_out, int out_fmt, size_t out_cap, size_t *out_len);
+/* The session's hipStream_t (for events), and a wait for everything queued on it. */
+void *mesh_session_stream(mesh_session *session);
+int mesh_session_synchronize(mesh_session *session);
+
+/* KV cache import/export for one sequence and one (absolute) layer: n_pos positions starting at pos0, host
+ * buffers of f16 bits laid out [n_pos][n_head_kv][head_dim].  (The reference has no KV hand-over; a restarted
+ * stage refills from the prompt -- mesh-llm/src/inference/election.rs:1894-1910.) */
+int mesh_session_kv_write(mesh_session *session, int layer, int seq_id, int pos0, int n_pos,
+                          const uint16_t *k, const uint16_t *v);
+int mesh_session_kv_read(mesh_session *session, int layer, int seq_id, int pos0, int n_pos,
+                         uint16_t *k, uint16_t *v);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,61 @@ SIGNATURES = {
     "mesh_dequantize_dev": (_i32, [_i32, _vp, _vp, _i64, _vp]),
 }
 
+
+
+class ModelInfo(ctypes.Structure):
+    """mesh_model_info"""
+    _fields_ = [("arch", ctypes.c_char * 32)] + [(n, ctypes.c_uint32) for n in (
+        "n_layer", "n_embd", "n_head", "n_head_kv", "head_dim", "n_ff", "n_vocab", "n_rot", "rope_mode",
+        "n_expert", "n_expert_used", "n_ff_exp")] + [("rms_eps", ctypes.c_float), ("rope_freq_base", ctypes.c_float),
+        ("gguf_version", ctypes.c_uint32), ("alignment", ctypes.c_uint32),
+        ("n_tensors", ctypes.c_uint64), ("data_offset", ctypes.c_uint64), ("file_size", ctypes.c_uint64)]
+
+
+class TensorInfo(ctypes.Structure):
+    """mesh_tensor_info"""
+    _fields_ = [("type", ctypes.c_uint32), ("n_dims", ctypes.c_uint32), ("ne", ctypes.c_uint64 * 4),
+                ("file_offset", ctypes.c_uint64), ("nbytes", ctypes.c_uint64)]
+
+
+class StageOpts(ctypes.Structure):
+    """mesh_stage_opts"""
+    _fields_ = [("device", ctypes.c_char_p), ("n_ctx", ctypes.c_int32), ("n_seq_max", ctypes.c_int32),
+                ("n_batch_max", ctypes.c_int32), ("kv_type", ctypes.c_int32)]
+
+
+class Batch(ctypes.Structure):
+    """mesh_batch"""
+    _fields_ = [("n_tokens", ctypes.c_int32), ("pos", ctypes.POINTER(ctypes.c_int32)),
+                ("seq_id", ctypes.POINTER(ctypes.c_int32))]
+
+
+TOKENS, LOGITS = 100, 101
+_pp = ctypes.POINTER(ctypes.c_void_p)
+_psz = ctypes.POINTER(ctypes.c_size_t)
+
+SIGNATURES.update({
+    "mesh_weight_upload": (_i32, [_i32, _vp, _i64, _i64, _pp]),
+    "mesh_weight_free": (None, [_vp]),
+    "mesh_weight_nbytes": (_sz, [_vp]),
+    "mesh_mul_mat_dev": (_i32, [_vp, _vp, _i64, _vp, _vp]),
+    "mesh_weight_download": (_i32, [_vp, _vp]),
+    "mesh_gguf_probe": (_i32, [_cp, ctypes.POINTER(ModelInfo)]),
+    "mesh_gguf_tensor": (_i32, [_cp, _cp, ctypes.POINTER(TensorInfo)]),
+    "mesh_stage_open": (_i32, [_cp, _i32, _i32, ctypes.POINTER(StageOpts), _pp]),
+    "mesh_stage_close": (None, [_vp]),
+    "mesh_stage_info": (_i32, [_vp, ctypes.POINTER(ModelInfo)]),
+    "mesh_stage_weight_bytes": (_sz, [_vp]),
+    "mesh_stage_session_new": (_i32, [_vp, _pp]),
+    "mesh_stage_session_free": (None, [_vp]),
+    "mesh_stage_decode": (_i32, [_vp, ctypes.POINTER(Batch), _vp, _i32, _vp, _i32, _sz, _psz]),
+    "mesh_stage_decode_dev": (_i32, [_vp, ctypes.POINTER(Batch), _vp, _i32, _vp, _i32, _sz, _psz]),
+    "mesh_session_stream": (_vp, [_vp]),
+    "mesh_session_synchronize": (_i32, [_vp]),
+    "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
+    "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
+})
+
 _lib = None
 
 
@@ -118,3 +173,147 @@ def act_unpack_dev(fmt, d_src, d_dst, n, stream=0):
 
 def dequantize_dev(type_, d_src, d_dst, n, stream=0):
     check(lib().mesh_dequantize_dev(type_, d_src, d_dst, n, stream))
+
+
+# ---------------------------------------------------------------------------------------------- weights
+class Weight:
+    """One matrix resident in HBM (mesh_weight)."""
+
+    def __init__(self, type_, data, n_rows, row_len):
+        import numpy as np
+        data = np.ascontiguousarray(data).view(np.uint8)
+        self._h = ctypes.c_void_p()
+        check(lib().mesh_weight_upload(type_, _np_ptr(data), n_rows, row_len, ctypes.byref(self._h)))
+        self.type, self.n_rows, self.row_len = type_, n_rows, row_len
+
+    @property
+    def nbytes(self):
+        return int(lib().mesh_weight_nbytes(self._h))
+
+    def mul_mat_dev(self, d_x, n_tokens, d_y, stream=0):
+        check(lib().mesh_mul_mat_dev(self._h, d_x, n_tokens, d_y, stream))
+
+    def download(self):
+        import numpy as np
+        out = np.empty(self.nbytes, dtype=np.uint8)
+        check(lib().mesh_weight_download(self._h, _np_ptr(out)))
+        return out
+
+    def close(self):
+        if self._h:
+            lib().mesh_weight_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------------------------------------- gguf
+def gguf_probe(path):
+    info = ModelInfo()
+    check(lib().mesh_gguf_probe(os.fsencode(path), ctypes.byref(info)))
+    return info
+
+
+def gguf_tensor(path, name):
+    info = TensorInfo()
+    check(lib().mesh_gguf_tensor(os.fsencode(path), name.encode(), ctypes.byref(info)))
+    return info
+
+
+# ---------------------------------------------------------------------------------------------- stage
+class Stage:
+    """Layers [layer_begin, layer_end) of a GGUF model resident on the GPU (mesh_stage)."""
+
+    def __init__(self, gguf_path, layer_begin, layer_end=-1, n_ctx=0, n_seq_max=0, n_batch_max=0, device=None):
+        opts = StageOpts(device.encode() if device else None, n_ctx, n_seq_max, n_batch_max, 0)
+        self._h = ctypes.c_void_p()
+        check(lib().mesh_stage_open(os.fsencode(gguf_path), layer_begin, layer_end, ctypes.byref(opts), ctypes.byref(self._h)))
+        self.info = ModelInfo()
+        check(lib().mesh_stage_info(self._h, ctypes.byref(self.info)))
+
+    @property
+    def weight_bytes(self):
+        return int(lib().mesh_stage_weight_bytes(self._h))
+
+    def session(self):
+        return Session(self)
+
+    def close(self):
+        if self._h:
+            lib().mesh_stage_close(self._h)
+            self._h = ctypes.c_void_p()
+
+
+class Session:
+    """KV cache + activation buffers of one set of sequences (mesh_session).  Single-threaded."""
+
+    def __init__(self, stage):
+        self.stage = stage
+        self._h = ctypes.c_void_p()
+        check(lib().mesh_stage_session_new(stage._h, ctypes.byref(self._h)))
+
+    @staticmethod
+    def _batch(pos, seq):
+        import numpy as np
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        seq = np.zeros_like(pos) if seq is None else np.ascontiguousarray(seq, dtype=np.int32)
+        b = Batch(pos.size, pos.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), seq.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+        return b, (pos, seq)
+
+    def decode(self, inp, pos, seq=None, in_fmt=F32, out_fmt=F32):
+        """Host form.  inp: numpy array holding the packed input (f32 rows, f16 bits, q8_0 bytes or int32 ids)."""
+        import numpy as np
+        b, keep = self._batch(pos, seq)
+        inp = np.ascontiguousarray(inp)
+        T = b.n_tokens
+        if out_fmt == LOGITS:
+            cap = T * max(self.stage.info.n_vocab, 1) * 4 + 16
+            cap = max(cap, 1 << 20)
+        else:
+            cap = T * self.stage.info.n_embd * 4
+        out = np.empty(cap, dtype=np.uint8)
+        n = ctypes.c_size_t(0)
+        rc = lib().mesh_stage_decode(self._h, ctypes.byref(b), _np_ptr(inp), in_fmt, _np_ptr(out), out_fmt, cap, ctypes.byref(n))
+        if rc == ERR_INVALID and out_fmt == LOGITS and n.value > cap:
+            cap = n.value
+            out = np.empty(cap, dtype=np.uint8)
+            rc = lib().mesh_stage_decode(self._h, ctypes.byref(b), _np_ptr(inp), in_fmt, _np_ptr(out), out_fmt, cap, ctypes.byref(n))
+        check(rc)
+        return out[:n.value]
+
+    def decode_dev(self, d_in, pos, d_out, out_cap, seq=None, in_fmt=F32, out_fmt=F32):
+        b, keep = self._batch(pos, seq)
+        n = ctypes.c_size_t(0)
+        check(lib().mesh_stage_decode_dev(self._h, ctypes.byref(b), d_in, in_fmt, d_out, out_fmt, out_cap, ctypes.byref(n)))
+        return n.value
+
+    @property
+    def stream(self):
+        return lib().mesh_session_stream(self._h) or 0
+
+    def synchronize(self):
+        check(lib().mesh_session_synchronize(self._h))
+
+    def kv_write(self, layer, seq_id, pos0, k, v):
+        """k, v: uint16 arrays [n_pos, n_head_kv, head_dim] of f16 bits."""
+        import numpy as np
+        k = np.ascontiguousarray(k, dtype=np.uint16)
+        v = np.ascontiguousarray(v, dtype=np.uint16)
+        check(lib().mesh_session_kv_write(self._h, layer, seq_id, pos0, k.shape[0], _np_ptr(k), _np_ptr(v)))
+
+    def kv_read(self, layer, seq_id, pos0, n_pos):
+        import numpy as np
+        i = self.stage.info
+        k = np.empty((n_pos, i.n_head_kv, i.head_dim), dtype=np.uint16)
+        v = np.empty_like(k)
+        check(lib().mesh_session_kv_read(self._h, layer, seq_id, pos0, n_pos, _np_ptr(k), _np_ptr(v)))
+        return k, v
+
+    def close(self):
+        if self._h:
+            lib().mesh_stage_session_free(self._h)
+            self._h = ctypes.c_void_p()

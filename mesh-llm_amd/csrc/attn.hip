@@ -1,0 +1,225 @@
+// RoPE + KV append, and GQA attention over the stage-local f16 KV cache (split-KV, online softmax).
+// Stands where the worker's graph runs rope -> kv store -> flash_attn_ext (-fa on, mesh-llm/src/inference/launch.rs:1350-1353;
+// f16 cache is the small-model tier of KvCacheQuant::for_model_size, launch.rs:568-591).
+//
+// Cache layout per layer: K and V as f16 [n_seq][n_head_kv][n_ctx][head_dim]; one (sequence, kv head) is a
+// contiguous run so a workgroup streams its key range linearly.  The `group` query heads that share a kv head
+// are processed together, so each K/V byte is read once per token.
+
+#include "attn.hpp"
+
+namespace mesh {
+
+// ------------------------------------------------------------------------------------------------ rope + append
+// grid (n_head + 2*n_head_kv, T), one wave per head vector.
+__global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvArgs a) {
+    const int hh = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    const int hd = a.head_dim;
+    const int pos = a.pos[t], seq = a.seq[t];
+    float *vec;
+    const float *nw = nullptr;
+    int kind, head;
+    if (hh < a.n_head) { kind = 0; head = hh; vec = a.q + ((size_t)t * a.n_head + head) * hd; nw = a.q_norm; }
+    else if (hh < a.n_head + a.n_kv) { kind = 1; head = hh - a.n_head; vec = const_cast<float *>(a.k) + ((size_t)t * a.n_kv + head) * hd; nw = a.k_norm; }
+    else { kind = 2; head = hh - a.n_head - a.n_kv; vec = const_cast<float *>(a.v) + ((size_t)t * a.n_kv + head) * hd; }
+
+    uint16_t *cache = nullptr;
+    if (kind) cache = (kind == 1 ? a.kcache : a.vcache) + (((size_t)seq * a.n_kv + head) * a.n_ctx + pos) * hd;
+
+    if (kind == 2) {
+        for (int i = lane; i < hd; i += 64) cache[i] = f32_to_f16_bits(vec[i]);
+        return;
+    }
+    // optional per-head RMS norm (qwen3: attn_q_norm / attn_k_norm over head_dim)
+    float nscale = 1.0f;
+    if (nw) {
+        float ss = 0.f;
+        for (int i = lane; i < hd; i += 64) ss += vec[i] * vec[i];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        nscale = 1.0f / sqrtf(ss / (float)hd + a.eps);
+    }
+    const int half = a.n_rot / 2;
+    for (int i = lane; i < half; i += 64) {
+        const int ia = a.rope_mode == ROPE_MODE_NEOX ? i : 2 * i;
+        const int ib = a.rope_mode == ROPE_MODE_NEOX ? i + half : 2 * i + 1;
+        float x0 = vec[ia], x1 = vec[ib];
+        if (nw) { x0 = x0 * nscale * nw[ia]; x1 = x1 * nscale * nw[ib]; }
+        float sn, cs;
+        sincosf((float)pos * a.inv_freq[i], &sn, &cs);
+        const float o0 = x0 * cs - x1 * sn;
+        const float o1 = x0 * sn + x1 * cs;
+        if (kind == 0) { vec[ia] = o0; vec[ib] = o1; }
+        else { cache[ia] = f32_to_f16_bits(o0); cache[ib] = f32_to_f16_bits(o1); }
+    }
+    // dimensions beyond n_rot are not rotated
+    for (int e = a.n_rot + lane; e < hd; e += 64) {
+        float x0 = vec[e];
+        if (nw) x0 = x0 * nscale * nw[e];
+        if (kind == 0) vec[e] = x0;
+        else cache[e] = f32_to_f16_bits(x0);
+    }
+}
+
+int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (a.head_dim % 2 || a.n_rot % 2 || a.n_rot > a.head_dim) return fail(MESH_ERR_INVALID, "rope: bad head_dim/n_rot %d/%d", a.head_dim, a.n_rot);
+    rope_kv_kernel<<<dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream>>>(a);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ attention
+constexpr int ATTN_THREADS = 256;
+
+__device__ __forceinline__ void load8h(const uint16_t *p, float (&o)[8]) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(p);
+    o[0] = f16_bits_to_f32((uint16_t)(v.x & 0xFFFF)); o[1] = f16_bits_to_f32((uint16_t)(v.x >> 16));
+    o[2] = f16_bits_to_f32((uint16_t)(v.y & 0xFFFF)); o[3] = f16_bits_to_f32((uint16_t)(v.y >> 16));
+    o[4] = f16_bits_to_f32((uint16_t)(v.z & 0xFFFF)); o[5] = f16_bits_to_f32((uint16_t)(v.z >> 16));
+    o[6] = f16_bits_to_f32((uint16_t)(v.w & 0xFFFF)); o[7] = f16_bits_to_f32((uint16_t)(v.w >> 16));
+}
+
+// grid (n_splits, n_kv * (group/G), T).  HD/8 lanes share one key; each thread keeps a private online-softmax
+// state (m, l, acc[8]) per query head over the keys its slot visits; slots are merged through LDS.
+template <int HD, int G>
+__global__ __launch_bounds__(ATTN_THREADS) void attn_split_kernel(AttnArgs a) {
+    constexpr int LPK = HD / 8;                 // lanes per key
+    constexpr int SLOTS = ATTN_THREADS / LPK;   // keys in flight per pass
+    __shared__ float s_m[SLOTS][G], s_l[SLOTS][G];
+    __shared__ float s_acc[ATTN_THREADS / 64][G][HD];   // per-wave sums of the slot states
+
+    const int split = blockIdx.x, t = blockIdx.z;
+    const int hgroups = a.group / G;            // G divides group (G == group, or G == 1)
+    const int kvh = blockIdx.y / hgroups;
+    const int h0 = kvh * a.group + (blockIdx.y % hgroups) * G;   // first query head of this workgroup
+    const int tid = threadIdx.x, slot = tid / LPK, ds = (tid % LPK) * 8;
+    const int seq = a.seq[t];
+    const int n_keys = a.pos[t] + 1;
+    const int per = (n_keys + a.n_splits - 1) / a.n_splits;
+    const int j0 = split * per;
+    const int j1 = j0 + per < n_keys ? j0 + per : n_keys;
+
+    float q[G][8], acc[G][8], m[G], l[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        const float *qp = a.q + ((size_t)t * a.n_head + h0 + h) * HD + ds;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { q[h][i] = qp[i] * a.scale; acc[h][i] = 0.f; }
+        m[h] = -INFINITY;
+        l[h] = 0.f;
+    }
+    const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
+    for (int j = j0 + slot; j < j1; j += SLOTS) {
+        float kf[8], vf[8];
+        load8h(a.kcache + (base + j) * HD + ds, kf);
+        load8h(a.vcache + (base + j) * HD + ds, vf);
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s = fmaf(q[h][i], kf[i], s);
+#pragma unroll
+            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            const float mn = fmaxf(m[h], s);
+            const float corr = expf(m[h] - mn);     // exp(-inf) = 0 on the first key
+            const float p = expf(s - mn);
+            l[h] = l[h] * corr + p;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, vf[i], acc[h][i] * corr);
+            m[h] = mn;
+        }
+    }
+    // merge the slots
+    if ((tid % LPK) == 0) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) { s_m[slot][h] = m[h]; s_l[slot][h] = l[h]; }
+    }
+    __syncthreads();
+    const int wave = tid >> 6;
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        float mm = -INFINITY;
+        for (int s2 = 0; s2 < SLOTS; ++s2) mm = fmaxf(mm, s_m[s2][h]);
+        const float w = (m[h] == -INFINITY) ? 0.f : expf(m[h] - mm);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float v = acc[h][i] * w;
+            // add up the slots that live in this wave (lanes with equal tid % LPK)
+#pragma unroll
+            for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o);
+            if ((tid & 63) < LPK) s_acc[wave][h][ds + i] = v;
+        }
+    }
+    __syncthreads();
+    for (int o = tid; o < G * HD; o += ATTN_THREADS) {
+        const int h = o / HD, dd = o % HD;
+        float sum = 0.f;
+        for (int w2 = 0; w2 < ATTN_THREADS / 64; ++w2) sum += s_acc[w2][h][dd];
+        a.part[(((size_t)t * a.n_head + h0 + h) * a.n_splits + split) * HD + dd] = sum;
+    }
+    if (tid < G) {
+        const int h = tid;
+        float mm = -INFINITY;
+        for (int s2 = 0; s2 < SLOTS; ++s2) mm = fmaxf(mm, s_m[s2][h]);
+        float ll = 0.f;
+        for (int s2 = 0; s2 < SLOTS; ++s2) ll += (s_m[s2][h] == -INFINITY) ? 0.f : s_l[s2][h] * expf(s_m[s2][h] - mm);
+        float *ml = a.ml + (((size_t)t * a.n_head + h0 + h) * a.n_splits + split) * 2;
+        ml[0] = mm;
+        ml[1] = ll;
+    }
+}
+
+// grid (n_head, T), block head_dim threads
+__global__ void attn_combine_kernel(AttnArgs a) {
+    const int h = blockIdx.x, t = blockIdx.y, dd = threadIdx.x;
+    const size_t row = (size_t)t * a.n_head + h;
+    const float *ml = a.ml + row * a.n_splits * 2;
+    float mm = -INFINITY;
+    for (int s = 0; s < a.n_splits; ++s) mm = fmaxf(mm, ml[2 * s]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < a.n_splits; ++s) {
+        const float ms = ml[2 * s];
+        if (ms == -INFINITY) continue;
+        const float w = expf(ms - mm);
+        num = fmaf(a.part[(row * a.n_splits + s) * a.head_dim + dd], w, num);
+        den = fmaf(ml[2 * s + 1], w, den);
+    }
+    a.out[row * a.head_dim + dd] = num / den;
+}
+
+template <int HD>
+static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
+    const dim3 block(ATTN_THREADS);
+#define MESH_ATTN_CASE(GG)                                                                          \
+    if (a.group == GG) {                                                                            \
+        attn_split_kernel<HD, GG><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
+        MESH_LAUNCH_CHECK();                                                                        \
+        return MESH_OK;                                                                             \
+    }
+    MESH_ATTN_CASE(1)
+    MESH_ATTN_CASE(2)
+    MESH_ATTN_CASE(4)
+    if (HD == 128) { MESH_ATTN_CASE(5) MESH_ATTN_CASE(8) }
+    if (HD == 64) { MESH_ATTN_CASE(7) }
+#undef MESH_ATTN_CASE
+    // any other group size: one query head per workgroup (K/V re-read per head)
+    attn_split_kernel<HD, 1><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+int attention(const AttnArgs &a, int T, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (a.n_splits < 1 || a.group < 1 || a.n_head != a.group * a.n_kv) return fail(MESH_ERR_INVALID, "attention: bad head layout");
+    int rc;
+    if (a.head_dim == 128) rc = launch_attn<128>(a, T, stream);
+    else if (a.head_dim == 64) rc = launch_attn<64>(a, T, stream);
+    else return fail(MESH_ERR_UNSUPPORTED, "attention: head_dim %d has no kernel (64 and 128 do)", a.head_dim);
+    if (rc != MESH_OK) return rc;
+    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+}  // namespace mesh

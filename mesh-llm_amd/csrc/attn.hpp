@@ -1,0 +1,39 @@
+// RoPE + KV append and GQA attention launchers (attn.hip).
+#pragma once
+
+#include "mesh_common.hpp"
+
+namespace mesh {
+
+constexpr int ROPE_MODE_NORM = 0, ROPE_MODE_NEOX = 2;
+
+struct RopeKvArgs {
+    float *q = nullptr;            // [T][n_head][head_dim], rotated in place
+    const float *k = nullptr;      // [T][n_kv][head_dim]
+    const float *v = nullptr;
+    uint16_t *kcache = nullptr;    // this layer's K: [n_seq][n_kv][n_ctx][head_dim] f16
+    uint16_t *vcache = nullptr;
+    const int32_t *pos = nullptr;  // device, [T]
+    const int32_t *seq = nullptr;  // device, [T]
+    const float *inv_freq = nullptr;   // device, [n_rot/2]
+    const float *q_norm = nullptr; // optional per-head RMS norm weights [head_dim]
+    const float *k_norm = nullptr;
+    float eps = 0.f;
+    int n_head = 0, n_kv = 0, head_dim = 0, n_rot = 0, rope_mode = ROPE_MODE_NORM, n_ctx = 0;
+};
+int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream);
+
+struct AttnArgs {
+    const float *q = nullptr;      // [T][n_head][head_dim]
+    const uint16_t *kcache = nullptr, *vcache = nullptr;
+    const int32_t *pos = nullptr, *seq = nullptr;
+    float *part = nullptr;         // [T][n_head][n_splits][head_dim]
+    float *ml = nullptr;           // [T][n_head][n_splits][2]
+    float *out = nullptr;          // [T][n_head][head_dim]
+    float scale = 1.f;
+    int n_head = 0, n_kv = 0, group = 1, head_dim = 0, n_ctx = 0, n_splits = 1;
+};
+// token t attends to cache positions [0, pos[t]] of sequence seq[t]
+int attention(const AttnArgs &a, int T, hipStream_t stream);
+
+}  // namespace mesh

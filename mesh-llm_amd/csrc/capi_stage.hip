@@ -1,0 +1,196 @@
+// extern "C" entry points for weights, GGUF inspection and the stage executor (include/mesh_stage.h).
+
+#include <cstring>
+#include <vector>
+
+#include "gemv.hpp"
+#include "stage.hpp"
+
+struct mesh_weight {
+    mesh::DevTensor t;
+    size_t gguf_bytes = 0;
+};
+
+using namespace mesh;
+
+extern "C" {
+
+int mesh_weight_upload(int type, const void *host_data, int64_t n_rows, int64_t row_len, mesh_weight **out) {
+    if (!host_data || !out || n_rows <= 0 || row_len <= 0) return fail(MESH_ERR_INVALID, "mesh_weight_upload: null pointer or empty shape");
+    *out = nullptr;
+    const int64_t rb = row_bytes(type, row_len);
+    if (rb < 0) return fail(block_elems(type) < 0 ? MESH_ERR_UNSUPPORTED : MESH_ERR_INVALID,
+                            "mesh_weight_upload: row length %lld is not a whole number of type-%d blocks", (long long)row_len, type);
+    mesh_weight *w = new mesh_weight();
+    w->t.type = type; w->t.K = row_len; w->t.M = n_rows; w->t.E = 1;
+    w->gguf_bytes = (size_t)(rb * n_rows);
+    w->t.tiled = type_is_tiled(type);
+    w->t.bytes = w->t.tiled ? (size_t)tiled_bytes(type, n_rows, row_len) : w->gguf_bytes;
+    hipError_t e = hipMalloc(&w->t.data, w->t.bytes);
+    if (e != hipSuccess) { delete w; return fail(MESH_ERR_NOMEM, "mesh_weight_upload: hipMalloc(%zu) failed: %s", w->t.bytes, hipGetErrorString(e)); }
+    int rc = MESH_OK;
+    if (!w->t.tiled) {
+        e = hipMemcpy(w->t.data, host_data, w->gguf_bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) rc = fail(MESH_ERR_DEVICE, "mesh_weight_upload: copy failed: %s", hipGetErrorString(e));
+    } else {
+        void *tmp = nullptr;
+        e = hipMalloc(&tmp, w->gguf_bytes);
+        if (e != hipSuccess) rc = fail(MESH_ERR_NOMEM, "mesh_weight_upload: hipMalloc(%zu) failed", w->gguf_bytes);
+        if (rc == MESH_OK && (e = hipMemcpy(tmp, host_data, w->gguf_bytes, hipMemcpyHostToDevice)) != hipSuccess)
+            rc = fail(MESH_ERR_DEVICE, "mesh_weight_upload: copy failed: %s", hipGetErrorString(e));
+        if (rc == MESH_OK) rc = repack_tiled(type, tmp, w->t.data, n_rows, row_len, nullptr);
+        if (rc == MESH_OK && (e = hipDeviceSynchronize()) != hipSuccess)
+            rc = fail(MESH_ERR_DEVICE, "mesh_weight_upload: repack failed: %s", hipGetErrorString(e));
+        if (tmp) (void)hipFree(tmp);
+    }
+    if (rc != MESH_OK) { (void)hipFree(w->t.data); delete w; return rc; }
+    *out = w;
+    return MESH_OK;
+}
+
+void mesh_weight_free(mesh_weight *w) {
+    if (!w) return;
+    if (w->t.data) (void)hipFree(w->t.data);
+    delete w;
+}
+
+size_t mesh_weight_nbytes(const mesh_weight *w) { return w ? w->gguf_bytes : 0; }
+
+int mesh_weight_download(const mesh_weight *w, void *host_data) {
+    if (!w || !host_data) return fail(MESH_ERR_INVALID, "mesh_weight_download: null argument");
+    if (!w->t.tiled) {
+        MESH_HIP_TRY(hipMemcpy(host_data, w->t.data, w->gguf_bytes, hipMemcpyDeviceToHost));
+        return MESH_OK;
+    }
+    void *tmp = nullptr;
+    MESH_HIP_TRY(hipMalloc(&tmp, w->gguf_bytes));
+    int rc = unpack_tiled(w->t.type, w->t.data, tmp, w->t.M, w->t.K, nullptr);
+    if (rc == MESH_OK && hipMemcpy(host_data, tmp, w->gguf_bytes, hipMemcpyDeviceToHost) != hipSuccess)
+        rc = fail(MESH_ERR_DEVICE, "mesh_weight_download: copy failed");
+    (void)hipFree(tmp);
+    return rc;
+}
+
+int mesh_mul_mat_dev(const mesh_weight *w, const float *d_x, int64_t n_tokens, float *d_y, void *stream) {
+    if (!w || !d_x || !d_y || n_tokens < 0) return fail(MESH_ERR_INVALID, "mesh_mul_mat_dev: null argument");
+    if (n_tokens == 0) return MESH_OK;
+    GemvArgs a;
+    a.n_mat = 1;
+    a.mat[0].W = w->t.data; a.mat[0].type = w->t.type; a.mat[0].M = (int)w->t.M; a.mat[0].y = d_y; a.mat[0].ldy = (int)w->t.M;
+    a.x = d_x; a.ldx = (int)w->t.K; a.K = (int)w->t.K; a.T = (int)n_tokens;
+    return gemv(a, static_cast<hipStream_t>(stream));
+}
+
+static void fill_info(const HParams &hp, mesh_model_info *o) {
+    memset(o, 0, sizeof *o);
+    strncpy(o->arch, hp.arch.c_str(), sizeof(o->arch) - 1);
+    o->n_layer = hp.n_layer; o->n_embd = hp.n_embd; o->n_head = hp.n_head; o->n_head_kv = hp.n_head_kv;
+    o->head_dim = hp.head_dim; o->n_ff = hp.n_ff; o->n_vocab = hp.n_vocab; o->n_rot = hp.n_rot; o->rope_mode = hp.rope_mode;
+    o->n_expert = hp.n_expert; o->n_expert_used = hp.n_expert_used; o->n_ff_exp = hp.n_ff_exp;
+    o->rms_eps = hp.rms_eps; o->rope_freq_base = hp.rope_freq_base;
+}
+
+int mesh_gguf_probe(const char *gguf_path, mesh_model_info *out) {
+    if (!out) return fail(MESH_ERR_INVALID, "mesh_gguf_probe: null output");
+    GgufFile g;
+    int rc = g.open(gguf_path);
+    if (rc != MESH_OK) return rc;
+    HParams hp;
+    if ((rc = hparams_from_gguf(g, hp)) != MESH_OK) return rc;
+    fill_info(hp, out);
+    out->gguf_version = g.version(); out->alignment = g.alignment();
+    out->n_tensors = g.tensors().size(); out->data_offset = g.data_offset(); out->file_size = g.file_size();
+    return MESH_OK;
+}
+
+int mesh_gguf_tensor(const char *gguf_path, const char *name, mesh_tensor_info *out) {
+    if (!name || !out) return fail(MESH_ERR_INVALID, "mesh_gguf_tensor: null argument");
+    GgufFile g;
+    int rc = g.open(gguf_path);
+    if (rc != MESH_OK) return rc;
+    const GgufTensorInfo *t = g.find(name);
+    if (!t) return fail(MESH_ERR_INVALID, "mesh_gguf_tensor: tensor '%s' not found", name);
+    memset(out, 0, sizeof *out);
+    out->type = t->type; out->n_dims = t->n_dims;
+    for (int i = 0; i < 4; ++i) out->ne[i] = t->ne[i];
+    out->file_offset = g.data_offset() + t->offset;
+    out->nbytes = t->nbytes;
+    if (t->nbytes == 0) return fail(MESH_ERR_UNSUPPORTED, "mesh_gguf_tensor: tensor '%s' has ggml type %u, unknown to this build", name, t->type);
+    if (!g.data(*t)) return fail(MESH_ERR_FORMAT, "mesh_gguf_tensor: tensor '%s' (%llu bytes at %llu) lies outside the file", name,
+                                 (unsigned long long)t->nbytes, (unsigned long long)out->file_offset);
+    return MESH_OK;
+}
+
+int mesh_stage_open(const char *gguf_path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out) {
+    return stage_open(gguf_path, layer_begin, layer_end, opts, out);
+}
+
+void mesh_stage_close(mesh_stage *stage) { delete stage; }
+
+int mesh_stage_info(const mesh_stage *stage, mesh_model_info *out) {
+    if (!stage || !out) return fail(MESH_ERR_INVALID, "mesh_stage_info: null argument");
+    fill_info(stage->hp, out);
+    return MESH_OK;
+}
+
+size_t mesh_stage_weight_bytes(const mesh_stage *stage) { return stage ? stage->weight_bytes : 0; }
+
+int mesh_stage_session_new(mesh_stage *stage, mesh_session **out) { return session_new(stage, out); }
+
+void mesh_stage_session_free(mesh_session *session) { delete session; }
+
+int mesh_stage_decode(mesh_session *session, const mesh_batch *batch, const void *in, int in_fmt, void *out, int out_fmt,
+                      size_t out_cap, size_t *out_len) {
+    return stage_decode(session, batch, in, in_fmt, out, out_fmt, out_cap, out_len);
+}
+
+int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const void *d_in, int in_fmt, void *d_out,
+                          int out_fmt, size_t out_cap, size_t *out_len) {
+    return stage_decode_dev(session, batch, d_in, in_fmt, d_out, out_fmt, out_cap, out_len);
+}
+
+void *mesh_session_stream(mesh_session *session) { return session ? static_cast<void *>(session->stream) : nullptr; }
+
+int mesh_session_synchronize(mesh_session *session) {
+    if (!session) return fail(MESH_ERR_INVALID, "mesh_session_synchronize: null session");
+    MESH_HIP_TRY(hipStreamSynchronize(session->stream));
+    return MESH_OK;
+}
+
+static int kv_xfer(mesh_session *s, int layer, int seq_id, int pos0, int n_pos, uint16_t *k, uint16_t *v, bool write) {
+    if (!s || !k || !v) return fail(MESH_ERR_INVALID, "mesh_session_kv: null argument");
+    const mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    if (layer < st->layer_begin || layer >= st->layer_end) return fail(MESH_ERR_INVALID, "mesh_session_kv: layer %d not in this stage [%d,%d)", layer, st->layer_begin, st->layer_end);
+    if (seq_id < 0 || seq_id >= st->n_seq_max || pos0 < 0 || n_pos <= 0 || pos0 + n_pos > st->n_ctx)
+        return fail(MESH_ERR_INVALID, "mesh_session_kv: sequence %d positions [%d,%d) outside the cache", seq_id, pos0, pos0 + n_pos);
+    MESH_HIP_TRY(hipSetDevice(st->device));
+    MESH_HIP_TRY(hipStreamSynchronize(s->stream));
+    const size_t hd = hp.head_dim, nkv = hp.n_head_kv;
+    std::vector<uint16_t> tmp((size_t)n_pos * hd);
+    for (int which = 0; which < 2; ++which) {
+        uint16_t *cache = (which ? s->vcache : s->kcache) + (size_t)(layer - st->layer_begin) * s->kv_layer_elems;
+        uint16_t *host = which ? v : k;
+        for (size_t h = 0; h < nkv; ++h) {
+            uint16_t *dev = cache + (((size_t)seq_id * nkv + h) * (size_t)st->n_ctx + (size_t)pos0) * hd;
+            if (write) {
+                for (int p = 0; p < n_pos; ++p) memcpy(&tmp[(size_t)p * hd], host + ((size_t)p * nkv + h) * hd, hd * 2);
+                MESH_HIP_TRY(hipMemcpy(dev, tmp.data(), tmp.size() * 2, hipMemcpyHostToDevice));
+            } else {
+                MESH_HIP_TRY(hipMemcpy(tmp.data(), dev, tmp.size() * 2, hipMemcpyDeviceToHost));
+                for (int p = 0; p < n_pos; ++p) memcpy(host + ((size_t)p * nkv + h) * hd, &tmp[(size_t)p * hd], hd * 2);
+            }
+        }
+    }
+    return MESH_OK;
+}
+
+int mesh_session_kv_write(mesh_session *session, int layer, int seq_id, int pos0, int n_pos, const uint16_t *k, const uint16_t *v) {
+    return kv_xfer(session, layer, seq_id, pos0, n_pos, const_cast<uint16_t *>(k), const_cast<uint16_t *>(v), true);
+}
+
+int mesh_session_kv_read(mesh_session *session, int layer, int seq_id, int pos0, int n_pos, uint16_t *k, uint16_t *v) {
+    return kv_xfer(session, layer, seq_id, pos0, n_pos, k, v, false);
+}
+
+}  // extern "C"

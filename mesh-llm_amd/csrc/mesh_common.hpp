@@ -39,6 +39,15 @@ constexpr int QK8_0 = 32, Q8_0_BYTES = 34;
 constexpr int QK5_0 = 32, Q5_0_BYTES = 22;
 constexpr int QK_K = 256, Q4_K_BYTES = 144, Q6_K_BYTES = 210;
 
+// device-side twins (int math)
+__host__ __device__ inline int block_elems_dev(int type) {
+    return (type == MESH_F32 || type == MESH_F16) ? 1 : (type == MESH_Q5_0 || type == MESH_Q8_0) ? 32 : 256;
+}
+__host__ __device__ inline int block_bytes_dev(int type) {
+    return type == MESH_F32 ? 4 : type == MESH_F16 ? 2 : type == MESH_Q5_0 ? Q5_0_BYTES : type == MESH_Q8_0 ? Q8_0_BYTES
+         : type == MESH_Q4_K ? Q4_K_BYTES : Q6_K_BYTES;
+}
+
 inline int64_t block_elems(int type) {
     switch (type) {
         case MESH_F32: case MESH_F16: return 1;

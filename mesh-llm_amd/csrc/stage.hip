@@ -1,0 +1,486 @@
+// The pipeline-stage executor: loads layers [begin, end) of a GGUF model into HBM and runs them over a batch of
+// token activations, keeping a stage-local f16 KV cache per session.
+//
+// It does, in one process and on one GPU, what a mesh-llm worker does today through llama.cpp RPC:
+//   * weight load by tensor name from the local GGUF  -- rpc_server::set_tensor_gguf,
+//     third_party/llama.cpp/patches/0001-rpc-optimize-local-GGUF-tensor-loading.patch:179-266
+//   * the per-layer graph  rms_norm -> q,k,v -> rope -> kv store -> attention -> o (+residual) -> rms_norm ->
+//     gate,up -> silu*mul -> down (+residual)  -- rpc_server::graph_compute, patches/0002-...:443-451
+//   * boundary hand-off of the hidden state -- push_tensor_to_peer, patches/0002-...:544-622 (packed here).
+
+#include "stage.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "attn.hpp"
+#include "gemv.hpp"
+
+namespace mesh {
+
+int act_pack_dev(int fmt, const float *src, void *dst, int64_t n, hipStream_t stream);
+int act_unpack_dev(int fmt, const void *src, float *dst, int64_t n, hipStream_t stream);
+int dequantize_dev(int type, const void *src, float *dst, int64_t n, hipStream_t stream);
+
+// ------------------------------------------------------------------------------------------------ hparams
+int hparams_from_gguf(const GgufFile &g, HParams &hp) {
+    if (!g.get_str("general.architecture", hp.arch)) return fail(MESH_ERR_FORMAT, "gguf: general.architecture missing");
+    const std::string &a = hp.arch;
+    if (a != "llama" && a != "qwen2" && a != "qwen3" && a != "qwen3moe")
+        return fail(MESH_ERR_UNSUPPORTED, "architecture '%s' is not supported (llama, qwen2, qwen3, qwen3moe are)", a.c_str());
+    auto need = [&](const char *suffix, uint32_t &out) -> int {
+        if (!g.get_u32(a + suffix, out)) return fail(MESH_ERR_FORMAT, "gguf: key %s%s missing or not an unsigned integer", a.c_str(), suffix);
+        return MESH_OK;
+    };
+    int rc;
+    if ((rc = need(".block_count", hp.n_layer)) || (rc = need(".embedding_length", hp.n_embd)) ||
+        (rc = need(".attention.head_count", hp.n_head)))
+        return rc;
+    hp.n_head_kv = hp.n_head;
+    g.get_u32(a + ".attention.head_count_kv", hp.n_head_kv);
+    g.get_u32(a + ".feed_forward_length", hp.n_ff);
+    g.get_u32(a + ".vocab_size", hp.n_vocab);
+    if (hp.n_head == 0 || hp.n_head_kv == 0 || hp.n_head % hp.n_head_kv) return fail(MESH_ERR_FORMAT, "gguf: head counts %u/%u inconsistent", hp.n_head, hp.n_head_kv);
+    hp.head_dim = hp.n_embd / hp.n_head;
+    g.get_u32(a + ".attention.key_length", hp.head_dim);
+    hp.n_rot = hp.head_dim;
+    g.get_u32(a + ".rope.dimension_count", hp.n_rot);
+    g.get_f32(a + ".attention.layer_norm_rms_epsilon", hp.rms_eps);
+    g.get_f32(a + ".rope.freq_base", hp.rope_freq_base);
+    g.get_u32(a + ".expert_count", hp.n_expert);
+    g.get_u32(a + ".expert_used_count", hp.n_expert_used);
+    g.get_u32(a + ".expert_feed_forward_length", hp.n_ff_exp);
+    hp.rope_mode = (a == "llama") ? ROPE_NORM : ROPE_NEOX;
+    if (hp.n_layer == 0 || hp.n_embd == 0 || hp.head_dim == 0) return fail(MESH_ERR_FORMAT, "gguf: zero-sized model dimensions");
+    if (hp.n_rot > hp.head_dim || hp.n_rot % 2) return fail(MESH_ERR_FORMAT, "gguf: rope dimension count %u does not fit head_dim %u", hp.n_rot, hp.head_dim);
+    if (a == "qwen3moe" && (hp.n_expert == 0 || hp.n_expert_used == 0 || hp.n_expert_used > hp.n_expert))
+        return fail(MESH_ERR_FORMAT, "gguf: qwen3moe without a usable expert_count / expert_used_count");
+    return MESH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ loading
+namespace {
+
+struct Loader {
+    const GgufFile &g;
+    mesh_stage &st;
+    void *staging = nullptr;
+    size_t staging_bytes = 0;
+
+    ~Loader() { if (staging) (void)hipFree(staging); }
+
+    int dev_alloc(void **p, size_t bytes) {
+        hipError_t e = hipMalloc(p, bytes ? bytes : 16);
+        if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? MESH_ERR_NOMEM : MESH_ERR_DEVICE, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        st.allocations.push_back(*p);
+        return MESH_OK;
+    }
+
+    // Loads tensor `name` into `out`.  want_K / want_M < 0 skip that check.  required=false: absent is fine.
+    int load(const std::string &name, DevTensor &out, int64_t want_K, int64_t want_M, int64_t want_E, bool required,
+             bool tile, bool f32_only) {
+        const GgufTensorInfo *ti = g.find(name);
+        if (!ti) return required ? fail(MESH_ERR_FORMAT, "gguf: tensor '%s' not found", name.c_str()) : MESH_OK;
+        const int64_t K = (int64_t)ti->ne[0], M = (int64_t)ti->ne[1], E = (int64_t)ti->ne[2];
+        if (ti->ne[3] != 1 || (want_K >= 0 && K != want_K) || (want_M >= 0 && M != want_M) || (want_E >= 0 && E != want_E))
+            return fail(MESH_ERR_FORMAT, "gguf: tensor '%s' has shape [%lld,%lld,%lld], expected [%lld,%lld,%lld]", name.c_str(),
+                        (long long)K, (long long)M, (long long)E, (long long)want_K, (long long)want_M, (long long)want_E);
+        if (block_elems((int)ti->type) < 0)
+            return fail(MESH_ERR_UNSUPPORTED, "gguf: tensor '%s' has ggml type %u, which this build has no kernel for", name.c_str(), ti->type);
+        if (f32_only && ti->type != MESH_F32) return fail(MESH_ERR_UNSUPPORTED, "gguf: tensor '%s' must be F32 (is type %u)", name.c_str(), ti->type);
+        const uint8_t *src = g.data(*ti);
+        if (!src) return fail(MESH_ERR_FORMAT, "gguf: tensor '%s' (%llu bytes at offset %llu) lies outside the file", name.c_str(),
+                              (unsigned long long)ti->nbytes, (unsigned long long)ti->offset);
+        out.type = (int)ti->type;
+        out.K = K; out.M = M; out.E = E;
+        out.tiled = tile && type_is_tiled(out.type);
+        st.weight_bytes += ti->nbytes;
+        int rc;
+        if (!out.tiled) {
+            out.bytes = ti->nbytes;
+            if ((rc = dev_alloc(&out.data, out.bytes)) != MESH_OK) return rc;
+            MESH_HIP_TRY(hipMemcpy(out.data, src, out.bytes, hipMemcpyHostToDevice));
+            return MESH_OK;
+        }
+        const size_t per_e = (size_t)tiled_bytes(out.type, M, K);
+        const size_t src_per_e = (size_t)(M * row_bytes(out.type, K));
+        out.bytes = per_e * (size_t)E;
+        if ((rc = dev_alloc(&out.data, out.bytes)) != MESH_OK) return rc;
+        if (staging_bytes < ti->nbytes) {
+            if (staging) (void)hipFree(staging);
+            staging = nullptr;
+            hipError_t e = hipMalloc(&staging, ti->nbytes);
+            if (e != hipSuccess) { staging_bytes = 0; return fail(MESH_ERR_NOMEM, "hipMalloc(%llu) for load staging failed", (unsigned long long)ti->nbytes); }
+            staging_bytes = ti->nbytes;
+        }
+        MESH_HIP_TRY(hipMemcpy(staging, src, ti->nbytes, hipMemcpyHostToDevice));
+        for (int64_t e = 0; e < E; ++e) {
+            rc = repack_tiled(out.type, static_cast<const uint8_t *>(staging) + e * src_per_e,
+                              static_cast<uint8_t *>(out.data) + e * per_e, M, K, nullptr);
+            if (rc != MESH_OK) return rc;
+        }
+        MESH_HIP_TRY(hipDeviceSynchronize());
+        return MESH_OK;
+    }
+};
+
+}  // namespace
+
+int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out) {
+    if (!path || !out) return fail(MESH_ERR_INVALID, "mesh_stage_open: null argument");
+    *out = nullptr;
+    GgufFile g;
+    int rc = g.open(path);
+    if (rc != MESH_OK) return rc;
+    std::unique_ptr<mesh_stage> st(new mesh_stage());
+    if ((rc = hparams_from_gguf(g, st->hp)) != MESH_OK) return rc;
+    const HParams &hp = st->hp;
+    if (layer_end < 0) layer_end = (int)hp.n_layer;
+    if (layer_begin < 0 || layer_begin >= layer_end || layer_end > (int)hp.n_layer)
+        return fail(MESH_ERR_INVALID, "mesh_stage_open: layer range [%d,%d) does not fit a %u-layer model", layer_begin, layer_end, hp.n_layer);
+    st->layer_begin = layer_begin;
+    st->layer_end = layer_end;
+    st->n_ctx = opts && opts->n_ctx > 0 ? opts->n_ctx : 4096;
+    st->n_seq_max = opts && opts->n_seq_max > 0 ? opts->n_seq_max : 1;
+    st->n_batch_max = opts && opts->n_batch_max > 0 ? opts->n_batch_max : 512;
+    if (opts && opts->kv_type != 0 && opts->kv_type != MESH_F16)
+        return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: KV cache type %d not supported (f16 is)", opts->kv_type);
+    if (opts && opts->device && opts->device[0]) {
+        if ((rc = mesh_device_select(opts->device)) != MESH_OK) return rc;
+    }
+    if (mesh_device_count() < 1) return fail(MESH_ERR_DEVICE, "mesh_stage_open: no GPU available");
+    MESH_HIP_TRY(hipGetDevice(&st->device));
+    if (hp.head_dim != 64 && hp.head_dim != 128)
+        return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: head_dim %u has no attention kernel (64 and 128 do)", hp.head_dim);
+
+    Loader ld{g, *st};
+    const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, KD = (int64_t)hp.n_head_kv * hp.head_dim;
+    const bool moe = hp.arch == "qwen3moe";
+    st->layers.resize((size_t)(layer_end - layer_begin));
+    for (int il = layer_begin; il < layer_end; ++il) {
+        LayerWeights &L = st->layers[(size_t)(il - layer_begin)];
+        const std::string p = "blk." + std::to_string(il) + ".";
+        if ((rc = ld.load(p + "attn_norm.weight", L.attn_norm, E, 1, 1, true, false, true)) ||
+            (rc = ld.load(p + "attn_q.weight", L.wq, E, QD, 1, true, true, false)) ||
+            (rc = ld.load(p + "attn_k.weight", L.wk, E, KD, 1, true, true, false)) ||
+            (rc = ld.load(p + "attn_v.weight", L.wv, E, KD, 1, true, true, false)) ||
+            (rc = ld.load(p + "attn_output.weight", L.wo, QD, E, 1, true, true, false)) ||
+            (rc = ld.load(p + "attn_q.bias", L.bq, QD, 1, 1, false, false, true)) ||
+            (rc = ld.load(p + "attn_k.bias", L.bk, KD, 1, 1, false, false, true)) ||
+            (rc = ld.load(p + "attn_v.bias", L.bv, KD, 1, 1, false, false, true)) ||
+            (rc = ld.load(p + "attn_q_norm.weight", L.q_norm, hp.head_dim, 1, 1, false, false, true)) ||
+            (rc = ld.load(p + "attn_k_norm.weight", L.k_norm, hp.head_dim, 1, 1, false, false, true)) ||
+            (rc = ld.load(p + "ffn_norm.weight", L.ffn_norm, E, 1, 1, true, false, true)))
+            return rc;
+        if (!moe) {
+            if (hp.n_ff == 0) return fail(MESH_ERR_FORMAT, "gguf: feed_forward_length missing");
+            if ((rc = ld.load(p + "ffn_gate.weight", L.w_gate, E, hp.n_ff, 1, true, true, false)) ||
+                (rc = ld.load(p + "ffn_up.weight", L.w_up, E, hp.n_ff, 1, true, true, false)) ||
+                (rc = ld.load(p + "ffn_down.weight", L.w_down, hp.n_ff, E, 1, true, true, false)))
+                return rc;
+        } else {
+            const GgufTensorInfo *gi = g.find(p + "ffn_gate_inp.weight");
+            if (!gi) return fail(MESH_ERR_FORMAT, "gguf: tensor '%sffn_gate_inp.weight' not found", p.c_str());
+            const int64_t ne = (int64_t)gi->ne[1];     // experts present in this file (a shard has fewer than the model)
+            const int64_t ffe = hp.n_ff_exp;
+            if (ffe == 0) return fail(MESH_ERR_FORMAT, "gguf: expert_feed_forward_length missing");
+            if ((rc = ld.load(p + "ffn_gate_inp.weight", L.gate_inp, E, ne, 1, true, false, false)) ||
+                (rc = ld.load(p + "ffn_gate_exps.weight", L.gate_exps, E, ffe, ne, true, true, false)) ||
+                (rc = ld.load(p + "ffn_up_exps.weight", L.up_exps, E, ffe, ne, true, true, false)) ||
+                (rc = ld.load(p + "ffn_down_exps.weight", L.down_exps, ffe, E, ne, true, true, false)))
+                return rc;
+        }
+    }
+    if (layer_begin == 0) {
+        if ((rc = ld.load("token_embd.weight", st->tok_embd, E, -1, 1, false, false, false)) != MESH_OK) return rc;
+    }
+    if (layer_end == (int)hp.n_layer) {
+        if ((rc = ld.load("output_norm.weight", st->output_norm, E, 1, 1, false, false, true)) != MESH_OK) return rc;
+        if (g.find("output.weight")) {
+            if ((rc = ld.load("output.weight", st->output, E, -1, 1, true, true, false)) != MESH_OK) return rc;
+        } else if (st->output_norm.present() && g.find("token_embd.weight")) {
+            // tied embeddings: the output projection is token_embd
+            if ((rc = ld.load("token_embd.weight", st->output, E, -1, 1, true, true, false)) != MESH_OK) return rc;
+        }
+    }
+    // inverse frequencies by ggml's f32 recurrence: theta_i = theta_{i-1} * base^(-2/n_rot)
+    {
+        std::vector<float> inv(hp.n_rot / 2);
+        const float theta_scale = powf(hp.rope_freq_base, -2.0f / (float)hp.n_rot);
+        float th = 1.0f;
+        for (size_t i = 0; i < inv.size(); ++i) { inv[i] = th; th *= theta_scale; }
+        void *p = nullptr;
+        if ((rc = ld.dev_alloc(&p, inv.size() * sizeof(float))) != MESH_OK) return rc;
+        st->rope_inv_freq = static_cast<float *>(p);
+        MESH_HIP_TRY(hipMemcpy(p, inv.data(), inv.size() * sizeof(float), hipMemcpyHostToDevice));
+    }
+    MESH_HIP_TRY(hipDeviceSynchronize());
+    *out = st.release();
+    return MESH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ session
+static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
+    hipError_t e = hipMalloc(p, bytes ? bytes : 16);
+    if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? MESH_ERR_NOMEM : MESH_ERR_DEVICE, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    s->allocations.push_back(*p);
+    return MESH_OK;
+}
+
+constexpr int ATTN_SPLITS_MAX = 64;
+constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
+constexpr int META_SLOTS = 8;
+
+int session_new(mesh_stage *st, mesh_session **out) {
+    if (!st || !out) return fail(MESH_ERR_INVALID, "mesh_stage_session_new: null argument");
+    *out = nullptr;
+    MESH_HIP_TRY(hipSetDevice(st->device));
+    std::unique_ptr<mesh_session> s(new mesh_session());
+    s->stage = st;
+    const HParams &hp = st->hp;
+    const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
+    MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
+    s->kv_layer_elems = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx * hp.head_dim;
+    int rc;
+    void *p = nullptr;
+    if ((rc = sess_alloc(s.get(), &p, nl * s->kv_layer_elems * 2)) != MESH_OK) return rc;
+    s->kcache = static_cast<uint16_t *>(p);
+    if ((rc = sess_alloc(s.get(), &p, nl * s->kv_layer_elems * 2)) != MESH_OK) return rc;
+    s->vcache = static_cast<uint16_t *>(p);
+    MESH_HIP_TRY(hipMemsetAsync(s->kcache, 0, nl * s->kv_layer_elems * 2, s->stream));
+    MESH_HIP_TRY(hipMemsetAsync(s->vcache, 0, nl * s->kv_layer_elems * 2, s->stream));
+    const size_t QD = (size_t)hp.n_head * hp.head_dim, KD = (size_t)hp.n_head_kv * hp.head_dim;
+    const size_t ff = std::max<size_t>(hp.n_ff, (size_t)hp.n_ff_exp * std::max<uint32_t>(hp.n_expert_used, 1));
+    auto fbuf = [&](float **dst, size_t n) -> int {
+        void *q = nullptr;
+        int r = sess_alloc(s.get(), &q, n * sizeof(float));
+        *dst = static_cast<float *>(q);
+        return r;
+    };
+    const size_t part_rows = std::max<size_t>(B, ATTN_PART_ROWS_MIN);
+    if ((rc = fbuf(&s->x, B * hp.n_embd)) || (rc = fbuf(&s->q, B * QD)) || (rc = fbuf(&s->k, B * KD)) ||
+        (rc = fbuf(&s->v, B * KD)) || (rc = fbuf(&s->attn, B * QD)) || (rc = fbuf(&s->ffn, B * ff)) ||
+        (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
+        return rc;
+    if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
+    if ((rc = sess_alloc(s.get(), &p, 3 * B * sizeof(int32_t))) != MESH_OK) return rc;
+    s->d_pos = static_cast<int32_t *>(p);
+    s->d_seq = s->d_pos + B;
+    s->d_tok = s->d_seq + B;
+    MESH_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->h_meta), META_SLOTS * 3 * B * sizeof(int32_t), hipHostMallocDefault));
+    // staging for packed in/out of the host-pointer entry point: f32 rows of n_embd (or logits) are the largest
+    const size_t out_row = std::max<size_t>(hp.n_embd, st->output.present() ? (size_t)st->output.M : 0);
+    s->io_stage_bytes = B * out_row * sizeof(float);
+    if ((rc = sess_alloc(s.get(), &s->io_stage, 2 * s->io_stage_bytes)) != MESH_OK) return rc;
+    MESH_HIP_TRY(hipHostMalloc(&s->h_io, 2 * s->io_stage_bytes, hipHostMallocDefault));
+    MESH_HIP_TRY(hipStreamSynchronize(s->stream));
+    *out = s.release();
+    return MESH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ decode
+static GemvMat mat_of(const DevTensor &w, float *y, int ldy, const DevTensor *bias) {
+    GemvMat m;
+    m.W = w.data; m.type = w.type; m.M = (int)w.M; m.y = y; m.ldy = ldy;
+    m.bias = bias && bias->present() ? static_cast<const float *>(bias->data) : nullptr;
+    return m;
+}
+
+static int attn_splits_for(int T, int n_kv, int max_keys) {
+    int s = 512 / std::max(1, T * n_kv);
+    s = std::min(s, (max_keys + 63) / 64);
+    return std::max(1, std::min(s, ATTN_SPLITS_MAX));
+}
+
+// Runs the layers over the T token rows already in s->x.  pos/seq are on the device in s->d_pos / s->d_seq.
+static int run_layers(mesh_session *s, int T, int max_keys) {
+    mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    hipStream_t stream = s->stream;
+    const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim);
+    int rc;
+    for (size_t il = 0; il < st->layers.size(); ++il) {
+        const LayerWeights &L = st->layers[il];
+        // q, k, v = W{q,k,v} . rms_norm(x)
+        GemvArgs qa;
+        qa.n_mat = 3;
+        qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
+        qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
+        qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
+        qa.x = s->x; qa.ldx = E; qa.K = E; qa.T = T;
+        qa.norm_w = static_cast<const float *>(L.attn_norm.data); qa.eps = hp.rms_eps;
+        if ((rc = gemv(qa, stream)) != MESH_OK) return rc;
+
+        RopeKvArgs ra;
+        ra.q = s->q; ra.k = s->k; ra.v = s->v;
+        ra.kcache = s->kcache + il * s->kv_layer_elems;
+        ra.vcache = s->vcache + il * s->kv_layer_elems;
+        ra.pos = s->d_pos; ra.seq = s->d_seq; ra.inv_freq = st->rope_inv_freq;
+        ra.q_norm = L.q_norm.present() ? static_cast<const float *>(L.q_norm.data) : nullptr;
+        ra.k_norm = L.k_norm.present() ? static_cast<const float *>(L.k_norm.data) : nullptr;
+        ra.eps = hp.rms_eps;
+        ra.n_head = (int)hp.n_head; ra.n_kv = (int)hp.n_head_kv; ra.head_dim = (int)hp.head_dim;
+        ra.n_rot = (int)hp.n_rot; ra.rope_mode = (int)hp.rope_mode; ra.n_ctx = st->n_ctx;
+        if ((rc = rope_kv(ra, T, stream)) != MESH_OK) return rc;
+
+        AttnArgs aa;
+        aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.pos = s->d_pos; aa.seq = s->d_seq;
+        aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = s->attn;
+        aa.scale = 1.0f / sqrtf((float)hp.head_dim);
+        aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
+        aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
+        aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys);
+        if ((rc = attention(aa, T, stream)) != MESH_OK) return rc;
+
+        // x += Wo . attn
+        GemvArgs oa;
+        oa.n_mat = 1;
+        oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
+        oa.x = s->attn; oa.ldx = QD; oa.K = QD; oa.T = T;
+        oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
+        if ((rc = gemv(oa, stream)) != MESH_OK) return rc;
+
+        if (!L.w_gate.present()) return fail(MESH_ERR_UNSUPPORTED, "mixture-of-experts layers are not executable yet");
+        // ffn = silu(Wgate . n) * (Wup . n),  n = rms_norm(x)
+        GemvArgs ga;
+        ga.n_mat = 2;
+        ga.mat[0] = mat_of(L.w_gate, s->ffn, (int)hp.n_ff, nullptr);
+        ga.mat[1] = mat_of(L.w_up, nullptr, (int)hp.n_ff, nullptr);
+        ga.x = s->x; ga.ldx = E; ga.K = E; ga.T = T;
+        ga.norm_w = static_cast<const float *>(L.ffn_norm.data); ga.eps = hp.rms_eps;
+        ga.epi = EPI_SWIGLU;
+        if ((rc = gemv(ga, stream)) != MESH_OK) return rc;
+
+        // x += Wdown . ffn
+        GemvArgs da;
+        da.n_mat = 1;
+        da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
+        da.x = s->ffn; da.ldx = (int)hp.n_ff; da.K = (int)hp.n_ff; da.T = T;
+        da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        if ((rc = gemv(da, stream)) != MESH_OK) return rc;
+    }
+    return MESH_OK;
+}
+
+static int validate_batch(const mesh_session *s, const mesh_batch *b, int *max_keys) {
+    const mesh_stage *st = s->stage;
+    if (!b || b->n_tokens <= 0 || !b->pos) return fail(MESH_ERR_INVALID, "mesh_stage_decode: empty batch or null positions");
+    if (b->n_tokens > st->n_batch_max) return fail(MESH_ERR_INVALID, "mesh_stage_decode: %d tokens exceed n_batch_max %d", b->n_tokens, st->n_batch_max);
+    int mk = 0;
+    for (int i = 0; i < b->n_tokens; ++i) {
+        const int p = b->pos[i], q = b->seq_id ? b->seq_id[i] : 0;
+        if (p < 0 || p >= st->n_ctx) return fail(MESH_ERR_INVALID, "mesh_stage_decode: position %d of token %d outside the context of %d", p, i, st->n_ctx);
+        if (q < 0 || q >= st->n_seq_max) return fail(MESH_ERR_INVALID, "mesh_stage_decode: sequence id %d of token %d outside [0,%d)", q, i, st->n_seq_max);
+        mk = std::max(mk, p + 1);
+    }
+    *max_keys = mk;
+    return MESH_OK;
+}
+
+int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int in_fmt, void *d_out, int out_fmt,
+                     size_t out_cap, size_t *out_len) {
+    if (!s || !d_in || !d_out) return fail(MESH_ERR_INVALID, "mesh_stage_decode: null argument");
+    mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    int max_keys = 0, rc;
+    if ((rc = validate_batch(s, b, &max_keys)) != MESH_OK) return rc;
+    const int T = b->n_tokens;
+    const bool tokens_in = in_fmt == MESH_TOKENS, logits_out = out_fmt == MESH_LOGITS;
+    if (tokens_in && (st->layer_begin != 0 || !st->tok_embd.present()))
+        return fail(MESH_ERR_INVALID, "mesh_stage_decode: token input needs a stage that starts at layer 0 of a file with token_embd");
+    if (!tokens_in && in_fmt != MESH_F32 && in_fmt != MESH_F16 && in_fmt != MESH_Q8_0)
+        return fail(MESH_ERR_INVALID, "mesh_stage_decode: input format %d unknown", in_fmt);
+    if (logits_out && !st->output.present())
+        return fail(MESH_ERR_INVALID, "mesh_stage_decode: logits output needs a stage that ends at the last layer of a file with output weights");
+    if (!logits_out && out_fmt != MESH_F32 && out_fmt != MESH_F16 && out_fmt != MESH_Q8_0)
+        return fail(MESH_ERR_INVALID, "mesh_stage_decode: output format %d unknown", out_fmt);
+    const size_t need = logits_out ? (size_t)T * (size_t)st->output.M * 4 : mesh_act_packed_size(out_fmt, T, hp.n_embd);
+    if (need == 0) return fail(MESH_ERR_INVALID, "mesh_stage_decode: n_embd %u is not a whole number of blocks of format %d", hp.n_embd, out_fmt);
+    if (out_len) *out_len = need;
+    if (out_cap < need) return fail(MESH_ERR_INVALID, "mesh_stage_decode: output needs %zu bytes, capacity is %zu", need, out_cap);
+    MESH_HIP_TRY(hipSetDevice(st->device));
+    hipStream_t stream = s->stream;
+
+    // positions / sequence ids -> device, through a ring of pinned slots so calls may be queued back to back
+    const size_t B = (size_t)st->n_batch_max;
+    if (s->meta_counter && s->meta_counter % META_SLOTS == 0) MESH_HIP_TRY(hipStreamSynchronize(stream));   // ring wraps: older copies are done
+    int32_t *slot = s->h_meta + (size_t)(s->meta_counter++ % META_SLOTS) * 3 * B;
+    for (int i = 0; i < T; ++i) { slot[i] = b->pos[i]; slot[B + i] = b->seq_id ? b->seq_id[i] : 0; }
+    MESH_HIP_TRY(hipMemcpyAsync(s->d_pos, slot, T * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+    MESH_HIP_TRY(hipMemcpyAsync(s->d_seq, slot + B, T * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+
+    if (tokens_in) {
+        // embedding rows: one dequantize per token (ids are read on the host side by the caller's contract)
+        return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_decode_dev: token input is only available through the host-pointer entry point");
+    }
+    if ((rc = act_unpack_dev(in_fmt, d_in, s->x, (int64_t)T * hp.n_embd, stream)) != MESH_OK) return rc;
+    if ((rc = run_layers(s, T, max_keys)) != MESH_OK) return rc;
+    if (logits_out) {
+        GemvArgs la;
+        la.n_mat = 1;
+        la.mat[0] = mat_of(st->output, static_cast<float *>(d_out), (int)st->output.M, nullptr);
+        la.x = s->x; la.ldx = (int)hp.n_embd; la.K = (int)hp.n_embd; la.T = T;
+        la.norm_w = static_cast<const float *>(st->output_norm.data); la.eps = hp.rms_eps;
+        return gemv(la, stream);
+    }
+    return act_pack_dev(out_fmt, s->x, d_out, (int64_t)T * hp.n_embd, stream);
+}
+
+int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fmt, void *out, int out_fmt, size_t out_cap,
+                 size_t *out_len) {
+    if (!s || !in || !out) return fail(MESH_ERR_INVALID, "mesh_stage_decode: null argument");
+    mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    if (!b || b->n_tokens <= 0) return fail(MESH_ERR_INVALID, "mesh_stage_decode: empty batch");
+    if (b->n_tokens > st->n_batch_max) return fail(MESH_ERR_INVALID, "mesh_stage_decode: %d tokens exceed n_batch_max %d", b->n_tokens, st->n_batch_max);
+    const int T = b->n_tokens;
+    MESH_HIP_TRY(hipSetDevice(st->device));
+    hipStream_t stream = s->stream;
+    uint8_t *d_in = static_cast<uint8_t *>(s->io_stage), *d_out = d_in + s->io_stage_bytes;
+    int rc;
+    int eff_in_fmt = in_fmt;
+    if (in_fmt == MESH_TOKENS) {
+        if (st->layer_begin != 0 || !st->tok_embd.present())
+            return fail(MESH_ERR_INVALID, "mesh_stage_decode: token input needs a stage that starts at layer 0 of a file with token_embd");
+        const int32_t *ids = static_cast<const int32_t *>(in);
+        const int64_t rb = row_bytes(st->tok_embd.type, hp.n_embd);
+        for (int i = 0; i < T; ++i) {
+            if (ids[i] < 0 || ids[i] >= st->tok_embd.M) return fail(MESH_ERR_INVALID, "mesh_stage_decode: token id %d outside the vocabulary of %lld", ids[i], (long long)st->tok_embd.M);
+            rc = dequantize_dev(st->tok_embd.type, static_cast<const uint8_t *>(st->tok_embd.data) + (size_t)ids[i] * rb,
+                                reinterpret_cast<float *>(d_in) + (size_t)i * hp.n_embd, hp.n_embd, stream);
+            if (rc != MESH_OK) return rc;
+        }
+        eff_in_fmt = MESH_F32;
+    } else {
+        const size_t in_bytes = mesh_act_packed_size(in_fmt, T, hp.n_embd);
+        if (in_bytes == 0) return fail(MESH_ERR_INVALID, "mesh_stage_decode: input format %d unknown or n_embd not a whole number of blocks", in_fmt);
+        memcpy(s->h_io, in, in_bytes);
+        MESH_HIP_TRY(hipMemcpyAsync(d_in, s->h_io, in_bytes, hipMemcpyHostToDevice, stream));
+    }
+    size_t len = 0;
+    if ((rc = stage_decode_dev(s, b, d_in, eff_in_fmt, d_out, out_fmt, std::min(out_cap, s->io_stage_bytes), &len)) != MESH_OK) {
+        if (out_len) *out_len = len;
+        return rc;
+    }
+    if (out_len) *out_len = len;
+    uint8_t *h_out = static_cast<uint8_t *>(s->h_io) + s->io_stage_bytes;
+    MESH_HIP_TRY(hipMemcpyAsync(h_out, d_out, len, hipMemcpyDeviceToHost, stream));
+    MESH_HIP_TRY(hipStreamSynchronize(stream));
+    memcpy(out, h_out, len);
+    return MESH_OK;
+}
+
+}  // namespace mesh
+
+mesh_stage::~mesh_stage() {
+    for (void *p : allocations) (void)hipFree(p);
+}
+
+mesh_session::~mesh_session() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (void *p : allocations) (void)hipFree(p);
+    if (h_meta) (void)hipHostFree(h_meta);
+    if (h_io) (void)hipHostFree(h_io);
+    if (stream) (void)hipStreamDestroy(stream);
+}

@@ -1,0 +1,87 @@
+// Internal types of the stage executor: hyper-parameters, device-resident weights, session state.
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "gguf.hpp"
+#include "mesh_common.hpp"
+
+namespace mesh {
+
+enum RopeMode { ROPE_NORM = 0, ROPE_NEOX = 2 };
+
+struct HParams {
+    std::string arch;
+    uint32_t n_layer = 0, n_embd = 0, n_head = 0, n_head_kv = 0, head_dim = 0, n_ff = 0, n_vocab = 0;
+    uint32_t n_rot = 0, rope_mode = ROPE_NORM;
+    uint32_t n_expert = 0, n_expert_used = 0, n_ff_exp = 0;
+    float rms_eps = 1e-5f, rope_freq_base = 10000.0f;
+};
+
+// Fills `hp` from the GGUF key/value table (keys of the form "<arch>.block_count", ...).
+int hparams_from_gguf(const GgufFile &g, HParams &hp);
+
+// A weight matrix resident in HBM.  K-quant matrices are stored in the tiled layout of gemv.hip
+// (same byte count as the GGUF tensor); everything else keeps the GGUF row-major layout.
+struct DevTensor {
+    void *data = nullptr;
+    int type = -1;
+    int64_t K = 0;       // row length (ggml ne[0])
+    int64_t M = 0;       // rows (ggml ne[1]); for 1-D tensors M = 1
+    int64_t E = 1;       // stacked expert matrices (ggml ne[2])
+    size_t bytes = 0;
+    bool tiled = false;
+    bool present() const { return data != nullptr; }
+};
+
+struct LayerWeights {
+    DevTensor attn_norm, wq, wk, wv, wo, bq, bk, bv, q_norm, k_norm;
+    DevTensor ffn_norm, w_gate, w_up, w_down;
+    DevTensor gate_inp, gate_exps, up_exps, down_exps;   // MoE
+};
+
+}  // namespace mesh
+
+namespace mesh {
+int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out);
+int session_new(mesh_stage *st, mesh_session **out);
+int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fmt, void *out, int out_fmt, size_t out_cap, size_t *out_len);
+int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int in_fmt, void *d_out, int out_fmt, size_t out_cap, size_t *out_len);
+}  // namespace mesh
+
+struct mesh_stage {
+    mesh::HParams hp;
+    int device = 0;
+    int layer_begin = 0, layer_end = 0;
+    int n_ctx = 0, n_seq_max = 1, n_batch_max = 0;
+    std::vector<mesh::LayerWeights> layers;
+    mesh::DevTensor tok_embd, output_norm, output;
+    std::vector<void *> allocations;
+    size_t weight_bytes = 0;      // GGUF bytes of everything resident (the algorithmic weight traffic of one decode step)
+    float *rope_inv_freq = nullptr;   // [n_rot/2] f32, theta_scale^i by the f32 recurrence ggml uses
+    ~mesh_stage();
+};
+
+struct mesh_session {
+    mesh_stage *stage = nullptr;
+    hipStream_t stream = nullptr;
+    // KV cache: per local layer, K and V as f16 [n_seq_max][n_head_kv][n_ctx][head_dim]
+    uint16_t *kcache = nullptr, *vcache = nullptr;
+    size_t kv_layer_elems = 0;
+    // activations (f32), sized for n_batch_max tokens
+    float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;
+    float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
+    float *moe_logits = nullptr, *moe_w = nullptr, *expert_mask = nullptr;
+    int32_t *moe_ids = nullptr;
+    int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
+    int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)
+    unsigned meta_counter = 0;
+    void *io_stage = nullptr;       // device staging for packed in/out of the host-pointer entry point
+    size_t io_stage_bytes = 0;
+    void *h_io = nullptr;           // pinned host staging
+    int attn_splits_max = 0;
+    std::vector<void *> allocations;
+    ~mesh_session();
+};

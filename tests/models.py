@@ -1,0 +1,167 @@
+"""Synthetic GGUF models of the benchmark shapes, generated directly in the block domain (no f32 -> K-quant
+quantiser is needed): random quants and sub-scales, super-scales chosen so the dequantized tensor has sigma ~0.02.
+
+  q4_K: qs uniform bytes; sub-scale sc uniform in [8,63], min m = sc, dmin = 7.5*d  =>  w = d*sc*(q - 7.5)
+  q6_K: ql/qh uniform; sub-scale uniform in [16,127]; d ~ 1.38e-5 is an fp16 SUBNORMAL, as in real files
+  q5_0 / q8_0 (fallback types of 896-wide rows): uniform quants, d = 0.02 / rms(q)
+The distribution is a uniform mixture, not Gaussian.
+"""
+import os
+
+import numpy as np
+
+import gguf_util as G
+
+F32, F16, Q5_0, Q8_0, Q4_K, Q6_K = 0, 1, 6, 8, 12, 14
+BLOCK = {F32: (1, 4), F16: (1, 2), Q5_0: (32, 22), Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+
+
+def pack_scales_k4(sc, m):
+    """sc, m: uint8 [n, 8] six-bit values -> uint8 [n, 12]."""
+    q = np.zeros((sc.shape[0], 12), np.uint8)
+    q[:, 0:4] = sc[:, 0:4] | ((sc[:, 4:8] >> 4) << 6)
+    q[:, 4:8] = m[:, 0:4] | ((m[:, 4:8] >> 4) << 6)
+    q[:, 8:12] = (sc[:, 4:8] & 0xF) | ((m[:, 4:8] & 0xF) << 4)
+    return q
+
+
+def random_tensor(rng, ttype, n_rows, row_len, sigma=0.02):
+    """uint8 array holding n_rows x row_len elements of `ttype` blocks."""
+    be, bb = BLOCK[ttype]
+    assert row_len % be == 0, (ttype, row_len)
+    nblk = n_rows * row_len // be
+    if ttype == F32:
+        return (rng.standard_normal(n_rows * row_len) * sigma).astype(np.float32).view(np.uint8)
+    if ttype == F16:
+        return (rng.standard_normal(n_rows * row_len) * sigma).astype(np.float16).view(np.uint8)
+    raw = rng.integers(0, 256, size=(nblk, bb), dtype=np.uint8)
+    if ttype == Q4_K:
+        sc = rng.integers(8, 64, size=(nblk, 8), dtype=np.uint8)
+        d = np.float16(sigma / (4.61 * 39.0))
+        raw[:, 0:2] = np.frombuffer(d.tobytes(), np.uint8)
+        raw[:, 2:4] = np.frombuffer(np.float16(7.5 * float(d)).tobytes(), np.uint8)
+        raw[:, 4:16] = pack_scales_k4(sc, sc)
+    elif ttype == Q6_K:
+        raw[:, 192:208] = rng.integers(16, 128, size=(nblk, 16), dtype=np.uint8)
+        raw[:, 208:210] = np.frombuffer(np.float16(sigma / (18.5 * 78.5)).tobytes(), np.uint8)
+    elif ttype == Q5_0:
+        raw[:, 0:2] = np.frombuffer(np.float16(sigma / 9.23).tobytes(), np.uint8)
+    elif ttype == Q8_0:
+        raw[:, 0:2] = np.frombuffer(np.float16(sigma / 73.9).tobytes(), np.uint8)
+    return raw.reshape(-1)
+
+
+def use_more_bits(i, n):
+    return i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2
+
+
+def q4km_type(name, i_layer, n_layer, row_len):
+    """Tensor -> type map of a Q4_K_M file: attn_v and ffn_down get Q6_K on 'more bits' layers, output Q6_K;
+    rows that are not a multiple of 256 fall back Q4_K -> Q5_0 and Q6_K -> Q8_0."""
+    t = Q4_K
+    if name in ("attn_v", "ffn_down", "ffn_down_exps") and use_more_bits(i_layer, n_layer):
+        t = Q6_K
+    if name in ("output", "token_embd_tied"):
+        t = Q6_K
+    if row_len % 256:
+        t = Q5_0 if t == Q4_K else Q8_0
+    return t
+
+
+CONFIGS = {
+    # name: arch, n_layer, n_embd, n_head, n_head_kv, head_dim, n_ff, vocab, eps, rope base
+    "qwen2.5-0.5b": dict(arch="qwen2", n_layer=24, n_embd=896, n_head=14, n_head_kv=2, head_dim=64, n_ff=4864, n_vocab=151936, eps=1e-6, rope=1e6, bias=True, tied=True),
+    "llama3-8b": dict(arch="llama", n_layer=32, n_embd=4096, n_head=32, n_head_kv=8, head_dim=128, n_ff=14336, n_vocab=128256, eps=1e-5, rope=5e5),
+    "qwen2.5-32b": dict(arch="qwen2", n_layer=64, n_embd=5120, n_head=40, n_head_kv=8, head_dim=128, n_ff=27648, n_vocab=152064, eps=1e-6, rope=1e6, bias=True),
+    "qwen3-30b-a3b": dict(arch="qwen3moe", n_layer=48, n_embd=2048, n_head=32, n_head_kv=4, head_dim=128, n_ff=6144, n_vocab=151936, eps=1e-6, rope=1e6, n_expert=128, n_expert_used=8, n_ff_exp=768, qk_norm=True),
+    # small shapes for fast parity tests
+    "tiny-llama": dict(arch="llama", n_layer=4, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_ff=512, n_vocab=512, eps=1e-5, rope=1e4),
+    "tiny-qwen2": dict(arch="qwen2", n_layer=3, n_embd=512, n_head=4, n_head_kv=1, head_dim=128, n_ff=768, n_vocab=768, eps=1e-6, rope=1e6, bias=True, tied=True),
+    "tiny-qwen3": dict(arch="qwen3", n_layer=2, n_embd=256, n_head=8, n_head_kv=4, head_dim=64, n_ff=768, n_vocab=256, eps=1e-6, rope=1e6, qk_norm=True),
+    "tiny-odd": dict(arch="qwen2", n_layer=2, n_embd=320, n_head=5, n_head_kv=1, head_dim=64, n_ff=640, n_vocab=96, eps=1e-6, rope=1e4, bias=True, tied=True),
+}
+
+
+def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_expert_local=None):
+    """Returns (kvs, tensors) for write_gguf; tensors only for `layers` (absolute indices)."""
+    c = cfg
+    a = c["arch"]
+    E, H, HK, HD, FF = c["n_embd"], c["n_head"], c["n_head_kv"], c["head_dim"], c["n_ff"]
+    kvs = [("general.architecture", G.T_STR, a), ("general.alignment", G.T_U32, 32),
+           (a + ".block_count", G.T_U32, c["n_layer"]), (a + ".embedding_length", G.T_U32, E),
+           (a + ".feed_forward_length", G.T_U32, FF), (a + ".attention.head_count", G.T_U32, H),
+           (a + ".attention.head_count_kv", G.T_U32, HK), (a + ".attention.layer_norm_rms_epsilon", G.T_F32, c["eps"]),
+           (a + ".rope.freq_base", G.T_F32, c["rope"]), (a + ".vocab_size", G.T_U32, c["n_vocab"]),
+           ("tokenizer.ggml.tokens", G.T_ARR, (G.T_STR, ["<a>", "<b>"]))]   # an array the reader has to skip
+    if E // H != HD:
+        kvs += [(a + ".attention.key_length", G.T_U32, HD), (a + ".attention.value_length", G.T_U32, HD)]
+    moe = a == "qwen3moe"
+    NE = c.get("n_expert", 0)
+    NEL = n_expert_local or NE
+    if moe:
+        kvs += [(a + ".expert_count", G.T_U32, NEL), (a + ".expert_used_count", G.T_U32, c["n_expert_used"]),
+                (a + ".expert_feed_forward_length", G.T_U32, c["n_ff_exp"])]
+    tensors = []
+
+    def add(name, ttype, rows, cols, rng, kind="w", n_e=1):
+        if kind == "norm":
+            data = (1.0 + 0.02 * rng.standard_normal(cols)).astype(np.float32).view(np.uint8)
+            tensors.append((name, F32, (cols,), data))
+        elif kind == "bias":
+            data = (0.02 * rng.standard_normal(cols)).astype(np.float32).view(np.uint8)
+            tensors.append((name, F32, (cols,), data))
+        elif n_e > 1:
+            tensors.append((name, ttype, (cols, rows, n_e), random_tensor(rng, ttype, rows * n_e, cols)))
+        else:
+            tensors.append((name, ttype, (cols, rows), random_tensor(rng, ttype, rows, cols)))
+
+    for il in layers:
+        def rng_for(j):
+            return np.random.Generator(np.random.PCG64(seed + 16 * il + j))
+        p = "blk.%d." % il
+        nl = c["n_layer"]
+        add(p + "attn_norm.weight", F32, 1, E, rng_for(0), "norm")
+        add(p + "attn_q.weight", q4km_type("attn_q", il, nl, E), H * HD, E, rng_for(1))
+        add(p + "attn_k.weight", q4km_type("attn_k", il, nl, E), HK * HD, E, rng_for(2))
+        add(p + "attn_v.weight", q4km_type("attn_v", il, nl, E), HK * HD, E, rng_for(3))
+        add(p + "attn_output.weight", q4km_type("attn_output", il, nl, H * HD), E, H * HD, rng_for(4))
+        if c.get("bias"):
+            add(p + "attn_q.bias", F32, 1, H * HD, rng_for(9), "bias")
+            add(p + "attn_k.bias", F32, 1, HK * HD, rng_for(10), "bias")
+            add(p + "attn_v.bias", F32, 1, HK * HD, rng_for(11), "bias")
+        if c.get("qk_norm"):
+            add(p + "attn_q_norm.weight", F32, 1, HD, rng_for(12), "norm")
+            add(p + "attn_k_norm.weight", F32, 1, HD, rng_for(13), "norm")
+        add(p + "ffn_norm.weight", F32, 1, E, rng_for(5), "norm")
+        if not moe:
+            add(p + "ffn_gate.weight", q4km_type("ffn_gate", il, nl, E), FF, E, rng_for(6))
+            add(p + "ffn_up.weight", q4km_type("ffn_up", il, nl, E), FF, E, rng_for(7))
+            add(p + "ffn_down.weight", q4km_type("ffn_down", il, nl, FF), E, FF, rng_for(8))
+        else:
+            FE = c["n_ff_exp"]
+            r = rng_for(14)
+            tensors.append((p + "ffn_gate_inp.weight", F32, (E, NEL), (r.standard_normal(NEL * E) * 0.02).astype(np.float32).view(np.uint8)))
+            add(p + "ffn_gate_exps.weight", q4km_type("ffn_gate_exps", il, nl, E), FE, E, rng_for(6), n_e=NEL)
+            add(p + "ffn_up_exps.weight", q4km_type("ffn_up_exps", il, nl, E), FE, E, rng_for(7), n_e=NEL)
+            add(p + "ffn_down_exps.weight", q4km_type("ffn_down_exps", il, nl, FE), E, FE, rng_for(8), n_e=NEL)
+    V = c["n_vocab"]
+    if with_embd or (with_output and c.get("tied")):
+        t = q4km_type("token_embd_tied" if c.get("tied") else "token_embd", 0, 1, E)
+        # sigma 1/sqrt(E)-ish embeddings would be tiny after the first norm anyway; use sigma 0.02 like the rest
+        add("token_embd.weight", t, V, E, np.random.Generator(np.random.PCG64(seed + 100000)))
+    if with_output:
+        add("output_norm.weight", F32, 1, E, np.random.Generator(np.random.PCG64(seed + 100001)), "norm")
+        if not c.get("tied"):
+            add("output.weight", q4km_type("output", 0, 1, E), V, E, np.random.Generator(np.random.PCG64(seed + 100002)))
+    return kvs, tensors
+
+
+def write_model(path, cfg, layers, **kw):
+    kvs, tensors = build_tensors(cfg, layers, **kw)
+    G.write_gguf(path, kvs, tensors)
+    return {name: (ttype, dims, data) for name, ttype, dims, data in tensors}
+
+
+def tmp_dir():
+    d = os.environ.get("MESH_TEST_TMP") or ("/dev/shm" if os.path.isdir("/dev/shm") else "/tmp")
+    return d
