@@ -1,13 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the pipeline-stage hot path on one MI355X.  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload codec]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stage|codec] [--batches 1,4,16]
 
 Workloads
-  codec   boundary activation codec alone: hidden state [4096, 4096] f32 -> q8_0 blocks (pack), inputs
-          resident in HBM; value = algorithmic GB/s of pack_q8_0 (5.0625 B/element).
+  stage   (default) Llama-3-8B-shaped stage, layers 0-15 of 32 (hidden 4096, 32/8 heads, head_dim 128, FFN 14336,
+          RoPE theta 5e5), random Q4_K_M weights generated in the block domain, 4096-token f16 KV context, input
+          hidden state resident in HBM, output the q8_0 boundary activation.  A step = one decode call of the
+          whole stage at batch 1; value = tokens/s.  Batch 4 and 16 and the boundary codec are reported beside it.
+  codec   boundary activation codec alone on [4096, 4096] f32; value = algorithmic GB/s of pack_q8_0.
 
-The kernel's launch duration is measured with HIP events recorded on the stream the kernels are queued on.
+Timing uses HIP events recorded on the stream the kernels run on (the session's own stream for the stage).
+The cpu_baseline leg times the CPU oracle (a restatement of ggml's reference routines, NOT llama.cpp) on the
+host cores, on a bounded sample.
 """
 import argparse
 import json
@@ -23,6 +28,9 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# algorithmic bytes per element of the codec (f32 in + packed out)
+Q8_BPE, F16_BPE = 4 + 34 / 32, 6.0
+
 
 def codec_input(T, h=4096):
     rng = np.random.Generator(np.random.PCG64(1234 + T))
@@ -32,35 +40,66 @@ def codec_input(T, h=4096):
     return x
 
 
-def time_events(torch, fn, steps, warmup):
-    """Average milliseconds per call of fn() over `steps` calls, HIP events on the current stream."""
-    for _ in range(warmup):
-        fn()
+def time_on_stream(torch, stream, fn, steps, warmup):
+    """Average ms per call of fn(i) over `steps` calls: events recorded on `stream`, host clock beside it."""
+    for i in range(warmup):
+        fn(i)
+    stream.synchronize()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        fn()
-    stop.record()
+    t0 = time.perf_counter()
+    start.record(stream)
+    for i in range(steps):
+        fn(i)
+    stop.record(stream)
+    stream.synchronize()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     return start.elapsed_time(stop) / steps, wall_ms
 
 
+# ------------------------------------------------------------------------------------------------ codec
+def run_codec(torch, m, steps, warmup, T=4096, h=4096):
+    """Each op cycles through enough distinct buffers (> 256 MiB in total) that no pass is served by the
+    memory-side cache."""
+    n = T * h
+    nbuf = 6
+    base = torch.from_numpy(codec_input(T, h)).cuda()
+    xs = [base.clone() if i else base for i in range(nbuf)]
+    packed = [torch.empty(m.act_packed_size(m.Q8_0, T, h), dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
+    halves = [torch.empty(n, dtype=torch.float16, device="cuda") for _ in range(nbuf)]
+    backs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(nbuf)]
+    stream = torch.cuda.current_stream()
+    s = stream.cuda_stream
+    for i in range(nbuf):   # valid packed inputs for the unpack runs
+        m.act_pack_dev(m.Q8_0, xs[i].data_ptr(), packed[i].data_ptr(), n, s)
+        m.act_pack_dev(m.F16, xs[i].data_ptr(), halves[i].data_ptr(), n, s)
+    ops = {
+        "pack_q8_0": (lambda i: m.act_pack_dev(m.Q8_0, xs[i % nbuf].data_ptr(), packed[i % nbuf].data_ptr(), n, s), Q8_BPE),
+        "unpack_q8_0": (lambda i: m.act_unpack_dev(m.Q8_0, packed[i % nbuf].data_ptr(), backs[i % nbuf].data_ptr(), n, s), Q8_BPE),
+        "pack_f16": (lambda i: m.act_pack_dev(m.F16, xs[i % nbuf].data_ptr(), halves[i % nbuf].data_ptr(), n, s), F16_BPE),
+        "unpack_f16": (lambda i: m.act_unpack_dev(m.F16, halves[i % nbuf].data_ptr(), backs[i % nbuf].data_ptr(), n, s), F16_BPE),
+    }
+    res = {}
+    for name, (fn, bpe) in ops.items():
+        ms, _ = time_on_stream(torch, stream, fn, steps, warmup)
+        gbs = n * bpe / ms / 1e6
+        res[name] = {"ms": round(ms, 5), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+    return res
+
+
 def cpu_codec_baseline(sample_T):
-    """The oracle's quantize_row_q8_0 restatement on the host, one thread, on `sample_T` rows of the workload."""
     import oracle
     x = codec_input(sample_T).reshape(-1)
-    oracle.quantize_q8_0(x[:32 * 1024])  # warm
+    oracle.quantize_q8_0(x[:32 * 1024])
     t0 = time.perf_counter()
     reps = 0
-    while time.perf_counter() - t0 < 10.0:
+    while time.perf_counter() - t0 < 8.0:
         oracle.quantize_q8_0(x)
         reps += 1
     dt = (time.perf_counter() - t0) / reps
-    return {"value": round(x.size * 5.0625 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+    return {"value": round(x.size * Q8_BPE / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "pack_q8_0 of [%d,4096] f32, %d repeats, scalar C restatement of quantize_row_q8_0_ref" % (sample_T, reps)}
 
 
@@ -69,25 +108,8 @@ def bench_codec(args):
     import __graft_entry__ as graft
     m = graft.load_package()
     m.lib()
-    T, h = 4096, 4096
-    n = T * h
-    x = torch.from_numpy(codec_input(T)).cuda()
-    packed = torch.empty(m.act_packed_size(m.Q8_0, T, h), dtype=torch.uint8, device="cuda")
-    half = torch.empty(n, dtype=torch.float16, device="cuda")
-    back = torch.empty(n, dtype=torch.float32, device="cuda")
-    s = torch.cuda.current_stream().cuda_stream
-    ops = {
-        "pack_q8_0": (lambda: m.act_pack_dev(m.Q8_0, x.data_ptr(), packed.data_ptr(), n, s), 5.0625),
-        "unpack_q8_0": (lambda: m.act_unpack_dev(m.Q8_0, packed.data_ptr(), back.data_ptr(), n, s), 5.0625),
-        "pack_f16": (lambda: m.act_pack_dev(m.F16, x.data_ptr(), half.data_ptr(), n, s), 6.0),
-        "unpack_f16": (lambda: m.act_unpack_dev(m.F16, half.data_ptr(), back.data_ptr(), n, s), 6.0),
-    }
-    res = {}
-    for name, (fn, bpe) in ops.items():
-        ms, wall = time_events(torch, fn, args.steps, args.warmup)
-        res[name] = {"ms": round(ms, 5), "GBps": round(n * bpe / ms / 1e6, 1), "frac_hbm": round(n * bpe / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    ms = res["pack_q8_0"]["ms"]
-    gbs = res["pack_q8_0"]["GBps"]
+    res = run_codec(torch, m, args.steps, args.warmup)
+    gbs, ms = res["pack_q8_0"]["GBps"], res["pack_q8_0"]["ms"]
     out = {
         "metric": "activation pack GB/s (q8_0, [4096,4096] f32)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -102,19 +124,136 @@ def bench_codec(args):
     return out
 
 
+# ------------------------------------------------------------------------------------------------ stage
+N_CTX = 4096
+STAGE_LAYERS = 16
+
+
+def build_stage_model(models, path):
+    cfg = models.CONFIGS["llama3-8b"]
+    t0 = time.perf_counter()
+    tensors = models.write_model(path, cfg, range(STAGE_LAYERS), seed=42, fast=True)
+    return cfg, tensors, time.perf_counter() - t0
+
+
+def cpu_stage_baseline(cfg, tensors, n_layers=2):
+    """One decode token through the first `n_layers` layers of the same stage on the host cores (all of them,
+    OpenMP), at KV depth 4095; scaled to the 16-layer stage."""
+    import oracle
+    from oracle.stage import StageOracle
+    orc = StageOracle(cfg, tensors, 0, n_layers, N_CTX)
+    rng = np.random.Generator(np.random.PCG64(5))
+    kv = (rng.standard_normal((cfg["n_head_kv"], N_CTX - 1, cfg["head_dim"])) * 0.1).astype(np.float16).view(np.uint16)
+    for li in range(n_layers):
+        orc.k[li, 0, :, :N_CTX - 1] = kv
+        orc.v[li, 0, :, :N_CTX - 1] = kv
+    x = rng.standard_normal((1, cfg["n_embd"])).astype(np.float32)
+    orc.forward(x, [N_CTX - 1])
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+        orc.forward(x, [N_CTX - 1])
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(1.0 / (dt * STAGE_LAYERS / n_layers), 3), "unit": "tok/s", "cores": oracle.get_threads(), "kind": "port",
+            "sample": "batch-1 decode of layers 0-%d of the same stage at KV depth 4095, %d repeats, time scaled x%d to 16 layers; "
+                      "CPU restatement of ggml's reference routines (f32 activations), not llama.cpp" % (n_layers - 1, reps, STAGE_LAYERS // n_layers)}
+
+
+def bench_stage(args):
+    import torch
+    import __graft_entry__ as graft
+    import models
+    m = graft.load_package()
+    m.lib()
+    tmp = models.tmp_dir()
+    path = os.path.join(tmp, "mesh_bench_llama3_8b_l0_15.gguf")
+    cfg, tensors, t_gen = build_stage_model(models, path)
+    batches = sorted(set(int(b) for b in args.batches.split(",")))
+    bmax = max(batches)
+    t0 = time.perf_counter()
+    st = m.Stage(path, 0, STAGE_LAYERS, n_ctx=N_CTX, n_seq_max=bmax, n_batch_max=max(bmax, 16))
+    t_load = time.perf_counter() - t0
+    os.unlink(path)
+    weight_bytes = st.weight_bytes
+    ses = st.session()
+    E, HK, HD = cfg["n_embd"], cfg["n_head_kv"], cfg["head_dim"]
+    # KV context: 4095 cached positions per sequence, f16 N(0,1)*0.1
+    rng = np.random.Generator(np.random.PCG64(99))
+    kv = (rng.standard_normal((N_CTX - 1, HK, HD)) * 0.1).astype(np.float16).view(np.uint16)
+    for il in range(STAGE_LAYERS):
+        for s in range(bmax):
+            ses.kv_write(il, s, 0, kv, kv)
+    kv_bytes_per_seq = STAGE_LAYERS * 2 * N_CTX * HK * HD * 2
+    stream = torch.cuda.ExternalStream(ses.stream)
+    results = {}
+    for B in batches:
+        x = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
+        out = torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        pos = np.full(B, N_CTX - 1, np.int32)
+        seq = np.arange(B, dtype=np.int32)
+
+        def step(i):
+            ses.decode_dev(x.data_ptr(), pos, out.data_ptr(), out.numel(), seq=seq, in_fmt=m.F32, out_fmt=m.Q8_0)
+
+        ms, wall = time_on_stream(torch, stream, step, args.steps, args.warmup)
+        # per-kernel-class durations, from a few extra steps with event brackets around every launch
+        ses.profile(True)
+        for i in range(5):
+            step(i)
+        prof = ses.profile_read()
+        ses.profile(False)
+        step_bytes = weight_bytes + kv_bytes_per_seq * B
+        results[B] = {"ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall, 4), "tok_s": round(B * 1e3 / ms, 1),
+                      "algorithmic_GB_per_step": round(step_bytes / 1e9, 4),
+                      "GBps": round(step_bytes / ms / 1e6, 1), "frac_hbm": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                      "kernel_ms_per_step": {k: round(v["ms"] / 5, 4) for k, v in prof.items()},
+                      "kernel_launches_per_step": {k: v["launches"] // 5 for k, v in prof.items()}}
+    b1 = results[batches[0]]
+    # roofline of the dominant kernel (the dequant-fused GEMV): all of a step's weight bytes pass through its
+    # launches, so the average launch moves weight_bytes / launches in kernel_ms / launches
+    g_ms = b1["kernel_ms_per_step"]["gemv"]
+    g_n = b1["kernel_launches_per_step"]["gemv"]
+    gemv_gbs = weight_bytes / g_ms / 1e6
+    codec = run_codec(torch, m, max(10, args.steps // 2), args.warmup)
+    out = {
+        "metric": "stage decode tok/s @8B Q4_K_M", "value": b1["tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": b1["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 activations x q4_K/q6_K weights, f16 KV", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B-shaped stage, layers 0-15 of 32, Q4_K_M block-domain random weights, decode batch %d, "
+                               "4096-token f16 KV context, f32 hidden state in HBM -> q8_0 boundary activation out" % batches[0],
+                   "weight_bytes": weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1> (q4_K/q6_K dequant-fused mat-vec)",
+                     "achieved": round(gemv_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gemv_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
+                     "algorithmic_bytes_per_launch": weight_bytes // g_n},
+        "stage_frac_hbm": b1["frac_hbm"],
+        "decode": {str(k): v for k, v in results.items()},
+        "codec": codec,
+        "setup_s": {"generate_gguf": round(t_gen, 1), "open_stage": round(t_load, 1)},
+    }
+    ses.close()
+    st.close()
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_stage_baseline(cfg, tensors)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="codec", choices=["codec"])
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="stage", choices=["stage", "codec"])
+    ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU's share of the stage path; --gpus %d is not supported (one GPU per box)" % args.gpus,
+        print("bench.py measures one GPU's share of the stage path (one GPU per box); --gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
-    out = bench_codec(args)
+    out = bench_stage(args) if args.workload == "stage" else bench_codec(args)
     print(json.dumps(out))
 
 

@@ -173,6 +173,20 @@ int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const 
 void *mesh_session_stream(mesh_session *session);
 int mesh_session_synchronize(mesh_session *session);
 
+/* Per-kernel-class timing of a session, measured with HIP events recorded on the session's stream around each
+ * launch.  Off by default (it adds two event records per launch).  Kinds index the arrays below. */
+#define MESH_PROF_GEMV 0      /* dequant-fused mat-vec launches (q/k/v, o, gate/up, down, output) */
+#define MESH_PROF_ROPE 1      /* rope + KV append */
+#define MESH_PROF_ATTN 2      /* attention (split + combine) */
+#define MESH_PROF_CODEC 3     /* boundary pack / unpack */
+#define MESH_PROF_KINDS 4
+typedef struct mesh_profile {
+    double ms[MESH_PROF_KINDS];           /* summed event time per kind since the last reset */
+    uint64_t launches[MESH_PROF_KINDS];   /* bracketed launch groups per kind */
+} mesh_profile;
+int mesh_session_profile(mesh_session *session, int enable);          /* also resets the counters */
+int mesh_session_profile_read(mesh_session *session, mesh_profile *out);   /* waits for the stream */
+
 /* KV cache import/export for one sequence and one (absolute) layer: n_pos positions starting at pos0, host
  * buffers of f16 bits laid out [n_pos][n_head_kv][head_dim].  (The reference has no KV hand-over; a restarted
  * stage refills from the prompt -- mesh-llm/src/inference/election.rs:1894-1910.) */

@@ -70,6 +70,12 @@ class Batch(ctypes.Structure):
                 ("seq_id", ctypes.POINTER(ctypes.c_int32))]
 
 
+class Profile(ctypes.Structure):
+    """mesh_profile"""
+    _fields_ = [("ms", ctypes.c_double * 4), ("launches", ctypes.c_uint64 * 4)]
+
+
+PROF_GEMV, PROF_ROPE, PROF_ATTN, PROF_CODEC = 0, 1, 2, 3
 TOKENS, LOGITS = 100, 101
 _pp = ctypes.POINTER(ctypes.c_void_p)
 _psz = ctypes.POINTER(ctypes.c_size_t)
@@ -92,6 +98,8 @@ SIGNATURES.update({
     "mesh_stage_decode_dev": (_i32, [_vp, ctypes.POINTER(Batch), _vp, _i32, _vp, _i32, _sz, _psz]),
     "mesh_session_stream": (_vp, [_vp]),
     "mesh_session_synchronize": (_i32, [_vp]),
+    "mesh_session_profile": (_i32, [_vp, _i32]),
+    "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
     "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
 })
@@ -297,6 +305,15 @@ class Session:
 
     def synchronize(self):
         check(lib().mesh_session_synchronize(self._h))
+
+    def profile(self, enable):
+        check(lib().mesh_session_profile(self._h, 1 if enable else 0))
+
+    def profile_read(self):
+        p = Profile()
+        check(lib().mesh_session_profile_read(self._h, ctypes.byref(p)))
+        names = ("gemv", "rope", "attn", "codec")
+        return {n: {"ms": p.ms[i], "launches": int(p.launches[i])} for i, n in enumerate(names)}
 
     def kv_write(self, layer, seq_id, pos0, k, v):
         """k, v: uint16 arrays [n_pos, n_head_kv, head_dim] of f16 bits."""

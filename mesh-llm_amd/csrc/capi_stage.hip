@@ -157,6 +157,23 @@ int mesh_session_synchronize(mesh_session *session) {
     return MESH_OK;
 }
 
+int mesh_session_profile(mesh_session *session, int enable) {
+    if (!session) return fail(MESH_ERR_INVALID, "mesh_session_profile: null session");
+    int rc = profile_collect(session);
+    if (rc != MESH_OK) return rc;
+    session->profile = enable != 0;
+    for (int i = 0; i < MESH_PROF_KINDS; ++i) { session->prof_ms[i] = 0; session->prof_launches[i] = 0; }
+    return MESH_OK;
+}
+
+int mesh_session_profile_read(mesh_session *session, mesh_profile *out) {
+    if (!session || !out) return fail(MESH_ERR_INVALID, "mesh_session_profile_read: null argument");
+    int rc = profile_collect(session);
+    if (rc != MESH_OK) return rc;
+    for (int i = 0; i < MESH_PROF_KINDS; ++i) { out->ms[i] = session->prof_ms[i]; out->launches[i] = session->prof_launches[i]; }
+    return MESH_OK;
+}
+
 static int kv_xfer(mesh_session *s, int layer, int seq_id, int pos0, int n_pos, uint16_t *k, uint16_t *v, bool write) {
     if (!s || !k || !v) return fail(MESH_ERR_INVALID, "mesh_session_kv: null argument");
     const mesh_stage *st = s->stage;

@@ -293,6 +293,43 @@ static int attn_splits_for(int T, int n_kv, int max_keys) {
     return std::max(1, std::min(s, ATTN_SPLITS_MAX));
 }
 
+// ---- optional timing -----------------------------------------------------------------------------
+struct ProfScope {
+    mesh_session *s;
+    bool on;
+    ProfScope(mesh_session *ses, int kind) : s(ses), on(ses->profile) {
+        if (!on) return;
+        if (s->prof_used + 2 > s->prof_events.size()) {
+            for (int i = 0; i < 2; ++i) {
+                hipEvent_t e;
+                if (hipEventCreate(&e) != hipSuccess) { on = false; return; }
+                s->prof_events.push_back(e);
+            }
+        }
+        s->prof_kinds.push_back(kind);
+        (void)hipEventRecord(s->prof_events[s->prof_used], s->stream);
+    }
+    ~ProfScope() {
+        if (!on) return;
+        (void)hipEventRecord(s->prof_events[s->prof_used + 1], s->stream);
+        s->prof_used += 2;
+    }
+};
+
+int profile_collect(mesh_session *s) {
+    MESH_HIP_TRY(hipStreamSynchronize(s->stream));
+    for (size_t i = 0; i + 1 < s->prof_used + 1 && i / 2 < s->prof_kinds.size(); i += 2) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, s->prof_events[i], s->prof_events[i + 1]) == hipSuccess) {
+            s->prof_ms[s->prof_kinds[i / 2]] += ms;
+            s->prof_launches[s->prof_kinds[i / 2]] += 1;
+        }
+    }
+    s->prof_used = 0;
+    s->prof_kinds.clear();
+    return MESH_OK;
+}
+
 // Runs the layers over the T token rows already in s->x.  pos/seq are on the device in s->d_pos / s->d_seq.
 static int run_layers(mesh_session *s, int T, int max_keys) {
     mesh_stage *st = s->stage;
@@ -310,7 +347,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = s->x; qa.ldx = E; qa.K = E; qa.T = T;
         qa.norm_w = static_cast<const float *>(L.attn_norm.data); qa.eps = hp.rms_eps;
-        if ((rc = gemv(qa, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(qa, stream); }
+        if (rc != MESH_OK) return rc;
 
         RopeKvArgs ra;
         ra.q = s->q; ra.k = s->k; ra.v = s->v;
@@ -322,7 +360,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         ra.eps = hp.rms_eps;
         ra.n_head = (int)hp.n_head; ra.n_kv = (int)hp.n_head_kv; ra.head_dim = (int)hp.head_dim;
         ra.n_rot = (int)hp.n_rot; ra.rope_mode = (int)hp.rope_mode; ra.n_ctx = st->n_ctx;
-        if ((rc = rope_kv(ra, T, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_ROPE); rc = rope_kv(ra, T, stream); }
+        if (rc != MESH_OK) return rc;
 
         AttnArgs aa;
         aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.pos = s->d_pos; aa.seq = s->d_seq;
@@ -331,7 +370,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
         aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
         aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys);
-        if ((rc = attention(aa, T, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
+        if (rc != MESH_OK) return rc;
 
         // x += Wo . attn
         GemvArgs oa;
@@ -339,7 +379,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
         oa.x = s->attn; oa.ldx = QD; oa.K = QD; oa.T = T;
         oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
-        if ((rc = gemv(oa, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(oa, stream); }
+        if (rc != MESH_OK) return rc;
 
         if (!L.w_gate.present()) return fail(MESH_ERR_UNSUPPORTED, "mixture-of-experts layers are not executable yet");
         // ffn = silu(Wgate . n) * (Wup . n),  n = rms_norm(x)
@@ -350,7 +391,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         ga.x = s->x; ga.ldx = E; ga.K = E; ga.T = T;
         ga.norm_w = static_cast<const float *>(L.ffn_norm.data); ga.eps = hp.rms_eps;
         ga.epi = EPI_SWIGLU;
-        if ((rc = gemv(ga, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ga, stream); }
+        if (rc != MESH_OK) return rc;
 
         // x += Wdown . ffn
         GemvArgs da;
@@ -358,7 +400,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
         da.x = s->ffn; da.ldx = (int)hp.n_ff; da.K = (int)hp.n_ff; da.T = T;
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
-        if ((rc = gemv(da, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(da, stream); }
+        if (rc != MESH_OK) return rc;
     }
     return MESH_OK;
 }
@@ -414,7 +457,8 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
         // embedding rows: one dequantize per token (ids are read on the host side by the caller's contract)
         return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_decode_dev: token input is only available through the host-pointer entry point");
     }
-    if ((rc = act_unpack_dev(in_fmt, d_in, s->x, (int64_t)T * hp.n_embd, stream)) != MESH_OK) return rc;
+    { ProfScope ps(s, MESH_PROF_CODEC); rc = act_unpack_dev(in_fmt, d_in, s->x, (int64_t)T * hp.n_embd, stream); }
+    if (rc != MESH_OK) return rc;
     if ((rc = run_layers(s, T, max_keys)) != MESH_OK) return rc;
     if (logits_out) {
         GemvArgs la;
@@ -422,8 +466,10 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
         la.mat[0] = mat_of(st->output, static_cast<float *>(d_out), (int)st->output.M, nullptr);
         la.x = s->x; la.ldx = (int)hp.n_embd; la.K = (int)hp.n_embd; la.T = T;
         la.norm_w = static_cast<const float *>(st->output_norm.data); la.eps = hp.rms_eps;
+        ProfScope ps(s, MESH_PROF_GEMV);
         return gemv(la, stream);
     }
+    ProfScope ps(s, MESH_PROF_CODEC);
     return act_pack_dev(out_fmt, s->x, d_out, (int64_t)T * hp.n_embd, stream);
 }
 
@@ -479,6 +525,7 @@ mesh_stage::~mesh_stage() {
 
 mesh_session::~mesh_session() {
     if (stream) (void)hipStreamSynchronize(stream);
+    for (hipEvent_t e : prof_events) (void)hipEventDestroy(e);
     for (void *p : allocations) (void)hipFree(p);
     if (h_meta) (void)hipHostFree(h_meta);
     if (h_io) (void)hipHostFree(h_io);

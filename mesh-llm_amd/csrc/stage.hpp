@@ -48,6 +48,7 @@ namespace mesh {
 int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out);
 int session_new(mesh_stage *st, mesh_session **out);
 int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fmt, void *out, int out_fmt, size_t out_cap, size_t *out_len);
+int profile_collect(mesh_session *s);
 int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int in_fmt, void *d_out, int out_fmt, size_t out_cap, size_t *out_len);
 }  // namespace mesh
 
@@ -83,5 +84,12 @@ struct mesh_session {
     void *h_io = nullptr;           // pinned host staging
     int attn_splits_max = 0;
     std::vector<void *> allocations;
+    // optional per-kernel-class timing (HIP events on `stream` around every launch group)
+    bool profile = false;
+    std::vector<hipEvent_t> prof_events;      // pairs (begin, end)
+    std::vector<int> prof_kinds;
+    size_t prof_used = 0;
+    double prof_ms[MESH_PROF_KINDS] = {0, 0, 0, 0};
+    uint64_t prof_launches[MESH_PROF_KINDS] = {0, 0, 0, 0};
     ~mesh_session();
 };

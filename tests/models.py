@@ -25,7 +25,22 @@ def pack_scales_k4(sc, m):
     return q
 
 
-def random_tensor(rng, ttype, n_rows, row_len, sigma=0.02):
+_BASE_BYTES = {}
+
+
+def _random_bytes(rng, n, variant):
+    """n uniform random bytes.  variant None: drawn from rng.  Otherwise: one cached draw per size (seeded by the
+    size), XOR-ed with a byte derived from `variant` -- still uniform, distinct per tensor, and ~10x cheaper, which
+    matters when a benchmark model holds gigabytes."""
+    if variant is None:
+        return rng.bit_generator.random_raw((n + 7) // 8).view(np.uint8)[:n].copy()
+    if n not in _BASE_BYTES:
+        g = np.random.Generator(np.random.PCG64(n))
+        _BASE_BYTES[n] = g.bit_generator.random_raw((n + 7) // 8).view(np.uint8)[:n]
+    return _BASE_BYTES[n] ^ np.uint8((variant * 37 + 11) & 0xFF)
+
+
+def random_tensor(rng, ttype, n_rows, row_len, sigma=0.02, variant=None):
     """uint8 array holding n_rows x row_len elements of `ttype` blocks."""
     be, bb = BLOCK[ttype]
     assert row_len % be == 0, (ttype, row_len)
@@ -34,7 +49,7 @@ def random_tensor(rng, ttype, n_rows, row_len, sigma=0.02):
         return (rng.standard_normal(n_rows * row_len) * sigma).astype(np.float32).view(np.uint8)
     if ttype == F16:
         return (rng.standard_normal(n_rows * row_len) * sigma).astype(np.float16).view(np.uint8)
-    raw = rng.integers(0, 256, size=(nblk, bb), dtype=np.uint8)
+    raw = _random_bytes(rng, nblk * bb, variant).reshape(nblk, bb)
     if ttype == Q4_K:
         sc = rng.integers(8, 64, size=(nblk, 8), dtype=np.uint8)
         d = np.float16(sigma / (4.61 * 39.0))
@@ -82,7 +97,7 @@ CONFIGS = {
 }
 
 
-def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_expert_local=None):
+def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_expert_local=None, fast=False):
     """Returns (kvs, tensors) for write_gguf; tensors only for `layers` (absolute indices)."""
     c = cfg
     a = c["arch"]
@@ -103,7 +118,11 @@ def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_ex
                 (a + ".expert_feed_forward_length", G.T_U32, c["n_ff_exp"])]
     tensors = []
 
+    counter = [0]
+
     def add(name, ttype, rows, cols, rng, kind="w", n_e=1):
+        counter[0] += 1
+        var = counter[0] if fast else None
         if kind == "norm":
             data = (1.0 + 0.02 * rng.standard_normal(cols)).astype(np.float32).view(np.uint8)
             tensors.append((name, F32, (cols,), data))
@@ -111,9 +130,9 @@ def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_ex
             data = (0.02 * rng.standard_normal(cols)).astype(np.float32).view(np.uint8)
             tensors.append((name, F32, (cols,), data))
         elif n_e > 1:
-            tensors.append((name, ttype, (cols, rows, n_e), random_tensor(rng, ttype, rows * n_e, cols)))
+            tensors.append((name, ttype, (cols, rows, n_e), random_tensor(rng, ttype, rows * n_e, cols, variant=var)))
         else:
-            tensors.append((name, ttype, (cols, rows), random_tensor(rng, ttype, rows, cols)))
+            tensors.append((name, ttype, (cols, rows), random_tensor(rng, ttype, rows, cols, variant=var)))
 
     for il in layers:
         def rng_for(j):
