@@ -71,29 +71,33 @@ int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream) {
 
 // ------------------------------------------------------------------------------------------------ attention
 constexpr int ATTN_THREADS = 256;
+constexpr int ATTN_WAVES = ATTN_THREADS / 64;
+constexpr int KPT = 4;                      // keys per thread per pass: 8 x 16-byte loads in flight per lane
 
-__device__ __forceinline__ void load8h(const uint16_t *p, float (&o)[8]) {
-    const uint4 v = *reinterpret_cast<const uint4 *>(p);
+__device__ __forceinline__ void unpack8h(const uint4 &v, float (&o)[8]) {
     o[0] = f16_bits_to_f32((uint16_t)(v.x & 0xFFFF)); o[1] = f16_bits_to_f32((uint16_t)(v.x >> 16));
     o[2] = f16_bits_to_f32((uint16_t)(v.y & 0xFFFF)); o[3] = f16_bits_to_f32((uint16_t)(v.y >> 16));
     o[4] = f16_bits_to_f32((uint16_t)(v.z & 0xFFFF)); o[5] = f16_bits_to_f32((uint16_t)(v.z >> 16));
     o[6] = f16_bits_to_f32((uint16_t)(v.w & 0xFFFF)); o[7] = f16_bits_to_f32((uint16_t)(v.w >> 16));
 }
 
-// grid (n_splits, n_kv * (group/G), T).  HD/8 lanes share one key; each thread keeps a private online-softmax
-// state (m, l, acc[8]) per query head over the keys its slot visits; slots are merged through LDS.
+// grid (n_splits, n_kv * (group/G), T).  HD/8 lanes share one key ("slot"); a thread visits keys
+// j0 + slot + SLOTS*i and keeps one online-softmax state (m, l, acc[8]) per query head.  Per pass all KPT keys'
+// K and V vectors are requested first, then scored, then folded in with a single rescale.  The slots of a
+// workgroup are merged through LDS.  With one split the normalised output is written directly; otherwise each
+// workgroup writes an un-normalised partial plus (max, sum) and attn_combine_kernel merges the splits.
 template <int HD, int G>
-__global__ __launch_bounds__(ATTN_THREADS) void attn_split_kernel(AttnArgs a) {
+__global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
     constexpr int LPK = HD / 8;                 // lanes per key
-    constexpr int SLOTS = ATTN_THREADS / LPK;   // keys in flight per pass
-    __shared__ float s_m[SLOTS][G], s_l[SLOTS][G];
-    __shared__ float s_acc[ATTN_THREADS / 64][G][HD];   // per-wave sums of the slot states
+    constexpr int SLOTS = ATTN_THREADS / LPK;   // keys visited side by side
+    __shared__ float s_m[SLOTS][G], s_l[ATTN_WAVES][G], s_mw[G];
+    __shared__ float s_acc[ATTN_WAVES][G][HD];  // per-wave sums of the slot states
 
     const int split = blockIdx.x, t = blockIdx.z;
     const int hgroups = a.group / G;            // G divides group (G == group, or G == 1)
     const int kvh = blockIdx.y / hgroups;
     const int h0 = kvh * a.group + (blockIdx.y % hgroups) * G;   // first query head of this workgroup
-    const int tid = threadIdx.x, slot = tid / LPK, ds = (tid % LPK) * 8;
+    const int tid = threadIdx.x, slot = tid / LPK, ds = (tid % LPK) * 8, wave = tid >> 6;
     const int seq = a.seq[t];
     const int n_keys = a.pos[t] + 1;
     const int per = (n_keys + a.n_splits - 1) / a.n_splits;
@@ -103,87 +107,135 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_split_kernel(AttnArgs a) {
     float q[G][8], acc[G][8], m[G], l[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-        const float *qp = a.q + ((size_t)t * a.n_head + h0 + h) * HD + ds;
+        const float4 qa = *reinterpret_cast<const float4 *>(a.q + ((size_t)t * a.n_head + h0 + h) * HD + ds);
+        const float4 qb = *reinterpret_cast<const float4 *>(a.q + ((size_t)t * a.n_head + h0 + h) * HD + ds + 4);
+        const float qs = a.scale * 1.44269504088896341f;      // scores in log2 units: softmax through exp2
+        q[h][0] = qa.x * qs; q[h][1] = qa.y * qs; q[h][2] = qa.z * qs; q[h][3] = qa.w * qs;
+        q[h][4] = qb.x * qs; q[h][5] = qb.y * qs; q[h][6] = qb.z * qs; q[h][7] = qb.w * qs;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { q[h][i] = qp[i] * a.scale; acc[h][i] = 0.f; }
+        for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
         m[h] = -INFINITY;
         l[h] = 0.f;
     }
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
-    for (int j = j0 + slot; j < j1; j += SLOTS) {
-        float kf[8], vf[8];
-        load8h(a.kcache + (base + j) * HD + ds, kf);
-        load8h(a.vcache + (base + j) * HD + ds, vf);
+    for (int jb = j0; jb < j1; jb += SLOTS * KPT) {
+        uint4 kr[KPT], vr[KPT];
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            const int j = jb + slot + SLOTS * i;
+            kr[i] = make_uint4(0, 0, 0, 0);
+            vr[i] = kr[i];
+            if (j < j1) {
+                kr[i] = *reinterpret_cast<const uint4 *>(a.kcache + (base + j) * HD + ds);
+                vr[i] = *reinterpret_cast<const uint4 *>(a.vcache + (base + j) * HD + ds);
+            }
+        }
+        float sc[KPT][G];
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            float kf[8];
+            unpack8h(kr[i], kf);
+            const bool ok = jb + slot + SLOTS * i < j1;
+#pragma unroll
+            for (int h = 0; h < G; ++h) {
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s = fmaf(q[h][e], kf[e], s);
+#pragma unroll
+                for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+                sc[i][h] = ok ? s : -INFINITY;
+            }
+        }
+        float vf[KPT][8];
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) unpack8h(vr[i], vf[i]);
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-            float s = 0.f;
+            float mn = m[h];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) s = fmaf(q[h][i], kf[i], s);
+            for (int i = 0; i < KPT; ++i) mn = fmaxf(mn, sc[i][h]);
+            if (mn == -INFINITY) continue;          // this slot had no key in range yet
+            const float corr = exp2f(m[h] - mn);    // exp2(-inf) = 0 the first time
+            float p[KPT], ps = 0.f;
 #pragma unroll
-            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
-            const float mn = fmaxf(m[h], s);
-            const float corr = expf(m[h] - mn);     // exp(-inf) = 0 on the first key
-            const float p = expf(s - mn);
-            l[h] = l[h] * corr + p;
+            for (int i = 0; i < KPT; ++i) { p[i] = exp2f(sc[i][h] - mn); ps += p[i]; }
+            l[h] = l[h] * corr + ps;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(p, vf[i], acc[h][i] * corr);
+            for (int e = 0; e < 8; ++e) {
+                float v = acc[h][e] * corr;
+#pragma unroll
+                for (int i = 0; i < KPT; ++i) v = fmaf(p[i], vf[i][e], v);
+                acc[h][e] = v;
+            }
             m[h] = mn;
         }
     }
-    // merge the slots
+    // merge the slots of this workgroup: every slot state is rescaled to the workgroup's maximum, slots sharing a
+    // wave are added with shuffles, the 4 waves meet in LDS
     if ((tid % LPK) == 0) {
 #pragma unroll
-        for (int h = 0; h < G; ++h) { s_m[slot][h] = m[h]; s_l[slot][h] = l[h]; }
+        for (int h = 0; h < G; ++h) s_m[slot][h] = m[h];
     }
     __syncthreads();
-    const int wave = tid >> 6;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-        float mm = -INFINITY;
-        for (int s2 = 0; s2 < SLOTS; ++s2) mm = fmaxf(mm, s_m[s2][h]);
-        const float w = (m[h] == -INFINITY) ? 0.f : expf(m[h] - mm);
+        float mh = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float v = acc[h][i] * w;
-            // add up the slots that live in this wave (lanes with equal tid % LPK)
+        for (int s2 = 0; s2 < SLOTS; ++s2) mh = fmaxf(mh, s_m[s2][h]);
+        const float w = (m[h] == -INFINITY) ? 0.f : exp2f(m[h] - mh);
+        float lw = l[h] * w;
 #pragma unroll
-            for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o);
-            if ((tid & 63) < LPK) s_acc[wave][h][ds + i] = v;
+        for (int o = LPK; o < 64; o <<= 1) lw += __shfl_xor(lw, o);
+        if ((tid & 63) == 0) { s_l[wave][h] = lw; s_mw[h] = mh; }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float v = acc[h][e] * w;
+#pragma unroll
+            for (int o = LPK; o < 64; o <<= 1) v += __shfl_xor(v, o);   // slots that live in this wave
+            if ((tid & 63) < LPK) s_acc[wave][h][ds + e] = v;
         }
     }
     __syncthreads();
+    const bool single = a.n_splits == 1;
     for (int o = tid; o < G * HD; o += ATTN_THREADS) {
         const int h = o / HD, dd = o % HD;
-        float sum = 0.f;
-        for (int w2 = 0; w2 < ATTN_THREADS / 64; ++w2) sum += s_acc[w2][h][dd];
-        a.part[(((size_t)t * a.n_head + h0 + h) * a.n_splits + split) * HD + dd] = sum;
-    }
-    if (tid < G) {
-        const int h = tid;
-        float mm = -INFINITY;
-        for (int s2 = 0; s2 < SLOTS; ++s2) mm = fmaxf(mm, s_m[s2][h]);
-        float ll = 0.f;
-        for (int s2 = 0; s2 < SLOTS; ++s2) ll += (s_m[s2][h] == -INFINITY) ? 0.f : s_l[s2][h] * expf(s_m[s2][h] - mm);
-        float *ml = a.ml + (((size_t)t * a.n_head + h0 + h) * a.n_splits + split) * 2;
-        ml[0] = mm;
-        ml[1] = ll;
+        float sum = 0.f, ll = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < ATTN_WAVES; ++w2) { sum += s_acc[w2][h][dd]; ll += s_l[w2][h]; }
+        const size_t row = (size_t)t * a.n_head + h0 + h;
+        if (single) {
+            a.out[row * HD + dd] = sum / ll;
+        } else {
+            a.part[(row * a.n_splits + split) * HD + dd] = sum;
+            if (dd == 0) {
+                a.ml[(row * a.n_splits + split) * 2 + 0] = s_mw[h];
+                a.ml[(row * a.n_splits + split) * 2 + 1] = ll;
+            }
+        }
     }
 }
 
-// grid (n_head, T), block head_dim threads
-__global__ void attn_combine_kernel(AttnArgs a) {
+// Merge of the KV splits: grid (n_head, T), head_dim threads.  Split statistics go through LDS so every thread
+// sees them with broadcast reads and the partial rows are fetched with independent loads.
+__global__ __launch_bounds__(128) void attn_combine_kernel(AttnArgs a) {
+    __shared__ float s_m[ATTN_SPLITS_CAP], s_l[ATTN_SPLITS_CAP];
     const int h = blockIdx.x, t = blockIdx.y, dd = threadIdx.x;
     const size_t row = (size_t)t * a.n_head + h;
-    const float *ml = a.ml + row * a.n_splits * 2;
-    float mm = -INFINITY;
-    for (int s = 0; s < a.n_splits; ++s) mm = fmaxf(mm, ml[2 * s]);
+    for (int s2 = dd; s2 < a.n_splits; s2 += blockDim.x) {
+        s_m[s2] = a.ml[(row * a.n_splits + s2) * 2 + 0];
+        s_l[s2] = a.ml[(row * a.n_splits + s2) * 2 + 1];
+    }
+    __syncthreads();
+    float mh = -INFINITY;
+    for (int s2 = 0; s2 < a.n_splits; ++s2) mh = fmaxf(mh, s_m[s2]);
     float num = 0.f, den = 0.f;
-    for (int s = 0; s < a.n_splits; ++s) {
-        const float ms = ml[2 * s];
-        if (ms == -INFINITY) continue;
-        const float w = expf(ms - mm);
-        num = fmaf(a.part[(row * a.n_splits + s) * a.head_dim + dd], w, num);
-        den = fmaf(ml[2 * s + 1], w, den);
+    const float *pp = a.part + row * a.n_splits * a.head_dim + dd;
+#pragma unroll 8
+    for (int s2 = 0; s2 < a.n_splits; ++s2) {
+        const float ms = s_m[s2];
+        const float w = ms == -INFINITY ? 0.f : exp2f(ms - mh);      // maxima are in log2 units
+        num = fmaf(pp[(size_t)s2 * a.head_dim], w, num);
+        den = fmaf(s_l[s2], w, den);
     }
     a.out[row * a.head_dim + dd] = num / den;
 }
@@ -193,7 +245,7 @@ static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     const dim3 block(ATTN_THREADS);
 #define MESH_ATTN_CASE(GG)                                                                          \
     if (a.group == GG) {                                                                            \
-        attn_split_kernel<HD, GG><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
+        attn_kernel<HD, GG><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
         MESH_LAUNCH_CHECK();                                                                        \
         return MESH_OK;                                                                             \
     }
@@ -204,19 +256,21 @@ static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     if (HD == 64) { MESH_ATTN_CASE(7) }
 #undef MESH_ATTN_CASE
     // any other group size: one query head per workgroup (K/V re-read per head)
-    attn_split_kernel<HD, 1><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
+    attn_kernel<HD, 1><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
 int attention(const AttnArgs &a, int T, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
-    if (a.n_splits < 1 || a.group < 1 || a.n_head != a.group * a.n_kv) return fail(MESH_ERR_INVALID, "attention: bad head layout");
+    if (a.n_splits < 1 || a.n_splits > ATTN_SPLITS_CAP || a.group < 1 || a.n_head != a.group * a.n_kv)
+        return fail(MESH_ERR_INVALID, "attention: bad head layout or split count");
+    if (a.n_splits > 1 && (!a.part || !a.ml)) return fail(MESH_ERR_INVALID, "attention: split buffers missing");
     int rc;
     if (a.head_dim == 128) rc = launch_attn<128>(a, T, stream);
     else if (a.head_dim == 64) rc = launch_attn<64>(a, T, stream);
     else return fail(MESH_ERR_UNSUPPORTED, "attention: head_dim %d has no kernel (64 and 128 do)", a.head_dim);
-    if (rc != MESH_OK) return rc;
+    if (rc != MESH_OK || a.n_splits == 1) return rc;
     attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;

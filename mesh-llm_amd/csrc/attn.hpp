@@ -6,6 +6,7 @@
 namespace mesh {
 
 constexpr int ROPE_MODE_NORM = 0, ROPE_MODE_NEOX = 2;
+constexpr int ATTN_SPLITS_CAP = 64;     // most KV splits per (token, kv head)
 
 struct RopeKvArgs {
     float *q = nullptr;            // [T][n_head][head_dim], rotated in place

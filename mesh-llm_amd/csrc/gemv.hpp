@@ -7,14 +7,15 @@ namespace mesh {
 
 // ---- tiled K-quant layout -----------------------------------------------------------------------------------
 // A K-quant matrix [M rows][K] is stored as tiles of 16 rows x one 256-element super-block, tile (R, sb) at
-// byte offset (R * K/256 + sb) * 16 * block_bytes: a workgroup streaming 16 rows along K reads one contiguous
-// run.  Byte count equals the GGUF tensor's (M is padded to 16 with zero blocks).  Inside a tile, lane
-// l = g*16 + r (r = row in tile, g = 0..3) owns the bytes that decode elements 32*s + 8*g + i, s = 0..7, i = 0..7:
-//   q4_K (2304 B): [16 x 16 B headers {d, dmin, scales[12]}] [plane0: 64 x 16 B] [plane1: 64 x 16 B];
-//                  lane's 16 B of plane p = qs[64p + 8g .. +8] | qs[64p + 32 + 8g .. +8]
-//   q6_K (3360 B): [ql plane n=0: 64 x 16 B] [ql plane n=1] [qh: 64 x 16 B] [16 x 16 B scales] [16 x fp16 d];
-//                  lane's 16 B of ql plane n = ql[64n + 8g .. +8] | ql[64n + 32 + 8g .. +8],
-//                  lane's 16 B of qh = qh[8g .. +8] | qh[32 + 8g .. +8]
+// byte offset (R * K/256 + sb) * 16 * block_bytes, so the workgroup that owns 16 rows streams one contiguous
+// run along K.  Byte count equals the GGUF tensor's (M is padded to 16 with zero blocks).  Inside a tile the
+// per-row fields are regrouped so that every access is an aligned 16-byte vector and a wave's loads are dense:
+//   q4_K (2304 B): [16 x 16 B headers {d, dmin, scales[12]}] [16 x 128 B qs]
+//   q6_K (3360 B): [16 x 128 B ql] [16 x 64 B qh] [16 x 16 B scales] [16 x fp16 d]
+// Lane l = 4*r + c of a wave works on row r, quarter c of the super-block:
+//   q4_K: qs[32c .. 32c+32)  -> sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
+//   q6_K: half n = c/2, u = c%2: ql[64n+16u..+16), ql[64n+32+16u..+16), qh[32n+16u..+16) -> elements
+//         128n + 32t + 16u + i, t = 0..3, i = 0..15 (one 16-element scale group per t)
 constexpr int TILE_ROWS = 16;
 constexpr int Q4K_TILE_BYTES = TILE_ROWS * Q4_K_BYTES;   // 2304
 constexpr int Q6K_TILE_BYTES = TILE_ROWS * Q6_K_BYTES;   // 3360
@@ -51,7 +52,7 @@ struct GemvArgs {
     const float *x = nullptr;  // [T][ldx]
     int ldx = 0;
     int K = 0;
-    int T = 0;                 // any T; processed 4 columns at a time
+    int T = 0;                 // any T; processed a few columns at a time
     const float *norm_w = nullptr;   // if set: x is RMS-normalised (eps) and scaled by norm_w[K] on the fly
     float eps = 0.f;
     const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y

@@ -5,73 +5,57 @@
 
 namespace mesh {
 
-// one wave per tile; lane l = g*16 + r
+// one wave per tile; lane l = 4*r + c copies a quarter of row r's block
 template <bool TO_TILED>
 __global__ __launch_bounds__(64) void repack_q4k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                         int M, int nsb) {
     const int sb = blockIdx.x, R = blockIdx.y, lane = threadIdx.x;
-    const int r = lane & 15, g = lane >> 4;
+    const int r = lane >> 2, c = lane & 3;
     const int row = R * TILE_ROWS + r;
-    const uint8_t *rm_c = (TO_TILED ? src : dst) + ((size_t)row * nsb + sb) * Q4_K_BYTES;   // row-major block
+    uint8_t *rm = const_cast<uint8_t *>(TO_TILED ? src : dst) + ((size_t)row * nsb + sb) * Q4_K_BYTES;
     uint8_t *tl = const_cast<uint8_t *>(TO_TILED ? dst : src) + ((size_t)R * nsb + sb) * Q4K_TILE_BYTES;
-    uint8_t *rm = const_cast<uint8_t *>(rm_c);
     const bool live = row < M;
+    uint4 *t_hdr = reinterpret_cast<uint4 *>(tl + r * 16);
+    uint4 *t_qs = reinterpret_cast<uint4 *>(tl + 256 + lane * 32);
     if (TO_TILED) {
-        if (g == 0) {
-            uint4 h = make_uint4(0, 0, 0, 0);
-            if (live) h = *reinterpret_cast<const uint4 *>(rm);
-            *reinterpret_cast<uint4 *>(tl + r * 16) = h;
-        }
-        for (int p = 0; p < 2; ++p) {
-            uint2 a = make_uint2(0, 0), b = make_uint2(0, 0);
-            if (live) {
-                a = *reinterpret_cast<const uint2 *>(rm + 16 + 64 * p + 8 * g);
-                b = *reinterpret_cast<const uint2 *>(rm + 16 + 64 * p + 32 + 8 * g);
-            }
-            *reinterpret_cast<uint4 *>(tl + 256 + p * 1024 + lane * 16) = make_uint4(a.x, a.y, b.x, b.y);
-        }
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        if (c == 0) *t_hdr = live ? *reinterpret_cast<const uint4 *>(rm) : z;
+        t_qs[0] = live ? *reinterpret_cast<const uint4 *>(rm + 16 + 32 * c) : z;
+        t_qs[1] = live ? *reinterpret_cast<const uint4 *>(rm + 16 + 32 * c + 16) : z;
     } else if (live) {
-        if (g == 0) *reinterpret_cast<uint4 *>(rm) = *reinterpret_cast<const uint4 *>(tl + r * 16);
-        for (int p = 0; p < 2; ++p) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(tl + 256 + p * 1024 + lane * 16);
-            *reinterpret_cast<uint2 *>(rm + 16 + 64 * p + 8 * g) = make_uint2(v.x, v.y);
-            *reinterpret_cast<uint2 *>(rm + 16 + 64 * p + 32 + 8 * g) = make_uint2(v.z, v.w);
-        }
+        if (c == 0) *reinterpret_cast<uint4 *>(rm) = *t_hdr;
+        *reinterpret_cast<uint4 *>(rm + 16 + 32 * c) = t_qs[0];
+        *reinterpret_cast<uint4 *>(rm + 16 + 32 * c + 16) = t_qs[1];
     }
 }
 
+// q6_K blocks are only 2-byte aligned in GGUF (210 bytes): move them as 16-bit words
 template <bool TO_TILED>
 __global__ __launch_bounds__(64) void repack_q6k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                         int M, int nsb) {
     const int sb = blockIdx.x, R = blockIdx.y, lane = threadIdx.x;
-    const int r = lane & 15, g = lane >> 4;
+    const int r = lane >> 2, c = lane & 3;
     const int row = R * TILE_ROWS + r;
-    uint8_t *rm = const_cast<uint8_t *>(TO_TILED ? src : dst) + ((size_t)row * nsb + sb) * Q6_K_BYTES;   // 2-byte aligned
+    uint16_t *rm = reinterpret_cast<uint16_t *>(const_cast<uint8_t *>(TO_TILED ? src : dst) + ((size_t)row * nsb + sb) * Q6_K_BYTES);
     uint8_t *tl = const_cast<uint8_t *>(TO_TILED ? dst : src) + ((size_t)R * nsb + sb) * Q6K_TILE_BYTES;
     const bool live = row < M;
     if (!TO_TILED && !live) return;
-    for (int n = 0; n < 2; ++n) {
-        for (int i = 0; i < 8; ++i) {
-            uint8_t *ta = tl + n * 1024 + lane * 16 + i, *tb = ta + 8;
-            uint8_t *ra = rm + 64 * n + 8 * g + i, *rb = ra + 32;
-            uint8_t *th = tl + 2048 + lane * 16 + 8 * n + i;
-            uint8_t *rh = rm + 128 + 32 * n + 8 * g + i;
-            if (TO_TILED) {
-                *ta = live ? *ra : 0; *tb = live ? *rb : 0; *th = live ? *rh : 0;
-            } else {
-                *ra = *ta; *rb = *tb; *rh = *th;
-            }
-        }
+    uint16_t *t_ql = reinterpret_cast<uint16_t *>(tl + r * 128 + 32 * c);          // 16 words
+    uint16_t *t_qh = reinterpret_cast<uint16_t *>(tl + 2048 + r * 64 + 16 * c);    // 8 words
+    uint16_t *t_sc = reinterpret_cast<uint16_t *>(tl + 3072 + r * 16);             // 8 words
+    uint16_t *t_d = reinterpret_cast<uint16_t *>(tl + 3328 + r * 2);
+    uint16_t *r_ql = rm + 16 * c, *r_qh = rm + 64 + 8 * c, *r_sc = rm + 96, *r_d = rm + 104;
+    for (int i = 0; i < 16; ++i) {
+        if (TO_TILED) t_ql[i] = live ? r_ql[i] : (uint16_t)0; else r_ql[i] = t_ql[i];
     }
-    if (g == 0) {
-        for (int i = 0; i < 16; ++i) {
-            if (TO_TILED) tl[3072 + r * 16 + i] = live ? rm[192 + i] : 0;
-            else rm[192 + i] = tl[3072 + r * 16 + i];
+    for (int i = 0; i < 8; ++i) {
+        if (TO_TILED) t_qh[i] = live ? r_qh[i] : (uint16_t)0; else r_qh[i] = t_qh[i];
+    }
+    if (c == 0) {
+        for (int i = 0; i < 8; ++i) {
+            if (TO_TILED) t_sc[i] = live ? r_sc[i] : (uint16_t)0; else r_sc[i] = t_sc[i];
         }
-        for (int i = 0; i < 2; ++i) {
-            if (TO_TILED) tl[3328 + r * 2 + i] = live ? rm[208 + i] : 0;
-            else rm[208 + i] = tl[3328 + r * 2 + i];
-        }
+        if (TO_TILED) *t_d = live ? *r_d : (uint16_t)0; else *r_d = *t_d;
     }
 }
 
@@ -79,8 +63,9 @@ static int repack_common(bool to_tiled, int type, const void *src, void *dst, in
     if (!type_is_tiled(type)) return fail(MESH_ERR_INVALID, "repack: type %d has no tiled layout", type);
     if (!src || !dst || M <= 0 || K <= 0 || K % QK_K) return fail(MESH_ERR_INVALID, "repack: bad shape M=%lld K=%lld", (long long)M, (long long)K);
     const int nsb = (int)(K / QK_K);
-    const dim3 grid((unsigned)nsb, (unsigned)(padded_rows(M) / TILE_ROWS));
-    if (grid.y > 65535u * 16u) return fail(MESH_ERR_INVALID, "repack: too many rows");
+    const int64_t tile_rows = padded_rows(M) / TILE_ROWS;
+    if (tile_rows > 65535) return fail(MESH_ERR_INVALID, "repack: %lld rows exceed the launch grid", (long long)M);
+    const dim3 grid((unsigned)nsb, (unsigned)tile_rows);
     const uint8_t *s = static_cast<const uint8_t *>(src);
     uint8_t *d = static_cast<uint8_t *>(dst);
     if (type == MESH_Q4_K) {

@@ -228,7 +228,7 @@ static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
     return MESH_OK;
 }
 
-constexpr int ATTN_SPLITS_MAX = 64;
+constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
 
