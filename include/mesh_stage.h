@@ -187,6 +187,15 @@ typedef struct mesh_profile {
 int mesh_session_profile(mesh_session *session, int enable);          /* also resets the counters */
 int mesh_session_profile_read(mesh_session *session, mesh_profile *out);   /* waits for the stream */
 
+/* Mixture-of-experts sessions: restrict routing to a subset of the file's experts.  allowed[e] != 0 keeps expert
+ * e; NULL clears the mask.  MESH_ERR_INVALID if n_mask differs from the expert count of the file.  The C API of
+ * llama_model_set_expert_mask (patches/0003:46-50: 0 on success, -1 on a count mismatch); the mask is added as
+ * 0 / -inf to the selection probabilities before top-k (patches/0003:86-104). */
+int mesh_session_set_expert_mask(mesh_session *session, const uint8_t *allowed, int32_t n_mask);
+/* Expert ids chosen for the tokens of the last decode call in the LAST mixture-of-experts layer of the stage:
+ * ids[n_tokens][n_expert_used].  For tests and for counting distinct experts touched. */
+int mesh_session_moe_last_ids(mesh_session *session, int32_t *ids, int32_t n_tokens);
+
 /* KV cache import/export for one sequence and one (absolute) layer: n_pos positions starting at pos0, host
  * buffers of f16 bits laid out [n_pos][n_head_kv][head_dim].  (The reference has no KV hand-over; a restarted
  * stage refills from the prompt -- mesh-llm/src/inference/election.rs:1894-1910.) */

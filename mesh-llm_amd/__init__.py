@@ -100,6 +100,8 @@ SIGNATURES.update({
     "mesh_session_synchronize": (_i32, [_vp]),
     "mesh_session_profile": (_i32, [_vp, _i32]),
     "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
+    "mesh_session_set_expert_mask": (_i32, [_vp, _vp, _i32]),
+    "mesh_session_moe_last_ids": (_i32, [_vp, _vp, _i32]),
     "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
 })
@@ -314,6 +316,21 @@ class Session:
         check(lib().mesh_session_profile_read(self._h, ctypes.byref(p)))
         names = ("gemv", "rope", "attn", "codec")
         return {n: {"ms": p.ms[i], "launches": int(p.launches[i])} for i, n in enumerate(names)}
+
+    def set_expert_mask(self, allowed):
+        """allowed: bool array over the file's experts, or None to clear."""
+        import numpy as np
+        if allowed is None:
+            check(lib().mesh_session_set_expert_mask(self._h, None, 0))
+            return
+        a = np.ascontiguousarray(allowed, dtype=np.uint8)
+        check(lib().mesh_session_set_expert_mask(self._h, _np_ptr(a), a.size))
+
+    def moe_last_ids(self, n_tokens):
+        import numpy as np
+        out = np.empty((n_tokens, self.stage.info.n_expert_used), dtype=np.int32)
+        check(lib().mesh_session_moe_last_ids(self._h, _np_ptr(out), n_tokens))
+        return out
 
     def kv_write(self, layer, seq_id, pos0, k, v):
         """k, v: uint16 arrays [n_pos, n_head_kv, head_dim] of f16 bits."""

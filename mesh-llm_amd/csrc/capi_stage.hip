@@ -1,5 +1,6 @@
 // extern "C" entry points for weights, GGUF inspection and the stage executor (include/mesh_stage.h).
 
+#include <cmath>
 #include <cstring>
 #include <vector>
 
@@ -171,6 +172,31 @@ int mesh_session_profile_read(mesh_session *session, mesh_profile *out) {
     int rc = profile_collect(session);
     if (rc != MESH_OK) return rc;
     for (int i = 0; i < MESH_PROF_KINDS; ++i) { out->ms[i] = session->prof_ms[i]; out->launches[i] = session->prof_launches[i]; }
+    return MESH_OK;
+}
+
+int mesh_session_set_expert_mask(mesh_session *session, const uint8_t *allowed, int32_t n_mask) {
+    if (!session) return fail(MESH_ERR_INVALID, "mesh_session_set_expert_mask: null session");
+    const mesh_stage *st = session->stage;
+    if (!session->expert_mask) return fail(MESH_ERR_INVALID, "mesh_session_set_expert_mask: the stage has no mixture-of-experts layers");
+    if (!allowed) { session->expert_mask_on = false; return MESH_OK; }
+    const int ne = (int)st->layers[0].gate_inp.M;
+    if (n_mask != ne) return fail(MESH_ERR_INVALID, "mesh_session_set_expert_mask: mask has %d entries, the file holds %d experts", n_mask, ne);
+    std::vector<float> m((size_t)ne);
+    for (int e = 0; e < ne; ++e) m[(size_t)e] = allowed[e] ? 0.0f : -INFINITY;
+    MESH_HIP_TRY(hipSetDevice(st->device));
+    MESH_HIP_TRY(hipStreamSynchronize(session->stream));
+    MESH_HIP_TRY(hipMemcpy(session->expert_mask, m.data(), m.size() * sizeof(float), hipMemcpyHostToDevice));
+    session->expert_mask_on = true;
+    return MESH_OK;
+}
+
+int mesh_session_moe_last_ids(mesh_session *session, int32_t *ids, int32_t n_tokens) {
+    if (!session || !ids || !session->moe_ids) return fail(MESH_ERR_INVALID, "mesh_session_moe_last_ids: no mixture-of-experts state");
+    const mesh_stage *st = session->stage;
+    if (n_tokens <= 0 || n_tokens > st->n_batch_max) return fail(MESH_ERR_INVALID, "mesh_session_moe_last_ids: bad token count");
+    MESH_HIP_TRY(hipStreamSynchronize(session->stream));
+    MESH_HIP_TRY(hipMemcpy(ids, session->moe_ids, (size_t)n_tokens * st->hp.n_expert_used * sizeof(int32_t), hipMemcpyDeviceToHost));
     return MESH_OK;
 }
 

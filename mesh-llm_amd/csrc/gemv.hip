@@ -47,6 +47,11 @@ struct GemvKernelArgs {
     int ldres;
     int epi;
     int ks;                // waves along K (the other 16/ks ways split the workgroup's tile-rows)
+    // expert indirection (MoE): blockIdx.y = (token, slot) pair p; it uses expert expert_ids[p]'s copy of every
+    // matrix (expert_stride bytes apart), reads activation column p / x_div and writes output row p
+    const int32_t *expert_ids;
+    size_t expert_stride;
+    int x_div;
 };
 
 // LDS view of the quantised activations of NB columns
@@ -89,14 +94,14 @@ struct XRegs {
 };
 
 template <int NB>
-__device__ __forceinline__ void x_fetch(XRegs<NB> &X, const GemvKernelArgs &a, int g, bool live) {
+__device__ __forceinline__ void x_fetch(XRegs<NB> &X, const float *__restrict__ x, int ldx, int g, bool live) {
 #pragma unroll
     for (int t = 0; t < NB; ++t) {
         X.a[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         X.b[t] = X.a[t];
         if (live) {
-            X.a[t] = *reinterpret_cast<const float4 *>(a.x + (size_t)t * a.ldx + g * 8);
-            X.b[t] = *reinterpret_cast<const float4 *>(a.x + (size_t)t * a.ldx + g * 8 + 4);
+            X.a[t] = *reinterpret_cast<const float4 *>(x + (size_t)t * ldx + g * 8);
+            X.b[t] = *reinterpret_cast<const float4 *>(x + (size_t)t * ldx + g * 8 + 4);
         }
     }
 }
@@ -299,8 +304,16 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
     GEMV_MARK(0);
     // activations first: they gate everything
     const int ng = K >> 3;
+    const float *xcol = a.x;
+    size_t eoff = 0, ycol = 0;
+    if (a.expert_ids) {
+        const int p = blockIdx.y;
+        xcol = a.x + (size_t)(p / a.x_div) * a.ldx;
+        eoff = (size_t)a.expert_ids[p] * a.expert_stride;
+        ycol = p;
+    }
     XRegs<NB> X;
-    x_fetch<NB>(X, a, tid, tid < ng);
+    x_fetch<NB>(X, xcol, a.ldx, tid, tid < ng);
 
     const int nsb = K / QK_K;
     const int KS = a.ks, RS = GEMV_WAVES / KS;
@@ -316,7 +329,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
         const int tr = tr0 + c.j;
         int mi = c.u;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        return a.wbase[mi] + (size_t)tr * row_stride + (size_t)(ks + KS * c.ii) * TB;
+        return a.wbase[mi] + eoff + (size_t)tr * row_stride + (size_t)(ks + KS * c.ii) * TB;
     };
 
     TileCursor<NU> ld{rs, 0, 0}, cp{rs, 0, 0};
@@ -334,7 +347,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
     for (int t = 0; t < NB; ++t) ss[t] = 0.f;
     x_quantise<NB, NEED_I16>(X, a, S, tid, tid < ng, ss);
     for (int g0 = GEMV_THREADS; g0 < ng; g0 += GEMV_THREADS) {
-        x_fetch<NB>(X, a, g0 + tid, g0 + tid < ng);
+        x_fetch<NB>(X, xcol, a.ldx, g0 + tid, g0 + tid < ng);
         x_quantise<NB, NEED_I16>(X, a, S, g0 + tid, g0 + tid < ng, ss);
     }
     if (a.norm_w) {
@@ -411,7 +424,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
         } else {
             out = s0;
         }
-        a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
+        a.y[mi][((size_t)t + ycol) * a.ldy[mi] + row] = out;
     }
     GEMV_MARK(5);
 }
@@ -425,20 +438,20 @@ static size_t dot_smem_bytes(int type, int NB, int K, int rows_here, int KS, int
 }
 
 template <int TYPE, int NB, int NU>
-static int launch_dot(const GemvKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
+static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
         MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dot_kernel<TYPE, NB, NU>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dot_kernel<TYPE, NB, NU><<<dim3((unsigned)grid), dim3(GEMV_THREADS), smem, stream>>>(ka);
+    gemv_dot_kernel<TYPE, NB, NU><<<grid, dim3(GEMV_THREADS), smem, stream>>>(ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
 template <int TYPE, int NU>
-static int launch_dot_nb(int nb, const GemvKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
+static int launch_dot_nb(int nb, const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
     if (nb == 4) return launch_dot<TYPE, 4, NU>(ka, grid, smem, stream);
     if (nb == 2) return launch_dot<TYPE, 2, NU>(ka, grid, smem, stream);
     return launch_dot<TYPE, 1, NU>(ka, grid, smem, stream);
@@ -486,13 +499,28 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     ka.epi = a.epi;
     const int KS = nsb < GEMV_WAVES ? nsb : GEMV_WAVES;
     ka.ks = KS;
+    const int n_pairs = a.expert_ids ? a.n_pairs : 1;
+    if (a.expert_ids) {
+        if (a.n_pairs <= 0 || a.x_div <= 0 || a.epi == EPI_RESIDUAL) return fail(MESH_ERR_INVALID, "gemv: bad expert-indirection arguments");
+        ka.expert_ids = a.expert_ids;
+        ka.expert_stride = (size_t)tiled_bytes(type, a.mat[0].M, a.K);
+        ka.x_div = a.x_div;
+    }
     // tile-rows per workgroup: spread over the CUs, bounded by the LDS partial buffer
-    const int ncu = n_compute_units();
+    const int ncu = std::max(1, n_compute_units() / n_pairs);
     int rows_per_wg = (total_rows + ncu - 1) / ncu;
     rows_per_wg = std::max(1, std::min(rows_per_wg, MAX_ROWS_X_KS / KS));
     const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
     const int rows_max = (total_rows + grid - 1) / grid;
     if (dot_smem_bytes(type, 1, a.K, rows_max, KS, NU) > LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemv: row length %d does not fit LDS", a.K);
+    if (a.expert_ids) {
+        // every pair is its own single-column product
+        ka.x = a.x;
+        const size_t smem = dot_smem_bytes(type, 1, a.K, rows_max, KS, NU);
+        const dim3 g((unsigned)grid, (unsigned)n_pairs);
+        if (type == MESH_Q4_K) return NU == 2 ? launch_dot_nb<MESH_Q4_K, 2>(1, ka, g, smem, stream) : launch_dot_nb<MESH_Q4_K, 1>(1, ka, g, smem, stream);
+        return NU == 2 ? launch_dot_nb<MESH_Q6_K, 2>(1, ka, g, smem, stream) : launch_dot_nb<MESH_Q6_K, 1>(1, ka, g, smem, stream);
+    }
     int t = 0;
     while (t < a.T) {
         const int left = a.T - t;
@@ -505,8 +533,9 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
             if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
         const size_t smem = dot_smem_bytes(type, nb, a.K, rows_max, KS, NU);
         int rc;
-        if (type == MESH_Q4_K) rc = NU == 2 ? launch_dot_nb<MESH_Q4_K, 2>(nb, kb, grid, smem, stream) : launch_dot_nb<MESH_Q4_K, 1>(nb, kb, grid, smem, stream);
-        else rc = NU == 2 ? launch_dot_nb<MESH_Q6_K, 2>(nb, kb, grid, smem, stream) : launch_dot_nb<MESH_Q6_K, 1>(nb, kb, grid, smem, stream);
+        const dim3 g((unsigned)grid);
+        if (type == MESH_Q4_K) rc = NU == 2 ? launch_dot_nb<MESH_Q4_K, 2>(nb, kb, g, smem, stream) : launch_dot_nb<MESH_Q4_K, 1>(nb, kb, g, smem, stream);
+        else rc = NU == 2 ? launch_dot_nb<MESH_Q6_K, 2>(nb, kb, g, smem, stream) : launch_dot_nb<MESH_Q6_K, 1>(nb, kb, g, smem, stream);
         if (rc != MESH_OK) return rc;
         t += nb;
     }
@@ -532,6 +561,8 @@ int gemv(const GemvArgs &a, hipStream_t stream) {
         uniform = uniform && same;
     }
     if (a.T == 0) return MESH_OK;
+    if (a.expert_ids && !(uniform && type_is_tiled(a.mat[0].type)))
+        return fail(MESH_ERR_UNSUPPORTED, "gemv: expert indirection needs K-quant expert matrices of one type");
     if (uniform) return type_is_tiled(a.mat[0].type) ? gemv_kquant(a, stream) : gemv_generic(a, stream);
     if (a.epi == EPI_SWIGLU) return fail(MESH_ERR_UNSUPPORTED, "gemv: gate and up of different types");
     // mixed types side by side (a q/k/v group whose v is q6_K): one launch per run of equal family

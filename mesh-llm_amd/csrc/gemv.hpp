@@ -58,6 +58,12 @@ struct GemvArgs {
     const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y
     int ldres = 0;
     int epi = EPI_STORE;
+    // Expert indirection (MoE): when expert_ids is set, the launch runs n_pairs independent single-column products;
+    // pair p uses expert expert_ids[p] (device array) of every matrix -- W points at expert 0, experts are stacked --
+    // reads activation column p / x_div of x and writes row p of y.  T is ignored.
+    const int32_t *expert_ids = nullptr;
+    int n_pairs = 0;
+    int x_div = 1;
 };
 
 int gemv(const GemvArgs &a, hipStream_t stream);

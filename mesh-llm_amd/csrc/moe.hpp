@@ -1,0 +1,19 @@
+// Mixture-of-experts routing launchers (moe.hip).
+#pragma once
+
+#include "mesh_common.hpp"
+
+namespace mesh {
+
+struct MoeRouteArgs {
+    const float *logits = nullptr;   // [T][n_expert] router outputs
+    const float *mask = nullptr;     // optional [n_expert]: 0 = allowed, -inf = masked out
+    int32_t *ids = nullptr;          // [T][top_k]
+    float *weights = nullptr;        // [T][top_k]
+    int n_expert = 0, top_k = 0, norm_w = 1;
+};
+int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream);
+// x[t] += sum_s weights[t][s] * y[t*top_k + s]
+int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
+
+}  // namespace mesh

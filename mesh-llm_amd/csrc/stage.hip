@@ -16,6 +16,7 @@
 
 #include "attn.hpp"
 #include "gemv.hpp"
+#include "moe.hpp"
 
 namespace mesh {
 
@@ -264,6 +265,15 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
     if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
+    if (hp.n_expert_used > 0 && !st->layers.empty() && st->layers[0].gate_inp.present()) {
+        const size_t ne = (size_t)st->layers[0].gate_inp.M, k = hp.n_expert_used;
+        if ((rc = fbuf(&s->moe_logits, B * ne)) || (rc = fbuf(&s->moe_w, B * k)) || (rc = fbuf(&s->moe_out, B * k * hp.n_embd)) ||
+            (rc = fbuf(&s->expert_mask, ne)))
+            return rc;
+        if ((rc = sess_alloc(s.get(), &p, B * k * sizeof(int32_t))) != MESH_OK) return rc;
+        s->moe_ids = static_cast<int32_t *>(p);
+        MESH_HIP_TRY(hipMemsetAsync(s->expert_mask, 0, ne * sizeof(float), s->stream));
+    }
     if ((rc = sess_alloc(s.get(), &p, 3 * B * sizeof(int32_t))) != MESH_OK) return rc;
     s->d_pos = static_cast<int32_t *>(p);
     s->d_seq = s->d_pos + B;
@@ -382,7 +392,40 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(oa, stream); }
         if (rc != MESH_OK) return rc;
 
-        if (!L.w_gate.present()) return fail(MESH_ERR_UNSUPPORTED, "mixture-of-experts layers are not executable yet");
+        if (!L.w_gate.present()) {
+            // mixture of experts: router -> top-k -> per-(token, slot) expert FFN -> weighted sum into x
+            const int ne = (int)L.gate_inp.M, k = (int)hp.n_expert_used, ffe = (int)hp.n_ff_exp;
+            GemvArgs ra2;
+            ra2.n_mat = 1;
+            ra2.mat[0] = mat_of(L.gate_inp, s->moe_logits, ne, nullptr);
+            ra2.x = s->x; ra2.ldx = E; ra2.K = E; ra2.T = T;
+            ra2.norm_w = static_cast<const float *>(L.ffn_norm.data); ra2.eps = hp.rms_eps;
+            { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ra2, stream); }
+            if (rc != MESH_OK) return rc;
+            MoeRouteArgs mr;
+            mr.logits = s->moe_logits; mr.mask = s->expert_mask_on ? s->expert_mask : nullptr;
+            mr.ids = s->moe_ids; mr.weights = s->moe_w; mr.n_expert = ne; mr.top_k = k; mr.norm_w = 1;
+            if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
+            GemvArgs ea;
+            ea.n_mat = 2;
+            ea.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);
+            ea.mat[1] = mat_of(L.up_exps, nullptr, ffe, nullptr);
+            ea.x = s->x; ea.ldx = E; ea.K = E; ea.T = 1;
+            ea.norm_w = static_cast<const float *>(L.ffn_norm.data); ea.eps = hp.rms_eps;
+            ea.epi = EPI_SWIGLU;
+            ea.expert_ids = s->moe_ids; ea.n_pairs = T * k; ea.x_div = k;
+            { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ea, stream); }
+            if (rc != MESH_OK) return rc;
+            GemvArgs xa;
+            xa.n_mat = 1;
+            xa.mat[0] = mat_of(L.down_exps, s->moe_out, E, nullptr);
+            xa.x = s->ffn; xa.ldx = ffe; xa.K = ffe; xa.T = 1;
+            xa.expert_ids = s->moe_ids; xa.n_pairs = T * k; xa.x_div = 1;
+            { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(xa, stream); }
+            if (rc != MESH_OK) return rc;
+            if ((rc = moe_combine(s->x, s->moe_out, s->moe_w, T, E, k, stream)) != MESH_OK) return rc;
+            continue;
+        }
         // ffn = silu(Wgate . n) * (Wup . n),  n = rms_norm(x)
         GemvArgs ga;
         ga.n_mat = 2;

@@ -74,7 +74,8 @@ struct mesh_session {
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
-    float *moe_logits = nullptr, *moe_w = nullptr, *expert_mask = nullptr;
+    float *moe_logits = nullptr, *moe_w = nullptr, *moe_out = nullptr, *expert_mask = nullptr;
+    bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)

@@ -368,27 +368,28 @@ void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcach
     }
 }
 
-/* MoE gating as llama.cpp's build_moe_ffn runs it for softmax-gated models, with the expert mask of
- * patches/0003:86-104 (a 0 / -inf vector ADDED to the router logits before selection). */
+/* MoE gating as llama.cpp's build_moe_ffn runs it for softmax-gated models (qwen3moe), with the expert mask of
+ * patches/0003:86-104: probs = softmax(logits) over every expert in the file; the 0 / -inf mask is ADDED to the
+ * probabilities used for selection only (selection_probs); the weights are the unmasked probs of the selected
+ * experts, divided by their sum when norm_w is set.  Ties go to the lower expert id. */
 void mo_moe_route(const float *logits, const float *mask, int n_expert, int top_k, int norm_w,
                   int32_t *ids, float *weights) {
     double *p = (double *)malloc((size_t)n_expert * sizeof(double));
     double mx = -INFINITY;
-    for (int e = 0; e < n_expert; e++) {
-        p[e] = (double)logits[e] + (mask ? (double)mask[e] : 0.0);
-        if (p[e] > mx) mx = p[e];
-    }
+    for (int e = 0; e < n_expert; e++) if ((double)logits[e] > mx) mx = (double)logits[e];
     double den = 0.0;
-    for (int e = 0; e < n_expert; e++) { p[e] = exp(p[e] - mx); den += p[e]; }
+    for (int e = 0; e < n_expert; e++) { p[e] = exp((double)logits[e] - mx); den += p[e]; }
     for (int e = 0; e < n_expert; e++) p[e] /= den;
     double wsum = 0.0;
     for (int k = 0; k < top_k; k++) {
         int best = -1;
+        double best_sel = 0.0;
         for (int e = 0; e < n_expert; e++) {
             int taken = 0;
             for (int j = 0; j < k; j++) taken |= (ids[j] == e);
             if (taken) continue;
-            if (best < 0 || p[e] > p[best]) best = e;
+            const double sel = p[e] + (mask ? (double)mask[e] : 0.0);
+            if (best < 0 || sel > best_sel) { best = e; best_sel = sel; }
         }
         ids[k] = best;
         weights[k] = (float)p[best];

@@ -66,8 +66,8 @@ void mo_swiglu(const float *gate, const float *up, float *out, int64_t n);
 void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcache,
                    int n_head, int n_kv, int head_dim, int64_t ctx_stride, int64_t n_past,
                    float scale, float *out);
-/* MoE router: probs = softmax(logits + mask) over n_expert, top-k ids by probability
- * (ties: lower id first), weights = selected probs, optionally renormalised to sum 1. */
+/* MoE router: probs = softmax(logits) over n_expert; top-k ids by (probs + mask), mask 0 / -inf (ties: lower id
+ * first); weights = unmasked probs of the selected experts, optionally renormalised to sum 1. */
 void mo_moe_route(const float *logits, const float *mask, int n_expert, int top_k, int norm_w,
                   int32_t *ids, float *weights);
 

@@ -176,3 +176,55 @@ def test_decode_argument_errors(tmp_path):
         ses.decode(x[:1], [0], out_fmt=m.LOGITS)
     ses.close()
     st.close()
+
+
+def test_moe_stage_matches_oracle_with_and_without_mask(tmp_path):
+    m, cfg, tensors, st = _open(tmp_path, "tiny-moe", range(0, 2), 0, 2)
+    ses = st.session()
+    rng = np.random.Generator(np.random.PCG64(21))
+    E = cfg["n_embd"]
+    x = rng.standard_normal((6, E)).astype(np.float32)
+    orc = StageOracle(cfg, tensors, 0, 2, 64)
+    got = ses.decode(x, np.arange(6)).view(np.float32).reshape(6, E)
+    ref = orc.forward(x, np.arange(6))
+    assert rel_l2(got, ref) <= 1e-3
+    assert np.array_equal(np.sort(ses.moe_last_ids(6), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+    # expert mask: only 3 of the 8 experts allowed (0 / -inf added to the selection probabilities)
+    allowed = np.zeros(8, bool)
+    allowed[[1, 4, 6]] = True
+    ses2 = st.session()
+    ses2.set_expert_mask(allowed)
+    orc2 = StageOracle(cfg, tensors, 0, 2, 64, expert_mask=np.where(allowed, 0.0, -np.inf).astype(np.float32))
+    got = ses2.decode(x, np.arange(6)).view(np.float32).reshape(6, E)
+    ref2 = orc2.forward(x, np.arange(6))
+    assert rel_l2(got, ref2) <= 1e-3
+    assert set(ses2.moe_last_ids(6).reshape(-1)) <= {1, 4, 6}
+    assert rel_l2(ref2, ref) > 1e-2            # the mask really changed the result
+    with pytest.raises(m.MeshError) as e:
+        ses2.set_expert_mask(np.ones(5, bool))
+    assert e.value.code == m.ERR_INVALID
+    ses2.set_expert_mask(None)
+    ses.close(); ses2.close(); st.close()
+
+
+def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
+    """One real-shape MoE layer of a 64-expert shard (of 128), decode batch 16, top-8 routing."""
+    m = mesh()
+    cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
+    path = os.path.join(str(tmp_path), "shard.gguf")
+    tensors = models.write_model(path, cfg, [5], seed=9, n_expert_local=64, fast=True)
+    st = m.Stage(path, 5, 6, n_ctx=64, n_seq_max=16, n_batch_max=16)
+    os.unlink(path)
+    assert st.info.n_expert == 64 and st.info.n_expert_used == 8
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 5, 6, 64, n_seq_max=16)
+    rng = np.random.Generator(np.random.PCG64(31))
+    x = rng.standard_normal((16, 2048)).astype(np.float32)
+    pos, seq = np.zeros(16, np.int32), np.arange(16, dtype=np.int32)
+    got = ses.decode(x, pos, seq=seq).view(np.float32).reshape(16, 2048)
+    ref = orc.forward(x, pos, seq=seq)
+    assert rel_l2(got, ref) <= 1e-3
+    ids = ses.moe_last_ids(16)
+    assert np.array_equal(np.sort(ids, axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+    assert len(set(ids.reshape(-1))) > 8
+    ses.close(); st.close()

@@ -117,12 +117,26 @@ def test_moe_route_vs_numpy():
         if trial % 2:
             mask[rng.choice(128, 64, replace=False)] = -np.inf
         ids, w = oracle.moe_route(logits, mask, 8, True)
-        z = logits.astype(np.float64) + mask
+        z = logits.astype(np.float64)
         p = np.exp(z - z.max())
-        p /= p.sum()
-        order = np.argsort(-p, kind="stable")[:8]
+        p /= p.sum()                                   # softmax over ALL experts; the mask only steers selection
+        order = np.argsort(-(p + mask), kind="stable")[:8]
         assert list(ids) == list(order)
         assert np.allclose(w, p[order] / p[order].sum(), rtol=1e-6)
         assert np.all(mask[ids] == 0)
         ids2, w2 = oracle.moe_route(logits, mask, 8, False)
         assert list(ids2) == list(order) and np.allclose(w2, p[order], rtol=1e-6)
+
+
+def test_moe_shard_equals_masked_full_model():
+    # a shard file holds the router rows of its experts only: with normalised weights, routing over the shard's
+    # logits equals routing over all logits with the other experts masked
+    rng = RNG(9)
+    logits = rng.standard_normal(128).astype(np.float32)
+    keep = np.sort(rng.choice(128, 64, replace=False))
+    mask = np.full(128, -np.inf, np.float32)
+    mask[keep] = 0
+    ids_full, w_full = oracle.moe_route(logits, mask, 8, True)
+    ids_shard, w_shard = oracle.moe_route(logits[keep], None, 8, True)
+    assert list(keep[ids_shard]) == list(ids_full)
+    assert np.allclose(w_shard, w_full, rtol=1e-5)
