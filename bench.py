@@ -224,7 +224,7 @@ def bench_stage(args):
         "config": {"workload": "Llama-3-8B-shaped stage, layers 0-15 of 32, Q4_K_M block-domain random weights, decode batch %d, "
                                "4096-token f16 KV context, f32 hidden state in HBM -> q8_0 boundary activation out" % batches[0],
                    "weight_bytes": weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<1> (q4_K/q6_K dequant-fused mat-vec)",
+        "roofline": {"bound": "hbm", "kernel": "gemv_dot_kernel<type,1,NU> (q4_K/q6_K dequant-fused mat-vec, all instantiations)",
                      "achieved": round(gemv_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gemv_gbs / HBM_PEAK_GBS, 4),
                      "traffic": None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
                      "algorithmic_bytes_per_launch": weight_bytes // g_n},
