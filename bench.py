@@ -127,6 +127,7 @@ def bench_codec(args):
 # ------------------------------------------------------------------------------------------------ stage
 N_CTX = 4096
 STAGE_LAYERS = 16
+PREFILL_T = 2048
 
 
 def build_stage_model(models, path):
@@ -172,7 +173,7 @@ def bench_stage(args):
     batches = sorted(set(int(b) for b in args.batches.split(",")))
     bmax = max(batches)
     t0 = time.perf_counter()
-    st = m.Stage(path, 0, STAGE_LAYERS, n_ctx=N_CTX, n_seq_max=bmax, n_batch_max=max(bmax, 16))
+    st = m.Stage(path, 0, STAGE_LAYERS, n_ctx=N_CTX, n_seq_max=bmax, n_batch_max=max(bmax, 16, PREFILL_T if args.prefill else 0))
     t_load = time.perf_counter() - t0
     os.unlink(path)
     weight_bytes = st.weight_bytes
@@ -210,6 +211,31 @@ def bench_stage(args):
                       "GBps": round(step_bytes / ms / 1e6, 1), "frac_hbm": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                       "kernel_ms_per_step": {k: round(v["ms"] / 5, 4) for k, v in prof.items()},
                       "kernel_launches_per_step": {k: v["launches"] // 5 for k, v in prof.items()}}
+    prefill = None
+    if args.prefill:
+        # prompt ingestion: 2048 tokens of sequence 0 in one call (MFMA GEMM path); done last, it overwrites the KV context
+        xp = torch.from_numpy(rng.standard_normal((PREFILL_T, E)).astype(np.float32)).cuda()
+        outp = torch.empty(m.act_packed_size(m.Q8_0, PREFILL_T, E), dtype=torch.uint8, device="cuda")
+        ppos = np.arange(PREFILL_T, dtype=np.int32)
+
+        def pstep(i):
+            ses.decode_dev(xp.data_ptr(), ppos, outp.data_ptr(), outp.numel(), in_fmt=m.F32, out_fmt=m.Q8_0)
+
+        pms, _ = time_on_stream(torch, stream, pstep, 3, 1)
+        ses.profile(True)
+        pstep(0)
+        pprof = ses.profile_read()
+        ses.profile(False)
+        H, HD, FF = cfg["n_head"], cfg["head_dim"], cfg["n_ff"]
+        mm_flop = 2.0 * PREFILL_T * STAGE_LAYERS * (E * H * HD * 2 + E * HK * HD * 2 + 3 * E * FF)
+        at_flop = 4.0 * STAGE_LAYERS * H * HD * PREFILL_T * (PREFILL_T + 1) / 2
+        gemm_ms = pprof["gemv"]["ms"]
+        prefill = {"tokens": PREFILL_T, "ms": round(pms, 2), "tok_s": round(PREFILL_T * 1e3 / pms, 1),
+                   "matmul_TFLOP": round(mm_flop / 1e12, 3), "attention_TFLOP": round(at_flop / 1e12, 3),
+                   "stage_TFLOPs": round((mm_flop + at_flop) / pms / 1e9, 1),
+                   "gemm_ms": round(gemm_ms, 2), "gemm_TFLOPs": round(mm_flop / gemm_ms / 1e9, 1),
+                   "gemm_frac_mfma_f16_peak": round(mm_flop / gemm_ms / 1e9 / 2500.0, 4),
+                   "kernel_ms": {k: round(v["ms"], 2) for k, v in pprof.items()}}
     b1 = results[batches[0]]
     # roofline of the dominant kernel (the dequant-fused GEMV): all of a step's weight bytes pass through its
     # launches, so the average launch moves weight_bytes / launches in kernel_ms / launches
@@ -230,6 +256,7 @@ def bench_stage(args):
                      "algorithmic_bytes_per_launch": weight_bytes // g_n},
         "stage_frac_hbm": b1["frac_hbm"],
         "decode": {str(k): v for k, v in results.items()},
+        "prefill": prefill,
         "codec": codec,
         "setup_s": {"generate_gguf": round(t_gen, 1), "open_stage": round(t_load, 1)},
     }
@@ -248,6 +275,7 @@ def main():
     ap.add_argument("--workload", default="stage", choices=["stage", "codec"])
     ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-prefill", dest="prefill", action="store_false", help="skip the 2048-token prefill measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the stage path (one GPU per box); --gpus %d is not supported" % args.gpus,

@@ -1,0 +1,243 @@
+// Prefill GEMM: Y[T][M] = X[T][K] . W^T with W in tiled q4_K / q6_K blocks (gemv.hpp) and X in f16.
+// The many-token counterpart of the decode GEMV -- what ggml_backend_graph_compute runs for mul_mat when a prompt is
+// ingested (third_party/llama.cpp/patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451).
+//
+// Design (gfx950): a 256-thread workgroup owns a 128 (weight rows) x 128 (tokens) output tile and walks K in
+// steps of 64.  Per step the 128 x 64 weight slab is dequantised from its K-quant blocks straight into LDS as
+// f16 (each thread: one row, one 32-element sub-block), the 128 x 64 activation slab is copied next to it, and
+// the four waves (2 x 2, 64 x 64 each) issue v_mfma_f32_32x32x16_f16 on 16-byte LDS fragments with f32
+// accumulation.  Weights cross HBM once per 128 tokens; dequantisation is amortised over 128 columns.
+//
+// MFMA operand layout used below (checked on hardware): A lane l = row l%32, k = 8*(l/32)+j; B lane l = column
+// l%32, same k; accumulator register i of lane l = D[8*(i/4) + 4*(l/32) + i%4][l%32].
+
+#include "gemm.hpp"
+
+namespace mesh {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int GM = 128, GN = 128, GK = 64;     // workgroup tile: weight rows x tokens x k-step
+constexpr int LDS_LD = GK + 8;                 // f16 elements per LDS row (16-byte pad against bank conflicts)
+constexpr int GEMM_THREADS = 256;
+
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+    return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+}
+
+// 32 dequantised elements (one sub-block of one row) -> 64 bytes of LDS
+__device__ __forceinline__ void store32(_Float16 *dst, const float (&v)[32]) {
+    uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        d4[i] = make_uint4(pack_h2(v[8 * i], v[8 * i + 1]), pack_h2(v[8 * i + 2], v[8 * i + 3]),
+                           pack_h2(v[8 * i + 4], v[8 * i + 5]), pack_h2(v[8 * i + 6], v[8 * i + 7]));
+}
+
+// q4_K: row r of tile, k-chunk c (64 elements) of the super-block, half h (sub-block 2c + h)
+__device__ __forceinline__ void dequant_q4k_32(const uint8_t *__restrict__ tile, int r, int c, int h, _Float16 *dst) {
+    const uint4 hdr = *reinterpret_cast<const uint4 *>(tile + r * 16);
+    const uint4 qa = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32);
+    const uint4 qb = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32 + 16);
+    const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+    const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
+    const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
+    const int sh = (c & 1) * 16 + h * 8;
+    const float ds = d * (float)((scw >> sh) & 0xFFu), dm = dmin * (float)((mnw >> sh) & 0xFFu);
+    const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t q = (w[j] >> (4 * h)) & 0x0F0F0F0Fu;
+        v[4 * j + 0] = fmaf(ds, (float)(q & 0xFFu), -dm);
+        v[4 * j + 1] = fmaf(ds, (float)((q >> 8) & 0xFFu), -dm);
+        v[4 * j + 2] = fmaf(ds, (float)((q >> 16) & 0xFFu), -dm);
+        v[4 * j + 3] = fmaf(ds, (float)(q >> 24), -dm);
+    }
+    store32(dst, v);
+}
+
+// q6_K: row r, k-chunk c: half n = c/2, elements 128n + 32*t4 + l with t4 = 2*(c%2) + h, l = 0..31
+__device__ __forceinline__ void dequant_q6k_32(const uint8_t *__restrict__ tile, int r, int c, int h, _Float16 *dst) {
+    const int n = c >> 1, t4 = 2 * (c & 1) + h;
+    const uint8_t *ql = tile + r * 128 + 64 * n + 32 * (t4 & 1);
+    const uint8_t *qh = tile + 2048 + r * 64 + 32 * n;
+    const uint4 la = *reinterpret_cast<const uint4 *>(ql), lb = *reinterpret_cast<const uint4 *>(ql + 16);
+    const uint4 ha = *reinterpret_cast<const uint4 *>(qh), hb = *reinterpret_cast<const uint4 *>(qh + 16);
+    const int8_t *sc = reinterpret_cast<const int8_t *>(tile + 3072 + r * 16) + 8 * n + 2 * t4;
+    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(tile + 3328 + r * 2));
+    const float ds0 = d * (float)sc[0], ds1 = d * (float)sc[1];
+    const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
+    const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t nib = (t4 & 2) ? (lw[j] >> 4) & 0x0F0F0F0Fu : lw[j] & 0x0F0F0F0Fu;
+        const uint32_t hb2 = ((hw[j] >> (2 * t4)) & 0x03030303u) << 4;
+        const uint32_t q = nib | hb2;
+        const float ds = j < 4 ? ds0 : ds1;
+        v[4 * j + 0] = ds * (float)((int)(q & 0xFFu) - 32);
+        v[4 * j + 1] = ds * (float)((int)((q >> 8) & 0xFFu) - 32);
+        v[4 * j + 2] = ds * (float)((int)((q >> 16) & 0xFFu) - 32);
+        v[4 * j + 3] = ds * (float)((int)(q >> 24) - 32);
+    }
+    store32(dst, v);
+}
+
+template <int TYPE>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
+    __shared__ __align__(16) _Float16 Ws[GM * LDS_LD];
+    __shared__ __align__(16) _Float16 Xs[GN * LDS_LD];
+    constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.x * GM, t0 = blockIdx.y * GN;
+    const int nsb = a.K / QK_K;
+    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;     // wave's 64 x 64 corner of the tile
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    // staging roles: weights -- row tid/2, sub-block half tid%2; activations -- token tid/2, 32 elements tid%2
+    const int srow = tid >> 1, sh = tid & 1;
+    const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
+    const bool wlive = wrow < a.M_pad;
+    const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)(wrow >> 4) * nsb * TB;
+    const int tok = t0 + srow;
+    const bool xlive = tok < a.T;
+    const _Float16 *xrow = a.X + (size_t)tok * a.ldx + 32 * sh;
+
+    for (int kc = 0; kc < a.K / GK; ++kc) {
+        const int sb = kc >> 2, c = kc & 3;
+        // stage the weight slab
+        if (wlive) {
+            const uint8_t *tile = wtile_row + (size_t)sb * TB;
+            if (TYPE == MESH_Q4_K) dequant_q4k_32(tile, wrow & 15, c, sh, Ws + srow * LDS_LD + 32 * sh);
+            else dequant_q6k_32(tile, wrow & 15, c, sh, Ws + srow * LDS_LD + 32 * sh);
+        } else {
+            uint4 *d4 = reinterpret_cast<uint4 *>(Ws + srow * LDS_LD + 32 * sh);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
+        }
+        // stage the activation slab
+        {
+            uint4 *d4 = reinterpret_cast<uint4 *>(Xs + srow * LDS_LD + 32 * sh);
+            const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) d4[i] = xlive ? s4[i] : make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < GK / 16; ++ks) {
+            half8 af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                af[i] = *reinterpret_cast<const half8 *>(Ws + (wm + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
+                bf[i] = *reinterpret_cast<const half8 *>(Xs + (wn + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // D[m][t]: lane holds column t = lane%32 and rows 8*(e/4) + 4*(lane/32) + e%4 -> four consecutive m per store
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int t = t0 + wn + 32 * j + (lane & 31);
+            if (t >= a.T) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int m = m0 + wm + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                if (m >= a.M) continue;      // M is a multiple of 4 for every projection
+                float4 o = make_float4(acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]);
+                if (a.bias) {
+                    const float4 b = *reinterpret_cast<const float4 *>(a.bias + m);
+                    o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w;
+                }
+                if (a.residual) {
+                    const float4 r = *reinterpret_cast<const float4 *>(a.residual + (size_t)t * a.ldres + m);
+                    o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
+                }
+                *reinterpret_cast<float4 *>(a.Y + (size_t)t * a.ldy + m) = o;
+            }
+        }
+}
+
+int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
+    if (!a.W || !a.X || !a.Y || a.M <= 0 || a.K <= 0 || a.T <= 0) return fail(MESH_ERR_INVALID, "gemm: null pointer or empty shape");
+    if (a.K % QK_K || a.M % 4 || a.ldx % 8 || a.ldy % 4 || (a.residual && a.ldres % 4))
+        return fail(MESH_ERR_INVALID, "gemm: shape M=%d K=%d not supported (K %% 256, M %% 4)", a.M, a.K);
+    if ((reinterpret_cast<uintptr_t>(a.X) | reinterpret_cast<uintptr_t>(a.Y)) & 15) return fail(MESH_ERR_INVALID, "gemm: X and Y must be 16-byte aligned");
+    GemmArgs k = a;
+    k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
+    const dim3 grid((unsigned)((a.M + GM - 1) / GM), (unsigned)((a.T + GN - 1) / GN));
+    if (a.type == MESH_Q4_K) gemm_kq_kernel<MESH_Q4_K><<<grid, dim3(GEMM_THREADS), 0, stream>>>(k);
+    else if (a.type == MESH_Q6_K) gemm_kq_kernel<MESH_Q6_K><<<grid, dim3(GEMM_THREADS), 0, stream>>>(k);
+    else return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// ---- small elementwise companions of the prefill path ---------------------------------------------------------
+// y16[t] = f16( x[t] * rsqrt(mean(x[t]^2) + eps) * w ), one workgroup per token
+__global__ __launch_bounds__(256) void rmsnorm_f16_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps,
+                                                          int n, _Float16 *__restrict__ y, int ldy) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float *xt = x + (size_t)t * n;
+    float ss = 0.f;
+    for (int i = tid * 4; i < n; i += 1024) {
+        const float4 v = *reinterpret_cast<const float4 *>(xt + i);
+        ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)n + eps);
+    for (int i = tid * 4; i < n; i += 1024) {
+        const float4 v = *reinterpret_cast<const float4 *>(xt + i);
+        const float4 g = *reinterpret_cast<const float4 *>(w + i);
+        *reinterpret_cast<uint2 *>(y + (size_t)t * ldy + i) =
+            make_uint2(pack_h2(v.x * scale * g.x, v.y * scale * g.y), pack_h2(v.z * scale * g.z, v.w * scale * g.w));
+    }
+}
+
+int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (n % 4 || ldy % 4) return fail(MESH_ERR_INVALID, "rmsnorm: row length %d not a multiple of 4", n);
+    rmsnorm_f16_kernel<<<dim3((unsigned)T), dim3(256), 0, stream>>>(x, w, eps, n, y, ldy);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// out16 = f16( silu(gate) * up )
+__global__ __launch_bounds__(256) void swiglu_f16_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                         _Float16 *__restrict__ o, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4 a = reinterpret_cast<const float4 *>(g)[i], b = reinterpret_cast<const float4 *>(u)[i];
+    const float r0 = a.x / (1.0f + expf(-a.x)) * b.x, r1 = a.y / (1.0f + expf(-a.y)) * b.y;
+    const float r2 = a.z / (1.0f + expf(-a.z)) * b.z, r3 = a.w / (1.0f + expf(-a.w)) * b.w;
+    reinterpret_cast<uint2 *>(o)[i] = make_uint2(pack_h2(r0, r1), pack_h2(r2, r3));
+}
+
+int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream) {
+    if (n <= 0) return MESH_OK;
+    if (n % 4) return fail(MESH_ERR_INVALID, "swiglu: count not a multiple of 4");
+    swiglu_f16_kernel<<<dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream>>>(gate, up, out, n / 4);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+}  // namespace mesh

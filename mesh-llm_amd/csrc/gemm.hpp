@@ -1,0 +1,26 @@
+// Prefill GEMM over tiled K-quant weights with f16 activations (gemm.hip), and its elementwise companions.
+#pragma once
+
+#include "gemv.hpp"
+
+namespace mesh {
+
+struct GemmArgs {
+    const void *W = nullptr;         // tiled q4_K / q6_K matrix [M][K]
+    int type = -1;
+    int M = 0, K = 0, T = 0;
+    int M_pad = 0;                   // filled in by gemm_kquant
+    const _Float16 *X = nullptr;     // [T][ldx] f16 activations
+    int ldx = 0;
+    float *Y = nullptr;              // [T][ldy] f32
+    int ldy = 0;
+    const float *bias = nullptr;     // [M] or null
+    const float *residual = nullptr; // [T][ldres] or null; may alias Y
+    int ldres = 0;
+};
+int gemm_kquant(const GemmArgs &a, hipStream_t stream);
+
+int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream);
+int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream);
+
+}  // namespace mesh

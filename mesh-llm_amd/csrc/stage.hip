@@ -15,6 +15,7 @@
 #include <cstring>
 
 #include "attn.hpp"
+#include "gemm.hpp"
 #include "gemv.hpp"
 #include "moe.hpp"
 
@@ -232,6 +233,7 @@ static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
 constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
+constexpr int PREFILL_MIN_TOKENS = 32;      // calls with at least this many tokens take the MFMA GEMM path
 
 int session_new(mesh_stage *st, mesh_session **out) {
     if (!st || !out) return fail(MESH_ERR_INVALID, "mesh_stage_session_new: null argument");
@@ -265,6 +267,13 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
     if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
+    if (B >= (size_t)PREFILL_MIN_TOKENS && hp.n_ff > 0) {
+        if ((rc = sess_alloc(s.get(), &p, B * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
+        s->xn16 = static_cast<uint16_t *>(p);
+        if ((rc = sess_alloc(s.get(), &p, B * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
+        s->ffn16 = static_cast<uint16_t *>(p);
+        if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
+    }
     if (hp.n_expert_used > 0 && !st->layers.empty() && st->layers[0].gate_inp.present()) {
         const size_t ne = (size_t)st->layers[0].gate_inp.M, k = hp.n_expert_used;
         if ((rc = fbuf(&s->moe_logits, B * ne)) || (rc = fbuf(&s->moe_w, B * k)) || (rc = fbuf(&s->moe_out, B * k * hp.n_embd)) ||
@@ -340,6 +349,81 @@ int profile_collect(mesh_session *s) {
     return MESH_OK;
 }
 
+static bool layer_is_kquant_dense(const LayerWeights &L) {
+    const DevTensor *w[] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down};
+    for (const DevTensor *t : w)
+        if (!t->present() || !t->tiled) return false;
+    return true;
+}
+
+static GemmArgs gemm_of(const DevTensor &w, const uint16_t *x16, int ldx, int T, float *y, int ldy, const DevTensor *bias) {
+    GemmArgs g;
+    g.W = w.data; g.type = w.type; g.M = (int)w.M; g.K = (int)w.K; g.T = T;
+    g.X = reinterpret_cast<const _Float16 *>(x16); g.ldx = ldx; g.Y = y; g.ldy = ldy;
+    g.bias = bias && bias->present() ? static_cast<const float *>(bias->data) : nullptr;
+    return g;
+}
+
+// One layer over many tokens: norms and activations are materialised in f16 and every projection is an MFMA GEMM.
+static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, int T, int max_keys) {
+    mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    hipStream_t stream = s->stream;
+    const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
+    _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
+    int rc;
+    if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
+    {
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_kquant(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv), stream)) != MESH_OK) return rc;
+    }
+    RopeKvArgs ra;
+    ra.q = s->q; ra.k = s->k; ra.v = s->v;
+    ra.kcache = s->kcache + il * s->kv_layer_elems;
+    ra.vcache = s->vcache + il * s->kv_layer_elems;
+    ra.pos = s->d_pos; ra.seq = s->d_seq; ra.inv_freq = st->rope_inv_freq;
+    ra.q_norm = L.q_norm.present() ? static_cast<const float *>(L.q_norm.data) : nullptr;
+    ra.k_norm = L.k_norm.present() ? static_cast<const float *>(L.k_norm.data) : nullptr;
+    ra.eps = hp.rms_eps;
+    ra.n_head = (int)hp.n_head; ra.n_kv = (int)hp.n_head_kv; ra.head_dim = (int)hp.head_dim;
+    ra.n_rot = (int)hp.n_rot; ra.rope_mode = (int)hp.rope_mode; ra.n_ctx = st->n_ctx;
+    { ProfScope ps(s, MESH_PROF_ROPE); rc = rope_kv(ra, T, stream); }
+    if (rc != MESH_OK) return rc;
+    AttnArgs aa;
+    aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.pos = s->d_pos; aa.seq = s->d_seq;
+    aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = s->attn;
+    aa.scale = 1.0f / sqrtf((float)hp.head_dim);
+    aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
+    aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
+    aa.n_splits = 1;
+    (void)max_keys;
+    { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
+    if (rc != MESH_OK) return rc;
+    if ((rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream)) != MESH_OK) return rc;
+    {
+        ProfScope ps(s, MESH_PROF_GEMV);
+        GemmArgs go = gemm_of(L.wo, s->xn16, QD, T, s->x, E, nullptr);
+        go.residual = s->x; go.ldres = E;
+        if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
+    }
+    if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
+    {
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_kquant(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr), stream)) != MESH_OK) return rc;
+    }
+    if ((rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream)) != MESH_OK) return rc;
+    {
+        ProfScope ps(s, MESH_PROF_GEMV);
+        GemmArgs gd = gemm_of(L.w_down, s->ffn16, FF, T, s->x, E, nullptr);
+        gd.residual = s->x; gd.ldres = E;
+        if ((rc = gemm_kquant(gd, stream)) != MESH_OK) return rc;
+    }
+    return MESH_OK;
+}
+
 // Runs the layers over the T token rows already in s->x.  pos/seq are on the device in s->d_pos / s->d_seq.
 static int run_layers(mesh_session *s, int T, int max_keys) {
     mesh_stage *st = s->stage;
@@ -349,6 +433,10 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     int rc;
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
+        if (T >= PREFILL_MIN_TOKENS && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
+            if ((rc = run_layer_prefill(s, L, il, T, max_keys)) != MESH_OK) return rc;
+            continue;
+        }
         // q, k, v = W{q,k,v} . rms_norm(x)
         GemvArgs qa;
         qa.n_mat = 3;

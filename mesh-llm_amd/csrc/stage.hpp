@@ -74,6 +74,9 @@ struct mesh_session {
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
+    // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
+    uint16_t *xn16 = nullptr, *ffn16 = nullptr;
+    float *ffn_up = nullptr;
     float *moe_logits = nullptr, *moe_w = nullptr, *moe_out = nullptr, *expert_mask = nullptr;
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;

@@ -228,3 +228,43 @@ def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
     assert np.array_equal(np.sort(ids, axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     assert len(set(ids.reshape(-1))) > 8
     ses.close(); st.close()
+
+
+def test_prefill_mfma_path_matches_oracle_and_decode_path(tmp_path):
+    """Calls with >= 32 tokens take the MFMA GEMM path (f16 activations, f32 accumulate): compare it with the oracle
+    and with the same tokens fed through the decode (GEMV) path, then keep decoding on top of the prefilled cache."""
+    m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [3, 4], 3, 5, n_ctx=256, n_seq=2, n_batch=160)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(41))
+    T = 150                                     # not a multiple of the 128-token tile
+    x = rng.standard_normal((T, E)).astype(np.float32)
+    ses = st.session()
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
+    orc = StageOracle(cfg, tensors, 3, 5, 256, n_seq_max=2)
+    ref = orc.forward(x, np.arange(T))
+    assert rel_l2(got, ref) <= 3e-3             # f16 GEMM inputs
+    # same tokens through the decode path, 16 at a time, into the other sequence
+    ses2 = st.session()
+    parts = [ses2.decode(x[i:i + 16], np.arange(i, min(i + 16, T)), seq=np.ones(min(16, T - i), np.int32)).view(np.float32)
+             for i in range(0, T, 16)]
+    step = np.concatenate(parts).reshape(T, E)
+    assert rel_l2(got, step) <= 3e-3
+    assert rel_l2(step, ref) <= 1e-3
+    # decode one more token on top of the prefilled cache
+    x1 = rng.standard_normal((1, E)).astype(np.float32)
+    got1 = ses.decode(x1, [T]).view(np.float32)
+    ref1 = orc.forward(x1, [T])
+    assert rel_l2(got1, ref1) <= 3e-3
+    ses.close(); ses2.close(); st.close()
+
+
+def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
+    m, cfg, tensors, st = _open(tmp_path, "tiny-qwen2", range(0, 3), 0, 3, n_ctx=128, n_seq=1, n_batch=64)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(43))
+    x = rng.standard_normal((47, E)).astype(np.float32)
+    ses = st.session()
+    got = ses.decode(x, np.arange(47)).view(np.float32).reshape(47, E)
+    ref = StageOracle(cfg, tensors, 0, 3, 128).forward(x, np.arange(47))
+    assert rel_l2(got, ref) <= 3e-3
+    ses.close(); st.close()
