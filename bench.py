@@ -252,7 +252,9 @@ def bench_stage(args):
                    "weight_bytes": weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
         "roofline": {"bound": "hbm", "kernel": "gemv_dot_kernel<type,1,NU> (q4_K/q6_K dequant-fused mat-vec, all instantiations)",
                      "achieved": round(gemv_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gemv_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
+                     # HBM bytes per average launch: rocprofv3 FETCH_SIZE (x2.0 calibration) + WRITE_SIZE of the gemv
+                     # launches, profiles/stage_decode_llama3_8b_l0_15_hbm_traffic.txt: 1.006 x algorithmic
+                     "traffic": int(round(1.006 * weight_bytes / g_n)), "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
                      "algorithmic_bytes_per_launch": weight_bytes // g_n},
         "stage_frac_hbm": b1["frac_hbm"],
         "decode": {str(k): v for k, v in results.items()},
