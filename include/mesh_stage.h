@@ -172,6 +172,11 @@ int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const 
 /* The session's hipStream_t (for events), and a wait for everything queued on it. */
 void *mesh_session_stream(mesh_session *session);
 int mesh_session_synchronize(mesh_session *session);
+/* Number of decode steps of this session that ran through the persistent single-launch decode kernel (batches of up
+ * to 4 single-token sequences on a dense K-quant stage with head_dim 128; environment MESH_STAGE_PERSISTENT=1 at
+ * session creation turns that kernel on).  -1 for a null session.  No counterpart in the reference; it lets tests and
+ * benchmarks tell which path produced a result. */
+int64_t mesh_session_persistent_steps(const mesh_session *session);
 
 /* Per-kernel-class timing of a session, measured with HIP events recorded on the session's stream around each
  * launch.  Off by default (it adds two event records per launch).  Kinds index the arrays below. */

@@ -98,6 +98,7 @@ SIGNATURES.update({
     "mesh_stage_decode_dev": (_i32, [_vp, ctypes.POINTER(Batch), _vp, _i32, _vp, _i32, _sz, _psz]),
     "mesh_session_stream": (_vp, [_vp]),
     "mesh_session_synchronize": (_i32, [_vp]),
+    "mesh_session_persistent_steps": (_i64, [_vp]),
     "mesh_session_profile": (_i32, [_vp, _i32]),
     "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
     "mesh_session_set_expert_mask": (_i32, [_vp, _vp, _i32]),
@@ -307,6 +308,11 @@ class Session:
 
     def synchronize(self):
         check(lib().mesh_session_synchronize(self._h))
+
+    @property
+    def persistent_steps(self):
+        """Decode steps so far that ran through the persistent single-launch kernel."""
+        return int(lib().mesh_session_persistent_steps(self._h))
 
     def profile(self, enable):
         check(lib().mesh_session_profile(self._h, 1 if enable else 0))
