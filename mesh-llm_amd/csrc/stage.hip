@@ -299,8 +299,10 @@ static int mega_setup(mesh_session *s) {
     const size_t nB = MEGA_BATCH_MAX;
     size_t off = 0;
     auto carve = [&](size_t floats) { const size_t o = off; off += (floats * 4 + 255) / 256 * 256; return o; };
-    const size_t o_x = carve(nB * E), o_q = carve(nB * QD), o_k = carve(nB * KD), o_v = carve(nB * KD), o_attn = carve(nB * QD),
-                 o_ffn = carve(nB * FF), o_part = carve(nB * QD * MEGA_SPLITS_MAX), o_ml = carve(nB * hp.n_head * MEGA_SPLITS_MAX * 2),
+    // replica strides are not multiples of a large power of two, so the copies fall on different memory channels
+    const size_t xs = nB * E + 1088, as = nB * QD + 1088, fs = nB * FF + 1088;
+    const size_t o_x = carve(MEGA_REPLICAS * xs), o_q = carve(nB * QD), o_k = carve(nB * KD), o_v = carve(nB * KD), o_attn = carve(MEGA_REPLICAS * as),
+                 o_ffn = carve(MEGA_REPLICAS * fs), o_part = carve(nB * QD * MEGA_SPLITS_MAX), o_ml = carve(nB * hp.n_head * MEGA_SPLITS_MAX * 2),
                  o_bar = carve(64);
     m.pool_bytes = off;
     m.pool = uncached_acquire(m.pool_bytes, st->device);
@@ -323,23 +325,23 @@ static int mega_setup(mesh_session *s) {
         auto f = [](const DevTensor &t) { return t.present() ? static_cast<const float *>(t.data) : nullptr; };
         MegaPhase &qkv = d.ph[0], &o = d.ph[1], &gu = d.ph[2], &dn = d.ph[3];
         qkv.n_part = 3;
-        qkv.part[0] = MegaPart{w(L.wq), nullptr, L.wq.type, QD, 0, QD, m.q, f(L.bq)};
-        qkv.part[1] = MegaPart{w(L.wk), nullptr, L.wk.type, KD, QD / TILE_ROWS, KD, m.k, f(L.bk)};
-        qkv.part[2] = MegaPart{w(L.wv), nullptr, L.wv.type, KD, (QD + KD) / TILE_ROWS, KD, m.v, f(L.bv)};
+        qkv.part[0] = MegaPart{w(L.wq), nullptr, L.wq.type, QD, 0, QD, m.q, f(L.bq), 1, 0};
+        qkv.part[1] = MegaPart{w(L.wk), nullptr, L.wk.type, KD, QD / TILE_ROWS, KD, m.k, f(L.bk), 1, 0};
+        qkv.part[2] = MegaPart{w(L.wv), nullptr, L.wv.type, KD, (QD + KD) / TILE_ROWS, KD, m.v, f(L.bv), 1, 0};
         qkv.total_rows = (QD + 2 * KD) / TILE_ROWS;
-        qkv.x = m.x; qkv.ldx = E; qkv.K = E; qkv.norm_w = f(L.attn_norm); qkv.epi = EPI_STORE;
+        qkv.x = m.x; qkv.x_rep_stride = xs; qkv.ldx = E; qkv.K = E; qkv.norm_w = f(L.attn_norm); qkv.epi = EPI_STORE;
         o.n_part = 1;
-        o.part[0] = MegaPart{w(L.wo), nullptr, L.wo.type, E, 0, E, m.x, nullptr};
+        o.part[0] = MegaPart{w(L.wo), nullptr, L.wo.type, E, 0, E, m.x, nullptr, MEGA_REPLICAS, xs};
         o.total_rows = E / TILE_ROWS;
-        o.x = m.attn; o.ldx = QD; o.K = QD; o.norm_w = nullptr; o.epi = EPI_RESIDUAL;
+        o.x = m.attn; o.x_rep_stride = as; o.ldx = QD; o.K = QD; o.norm_w = nullptr; o.epi = EPI_RESIDUAL;
         gu.n_part = 1;
-        gu.part[0] = MegaPart{w(L.w_gate), w(L.w_up), L.w_gate.type, FF, 0, FF, m.ffn, nullptr};
+        gu.part[0] = MegaPart{w(L.w_gate), w(L.w_up), L.w_gate.type, FF, 0, FF, m.ffn, nullptr, MEGA_REPLICAS, fs};
         gu.total_rows = FF / TILE_ROWS;
-        gu.x = m.x; gu.ldx = E; gu.K = E; gu.norm_w = f(L.ffn_norm); gu.epi = EPI_SWIGLU;
+        gu.x = m.x; gu.x_rep_stride = xs; gu.ldx = E; gu.K = E; gu.norm_w = f(L.ffn_norm); gu.epi = EPI_SWIGLU;
         dn.n_part = 1;
-        dn.part[0] = MegaPart{w(L.w_down), nullptr, L.w_down.type, E, 0, E, m.x, nullptr};
+        dn.part[0] = MegaPart{w(L.w_down), nullptr, L.w_down.type, E, 0, E, m.x, nullptr, MEGA_REPLICAS, xs};
         dn.total_rows = E / TILE_ROWS;
-        dn.x = m.ffn; dn.ldx = FF; dn.K = FF; dn.norm_w = nullptr; dn.epi = EPI_RESIDUAL;
+        dn.x = m.ffn; dn.x_rep_stride = fs; dn.ldx = FF; dn.K = FF; dn.norm_w = nullptr; dn.epi = EPI_RESIDUAL;
         d.kc = s->kcache + il * s->kv_layer_elems;
         d.vc = s->vcache + il * s->kv_layer_elems;
     }
@@ -355,6 +357,12 @@ static int mega_setup(mesh_session *s) {
     if (m.max_batch == 0) return MESH_OK;
     int rc = sess_alloc(s, &m.layers, tbl.size() * sizeof(MegaLayer));
     if (rc != MESH_OK) return rc;
+    void *rope_tab = nullptr;
+    if ((rc = sess_alloc(s, &rope_tab, 2 * nB * 64 * sizeof(float))) != MESH_OK) return rc;
+    m.rope_cs = static_cast<float *>(rope_tab);
+    m.rope_sn = m.rope_cs + nB * 64;
+    m.x_rep_stride = xs;
+    m.attn_rep_stride = as;
     MESH_HIP_TRY(hipMemcpy(m.layers, tbl.data(), tbl.size() * sizeof(MegaLayer), hipMemcpyHostToDevice));
     m.grid = grid;
     m.ready = true;
@@ -371,13 +379,16 @@ static int mega_step(mesh_session *s, int T, int max_keys) {
     ma.layers = static_cast<const MegaLayer *>(m.layers);
     ma.n_layers = (int)st->layers.size();
     ma.B = T;
+    ma.E = (int)hp.n_embd;
     ma.n_head = (int)hp.n_head; ma.n_kv = (int)hp.n_head_kv; ma.group = (int)(hp.n_head / hp.n_head_kv);
     ma.n_rot = (int)hp.n_rot; ma.rope_mode = (int)hp.rope_mode; ma.n_ctx = st->n_ctx;
     int ns = 1;
     while (ns * 2 <= MEGA_SPLITS_MAX && T * ma.n_kv * ns * 2 <= m.grid && ns * 2 * 32 <= max_keys) ns *= 2;
     ma.n_splits = ns;
     ma.eps = hp.rms_eps; ma.attn_scale = 1.0f / sqrtf((float)hp.head_dim);
+    ma.x = m.x; ma.x_rep_stride = m.x_rep_stride; ma.attn_rep_stride = m.attn_rep_stride;
     ma.q = m.q; ma.k = m.k; ma.v = m.v; ma.attn = m.attn; ma.part = m.part; ma.ml = m.ml;
+    ma.rope_cs = m.rope_cs; ma.rope_sn = m.rope_sn;
     ma.pos = s->d_pos; ma.seq = s->d_seq; ma.inv_freq = st->rope_inv_freq;
     ma.bar = m.bar; ma.bar_base = m.bar_value; ma.abort_flag = m.abort_flag;
     ma.spin_limit = 400000;

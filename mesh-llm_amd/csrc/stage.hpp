@@ -95,6 +95,8 @@ struct mesh_session {
         void *pool = nullptr;             // one uncached block, returned to a process-wide free list, never hipFree'd
         size_t pool_bytes = 0;
         float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *part = nullptr, *ml = nullptr;
+        float *rope_cs = nullptr, *rope_sn = nullptr;   // ordinary device memory
+        size_t x_rep_stride = 0, attn_rep_stride = 0;
         unsigned *bar = nullptr;
         int *abort_flag = nullptr;
         void *layers = nullptr;           // device array of MegaLayer
