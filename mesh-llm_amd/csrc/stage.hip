@@ -411,7 +411,25 @@ static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
 constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
-constexpr int PREFILL_MIN_TOKENS = 32;      // calls with at least this many tokens take the MFMA GEMM path
+// calls with at least this many tokens take the MFMA GEMM path (MESH_GEMM_MIN_TOKENS overrides, for tuning)
+static int gemm_min_tokens() {
+    static int v = 0;
+    if (!v) {
+        const char *e = getenv("MESH_GEMM_MIN_TOKENS");
+        v = e && atoi(e) > 0 ? atoi(e) : 192;
+    }
+    return v;
+}
+#define PREFILL_MIN_TOKENS gemm_min_tokens()
+// calls with at least this many tokens (and fewer than the above) take the skinny MFMA GEMM (MESH_SKINNY_MIN_TOKENS)
+static int skinny_min_tokens() {
+    static int v = 0;
+    if (!v) {
+        const char *e = getenv("MESH_SKINNY_MIN_TOKENS");
+        v = e && atoi(e) > 0 ? atoi(e) : 5;
+    }
+    return v;
+}
 
 int session_new(mesh_stage *st, mesh_session **out) {
     if (!st || !out) return fail(MESH_ERR_INVALID, "mesh_stage_session_new: null argument");
@@ -445,7 +463,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
     if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
-    if (B >= (size_t)PREFILL_MIN_TOKENS && hp.n_ff > 0) {
+    if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && hp.n_ff > 0) {
         if ((rc = sess_alloc(s.get(), &p, B * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
         if ((rc = sess_alloc(s.get(), &p, B * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
@@ -544,7 +562,9 @@ static GemmArgs gemm_of(const DevTensor &w, const uint16_t *x16, int ldx, int T,
 }
 
 // One layer over many tokens: norms and activations are materialised in f16 and every projection is an MFMA GEMM.
-static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, int T, int max_keys) {
+// One dense K-quant layer over f16 activations on the matrix cores: `skinny` selects the batched-decode GEMM (few
+// tokens, weight-streaming bound) instead of the large-tile prefill GEMM.
+static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, int T, int max_keys, bool skinny) {
     mesh_stage *st = s->stage;
     const HParams &hp = st->hp;
     hipStream_t stream = s->stream;
@@ -552,7 +572,16 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
     if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
-    {
+    if (skinny) {
+        SkinnyArgs qa;
+        qa.n_mat = 3;
+        qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
+        qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
+        qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
+        qa.x = xn; qa.ldx = E; qa.K = E; qa.T = T;
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
+    } else {
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_kquant(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq), stream)) != MESH_OK) return rc;
         if ((rc = gemm_kquant(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk), stream)) != MESH_OK) return rc;
@@ -576,18 +605,42 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-    aa.n_splits = 1;
-    (void)max_keys;
+    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;     // a batch of decode steps still splits the long KV
     { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
     if (rc != MESH_OK) return rc;
     if ((rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream)) != MESH_OK) return rc;
-    {
+    if (skinny) {
+        SkinnyArgs oa;
+        oa.n_mat = 1;
+        oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
+        oa.x = xn; oa.ldx = QD; oa.K = QD; oa.T = T;
+        oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny(oa, stream)) != MESH_OK) return rc;
+    } else {
         ProfScope ps(s, MESH_PROF_GEMV);
         GemmArgs go = gemm_of(L.wo, s->xn16, QD, T, s->x, E, nullptr);
         go.residual = s->x; go.ldres = E;
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
     if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
+    if (skinny && L.w_gate.type == L.w_up.type) {
+        // gate and up in one pass with the SwiGLU epilogue, written as f16 straight into the down projection's input
+        SkinnyArgs ga;
+        ga.n_mat = 2;
+        ga.mat[0] = mat_of(L.w_gate, nullptr, FF, nullptr);
+        ga.mat[1] = mat_of(L.w_up, nullptr, FF, nullptr);
+        ga.x = xn; ga.ldx = E; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
+        ga.y16 = f16ffn; ga.ldy16 = FF;
+        SkinnyArgs da;
+        da.n_mat = 1;
+        da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
+        da.x = f16ffn; da.ldx = FF; da.K = FF; da.T = T;
+        da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny(ga, stream)) != MESH_OK) return rc;
+        return gemm_skinny(da, stream);
+    }
     {
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_kquant(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr), stream)) != MESH_OK) return rc;
@@ -612,9 +665,12 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     int rc;
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
-        if (T >= PREFILL_MIN_TOKENS && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
-            if ((rc = run_layer_prefill(s, L, il, T, max_keys)) != MESH_OK) return rc;
-            continue;
+        if (T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
+            const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0;
+            if (skinny || T >= PREFILL_MIN_TOKENS) {
+                if ((rc = run_layer_prefill(s, L, il, T, max_keys, skinny)) != MESH_OK) return rc;
+                continue;
+            }
         }
         // q, k, v = W{q,k,v} . rms_norm(x)
         GemvArgs qa;
