@@ -274,7 +274,8 @@ __device__ __forceinline__ void gemv_phase(const MegaPhase &ph, float eps, const
         for (int gg = tid; gg - tid < ng; gg += MEGA_THREADS) {
             XRegs<NB> X;
             x_fetch_exchange<NB>(X, xin, ph.ldx, gg, gg < ng);
-            x_quantise<NB, true>(X, norm_w, K, S, gg, gg < ng, ss);
+            norm_fetch<NB>(X, norm_w, gg, gg < ng);
+            x_quantise<NB, true>(X, K, S, gg, gg < ng, ss);
         }
         if (norm_w) {
 #pragma unroll

@@ -21,20 +21,23 @@ struct GemmArgs {
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
 
 // Skinny GEMM for a batch of decode steps (gemm_skinny.hip): up to three tiled K-quant matrices sharing the f16
-// activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel.
+// activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel.  Activations are in the
+// "k8-major" layout: blocks of 16 tokens, element (t, k) of block t / 16 at ((k / 8) * 16 + t % 16) * 8 + k % 8 within
+// the block of 16 * K halfs; columns beyond T hold zeros.  rmsnorm_f16_k8 / pack_f16_k8 produce it.
 struct SkinnyArgs {
     GemvMat mat[3];
     int n_mat = 1;                   // for EPI_SWIGLU exactly 2 (gate, up), written through mat[0].y and/or y16
-    const _Float16 *x = nullptr;     // [T][ldx] f16, rows 16-byte aligned
-    int ldx = 0;
+    const _Float16 *x = nullptr;     // k8-major, ceil(T / 16) blocks of 16 * K halfs, 16-byte aligned
     int K = 0, T = 0;
     int epi = EPI_STORE;
     const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y
     int ldres = 0;
-    _Float16 *y16 = nullptr;         // optional f16 copy of matrix 0's output (feeds the next GEMM), [T][ldy16]
-    int ldy16 = 0;
+    _Float16 *y16 = nullptr;         // optional f16 copy of matrix 0's output in the k8-major layout (feeds the next GEMM)
 };
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
+// y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
+int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream);
+int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream);
 
 int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream);
 int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream);

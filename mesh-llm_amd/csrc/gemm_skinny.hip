@@ -15,6 +15,14 @@
 // (0x6400 | q is 1024 + q exactly), the offset is removed exactly, and the sub-block scale and minimum are applied
 // with one packed fma, all in f16 (sums are f32, in the MFMA accumulator).
 //
+// Activation layout ("k8-major"): X is not read as [T][K] rows.  Tokens are grouped in blocks of 16 columns, and
+// within a block the 8 consecutive k of every column sit together: element (t, k) of block b = t / 16 is at
+// ((b * K/8 + k/8) * 16 + t % 16) * 8 + k % 8.  The 16 lanes that supply the 16 columns of one MFMA B fragment then
+// read 256 contiguous bytes, where row-major activations would cost one cache line per lane.  The producers
+// (rmsnorm_f16_k8, pack_f16_k8, this kernel's own f16 output) write that layout, zero-filling the unused columns.
+// Weight tiles are loaded with the mat-vec kernel's dense lane mapping and moved to the MFMA lanes with
+// ds_bpermute (register crossbar), again so that a wave's load touches whole cache lines.
+//
 // Same math as ggml's mul_mat for K-quant weights (ggml_vec_dot_q4_K_q8_K / q6_K in
 // third_party/llama.cpp ggml-cpu/quants.c, reached from rpc_server::graph_compute,
 // patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451) except that activations are rounded to f16
@@ -29,12 +37,13 @@ constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
 constexpr int SK_DEPTH = 4;               // weight tiles a wave keeps in flight
 constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA N)
-constexpr int SK_SEGS_MAX = 8;            // (tile-row, matrix) segments one wave may own
+constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 
 struct SkinnyKernelArgs {
     const uint8_t *wbase[3];      // matrix base minus its first tile-row, so a global tile-row index addresses it
@@ -43,13 +52,13 @@ struct SkinnyKernelArgs {
     const float *bias[3];
     int M[3];
     int ldy[3];
-    const _Float16 *x;            // [T][ldx]
-    int ldx, K, T;
+    const _Float16 *x;            // k8-major block of 16 columns
+    int K, T;
     const float *residual;
     int ldres;
     int epi;
-    _Float16 *y16;                // optional f16 copy of the output (matrix 0), [T][ldy16]
-    int ldy16;
+    _Float16 *y16;                // optional f16 copy of the output (matrix 0): k8-major block with M16 rows as its k
+    int M16;
     int ks;                       // waves along K
 };
 
@@ -64,15 +73,13 @@ __device__ __forceinline__ h8_t dequant8(uint32_t v0, uint32_t v1, h2_t off, h2_
     h2_t p[4];
     bytes_to_h1024(v0, p[0], p[1]);
     bytes_to_h1024(v1, p[2], p[3]);
-    h8_t a;
+    u4_t a;                                                          // built as four dwords: no half-register moves
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const h2_t q = p[i] - off;                                   // exact
-        const h2_t w = __builtin_elementwise_fma(q, s, mn);
-        a[2 * i] = w[0];
-        a[2 * i + 1] = w[1];
+        a[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, s, mn));
     }
-    return a;
+    return __builtin_bit_cast(h8_t, a);
 }
 
 __device__ __forceinline__ h2_t h2_of(float v) {
@@ -152,27 +159,50 @@ template <> struct TileFrags<MESH_Q6_K> {
 template <int TYPE>
 struct BFrags {
     uint4 b[8];
-    __device__ __forceinline__ void load(const _Float16 *xcol, bool live, int sb, int g) {
+    // x: the k8-major block (uniform), lane_off: this lane's column and quarter offset in halfs
+    __device__ __forceinline__ void load(const _Float16 *x, int lane_off, int sb) {
+        const _Float16 *base = x + (size_t)sb * (QK_K * 16);      // uniform
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            int koff;
-            if (TYPE == MESH_Q4_K) koff = 64 * g + 32 * (t >> 2) + 8 * (t & 3);
-            else koff = 128 * (g >> 1) + 16 * (g & 1) + 32 * (t >> 1) + 8 * (t & 1);
-            b[t] = live ? ldg<uint4>(xcol + sb * QK_K + koff) : make_uint4(0u, 0u, 0u, 0u);
+            int koff;                                      // compile-time part of the element offset
+            if (TYPE == MESH_Q4_K) koff = 32 * (t >> 2) + 8 * (t & 3);
+            else koff = 32 * (t >> 1) + 8 * (t & 1);
+            b[t] = ldg<uint4>(base + lane_off + koff * 16);
         }
     }
 };
+
+// Moves a tile loaded with the dense mapping (lane 4r + c holds row r, quarter c) to the MFMA mapping
+// (lane m + 16 g holds row m, quarter g).
+__device__ __forceinline__ uint32_t lane_gather(uint32_t v, int src_lane4) {
+    return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane4, (int)v);
+}
+__device__ __forceinline__ uint4 lane_gather(const uint4 &v, int src_lane4) {
+    return make_uint4(lane_gather(v.x, src_lane4), lane_gather(v.y, src_lane4), lane_gather(v.z, src_lane4), lane_gather(v.w, src_lane4));
+}
+__device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q4_K> &R, int src_lane4) {
+    R.hdr = lane_gather(R.hdr, src_lane4);
+    R.qa = lane_gather(R.qa, src_lane4);
+    R.qb = lane_gather(R.qb, src_lane4);
+}
+__device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_lane4) {
+    R.qla = lane_gather(R.qla, src_lane4);
+    R.qlb = lane_gather(R.qlb, src_lane4);
+    R.qh = lane_gather(R.qh, src_lane4);
+    R.sc = lane_gather(R.sc, src_lane4);
+    R.d = lane_gather(R.d, src_lane4);
+}
 
 template <int TYPE, int NU, int SEGS>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKernelArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
     constexpr int TB = TileRegs<TYPE>::BYTES;
-    constexpr int U = 2 * (SEGS > SK_DEPTH ? SEGS : SK_DEPTH);       // flat tile indices per unrolled round
     const int K = a.K, nsb = K / QK_K;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: tile addresses become SGPR base + lane offset
     const int m = lane & 15, g = lane >> 4;
-    const int lane_perm = 4 * m + g;                      // the mat-vec kernel's lane that loads row m, quarter g
+    const int src_lane4 = 4 * (4 * m + g);                // byte address, for ds_bpermute, of the lane that loaded row m, quarter g
     const int KS = a.ks, RS = SK_WAVES / KS;
     const int ks = wave % KS, rs = wave / KS;
     const int total_rows = a.tile_begin[3];
@@ -181,18 +211,22 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
     const int rows_here = tr1 - tr0;
     const int n_i = rs < RS ? (nsb - ks + KS - 1) / KS : 0;         // super-blocks of this wave (ks < KS <= nsb)
     const size_t row_stride = (size_t)nsb * TB;
-    const bool col_live = m < a.T;                        // B fragments: lane (n = m, g) supplies column n
-    const _Float16 *xcol = a.x + (size_t)(col_live ? m : 0) * a.ldx;
-
+    // B fragments: lane (n = m, g) supplies column n, quarter g (columns beyond T hold zeros)
+    const int lane_off = (TYPE == MESH_Q4_K ? 64 * g : 128 * (g >> 1) + 16 * (g & 1)) * 16 + m * 8;
     // flat tile index f -> (ii, seg); seg -> (local tile-row j, matrix u)
     auto seg_valid = [&](int seg) { return rs + RS * (seg / NU) < rows_here; };
     auto tile_ptr = [&](int ii, int seg) -> const uint8_t * {
         const int tr = tr0 + rs + RS * (seg / NU);
         int mi = seg % NU;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        return a.wbase[mi] + (size_t)tr * row_stride + (size_t)(ks + KS * ii) * TB;
+        // (selected, not indexed: a dynamically indexed kernel-argument array is fetched with a load, and waiting for
+        // that address would drain every tile load in flight)
+        const uint8_t *wb = mi == 0 ? a.wbase[0] : mi == 1 ? a.wbase[1] : a.wbase[2];
+        return wb + (size_t)tr * row_stride + (size_t)(ks + KS * ii) * TB;
     };
-    const int total = n_i * SEGS;                         // flat indices, invalid segments included as bubbles
+    // flat tile index f = ii * SEGS + seg, invalid segments included as bubbles; a wave without a valid first
+    // segment has nothing at all
+    const int total = seg_valid(0) ? n_i * SEGS : 0;
 
     TileRegs<TYPE> ring[SK_DEPTH];
     BFrags<TYPE> B[2];
@@ -200,39 +234,49 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
 #pragma unroll
     for (int s = 0; s < SEGS; ++s) D[s] = f4_t{0.f, 0.f, 0.f, 0.f};
 
-    // prologue: the first DEPTH tiles and the activations of the first two super-blocks
+    // Loads are never under a branch of their own: an index past the end or an invalid segment is clamped to a tile
+    // the wave owns (a cache hit).  The compiler then knows exactly how many loads are in flight at every point
+    // and waits for one tile without draining the others; a load under a branch makes it assume the worst at the
+    // join, which in an unrolled pipeline degenerates to waiting for everything.
+    auto load_tile = [&](TileRegs<TYPE> &dst, int f, int seg) {
+        const bool ok = f < total && seg_valid(seg);
+        dst.load(tile_ptr(ok ? f / SEGS : n_i - 1, ok ? seg : 0), lane);
+    };
+    auto compute = [&](const TileRegs<TYPE> &loaded, const BFrags<TYPE> &bf, f4_t &acc) {
+        TileRegs<TYPE> tile = loaded;
+        to_mfma_lanes(tile, src_lane4);
+        TileFrags<TYPE> F;
+        F.prepare(tile, g);
 #pragma unroll
-    for (int f = 0; f < SK_DEPTH; ++f) {
-        const int ii = f / SEGS, seg = f % SEGS;
-        if (f < total && seg_valid(seg)) ring[f].load(tile_ptr(ii, seg), lane_perm);
-    }
-    if (n_i > 0) B[0].load(xcol, col_live, ks, g);
-    if (n_i > 1) B[1].load(xcol, col_live, ks + KS, g);
-
-    for (int f0 = 0; f0 < total; f0 += U) {
+        for (int t = 0; t < 8; ++t)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
+    };
+    if (total > 0) {
 #pragma unroll
-        for (int q = 0; q < U; ++q) {
-            const int f = f0 + q;
-            constexpr int dummy = 0; (void)dummy;
-            const int seg = q % SEGS, slot = q % SK_DEPTH, buf = (q / SEGS) % 2;
-            const int ii = f / SEGS;
-            if (f < total) {
-                if (seg_valid(seg)) {
-                    TileFrags<TYPE> F;
-                    F.prepare(ring[slot], g);
+        for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
+        B[0].load(a.x, lane_off, ks);
+        B[1].load(a.x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
+        if (n_i <= 2 && total <= SK_DEPTH) {
+            // short walk: everything it needs is already in flight
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const h8_t af = F.frag(t);
-                        const h8_t bf = __builtin_bit_cast(h8_t, B[buf].b[t]);
-                        D[seg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, D[seg], 0, 0, 0);
-                    }
+            for (int q = 0; q < SK_DEPTH; ++q)
+                if (q < total && seg_valid(q % SEGS)) compute(ring[q], B[(q / SEGS) % 2], D[q % SEGS]);
+        } else {
+            constexpr int RB = SEGS >= 2 ? 2 : 4;            // super-block rounds per unrolled block (even: B parity is static)
+            constexpr int UB = RB * SEGS;                    // tiles per block, a multiple of the ring depth
+            static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
+            for (int blk = 0; blk * RB < n_i; ++blk) {
+#pragma unroll
+                for (int q = 0; q < UB; ++q) {
+                    const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
+                    const int ii = blk * RB + r, f = ii * SEGS + seg;
+                    if (ii < n_i && seg_valid(seg)) compute(ring[slot], B[r % 2], D[seg]);
+                    // refill this slot with the tile DEPTH positions ahead
+                    load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
+                    // last segment of a super-block: its activation buffer is free for the one after next
+                    if (seg == SEGS - 1) B[r % 2].load(a.x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
+                    __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
                 }
-                // refill this slot with the tile DEPTH positions ahead
-                const int fn = f + SK_DEPTH;
-                const int segn = (q + SK_DEPTH) % SEGS;
-                if (fn < total && seg_valid(segn)) ring[slot].load(tile_ptr(fn / SEGS, segn), lane_perm);
-                // last segment of a super-block: its activation buffer is free for the one after next
-                if (seg == SEGS - 1 && ii + 2 < n_i) B[buf].load(xcol, col_live, ks + KS * (ii + 2), g);
             }
         }
     }
@@ -240,7 +284,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
     // partial sums of this wave: D[seg] holds rows 4g..4g+3, column m of segment seg
 #pragma unroll
     for (int seg = 0; seg < SEGS; ++seg) {
-        if (n_i > 0 && seg_valid(seg)) {
+        if (total > 0 && seg_valid(seg)) {
             const int j = rs + RS * (seg / NU), u = seg % NU;
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + 4 * g + i) * 16 + m] = D[seg][i];
@@ -251,12 +295,15 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
     // outputs of this workgroup: rows_here x 16 rows x T columns
     for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
-        if (t >= a.T) continue;
         const int tr = tr0 + j;
         int mi = 0;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
         const int row = (tr - a.tile_begin[mi]) * TILE_ROWS + r;
         if (row >= a.M[mi]) continue;
+        if (t >= a.T) {                                    // unused columns of the f16 output block stay finite
+            if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
+            continue;
+        }
         float s0 = 0.f, s1 = 0.f;
         for (int k2 = 0; k2 < KS; ++k2) {
             s0 += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + r) * 16 + t];
@@ -273,7 +320,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
             out = s0;
         }
         if (a.y[mi]) a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
-        if (a.y16 && mi == 0) a.y16[(size_t)t * a.ldy16 + row] = (_Float16)out;
+        if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)out;
     }
 }
 
@@ -294,8 +341,7 @@ template <int TYPE, int NU>
 static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
     if (segs <= 1) return launch_skinny<TYPE, NU, NU>(ka, grid, smem, stream);       // NU == 2 needs two segments at least
     if (segs <= 2) return launch_skinny<TYPE, NU, 2>(ka, grid, smem, stream);
-    if (segs <= 4) return launch_skinny<TYPE, NU, 4>(ka, grid, smem, stream);
-    return launch_skinny<TYPE, NU, 8>(ka, grid, smem, stream);
+    return launch_skinny<TYPE, NU, 4>(ka, grid, smem, stream);
 }
 
 static int skinny_n_cu() {
@@ -328,9 +374,9 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     }
     const int n_bound = NU == 2 ? 1 : a.n_mat;          // matrix boundaries the kernel searches
     for (int i = n_bound; i < 4; ++i) ka.tile_begin[i] = total_rows;
-    ka.ldx = a.ldx; ka.K = a.K;
+    ka.K = a.K;
     ka.ldres = a.ldres; ka.epi = a.epi;
-    ka.ldy16 = a.ldy16;
+    ka.M16 = a.mat[0].M;
     const int KS = nsb < SK_WAVES ? nsb : SK_WAVES, RS = SK_WAVES / KS;
     ka.ks = KS;
     // tile-rows per workgroup: spread over the CUs, bounded by the segments a wave can hold
@@ -347,9 +393,9 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     for (int t = 0; t < a.T; t += SK_NT) {
         SkinnyKernelArgs kb = ka;
         kb.T = std::min(SK_NT, a.T - t);
-        kb.x = a.x + (size_t)t * a.ldx;
+        kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
-        kb.y16 = a.y16 ? a.y16 + (size_t)t * a.ldy16 : nullptr;
+        kb.y16 = a.y16 ? a.y16 + (size_t)t * a.mat[0].M : nullptr;
         for (int i = 0; i < a.n_mat; ++i)
             if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
         int rc;
@@ -360,10 +406,64 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     return MESH_OK;
 }
 
+// ---- producers of the k8-major activation layout ------------------------------------------------------------------
+__device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {
+    const h2_t h = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// y = f16(x[t] * rsqrt(mean(x[t]^2) + eps) * w), or with w == null just f16(x[t]); one workgroup per token slot of the
+// padded batch (slots >= T write zeros).
+__global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int T, int n,
+                                                    _Float16 *__restrict__ y) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    _Float16 *yb = y + (size_t)(t / 16) * 16 * n + (size_t)(t % 16) * 8;        // element (t, k) at yb + (k / 8) * 128 + k % 8
+    if (t >= T) {
+        for (int i = tid * 8; i < n; i += 2048) *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
+    const float *xt = x + (size_t)t * n;
+    float scale = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int i = tid * 4; i < n; i += 1024) {
+            const float4 v = *reinterpret_cast<const float4 *>(xt + i);
+            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)n + eps);
+    }
+    for (int i = tid * 8; i < n; i += 2048) {
+        const float4 v0 = *reinterpret_cast<const float4 *>(xt + i), v1 = *reinterpret_cast<const float4 *>(xt + i + 4);
+        float4 g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
+        if (w) { g0 = *reinterpret_cast<const float4 *>(w + i); g1 = *reinterpret_cast<const float4 *>(w + i + 4); }
+        *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) =
+            make_uint4(sk_pack_h2(v0.x * scale * g0.x, v0.y * scale * g0.y), sk_pack_h2(v0.z * scale * g0.z, v0.w * scale * g0.w),
+                       sk_pack_h2(v1.x * scale * g1.x, v1.y * scale * g1.y), sk_pack_h2(v1.z * scale * g1.z, v1.w * scale * g1.w));
+    }
+}
+
+int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
+    to_k8_kernel<<<dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream>>>(x, w, eps, T, n, y);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream) {
+    return rmsnorm_f16_k8(x, nullptr, 0.f, T, n, y, stream);
+}
+
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
     if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.T <= 0 || a.K <= 0) return fail(MESH_ERR_INVALID, "gemm_skinny: bad arguments");
-    if (a.K % QK_K || a.ldx % 8 || (reinterpret_cast<uintptr_t>(a.x) & 15))
-        return fail(MESH_ERR_INVALID, "gemm_skinny: K %d must be a multiple of 256 and the activations 16-byte aligned rows (ldx %d)", a.K, a.ldx);
+    if (a.K % QK_K || (reinterpret_cast<uintptr_t>(a.x) & 15))
+        return fail(MESH_ERR_INVALID, "gemm_skinny: K %d must be a multiple of 256 and the activations 16-byte aligned", a.K);
+    if (a.y16 && a.mat[0].M % 8) return fail(MESH_ERR_INVALID, "gemm_skinny: f16 output needs a row count that is a multiple of 8");
     if (a.epi == EPI_SWIGLU && (a.n_mat != 2 || a.mat[0].M != a.mat[1].M || a.mat[0].type != a.mat[1].type))
         return fail(MESH_ERR_INVALID, "gemm_skinny: SwiGLU needs a gate and an up matrix of equal shape and type");
     if (a.epi == EPI_RESIDUAL && !a.residual) return fail(MESH_ERR_INVALID, "gemm_skinny: residual epilogue without residual");

@@ -91,7 +91,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
     S.ssq = reinterpret_cast<float *>(S.xi16 + (NEED_I16 ? NB * (K >> 4) : 0));
     S.red = S.ssq + GEMV_WAVES * NB;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // scalar, so that tile addresses and matrix selection stay in SGPRs
     GEMV_MARK(0);
     // activations first: they gate everything
     const int ng = K >> 3;
@@ -105,11 +106,12 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
     }
     XRegs<NB> X;
     x_fetch<NB>(X, xcol, a.ldx, tid, tid < ng);
+    norm_fetch<NB>(X, a.norm_w, tid, tid < ng);
 
     const int nsb = K / QK_K;
     const int KS = a.ks, RS = GEMV_WAVES / KS;
     const int ks = wave % KS, rs = wave / KS;
-    const int total_rows = a.tile_begin[a.n_mat];
+    const int total_rows = a.tile_begin[3];       // (a constant index: the host fills every unused slot with the total)
     const int tr0 = (int)(((long long)blockIdx.x * total_rows) / gridDim.x);
     const int tr1 = (int)(((long long)(blockIdx.x + 1) * total_rows) / gridDim.x);
     const int rows_here = tr1 - tr0;
@@ -120,26 +122,38 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
         const int tr = tr0 + c.j;
         int mi = c.u;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        return a.wbase[mi] + eoff + (size_t)tr * row_stride + (size_t)(ks + KS * c.ii) * TB;
+        // (selected, not indexed: a dynamically indexed kernel-argument array is fetched with a load, and waiting for
+        // that address would drain every tile load in flight)
+        const uint8_t *wb = mi == 0 ? a.wbase[0] : mi == 1 ? a.wbase[1] : a.wbase[2];
+        return wb + eoff + (size_t)tr * row_stride + (size_t)(ks + KS * c.ii) * TB;
     };
 
+    // Loads are unconditional: past its last tile a wave simply re-reads that tile (a cache hit).  With no load
+    // under a branch the compiler counts outstanding loads exactly and never has to drain the queue at a join.
     TileCursor<NU> ld{rs, 0, 0}, cp{rs, 0, 0};
     TileRegs<TYPE> t0, t1;
     const bool any = n_i > 0 && rs < rows_here;
+    auto advance_load = [&]() {
+        TileCursor<NU> nx = ld;
+        nx.advance(n_i, RS);
+        if (nx.j < rows_here) ld = nx;
+    };
     if (any) {
         t0.load(tile_ptr(ld), lane);
-        ld.advance(n_i, RS);
-        if (ld.j < rows_here) { t1.load(tile_ptr(ld), lane); ld.advance(n_i, RS); }
+        advance_load();
+        t1.load(tile_ptr(ld), lane);
+        advance_load();
     }
     GEMV_MARK(1);
 
     float ss[NB];
 #pragma unroll
     for (int t = 0; t < NB; ++t) ss[t] = 0.f;
-    x_quantise<NB, NEED_I16>(X, a.norm_w, K, S, tid, tid < ng, ss);
+    x_quantise<NB, NEED_I16>(X, K, S, tid, tid < ng, ss);
     for (int g0 = GEMV_THREADS; g0 < ng; g0 += GEMV_THREADS) {
         x_fetch<NB>(X, xcol, a.ldx, g0 + tid, g0 + tid < ng);
-        x_quantise<NB, NEED_I16>(X, a.norm_w, K, S, g0 + tid, g0 + tid < ng, ss);
+        norm_fetch<NB>(X, a.norm_w, g0 + tid, g0 + tid < ng);
+        x_quantise<NB, NEED_I16>(X, K, S, g0 + tid, g0 + tid < ng, ss);
     }
     if (a.norm_w) {
 #pragma unroll
@@ -171,12 +185,14 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
             tile_compute<NB>(t0, lane, ks + KS * cp.ii, S, K, acc);
             if (cp.ii + 1 == n_i) finish_segment(cp);
             cp.advance(n_i, RS);
-            if (ld.j < rows_here) { t0.load(tile_ptr(ld), lane); ld.advance(n_i, RS); }
+            t0.load(tile_ptr(ld), lane);
+            advance_load();
             if (cp.j >= rows_here) break;
             tile_compute<NB>(t1, lane, ks + KS * cp.ii, S, K, acc);
             if (cp.ii + 1 == n_i) finish_segment(cp);
             cp.advance(n_i, RS);
-            if (ld.j < rows_here) { t1.load(tile_ptr(ld), lane); ld.advance(n_i, RS); }
+            t1.load(tile_ptr(ld), lane);
+            advance_load();
             if (cp.j >= rows_here) break;
         }
     }

@@ -49,7 +49,20 @@ struct XStage {
 template <int NB>
 struct XRegs {
     float4 a[NB], b[NB];
+    float4 w0, w1;           // the norm weights of the same eight elements (ones without a norm)
 };
+
+// Issued together with the activation loads, i.e. before the first weight-tile loads: loads return in order, so a
+// norm-weight load issued after the tiles would make the prologue wait for the tiles as well.
+template <int NB>
+__device__ __forceinline__ void norm_fetch(XRegs<NB> &X, const float *__restrict__ norm_w, int g, bool live) {
+    X.w0 = make_float4(1.f, 1.f, 1.f, 1.f);
+    X.w1 = X.w0;
+    if (norm_w && live) {
+        X.w0 = ldg<float4>(norm_w + g * 8);
+        X.w1 = ldg<float4>(norm_w + g * 8 + 4);
+    }
+}
 
 template <int NB>
 __device__ __forceinline__ void x_fetch(XRegs<NB> &X, const float *__restrict__ x, int ldx, int g, bool live) {
@@ -65,14 +78,9 @@ __device__ __forceinline__ void x_fetch(XRegs<NB> &X, const float *__restrict__ 
 }
 
 template <int NB, bool NEED_I16>
-__device__ __forceinline__ void x_quantise(const XRegs<NB> &X, const float *__restrict__ norm_w, int K, const XStage &S, int g,
-                                           bool live, float (&ss)[NB]) {
+__device__ __forceinline__ void x_quantise(const XRegs<NB> &X, int K, const XStage &S, int g, bool live, float (&ss)[NB]) {
     const int lane = threadIdx.x & 63;
-    float4 w0 = make_float4(1.f, 1.f, 1.f, 1.f), w1 = w0;
-    if (norm_w && live) {
-        w0 = ldg<float4>(norm_w + g * 8);
-        w1 = ldg<float4>(norm_w + g * 8 + 4);
-    }
+    const float4 w0 = X.w0, w1 = X.w1;
 #pragma unroll
     for (int t = 0; t < NB; ++t) {
         const float4 a0 = X.a[t], a1 = X.b[t];

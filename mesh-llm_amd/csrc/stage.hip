@@ -464,9 +464,10 @@ int session_new(mesh_stage *st, mesh_session **out) {
         return rc;
     if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
     if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && hp.n_ff > 0) {
-        if ((rc = sess_alloc(s.get(), &p, B * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
+        const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
+        if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
-        if ((rc = sess_alloc(s.get(), &p, B * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
+        if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
         s->ffn16 = static_cast<uint16_t *>(p);
         if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
     }
@@ -571,14 +572,16 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
-    if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
+    if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
+    else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    if (rc != MESH_OK) return rc;
     if (skinny) {
         SkinnyArgs qa;
         qa.n_mat = 3;
         qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
-        qa.x = xn; qa.ldx = E; qa.K = E; qa.T = T;
+        qa.x = xn; qa.K = E; qa.T = T;
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
     } else {
@@ -608,12 +611,14 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;     // a batch of decode steps still splits the long KV
     { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
     if (rc != MESH_OK) return rc;
-    if ((rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream)) != MESH_OK) return rc;
+    if (skinny) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
+    else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
+    if (rc != MESH_OK) return rc;
     if (skinny) {
         SkinnyArgs oa;
         oa.n_mat = 1;
         oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
-        oa.x = xn; oa.ldx = QD; oa.K = QD; oa.T = T;
+        oa.x = xn; oa.K = QD; oa.T = T;
         oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny(oa, stream)) != MESH_OK) return rc;
@@ -623,19 +628,21 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         go.residual = s->x; go.ldres = E;
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
-    if ((rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream)) != MESH_OK) return rc;
-    if (skinny && L.w_gate.type == L.w_up.type) {
+    if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
+    else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    if (rc != MESH_OK) return rc;
+    if (skinny) {
         // gate and up in one pass with the SwiGLU epilogue, written as f16 straight into the down projection's input
         SkinnyArgs ga;
         ga.n_mat = 2;
         ga.mat[0] = mat_of(L.w_gate, nullptr, FF, nullptr);
         ga.mat[1] = mat_of(L.w_up, nullptr, FF, nullptr);
-        ga.x = xn; ga.ldx = E; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
-        ga.y16 = f16ffn; ga.ldy16 = FF;
+        ga.x = xn; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
+        ga.y16 = f16ffn;
         SkinnyArgs da;
         da.n_mat = 1;
         da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
-        da.x = f16ffn; da.ldx = FF; da.K = FF; da.T = T;
+        da.x = f16ffn; da.K = FF; da.T = T;
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny(ga, stream)) != MESH_OK) return rc;
@@ -666,7 +673,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
         if (T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
-            const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0;
+            const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0 &&
+                                L.w_gate.type == L.w_up.type;
             if (skinny || T >= PREFILL_MIN_TOKENS) {
                 if ((rc = run_layer_prefill(s, L, il, T, max_keys, skinny)) != MESH_OK) return rc;
                 continue;
