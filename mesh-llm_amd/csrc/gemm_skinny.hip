@@ -35,9 +35,10 @@ namespace mesh {
 
 constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
-constexpr int SK_DEPTH = 4;               // weight tiles a wave keeps in flight
+constexpr int SK_DEPTH_Q4 = 4;            // weight tiles a wave keeps in flight (2304 B each)
+constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B and their fragments need more registers
 constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA N)
-constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own
+constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
@@ -198,6 +199,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
     extern __shared__ __align__(16) uint8_t smem[];
     float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
     constexpr int TB = TileRegs<TYPE>::BYTES;
+    constexpr int SK_DEPTH = TYPE == MESH_Q4_K ? SK_DEPTH_Q4 : SK_DEPTH_Q6;
     const int K = a.K, nsb = K / QK_K;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: tile addresses become SGPR base + lane offset

@@ -80,7 +80,8 @@ def test_persistent_decode_matches_oracle_and_plain_path(tmp_path, name, depth):
             expected_steps += 1
             assert fast.persistent_steps == expected_steps, "the persistent kernel did not take this batch"
             assert rel_l2(got, ref) <= 1e-3, (name, rnd, T)
-            assert rel_l2(got, alt) <= 2e-4, (name, rnd, T)
+            # the default session runs batches of three and more through the skinny MFMA GEMM (f16 activations)
+            assert rel_l2(got, alt) <= (2e-4 if T < 3 else 3e-3), (name, rnd, T)
     assert plain.persistent_steps == 0
     # both paths appended the same keys and values (f16 of nearly equal f32 numbers)
     for il in range(nl):
@@ -90,7 +91,7 @@ def test_persistent_decode_matches_oracle_and_plain_path(tmp_path, name, depth):
             k2, v2 = plain.kv_read(il, s, depth, n_new)
             ko = orc.k[il, s, :, depth:depth + n_new].transpose(1, 0, 2)
             f = lambda a: np.asarray(a).view(np.float16).astype(np.float32)
-            assert rel_l2(f(k1), f(k2)) <= 1e-3 and rel_l2(f(v1), f(v2)) <= 1e-3
+            assert rel_l2(f(k1), f(k2)) <= 3e-3 and rel_l2(f(v1), f(v2)) <= 3e-3
             assert rel_l2(f(k1), f(ko)) <= 2e-3
     fast.close()
     plain.close()
