@@ -36,5 +36,8 @@ struct AttnArgs {
 };
 // token t attends to cache positions [0, pos[t]] of sequence seq[t]
 int attention(const AttnArgs &a, int T, hipStream_t stream);
+// The same for a chunk of T consecutive positions pos0 .. pos0 + T - 1 of one sequence, on the matrix cores
+// (attn_prefill.hip; head_dim 128).  a.pos / a.seq / a.part / a.ml are not used.
+int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t stream);
 
 }  // namespace mesh

@@ -1,0 +1,161 @@
+// Causal GQA attention for a prefill chunk on the matrix cores (head_dim 128, f16 KV cache).
+//
+// The chunk is T consecutive positions pos0 .. pos0 + T - 1 of one sequence whose keys and values are already in
+// the cache (rope_kv appended them); token t attends to cache positions [0, pos0 + t].  A workgroup takes 32
+// queries of every head of one KV-head group (one wave per head), walks the keys in tiles of 32 and keeps the
+// running softmax in registers:
+//   S^T = K . Q^T        (32 keys x 32 queries, v_mfma_f32_32x32x16_f16 over the 128 dims)
+//   O^T += V^T . P^T     (128 dims x 32 queries, contraction over the 32 keys)
+// Both products are arranged transposed so that a lane owns ONE query column: the softmax maximum and sum of a
+// query are reductions over the lane's own 16 registers plus one cross-half shuffle, and the rescale of O is a
+// per-lane scalar.  K and V tiles are staged once per workgroup in LDS (all heads of the group share them), V
+// transposed on the way in because the contraction index (keys) has to be contiguous in an MFMA operand.
+// The MFMA k-slots of the second product are the lane's own S^T registers, in the order the hardware leaves them:
+// slot (half, j) of the first MFMA is key 4*half + j (j < 4) or 8 + 4*half + j - 4; the V^T operand is read from LDS
+// with the same key order, so no data moves between lanes.
+//
+// Same result as the per-token kernel of attn.hip (ggml's soft_max + mul_mat of the attention block, reached from
+// rpc_server::graph_compute, third_party/llama.cpp/patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451)
+// except that Q and the probabilities are rounded to f16 for the matrix cores; sums are f32.
+
+#include "attn.hpp"
+
+namespace mesh {
+
+constexpr int PF_HD = 128;
+constexpr int PF_TILE = 32;                 // queries per workgroup and keys per step
+constexpr int PF_KPITCH = PF_HD + 8;        // halfs per key row of the K tile in LDS (bank-conflict padding)
+constexpr int PF_VPITCH = PF_TILE + 4;      // halfs per dim row of the transposed V tile
+
+typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 pf_h2 __attribute__((ext_vector_type(2)));
+typedef float pf_f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t pf_u4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t pf_pack(float a, float b) {
+    const pf_h2 h = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw) {
+    __shared__ __align__(16) _Float16 sK[PF_TILE * PF_KPITCH];
+    __shared__ __align__(16) _Float16 sVt[PF_HD * PF_VPITCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+    const int qcol = lane & 31, half = lane >> 5;
+    const int qt = blockIdx.x, kvh = blockIdx.y;
+    const int h = kvh * a.group + blockIdx.z * hpw + wave;
+    const int tq = qt * PF_TILE + qcol;
+    const bool q_live = tq < T;
+    const int pos_q = pos0 + tq;
+
+    // Q^T fragments of this lane's query, scaled so that the scores are in log2 units
+    const float qs = a.scale * 1.44269504088896341f;
+    pf_h8 qf[8];
+    {
+        const float *qp = a.q + ((size_t)(q_live ? tq : 0) * a.n_head + h) * PF_HD + 8 * half;
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc) {
+            const float4 v0 = *reinterpret_cast<const float4 *>(qp + kc * 16), v1 = *reinterpret_cast<const float4 *>(qp + kc * 16 + 4);
+            const float z = q_live ? qs : 0.f;
+            const pf_u4 p = {pf_pack(v0.x * z, v0.y * z), pf_pack(v0.z * z, v0.w * z), pf_pack(v1.x * z, v1.y * z), pf_pack(v1.z * z, v1.w * z)};
+            qf[kc] = __builtin_bit_cast(pf_h8, p);
+        }
+    }
+    pf_f16v o[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
+    const int q_end = qt * PF_TILE + PF_TILE < T ? qt * PF_TILE + PF_TILE : T;      // queries of this tile: [qt*32, q_end)
+    const int n_keys = pos0 + q_end;                                                // keys any of them may see
+    for (int k0 = 0; k0 < n_keys; k0 += PF_TILE) {
+        // stage the K tile as it is and the V tile transposed; rows past the context end are clamped (masked below)
+        for (int p = tid; p < PF_TILE * 16; p += nthreads) {
+            const int key = p >> 4, piece = p & 15;
+            int kr = k0 + key;
+            kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
+            const uint4 kv = *reinterpret_cast<const uint4 *>(a.kcache + (base + kr) * PF_HD + piece * 8);
+            const uint4 vv = *reinterpret_cast<const uint4 *>(a.vcache + (base + kr) * PF_HD + piece * 8);
+            *reinterpret_cast<uint4 *>(sK + key * PF_KPITCH + piece * 8) = kv;
+            const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                reinterpret_cast<uint16_t *>(sVt)[(piece * 8 + e) * PF_VPITCH + key] = (uint16_t)(vw[e >> 1] >> (16 * (e & 1)));
+        }
+        __syncthreads();
+
+        // S^T = K . Q^T : lane (key row = lane % 32 of the A operand, query column = lane % 32 of the result)
+        pf_f16v s;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc) {
+            const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + qcol * PF_KPITCH + kc * 16 + 8 * half);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s, 0, 0, 0);
+        }
+        // register i of the result is key k0 + 8 * (i / 4) + 4 * half + i % 4 for query qcol
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = k0 + 8 * (i >> 2) + 4 * half + (i & 3);
+            s[i] = (q_live && key <= pos_q) ? s[i] : -INFINITY;
+            mx = fmaxf(mx, s[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;       // a query that has seen no key yet
+        const float corr = exp2f(m - m_use);                        // exp2(-inf) = 0 while nothing is accumulated
+        float p[16], ps = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { p[i] = exp2f(s[i] - m_use); ps += p[i]; }
+        ps += __shfl_xor(ps, 32);
+        l = l * corr + ps;
+        m = m_new;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+        // P^T as the B operand: the lane's own registers, 8 per MFMA
+        const pf_u4 pu1 = {pf_pack(p[0], p[1]), pf_pack(p[2], p[3]), pf_pack(p[4], p[5]), pf_pack(p[6], p[7])};
+        const pf_u4 pu2 = {pf_pack(p[8], p[9]), pf_pack(p[10], p[11]), pf_pack(p[12], p[13]), pf_pack(p[14], p[15])};
+        const pf_h8 p1 = __builtin_bit_cast(pf_h8, pu1), p2 = __builtin_bit_cast(pf_h8, pu2);
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+            const _Float16 *vrow = sVt + (db * 32 + qcol) * PF_VPITCH + 4 * half;     // dim row, this half's keys
+            const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow), a1 = *reinterpret_cast<const uint2 *>(vrow + 8);
+            const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 16), a3 = *reinterpret_cast<const uint2 *>(vrow + 24);
+            const pf_u4 v1 = {a0.x, a0.y, a1.x, a1.y}, v2 = {a2.x, a2.y, a3.x, a3.y};
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v1), p1, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v2), p2, o[db], 0, 0, 0);
+        }
+        __syncthreads();        // the tiles are overwritten by the next step
+    }
+    if (q_live) {
+        const float inv = 1.0f / l;
+        float *op = a.out + ((size_t)tq * a.n_head + h) * PF_HD;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4)
+                *reinterpret_cast<float4 *>(op + db * 32 + 8 * i4 + 4 * half) =
+                    make_float4(o[db][4 * i4] * inv, o[db][4 * i4 + 1] * inv, o[db][4 * i4 + 2] * inv, o[db][4 * i4 + 3] * inv);
+    }
+}
+
+int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (a.head_dim != PF_HD) return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: head_dim %d (128 only)", a.head_dim);
+    if (a.group < 1 || a.n_head != a.group * a.n_kv || pos0 < 0 || pos0 + T > a.n_ctx || seq < 0)
+        return fail(MESH_ERR_INVALID, "attention_chunk: bad head layout or chunk [%d, %d) outside the context of %d", pos0, pos0 + T, a.n_ctx);
+    int hpw = a.group;                       // heads (waves) per workgroup: the largest divisor of the group up to 8
+    while (hpw > 8 || a.group % hpw) --hpw;
+    const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
+    attn_chunk_kernel<<<grid, dim3((unsigned)(64 * hpw)), 0, stream>>>(a, T, pos0, seq, hpw);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+}  // namespace mesh

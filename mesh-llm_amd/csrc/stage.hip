@@ -609,7 +609,11 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
     aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;     // a batch of decode steps still splits the long KV
-    { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
+    {
+        ProfScope ps(s, MESH_PROF_ATTN);
+        if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
+        else rc = attention(aa, T, stream);
+    }
     if (rc != MESH_OK) return rc;
     if (skinny) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
     else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
@@ -819,6 +823,11 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
     MESH_HIP_TRY(hipSetDevice(st->device));
     hipStream_t stream = s->stream;
 
+    // a run of consecutive positions of one sequence (a prefill chunk) can use the chunk attention kernel
+    s->chunk_pos0 = b->pos[0];
+    s->chunk_seq = b->seq_id ? b->seq_id[0] : 0;
+    for (int i = 1; i < T && s->chunk_pos0 >= 0; ++i)
+        if (b->pos[i] != b->pos[0] + i || (b->seq_id ? b->seq_id[i] : 0) != s->chunk_seq) s->chunk_pos0 = -1;
     // positions / sequence ids -> device, through a ring of pinned slots so calls may be queued back to back
     const size_t B = (size_t)st->n_batch_max;
     if (s->meta_counter && s->meta_counter % META_SLOTS == 0) MESH_HIP_TRY(hipStreamSynchronize(stream));   // ring wraps: older copies are done

@@ -89,6 +89,8 @@ struct mesh_session {
     size_t io_stage_bytes = 0;
     void *h_io = nullptr;           // pinned host staging
     int attn_splits_max = 0;
+    // set per call: the batch is one run of consecutive positions of one sequence (first position, sequence), else -1
+    int chunk_pos0 = -1, chunk_seq = -1;
     // persistent decode kernel (decode_mega.hip): exchange buffers in uncached device memory, per-layer table
     struct Mega {
         bool ready = false;

@@ -259,17 +259,20 @@ def test_prefill_mfma_path_matches_oracle_and_decode_path(tmp_path):
 
 
 def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
-    m, cfg, tensors, st = _open(tmp_path, "tiny-qwen2", range(0, 3), 0, 3, n_ctx=256, n_seq=2, n_batch=208)
+    m, cfg, tensors, st = _open(tmp_path, "tiny-qwen2", range(0, 3), 0, 3, n_ctx=512, n_seq=2, n_batch=208)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(43))
-    orc = StageOracle(cfg, tensors, 0, 3, 256, n_seq_max=2)
+    orc = StageOracle(cfg, tensors, 0, 3, 512, n_seq_max=2)
     ses = st.session()
-    for T, seq in ((200, 0), (47, 1)):          # large-tile GEMM, then the skinny GEMM (three 16-column passes, ragged)
+    # large-tile GEMM + chunk attention from position 0, a second chunk on top of the first (ragged: 200 = 6 * 32 + 8),
+    # then the skinny GEMM (three 16-column passes, ragged) on the other sequence
+    for T, pos0, seq in ((200, 0, 0), (200, 200, 0), (47, 0, 1)):
         x = rng.standard_normal((T, E)).astype(np.float32)
         sq = np.full(T, seq, np.int32)
-        got = ses.decode(x, np.arange(T), seq=sq).view(np.float32).reshape(T, E)
-        ref = orc.forward(x, np.arange(T), seq=sq)
-        assert rel_l2(got, ref) <= 3e-3, T
+        pos = np.arange(pos0, pos0 + T)
+        got = ses.decode(x, pos, seq=sq).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos, seq=sq)
+        assert rel_l2(got, ref) <= 3e-3, (T, pos0)
     ses.close(); st.close()
 
 
