@@ -161,6 +161,34 @@ def test_llama3_8b_shaped_layers_decode_with_long_kv(tmp_path):
     st.close()
 
 
+def test_qwen25_32b_shaped_layer_all_decode_paths(tmp_path):
+    """One real-shape Qwen2.5-32B layer (hidden 5120 = 20 super-blocks, 40 heads / 8 KV heads = 5 per group, FFN 27648, q/k/v
+    bias, NEOX rope): batch 1 and 4 on the mat-vec kernel, 16 and a ragged 11 on the skinny MFMA GEMM, at KV depth 100."""
+    name = "qwen2.5-32b"
+    m, cfg, tensors, st = _open(tmp_path, name, [7], 7, 8, n_ctx=128, n_seq=16, n_batch=16)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 7, 8, 128, n_seq_max=16)
+    rng = np.random.Generator(np.random.PCG64(14))
+    n_past = 100
+    for s_ in range(16):
+        k = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
+        v = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
+        ses.kv_write(7, s_, 0, k, v)
+        orc.k[0, s_, :, :n_past] = k.transpose(1, 0, 2)
+        orc.v[0, s_, :, :n_past] = v.transpose(1, 0, 2)
+    nxt = [n_past] * 16
+    for seqs, tol in (([3], 1e-3), ([0, 5, 9, 12], 1e-3), (list(range(16)), 3e-3), ([1, 2, 3, 4, 6, 7, 8, 10, 11, 13, 15], 3e-3)):
+        T = len(seqs)
+        pos = [nxt[q] for q in seqs]
+        for q in seqs:
+            nxt[q] += 1
+        x = rng.standard_normal((T, 5120)).astype(np.float32)
+        got = ses.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 5120)
+        ref = orc.forward(x, pos, seq=seqs)
+        assert rel_l2(got, ref) <= tol, T
+    ses.close(); st.close()
+
+
 def test_decode_argument_errors(tmp_path):
     m, cfg, tensors, st = _open(tmp_path, "tiny-llama", range(0, 2), 0, 2, n_ctx=32, n_seq=1, n_batch=4)
     ses = st.session()
