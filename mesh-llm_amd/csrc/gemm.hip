@@ -6,7 +6,10 @@
 // steps of 64.  Per step the 128 x 64 weight slab is dequantised from its K-quant blocks straight into LDS as
 // f16 (each thread: one row, one 32-element sub-block), the 128 x 64 activation slab is copied next to it, and
 // the four waves (2 x 2, 64 x 64 each) issue v_mfma_f32_32x32x16_f16 on 16-byte LDS fragments with f32
-// accumulation.  Weights cross HBM once per 128 tokens; dequantisation is amortised over 128 columns.
+// accumulation.  Weights cross HBM once per 128 tokens; dequantisation is amortised over 128 columns.  The two
+// LDS stages alternate: the raw bytes of step k+1 are fetched into registers before the MFMAs of step k and
+// dequantised after them, so global-memory latency and the dequant VALU work overlap the matrix cores (two
+// workgroups fit a CU).
 //
 // MFMA operand layout used below (checked on hardware): A lane l = row l%32, k = 8*(l/32)+j; B lane l = column
 // l%32, same k; accumulator register i of lane l = D[8*(i/4) + 4*(l/32) + i%4][l%32].
@@ -26,73 +29,101 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
 }
 
-// 32 dequantised elements (one sub-block of one row) -> 64 bytes of LDS
-__device__ __forceinline__ void store32(_Float16 *dst, const float (&v)[32]) {
-    uint4 *d4 = reinterpret_cast<uint4 *>(dst);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        d4[i] = make_uint4(pack_h2(v[8 * i], v[8 * i + 1]), pack_h2(v[8 * i + 2], v[8 * i + 3]),
-                           pack_h2(v[8 * i + 4], v[8 * i + 5]), pack_h2(v[8 * i + 6], v[8 * i + 7]));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// four bytes (values < 64) -> four f16 holding (value - off) * s + mn, as two packed dwords.  0x6400 | q is the f16
+// 1024 + q exactly; the offset comes off exactly, then one packed fma applies the block scale and minimum.
+__device__ __forceinline__ void dequant4(uint32_t q, half2v off, half2v s, half2v mn, uint32_t &lo, uint32_t &hi) {
+    const half2v a = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04010400u)) - off;
+    const half2v b = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04030402u)) - off;
+    lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(a, s, mn));
+    hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(b, s, mn));
+}
+__device__ __forceinline__ half2v h2_splat(float v) {
+    const _Float16 h = (_Float16)v;
+    return half2v{h, h};
 }
 
-// q4_K: row r of tile, k-chunk c (64 elements) of the super-block, half h (sub-block 2c + h)
-__device__ __forceinline__ void dequant_q4k_32(const uint8_t *__restrict__ tile, int r, int c, int h, _Float16 *dst) {
-    const uint4 hdr = *reinterpret_cast<const uint4 *>(tile + r * 16);
-    const uint4 qa = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32);
-    const uint4 qb = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32 + 16);
-    const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
-    const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
-    const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
-    const int sh = (c & 1) * 16 + h * 8;
-    const float ds = d * (float)((scw >> sh) & 0xFFu), dm = dmin * (float)((mnw >> sh) & 0xFFu);
-    const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-    float v[32];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t q = (w[j] >> (4 * h)) & 0x0F0F0F0Fu;
-        v[4 * j + 0] = fmaf(ds, (float)(q & 0xFFu), -dm);
-        v[4 * j + 1] = fmaf(ds, (float)((q >> 8) & 0xFFu), -dm);
-        v[4 * j + 2] = fmaf(ds, (float)((q >> 16) & 0xFFu), -dm);
-        v[4 * j + 3] = fmaf(ds, (float)(q >> 24), -dm);
+// Raw bytes of one (row, 32-element sub-block) of a tile: what a staging thread prefetches one k-step ahead.
+template <int TYPE> struct RawSub;
+
+// q4_K: row r of the tile, k-chunk c (64 elements) of the super-block, half h (sub-block 2c + h)
+template <> struct RawSub<MESH_Q4_K> {
+    uint4 hdr, qa, qb;
+    __device__ __forceinline__ void load(const uint8_t *__restrict__ tile, int r, int c, int) {
+        hdr = *reinterpret_cast<const uint4 *>(tile + r * 16);
+        qa = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32);
+        qb = *reinterpret_cast<const uint4 *>(tile + 256 + r * 128 + c * 32 + 16);
     }
-    store32(dst, v);
-}
+    __device__ __forceinline__ void store(int c, int h, _Float16 *dst) const {
+        const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+        const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
+        const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
+        const int sh = (c & 1) * 16 + h * 8;
+        const half2v s = h2_splat(d * (float)((scw >> sh) & 0xFFu)), mn = h2_splat(-dmin * (float)((mnw >> sh) & 0xFFu));
+        const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 o;
+            dequant4((w[2 * i] >> (4 * h)) & 0x0F0F0F0Fu, off, s, mn, o.x, o.y);
+            dequant4((w[2 * i + 1] >> (4 * h)) & 0x0F0F0F0Fu, off, s, mn, o.z, o.w);
+            d4[i] = o;
+        }
+    }
+};
 
 // q6_K: row r, k-chunk c: half n = c/2, elements 128n + 32*t4 + l with t4 = 2*(c%2) + h, l = 0..31
-__device__ __forceinline__ void dequant_q6k_32(const uint8_t *__restrict__ tile, int r, int c, int h, _Float16 *dst) {
-    const int n = c >> 1, t4 = 2 * (c & 1) + h;
-    const uint8_t *ql = tile + r * 128 + 64 * n + 32 * (t4 & 1);
-    const uint8_t *qh = tile + 2048 + r * 64 + 32 * n;
-    const uint4 la = *reinterpret_cast<const uint4 *>(ql), lb = *reinterpret_cast<const uint4 *>(ql + 16);
-    const uint4 ha = *reinterpret_cast<const uint4 *>(qh), hb = *reinterpret_cast<const uint4 *>(qh + 16);
-    const int8_t *sc = reinterpret_cast<const int8_t *>(tile + 3072 + r * 16) + 8 * n + 2 * t4;
-    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(tile + 3328 + r * 2));
-    const float ds0 = d * (float)sc[0], ds1 = d * (float)sc[1];
-    const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
-    const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
-    float v[32];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const uint32_t nib = (t4 & 2) ? (lw[j] >> 4) & 0x0F0F0F0Fu : lw[j] & 0x0F0F0F0Fu;
-        const uint32_t hb2 = ((hw[j] >> (2 * t4)) & 0x03030303u) << 4;
-        const uint32_t q = nib | hb2;
-        const float ds = j < 4 ? ds0 : ds1;
-        v[4 * j + 0] = ds * (float)((int)(q & 0xFFu) - 32);
-        v[4 * j + 1] = ds * (float)((int)((q >> 8) & 0xFFu) - 32);
-        v[4 * j + 2] = ds * (float)((int)((q >> 16) & 0xFFu) - 32);
-        v[4 * j + 3] = ds * (float)((int)(q >> 24) - 32);
+template <> struct RawSub<MESH_Q6_K> {
+    uint4 la, lb, ha, hb;
+    uint32_t sc, d;
+    __device__ __forceinline__ void load(const uint8_t *__restrict__ tile, int r, int c, int h) {
+        const int n = c >> 1, t4 = 2 * (c & 1) + h;
+        const uint8_t *ql = tile + r * 128 + 64 * n + 32 * (t4 & 1);
+        const uint8_t *qh = tile + 2048 + r * 64 + 32 * n;
+        la = *reinterpret_cast<const uint4 *>(ql); lb = *reinterpret_cast<const uint4 *>(ql + 16);
+        ha = *reinterpret_cast<const uint4 *>(qh); hb = *reinterpret_cast<const uint4 *>(qh + 16);
+        sc = *reinterpret_cast<const uint16_t *>(tile + 3072 + r * 16 + 8 * n + 2 * t4);
+        d = *reinterpret_cast<const uint16_t *>(tile + 3328 + r * 2);
     }
-    store32(dst, v);
-}
+    __device__ __forceinline__ void store(int c, int h, _Float16 *dst) const {
+        const int t4 = 2 * (c & 1) + h;
+        const float df = f16_bits_to_f32((uint16_t)d);
+        const half2v s0 = h2_splat(df * (float)(int8_t)(sc & 0xFFu)), s1 = h2_splat(df * (float)(int8_t)(sc >> 8));
+        const half2v off = {(_Float16)1056.f, (_Float16)1056.f}, zero = {(_Float16)0.f, (_Float16)0.f};
+        const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
+        const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t q[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int j = 2 * i + e;
+                const uint32_t nib = (t4 & 2) ? (lw[j] >> 4) & 0x0F0F0F0Fu : lw[j] & 0x0F0F0F0Fu;
+                q[e] = nib | (((hw[j] >> (2 * t4)) & 0x03030303u) << 4);
+            }
+            const half2v s = i < 2 ? s0 : s1;       // one scale per 16 elements
+            uint4 o;
+            dequant4(q[0], off, s, zero, o.x, o.y);
+            dequant4(q[1], off, s, zero, o.z, o.w);
+            d4[i] = o;
+        }
+    }
+};
 
+// Software pipeline: while the matrix cores work on LDS stage kc & 1, the staging threads hold the raw weight
+// bytes and activations of step kc + 1 in registers (loads in flight), then dequantise them into the other stage.
 template <int TYPE>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
-    __shared__ __align__(16) _Float16 Ws[GM * LDS_LD];
-    __shared__ __align__(16) _Float16 Xs[GN * LDS_LD];
+    extern __shared__ __align__(16) _Float16 gemm_smem[];
+    _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
+    _Float16 *Xs = gemm_smem + 2 * GM * LDS_LD;                // [2][GN][LDS_LD]
     constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m0 = blockIdx.x * GM, t0 = blockIdx.y * GN;
-    const int nsb = a.K / QK_K;
+    const int nsb = a.K / QK_K, n_steps = a.K / GK;
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;     // wave's 64 x 64 corner of the tile
 
     float16v acc[2][2];
@@ -107,44 +138,55 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     const int srow = tid >> 1, sh = tid & 1;
     const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
     const bool wlive = wrow < a.M_pad;
-    const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)(wrow >> 4) * nsb * TB;
+    const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
     const int tok = t0 + srow;
     const bool xlive = tok < a.T;
-    const _Float16 *xrow = a.X + (size_t)tok * a.ldx + 32 * sh;
+    const _Float16 *xrow = a.X + (size_t)(xlive ? tok : 0) * a.ldx + 32 * sh;
 
-    for (int kc = 0; kc < a.K / GK; ++kc) {
-        const int sb = kc >> 2, c = kc & 3;
-        // stage the weight slab
+    RawSub<TYPE> rw;
+    uint4 rx[4];
+    auto fetch = [&](int kc) {
+        rw.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
+        const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rx[i] = s4[i];
+    };
+    auto stage = [&](int kc, int buf) {
+        _Float16 *wdst = Ws + (buf * GM + srow) * LDS_LD + 32 * sh;
         if (wlive) {
-            const uint8_t *tile = wtile_row + (size_t)sb * TB;
-            if (TYPE == MESH_Q4_K) dequant_q4k_32(tile, wrow & 15, c, sh, Ws + srow * LDS_LD + 32 * sh);
-            else dequant_q6k_32(tile, wrow & 15, c, sh, Ws + srow * LDS_LD + 32 * sh);
+            rw.store(kc & 3, sh, wdst);
         } else {
-            uint4 *d4 = reinterpret_cast<uint4 *>(Ws + srow * LDS_LD + 32 * sh);
+            uint4 *d4 = reinterpret_cast<uint4 *>(wdst);
 #pragma unroll
             for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
         }
-        // stage the activation slab
-        {
-            uint4 *d4 = reinterpret_cast<uint4 *>(Xs + srow * LDS_LD + 32 * sh);
-            const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+        uint4 *x4 = reinterpret_cast<uint4 *>(Xs + (buf * GN + srow) * LDS_LD + 32 * sh);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) d4[i] = xlive ? s4[i] : make_uint4(0, 0, 0, 0);
-        }
-        __syncthreads();
+        for (int i = 0; i < 4; ++i) x4[i] = xlive ? rx[i] : make_uint4(0, 0, 0, 0);
+    };
+
+    fetch(0);
+    stage(0, 0);
+    __syncthreads();
+    for (int kc = 0; kc < n_steps; ++kc) {
+        const int buf = kc & 1;
+        const bool more = kc + 1 < n_steps;
+        if (more) fetch(kc + 1);
+        const _Float16 *Wb = Ws + buf * GM * LDS_LD, *Xb = Xs + buf * GN * LDS_LD;
 #pragma unroll
         for (int ks = 0; ks < GK / 16; ++ks) {
             half8 af[2], bf[2];
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                af[i] = *reinterpret_cast<const half8 *>(Ws + (wm + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
-                bf[i] = *reinterpret_cast<const half8 *>(Xs + (wn + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
+                af[i] = *reinterpret_cast<const half8 *>(Wb + (wm + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
+                bf[i] = *reinterpret_cast<const half8 *>(Xb + (wn + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
+        if (more) stage(kc + 1, buf ^ 1);
         __syncthreads();
     }
 
@@ -181,8 +223,15 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     GemmArgs k = a;
     k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
     const dim3 grid((unsigned)((a.M + GM - 1) / GM), (unsigned)((a.T + GN - 1) / GN));
-    if (a.type == MESH_Q4_K) gemm_kq_kernel<MESH_Q4_K><<<grid, dim3(GEMM_THREADS), 0, stream>>>(k);
-    else if (a.type == MESH_Q6_K) gemm_kq_kernel<MESH_Q6_K><<<grid, dim3(GEMM_THREADS), 0, stream>>>(k);
+    constexpr size_t smem = sizeof(_Float16) * 2 * (GM + GN) * LDS_LD;        // two stages of both slabs: 73 728 B
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<MESH_Q4_K>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<MESH_Q6_K>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    if (a.type == MESH_Q4_K) gemm_kq_kernel<MESH_Q4_K><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
+    else if (a.type == MESH_Q6_K) gemm_kq_kernel<MESH_Q6_K><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
     else return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
