@@ -78,162 +78,26 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p) {
 // KS partials of a row meet after one barrier.
 template <int TYPE, int NB, int NU>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernelArgs a) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int TB = TileRegs<TYPE>::BYTES;
-    constexpr bool NEED_I16 = TYPE == MESH_Q6_K;
-    const int K = a.K;
-    XStage S;
-    S.xh = reinterpret_cast<int8_t *>(smem);
-    S.xl = S.xh + NB * K;
-    S.xd = reinterpret_cast<float *>(S.xl + NB * K);
-    S.xs = S.xd + NB * (K >> 5);
-    S.xi16 = reinterpret_cast<int *>(S.xs + NB * (K >> 5));
-    S.ssq = reinterpret_cast<float *>(S.xi16 + (NEED_I16 ? NB * (K >> 4) : 0));
-    S.red = S.ssq + GEMV_WAVES * NB;
+    const int bid = blockIdx.x, nblk = gridDim.x;
+#include "gemv_body.inc"
+}
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // scalar, so that tile addresses and matrix selection stay in SGPRs
-    GEMV_MARK(0);
-    // activations first: they gate everything
-    const int ng = K >> 3;
-    const float *xcol = a.x;
-    size_t eoff = 0, ycol = 0;
-    if (a.expert_ids) {
-        const int p = blockIdx.y;
-        xcol = a.x + (size_t)(p / a.x_div) * a.ldx;
-        eoff = (size_t)a.expert_ids[p] * a.expert_stride;
-        ycol = p;
+// q/k/v groups whose matrices are of both K-quant types (attn_v in q6_K on the "more bits" layers of a Q4_K_M
+// file): one launch, the first n4 workgroups run the q4_K matrices, the rest the q6_K ones.
+template <int NB>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const GemvKernelArgs a4, const GemvKernelArgs a6, int n4) {
+    constexpr int NU = 1;
+    if ((int)blockIdx.x < n4) {
+        const GemvKernelArgs &a = a4;
+        constexpr int TYPE = MESH_Q4_K;
+        const int bid = blockIdx.x, nblk = n4;
+#include "gemv_body.inc"
+    } else {
+        const GemvKernelArgs &a = a6;
+        constexpr int TYPE = MESH_Q6_K;
+        const int bid = (int)blockIdx.x - n4, nblk = (int)gridDim.x - n4;
+#include "gemv_body.inc"
     }
-    XRegs<NB> X;
-    x_fetch<NB>(X, xcol, a.ldx, tid, tid < ng);
-    norm_fetch<NB>(X, a.norm_w, tid, tid < ng);
-
-    const int nsb = K / QK_K;
-    const int KS = a.ks, RS = GEMV_WAVES / KS;
-    const int ks = wave % KS, rs = wave / KS;
-    const int total_rows = a.tile_begin[3];       // (a constant index: the host fills every unused slot with the total)
-    const int tr0 = (int)(((long long)blockIdx.x * total_rows) / gridDim.x);
-    const int tr1 = (int)(((long long)(blockIdx.x + 1) * total_rows) / gridDim.x);
-    const int rows_here = tr1 - tr0;
-    const int n_i = rs < RS ? (nsb - ks + KS - 1) / KS : 0;      // tiles per segment (ks < KS <= nsb)
-    const size_t row_stride = (size_t)nsb * TB;
-
-    auto tile_ptr = [&](const TileCursor<NU> &c) -> const uint8_t * {
-        const int tr = tr0 + c.j;
-        int mi = c.u;
-        if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        // (selected, not indexed: a dynamically indexed kernel-argument array is fetched with a load, and waiting for
-        // that address would drain every tile load in flight)
-        const uint8_t *wb = mi == 0 ? a.wbase[0] : mi == 1 ? a.wbase[1] : a.wbase[2];
-        return wb + eoff + (size_t)tr * row_stride + (size_t)(ks + KS * c.ii) * TB;
-    };
-
-    // Loads are unconditional: past its last tile a wave simply re-reads that tile (a cache hit).  With no load
-    // under a branch the compiler counts outstanding loads exactly and never has to drain the queue at a join.
-    TileCursor<NU> ld{rs, 0, 0}, cp{rs, 0, 0};
-    TileRegs<TYPE> t0, t1;
-    const bool any = n_i > 0 && rs < rows_here;
-    auto advance_load = [&]() {
-        TileCursor<NU> nx = ld;
-        nx.advance(n_i, RS);
-        if (nx.j < rows_here) ld = nx;
-    };
-    if (any) {
-        t0.load(tile_ptr(ld), lane);
-        advance_load();
-        t1.load(tile_ptr(ld), lane);
-        advance_load();
-    }
-    GEMV_MARK(1);
-
-    float ss[NB];
-#pragma unroll
-    for (int t = 0; t < NB; ++t) ss[t] = 0.f;
-    x_quantise<NB, NEED_I16>(X, K, S, tid, tid < ng, ss);
-    for (int g0 = GEMV_THREADS; g0 < ng; g0 += GEMV_THREADS) {
-        x_fetch<NB>(X, xcol, a.ldx, g0 + tid, g0 + tid < ng);
-        norm_fetch<NB>(X, a.norm_w, g0 + tid, g0 + tid < ng);
-        x_quantise<NB, NEED_I16>(X, K, S, g0 + tid, g0 + tid < ng, ss);
-    }
-    if (a.norm_w) {
-#pragma unroll
-        for (int t = 0; t < NB; ++t) {
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) ss[t] += __shfl_xor(ss[t], o);
-            if (lane == 0) S.ssq[wave * NB + t] = ss[t];
-        }
-    }
-    __syncthreads();
-    GEMV_MARK(2);
-
-    float acc[NB];
-#pragma unroll
-    for (int t = 0; t < NB; ++t) acc[t] = 0.f;
-    auto finish_segment = [&](const TileCursor<NU> &c) {
-#pragma unroll
-        for (int t = 0; t < NB; ++t) {
-            float v = acc[t];
-            v += __shfl_xor(v, 1);
-            v += __shfl_xor(v, 2);
-            if ((lane & 3) == 0) S.red[(((ks * rows_here + c.j) * NU + c.u) * 16 + (lane >> 2)) * NB + t] = v;
-            acc[t] = 0.f;
-        }
-    };
-    if (any) {
-        // two tiles alternate between the register sets; each is reloaded as soon as it has been consumed
-        while (true) {
-            tile_compute<NB>(t0, lane, ks + KS * cp.ii, S, K, acc);
-            if (cp.ii + 1 == n_i) finish_segment(cp);
-            cp.advance(n_i, RS);
-            t0.load(tile_ptr(ld), lane);
-            advance_load();
-            if (cp.j >= rows_here) break;
-            tile_compute<NB>(t1, lane, ks + KS * cp.ii, S, K, acc);
-            if (cp.ii + 1 == n_i) finish_segment(cp);
-            cp.advance(n_i, RS);
-            t1.load(tile_ptr(ld), lane);
-            advance_load();
-            if (cp.j >= rows_here) break;
-        }
-    }
-    GEMV_MARK(3);
-    __syncthreads();
-    GEMV_MARK(4);
-
-    // outputs of this workgroup: rows_here x 16 rows x NB columns
-    for (int o = tid; o < rows_here * 16 * NB; o += GEMV_THREADS) {
-        const int t = o % NB, r = (o / NB) % 16, j = o / (NB * 16);
-        const int tr = tr0 + j;
-        int mi = 0;
-        if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        const int row = (tr - a.tile_begin[mi]) * TILE_ROWS + r;
-        if (row >= a.M[mi]) continue;
-        float s0 = 0.f, s1 = 0.f;
-        for (int k2 = 0; k2 < KS; ++k2) {
-            s0 += S.red[(((k2 * rows_here + j) * NU + 0) * 16 + r) * NB + t];
-            if (NU == 2) s1 += S.red[(((k2 * rows_here + j) * NU + 1) * 16 + r) * NB + t];
-        }
-        if (a.norm_w) {
-            float q = 0.f;
-#pragma unroll
-            for (int w = 0; w < GEMV_WAVES; ++w) q += S.ssq[w * NB + t];
-            const float scale = 1.0f / sqrtf(q / (float)K + a.eps);
-            s0 *= scale;
-            s1 *= scale;
-        }
-        if (a.bias[mi]) s0 += a.bias[mi][row];
-        float out;
-        if (NU == 2) {
-            if (a.bias[1]) s1 += a.bias[1][row];
-            out = (s0 / (1.0f + expf(-s0))) * s1;
-        } else if (a.epi == EPI_RESIDUAL) {
-            out = a.residual[(size_t)t * a.ldres + row] + s0;
-        } else {
-            out = s0;
-        }
-        a.y[mi][((size_t)t + ycol) * a.ldy[mi] + row] = out;
-    }
-    GEMV_MARK(5);
 }
 
 constexpr size_t LDS_LIMIT = 160 * 1024;
@@ -275,12 +139,17 @@ static int n_compute_units() {
     return n;
 }
 
-// All matrices of `a` are tiled K-quants of one type.
-static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
+// Launch geometry of the K-quant matrices of `a` (all of one type) over `ncu` compute units.
+struct KquantPlan {
+    GemvKernelArgs ka;
+    int type, NU, KS, grid, rows_max;
+};
+static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
     const int type = a.mat[0].type;
     const int nsb = a.K / QK_K, NU = a.epi == EPI_SWIGLU ? 2 : 1;
     const size_t row_stride = (size_t)nsb * (type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES);
-    GemvKernelArgs ka{};
+    GemvKernelArgs &ka = p.ka;
+    ka = GemvKernelArgs{};
     int total_rows = 0;
     for (int i = 0; i < a.n_mat; ++i) {
         const int begin = (NU == 2 && i == 1) ? 0 : total_rows;     // gate and up share tile-row indices
@@ -293,11 +162,8 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
         if (!(NU == 2 && i == 1)) total_rows += (a.mat[i].M + TILE_ROWS - 1) / TILE_ROWS;
     }
     const int n_mat_k = NU == 2 ? 1 : a.n_mat;      // boundaries the kernel searches
-    for (int i = n_mat_k; i < 4; ++i) ka.tile_begin[i] = total_rows;
-    if (NU == 2) ka.tile_begin[1] = total_rows;
+    for (int i = n_mat_k; i < 4; ++i) ka.tile_begin[i] = total_rows;      // unused slots compare as "beyond the end"
     ka.n_mat = n_mat_k;
-    // unused boundary slots must compare as "beyond the end"
-    for (int i = n_mat_k; i < 3; ++i) { ka.tile_begin[i] = total_rows; }
     ka.ldx = a.ldx;
     ka.K = a.K;
     ka.norm_w = a.norm_w;
@@ -306,20 +172,30 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     ka.epi = a.epi;
     const int KS = nsb < GEMV_WAVES ? nsb : GEMV_WAVES;
     ka.ks = KS;
+    // tile-rows per workgroup: spread over the CUs, bounded by the LDS partial buffer
+    int rows_per_wg = (total_rows + ncu - 1) / ncu;
+    rows_per_wg = std::max(1, std::min(rows_per_wg, MAX_ROWS_X_KS / KS));
+    p.grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
+    p.rows_max = (total_rows + p.grid - 1) / p.grid;
+    p.type = type; p.NU = NU; p.KS = KS;
+    if (dot_smem_bytes(type, 1, a.K, p.rows_max, KS, NU) > LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemv: row length %d does not fit LDS", a.K);
+    return MESH_OK;
+}
+
+// All matrices of `a` are tiled K-quants of one type.
+static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     const int n_pairs = a.expert_ids ? a.n_pairs : 1;
+    if (a.expert_ids && (a.n_pairs <= 0 || a.x_div <= 0 || a.epi == EPI_RESIDUAL)) return fail(MESH_ERR_INVALID, "gemv: bad expert-indirection arguments");
+    KquantPlan plan;
+    int rc0 = plan_kquant(a, std::max(1, n_compute_units() / n_pairs), plan);
+    if (rc0 != MESH_OK) return rc0;
+    GemvKernelArgs &ka = plan.ka;
+    const int type = plan.type, NU = plan.NU, KS = plan.KS, grid = plan.grid, rows_max = plan.rows_max;
     if (a.expert_ids) {
-        if (a.n_pairs <= 0 || a.x_div <= 0 || a.epi == EPI_RESIDUAL) return fail(MESH_ERR_INVALID, "gemv: bad expert-indirection arguments");
         ka.expert_ids = a.expert_ids;
         ka.expert_stride = (size_t)tiled_bytes(type, a.mat[0].M, a.K);
         ka.x_div = a.x_div;
     }
-    // tile-rows per workgroup: spread over the CUs, bounded by the LDS partial buffer
-    const int ncu = std::max(1, n_compute_units() / n_pairs);
-    int rows_per_wg = (total_rows + ncu - 1) / ncu;
-    rows_per_wg = std::max(1, std::min(rows_per_wg, MAX_ROWS_X_KS / KS));
-    const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
-    const int rows_max = (total_rows + grid - 1) / grid;
-    if (dot_smem_bytes(type, 1, a.K, rows_max, KS, NU) > LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemv: row length %d does not fit LDS", a.K);
     if (a.expert_ids) {
         // every pair is its own single-column product
         ka.x = a.x;
@@ -349,6 +225,48 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     return MESH_OK;
 }
 
+template <int NB>
+static int launch_dual(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int n4, int n6, size_t smem, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dual_kernel<NB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
+        attr_set = true;
+    }
+    gemv_dual_kernel<NB><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(k4, k6, n4);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// a4: the q4_K matrices of a group, a6: its q6_K matrices; same activations, plain store epilogue
+static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream) {
+    const int ncu = n_compute_units();
+    double b4 = 0, b6 = 0;
+    for (int i = 0; i < a4.n_mat; ++i) b4 += (double)tiled_bytes(MESH_Q4_K, a4.mat[i].M, a4.K);
+    for (int i = 0; i < a6.n_mat; ++i) b6 += (double)tiled_bytes(MESH_Q6_K, a6.mat[i].M, a6.K);
+    int c6 = (int)(ncu * b6 / (b4 + b6) + 0.5);              // compute units in proportion to the bytes streamed
+    c6 = std::max(1, std::min(ncu - 1, c6));
+    KquantPlan p4, p6;
+    int rc;
+    if ((rc = plan_kquant(a4, ncu - c6, p4)) != MESH_OK || (rc = plan_kquant(a6, c6, p6)) != MESH_OK) return rc;
+    int t = 0;
+    while (t < a4.T) {
+        const int left = a4.T - t;
+        int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        auto need = [&](int n) { return std::max(dot_smem_bytes(MESH_Q4_K, n, a4.K, p4.rows_max, p4.KS, 1), dot_smem_bytes(MESH_Q6_K, n, a6.K, p6.rows_max, p6.KS, 1)); };
+        while (nb > 1 && need(nb) > LDS_LIMIT) nb >>= 1;
+        GemvKernelArgs k4 = p4.ka, k6 = p6.ka;
+        k4.x = k6.x = a4.x + (size_t)t * a4.ldx;
+        for (int i = 0; i < a4.n_mat; ++i) k4.y[i] = a4.mat[i].y + (size_t)t * a4.mat[i].ldy;
+        for (int i = 0; i < a6.n_mat; ++i) k6.y[i] = a6.mat[i].y + (size_t)t * a6.mat[i].ldy;
+        if (nb == 4) rc = launch_dual<4>(k4, k6, p4.grid, p6.grid, need(4), stream);
+        else if (nb == 2) rc = launch_dual<2>(k4, k6, p4.grid, p6.grid, need(2), stream);
+        else rc = launch_dual<1>(k4, k6, p4.grid, p6.grid, need(1), stream);
+        if (rc != MESH_OK) return rc;
+        t += nb;
+    }
+    return MESH_OK;
+}
+
 int gemv(const GemvArgs &a, hipStream_t stream) {
     if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.K <= 0 || a.T < 0)
         return fail(MESH_ERR_INVALID, "gemv: bad arguments (n_mat %d, K %d, T %d)", a.n_mat, a.K, a.T);
@@ -372,6 +290,18 @@ int gemv(const GemvArgs &a, hipStream_t stream) {
         return fail(MESH_ERR_UNSUPPORTED, "gemv: expert indirection needs K-quant expert matrices of one type");
     if (uniform) return type_is_tiled(a.mat[0].type) ? gemv_kquant(a, stream) : gemv_generic(a, stream);
     if (a.epi == EPI_SWIGLU) return fail(MESH_ERR_UNSUPPORTED, "gemv: gate and up of different types");
+    // the common mix -- every matrix q4_K or q6_K, plain store -- runs as one two-type launch
+    {
+        GemvArgs a4 = a, a6 = a;
+        a4.n_mat = a6.n_mat = 0;
+        bool kq_only = a.epi == EPI_STORE && !a.expert_ids;
+        for (int i = 0; i < a.n_mat && kq_only; ++i) {
+            if (a.mat[i].type == MESH_Q4_K) a4.mat[a4.n_mat++] = a.mat[i];
+            else if (a.mat[i].type == MESH_Q6_K) a6.mat[a6.n_mat++] = a.mat[i];
+            else kq_only = false;
+        }
+        if (kq_only && a4.n_mat > 0 && a6.n_mat > 0) return gemv_dual(a4, a6, stream);
+    }
     // mixed types side by side (a q/k/v group whose v is q6_K): one launch per run of equal family
     int i = 0;
     while (i < a.n_mat) {
