@@ -8,84 +8,18 @@
 // All four kernels are HBM-bound (5.0625 B/element for q8_0, 6 B/element for f16).  The q8_0 block is 34 bytes
 // and only 2-byte aligned, so packed bytes are staged through LDS and cross HBM as aligned 16-byte vectors.
 //
-// Must be compiled with -ffp-contract=off: x*id feeds roundf, and fusing that multiply into roundf's
-// internal subtraction would change results.
+// Must be compiled with -ffp-contract=off: x*id feeds the rounding, and fusing that multiply into the rounding's
+// addition would change results.
 
 #include "mesh_common.hpp"
 
 namespace mesh {
 
 constexpr int CODEC_THREADS = 256;
-constexpr int Q8_WG_BLOCKS = 256;                      // q8_0 blocks per workgroup: 32 KiB of f32, 8704 B packed
+constexpr int Q8_WG_BLOCKS = 256;                      // unpack: q8_0 blocks per workgroup, 8704 B packed in, 32 KiB of f32 out
 constexpr int Q8_ITERS = Q8_WG_BLOCKS / 32;            // 8 lanes per block, 32 blocks per pass
-static_assert((Q8_WG_BLOCKS * Q8_0_BYTES) % 16 == 0, "workgroup output must start 16-byte aligned");
-
-__device__ __forceinline__ uint32_t pack4_i8(float a, float b, float c, float d) {
-    const int qa = (int)roundf(a), qb = (int)roundf(b), qc = (int)roundf(c), qd = (int)roundf(d);
-    return (uint32_t)(qa & 0xFF) | ((uint32_t)(qb & 0xFF) << 8) | ((uint32_t)(qc & 0xFF) << 16) |
-           ((uint32_t)(qd & 0xFF) << 24);
-}
-
-template <bool ALIGNED>
-__global__ __launch_bounds__(CODEC_THREADS) void pack_q8_0_kernel(const float *__restrict__ x,
-                                                                  uint8_t *__restrict__ y, int64_t nblk) {
-    __shared__ __align__(16) uint8_t stage[Q8_WG_BLOCKS * Q8_0_BYTES];
-    const int tid = threadIdx.x;
-    const int part = tid & 7;    // which 4 of the block's 32 values
-    const int sub = tid >> 3;    // block within a pass
-    const int64_t blk0 = (int64_t)blockIdx.x * Q8_WG_BLOCKS;
-    const int64_t left = nblk - blk0;
-    const int nb_here = left < Q8_WG_BLOCKS ? (int)left : Q8_WG_BLOCKS;
-
-    float4 v[Q8_ITERS];
-#pragma unroll
-    for (int it = 0; it < Q8_ITERS; ++it) {
-        const int b = it * 32 + sub;
-        v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (b < nb_here) {
-            const float *p = x + (blk0 + b) * QK8_0 + part * 4;
-            if (ALIGNED) {
-                v[it] = *reinterpret_cast<const float4 *>(p);
-            } else {
-                v[it] = make_float4(p[0], p[1], p[2], p[3]);
-            }
-        }
-    }
-#pragma unroll
-    for (int it = 0; it < Q8_ITERS; ++it) {
-        const int b = it * 32 + sub;
-        float amax = fmaxf(fmaxf(fabsf(v[it].x), fabsf(v[it].y)), fmaxf(fabsf(v[it].z), fabsf(v[it].w)));
-        amax = fmaxf(amax, __shfl_xor(amax, 1));
-        amax = fmaxf(amax, __shfl_xor(amax, 2));
-        amax = fmaxf(amax, __shfl_xor(amax, 4));
-        const float d = amax / 127.0f;                 // IEEE divide
-        const float id = d != 0.0f ? 1.0f / d : 0.0f;  // from the unrounded f32 d
-        const uint32_t q = pack4_i8(v[it].x * id, v[it].y * id, v[it].z * id, v[it].w * id);
-        uint8_t *o = stage + b * Q8_0_BYTES;
-        if (part == 0) *reinterpret_cast<uint16_t *>(o) = f32_to_f16_bits(d);
-        uint16_t *oq = reinterpret_cast<uint16_t *>(o + 2 + part * 4);
-        oq[0] = (uint16_t)(q & 0xFFFFu);
-        oq[1] = (uint16_t)(q >> 16);
-    }
-    __syncthreads();
-
-    const int nbytes = nb_here * Q8_0_BYTES;
-    uint8_t *out = y + blk0 * Q8_0_BYTES;
-    if (ALIGNED) {
-        const int n16 = nbytes >> 4;
-        const uint4 *s4 = reinterpret_cast<const uint4 *>(stage);
-        uint4 *o4 = reinterpret_cast<uint4 *>(out);
-        for (int i = tid; i < n16; i += CODEC_THREADS) o4[i] = s4[i];
-        const int done = n16 << 4;
-        const uint16_t *s2 = reinterpret_cast<const uint16_t *>(stage + done);
-        uint16_t *o2 = reinterpret_cast<uint16_t *>(out + done);
-        for (int i = tid; i < ((nbytes - done) >> 1); i += CODEC_THREADS) o2[i] = s2[i];
-    } else {
-        const uint16_t *s2 = reinterpret_cast<const uint16_t *>(stage);
-        uint16_t *o2 = reinterpret_cast<uint16_t *>(out);
-        for (int i = tid; i < (nbytes >> 1); i += CODEC_THREADS) o2[i] = s2[i];
-    }
-}
+static_assert((Q8_WG_BLOCKS * Q8_0_BYTES) % 16 == 0, "workgroup input must start 16-byte aligned");
+constexpr int Q8_PACK_WG_BLOCKS = 16 * (CODEC_THREADS / 64);   // pack: 4 lanes per block, 16 blocks (544 B packed) per wave
 
 template <bool ALIGNED>
 __global__ __launch_bounds__(CODEC_THREADS) void unpack_q8_0_kernel(const uint8_t *__restrict__ x,
@@ -139,7 +73,123 @@ __global__ __launch_bounds__(CODEC_THREADS) void unpack_q8_0_kernel(const uint8_
     }
 }
 
-// 8 elements per thread: two 16-byte loads, one 16-byte store
+// Orders a wave's own LDS writes before its own LDS reads of other lanes' data (no workgroup barrier involved).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// roundf (half away from zero) followed by the float -> int conversion, for |x| < 2^23: adding the largest float
+// below one half, with the sign of x, and truncating gives the same integer as roundf for every float (the sum of
+// k + 0.5 and the constant is a tie that rounds up to k + 1; every smaller fraction stays below k + 1).
+__device__ __forceinline__ int round_half_away_i32(float x) { return (int)(x + copysignf(0.49999997f, x)); }
+
+__device__ __forceinline__ uint32_t pack4_i8_fast(float a, float b, float c, float d) {
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)round_half_away_i32(b), (uint32_t)round_half_away_i32(a), 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)round_half_away_i32(d), (uint32_t)round_half_away_i32(c), 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float quad_swizzle(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+
+// f32 -> q8_0.  Four lanes per block (8 values each), 16 blocks per wave; the wave stages its 544 packed bytes (a
+// multiple of 16) in its own LDS region and copies them out itself, so no workgroup barrier separates loads and
+// stores.  The kernel is as much VALU- as HBM-bound (two IEEE divides, 32 roundings and the byte packing per block),
+// hence the quad-wide maximum through DPP, the add-and-truncate rounding and v_perm packing.
+template <bool ALIGNED>
+__global__ __launch_bounds__(CODEC_THREADS) void pack_q8_0_kernel(const float *__restrict__ x,
+                                                                       uint8_t *__restrict__ y, int64_t nblk) {
+    constexpr int ITERS = 1, WB = 16 * ITERS, WAVES = CODEC_THREADS / 64;
+    __shared__ __align__(16) uint8_t stage_all[WAVES][WB * Q8_0_BYTES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int part = lane & 3, sub = lane >> 2;
+    uint8_t *stage = stage_all[wave];
+    const int64_t blk0 = ((int64_t)blockIdx.x * WAVES + wave) * WB;
+    const int64_t left = nblk - blk0;
+    if (left <= 0) return;
+    const int nb_here = left < WB ? (int)left : WB;
+
+    float4 va[ITERS], vb[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int b = it * 16 + sub;
+        va[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        vb[it] = va[it];
+        if (b < nb_here) {
+            const float *p = x + (blk0 + b) * QK8_0 + part * 8;
+            if (ALIGNED) {
+                va[it] = *reinterpret_cast<const float4 *>(p);
+                vb[it] = *reinterpret_cast<const float4 *>(p + 4);
+            } else {
+                va[it] = make_float4(p[0], p[1], p[2], p[3]);
+                vb[it] = make_float4(p[4], p[5], p[6], p[7]);
+            }
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int b = it * 16 + sub;
+        const float4 a = va[it], c = vb[it];
+        float amax = fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
+                           fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+        amax = fmaxf(amax, quad_swizzle<0xB1>(amax));      // lanes 1,0,3,2 of the quad
+        amax = fmaxf(amax, quad_swizzle<0x4E>(amax));      // lanes 2,3,0,1
+        const float d = amax / 127.0f;                 // IEEE divide
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;  // from the unrounded f32 d
+        const uint32_t q0 = pack4_i8_fast(a.x * id, a.y * id, a.z * id, a.w * id);
+        const uint32_t q1 = pack4_i8_fast(c.x * id, c.y * id, c.z * id, c.w * id);
+        uint8_t *o = stage + b * Q8_0_BYTES;
+        if (part == 0) *reinterpret_cast<uint16_t *>(o) = f32_to_f16_bits(d);
+        uint16_t *oq = reinterpret_cast<uint16_t *>(o + 2 + part * 8);
+        oq[0] = (uint16_t)(q0 & 0xFFFFu);
+        oq[1] = (uint16_t)(q0 >> 16);
+        oq[2] = (uint16_t)(q1 & 0xFFFFu);
+        oq[3] = (uint16_t)(q1 >> 16);
+    }
+    wave_lds_sync();
+
+    const int nbytes = nb_here * Q8_0_BYTES;
+    uint8_t *out = y + blk0 * Q8_0_BYTES;
+    if (ALIGNED) {
+        const int n16 = nbytes >> 4;
+        const uint4 *s4 = reinterpret_cast<const uint4 *>(stage);
+        uint4 *o4 = reinterpret_cast<uint4 *>(out);
+        for (int i = lane; i < n16; i += 64) o4[i] = s4[i];
+        const int done = n16 << 4;
+        const uint16_t *s2 = reinterpret_cast<const uint16_t *>(stage + done);
+        uint16_t *o2 = reinterpret_cast<uint16_t *>(out + done);
+        for (int i = lane; i < ((nbytes - done) >> 1); i += 64) o2[i] = s2[i];
+    } else {
+        const uint16_t *s2 = reinterpret_cast<const uint16_t *>(stage);
+        uint16_t *o2 = reinterpret_cast<uint16_t *>(out);
+        for (int i = lane; i < (nbytes >> 1); i += 64) o2[i] = s2[i];
+    }
+}
+
+// f16 -> f32, 4 elements per thread: one 8-byte load and one 16-byte store, so that every store instruction of a wave
+// covers whole cache lines (8 elements per thread would write each line in two halves)
+template <bool ALIGNED>
+__global__ __launch_bounds__(CODEC_THREADS) void unpack_f16_kernel(const uint16_t *__restrict__ x,
+                                                                   float *__restrict__ y, int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * CODEC_THREADS + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (ALIGNED && i + 4 <= n) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(x + i);
+        float4 a;
+        a.x = f16_bits_to_f32((uint16_t)(v.x & 0xFFFF)); a.y = f16_bits_to_f32((uint16_t)(v.x >> 16));
+        a.z = f16_bits_to_f32((uint16_t)(v.y & 0xFFFF)); a.w = f16_bits_to_f32((uint16_t)(v.y >> 16));
+        *reinterpret_cast<float4 *>(y + i) = a;
+    } else {
+        const int64_t e = i + 4 < n ? i + 4 : n;
+        for (int64_t j = i; j < e; ++j) y[j] = f16_bits_to_f32(x[j]);
+    }
+}
+
+// f32 -> f16, 8 elements per thread: two 16-byte loads, one 16-byte store
 template <bool ALIGNED>
 __global__ __launch_bounds__(CODEC_THREADS) void pack_f16_kernel(const float *__restrict__ x,
                                                                  uint16_t *__restrict__ y, int64_t n) {
@@ -157,26 +207,6 @@ __global__ __launch_bounds__(CODEC_THREADS) void pack_f16_kernel(const float *__
     } else {
         const int64_t e = i + 8 < n ? i + 8 : n;
         for (int64_t j = i; j < e; ++j) y[j] = f32_to_f16_bits(x[j]);
-    }
-}
-
-template <bool ALIGNED>
-__global__ __launch_bounds__(CODEC_THREADS) void unpack_f16_kernel(const uint16_t *__restrict__ x,
-                                                                   float *__restrict__ y, int64_t n) {
-    const int64_t i = ((int64_t)blockIdx.x * CODEC_THREADS + threadIdx.x) * 8;
-    if (i >= n) return;
-    if (ALIGNED && i + 8 <= n) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(x + i);
-        float4 a, b;
-        a.x = f16_bits_to_f32((uint16_t)(v.x & 0xFFFF)); a.y = f16_bits_to_f32((uint16_t)(v.x >> 16));
-        a.z = f16_bits_to_f32((uint16_t)(v.y & 0xFFFF)); a.w = f16_bits_to_f32((uint16_t)(v.y >> 16));
-        b.x = f16_bits_to_f32((uint16_t)(v.z & 0xFFFF)); b.y = f16_bits_to_f32((uint16_t)(v.z >> 16));
-        b.z = f16_bits_to_f32((uint16_t)(v.w & 0xFFFF)); b.w = f16_bits_to_f32((uint16_t)(v.w >> 16));
-        *reinterpret_cast<float4 *>(y + i) = a;
-        *reinterpret_cast<float4 *>(y + i + 4) = b;
-    } else {
-        const int64_t e = i + 8 < n ? i + 8 : n;
-        for (int64_t j = i; j < e; ++j) y[j] = f16_bits_to_f32(x[j]);
     }
 }
 
@@ -202,7 +232,7 @@ int act_pack_dev(int fmt, const float *src, void *dst, int64_t n, hipStream_t st
         case MESH_Q8_0: {
             if (n % QK8_0) return fail(MESH_ERR_INVALID, "mesh_act_pack: q8_0 needs a multiple of 32 elements, got %lld", (long long)n);
             const int64_t nblk = n / QK8_0;
-            const int64_t grid = (nblk + Q8_WG_BLOCKS - 1) / Q8_WG_BLOCKS;
+            const int64_t grid = (nblk + Q8_PACK_WG_BLOCKS - 1) / Q8_PACK_WG_BLOCKS;
             if (al) pack_q8_0_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint8_t *)dst, nblk);
             else pack_q8_0_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint8_t *)dst, nblk);
             MESH_LAUNCH_CHECK();
@@ -222,7 +252,7 @@ int act_unpack_dev(int fmt, const void *src, float *dst, int64_t n, hipStream_t 
             MESH_HIP_TRY(hipMemcpyAsync(dst, src, (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
             return MESH_OK;
         case MESH_F16: {
-            const int64_t grid = (n + CODEC_THREADS * 8 - 1) / (CODEC_THREADS * 8);
+            const int64_t grid = (n + CODEC_THREADS * 4 - 1) / (CODEC_THREADS * 4);
             if (al) unpack_f16_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint16_t *)src, dst, n);
             else unpack_f16_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint16_t *)src, dst, n);
             MESH_LAUNCH_CHECK();

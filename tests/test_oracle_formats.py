@@ -131,3 +131,18 @@ def test_row_bytes():
     assert oracle.row_bytes(oracle.Q5_0, 896) == 28 * 22
     assert oracle.row_bytes(oracle.Q4_K, 896) == -1
     assert oracle.row_bytes(oracle.F16, 7) == 14 and oracle.row_bytes(oracle.F32, 7) == 28
+
+
+def test_add_and_truncate_equals_round_half_away():
+    """The q8_0 pack kernel rounds x*id with trunc(x + copysign(nextbelow(0.5), x)) instead of roundf; the two agree
+    for every float of magnitude below 2^23.  Checked here on every tie k + 0.5, its two float neighbours, and a dense
+    stride through all floats in [0, 256) (the quantiser's products stay within +-127.5)."""
+    c = np.nextafter(np.float32(0.5), np.float32(0))
+    assert c == np.float32(0.49999997)
+    ties = np.arange(0, 4096, dtype=np.float32) + np.float32(0.5)
+    cand = np.concatenate([ties, np.nextafter(ties, np.float32(0)), np.nextafter(ties, np.float32(1e9)),
+                           np.arange(0, 0x43800000, 37, dtype=np.uint32).view(np.float32)])
+    for x in (cand, -cand):
+        fast = np.trunc(x + np.copysign(c, x))                                   # float32 add, round to nearest even
+        exact = np.copysign(np.floor(np.abs(x).astype(np.float64) + 0.5), x)     # roundf
+        assert np.array_equal(fast.astype(np.float64), exact)
