@@ -127,6 +127,8 @@ def bench_codec(args):
 # ------------------------------------------------------------------------------------------------ stage
 N_CTX = 4096
 STAGE_LAYERS = 16
+# bytes of one head_dim-128 cache row: f16, q8_0 (32 x 34-byte blocks' worth: 128 quants + 4 scales), q4_0 (64 + 8)
+HD_BYTES_F16, HD_BYTES_Q8_0, HD_BYTES_Q4_0 = 256, 136, 72
 PREFILL_T = 2048
 
 
@@ -173,7 +175,10 @@ def bench_stage(args):
     batches = sorted(set(int(b) for b in args.batches.split(",")))
     bmax = max(batches)
     t0 = time.perf_counter()
-    st = m.Stage(path, 0, STAGE_LAYERS, n_ctx=N_CTX, n_seq_max=bmax, n_batch_max=max(bmax, 16, PREFILL_T if args.prefill else 0))
+    kv_types = {"f16": (m.F16, m.F16), "q8_0/q4_0": (m.Q8_0, m.Q4_0), "q4_0/q4_0": (m.Q4_0, m.Q4_0)}[args.kv]
+    kv_row = {m.F16: HD_BYTES_F16, m.Q8_0: HD_BYTES_Q8_0, m.Q4_0: HD_BYTES_Q4_0}
+    st = m.Stage(path, 0, STAGE_LAYERS, n_ctx=N_CTX, n_seq_max=bmax, n_batch_max=max(bmax, 16, PREFILL_T if args.prefill else 0),
+                 kv_types=kv_types)
     t_load = time.perf_counter() - t0
     os.unlink(path)
     weight_bytes = st.weight_bytes
@@ -185,7 +190,7 @@ def bench_stage(args):
     for il in range(STAGE_LAYERS):
         for s in range(bmax):
             ses.kv_write(il, s, 0, kv, kv)
-    kv_bytes_per_seq = STAGE_LAYERS * 2 * N_CTX * HK * HD * 2
+    kv_bytes_per_seq = STAGE_LAYERS * N_CTX * HK * (kv_row[kv_types[0]] + kv_row[kv_types[1]])
     stream = torch.cuda.ExternalStream(ses.stream)
     results = {}
     for B in batches:
@@ -246,9 +251,9 @@ def bench_stage(args):
     out = {
         "metric": "stage decode tok/s @8B Q4_K_M", "value": b1["tok_s"], "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": b1["ms_per_step"], "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32 activations x q4_K/q6_K weights, f16 KV", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 activations x q4_K/q6_K weights, %s KV" % args.kv, "data": "synthetic",
         "config": {"workload": "Llama-3-8B-shaped stage, layers 0-15 of 32, Q4_K_M block-domain random weights, decode batch %d, "
-                               "4096-token f16 KV context, f32 hidden state in HBM -> q8_0 boundary activation out" % batches[0],
+                               "4096-token %s KV context, f32 hidden state in HBM -> q8_0 boundary activation out" % (batches[0], args.kv),
                    "weight_bytes": weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
         "roofline": {"bound": "hbm", "kernel": "gemv_dot_kernel<type,1,NU> (q4_K/q6_K dequant-fused mat-vec, all instantiations)",
                      "achieved": round(gemv_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gemv_gbs / HBM_PEAK_GBS, 4),
@@ -276,6 +281,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="stage", choices=["stage", "codec"])
     ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
+    ap.add_argument("--kv", default="f16", choices=["f16", "q8_0/q4_0", "q4_0/q4_0"],
+                    help="KV cache row types K/V (default f16: the tier the reference picks for an 8B Q4_K_M model)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", dest="prefill", action="store_false", help="skip the 2048-token prefill measurement")
     args = ap.parse_args()

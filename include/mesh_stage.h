@@ -41,6 +41,7 @@ typedef enum mesh_status {
 typedef enum mesh_dtype {
     MESH_F32 = 0,
     MESH_F16 = 1,
+    MESH_Q4_0 = 2,
     MESH_Q5_0 = 6,
     MESH_Q8_0 = 8,
     MESH_Q4_K = 12,
@@ -137,7 +138,9 @@ typedef struct mesh_stage_opts {
     int32_t n_ctx;          /* KV positions per sequence; 0 = 4096                          (-c, launch.rs:474-504) */
     int32_t n_seq_max;      /* sequences the KV cache holds; 0 = 1                          (--parallel, launch.rs:1338-1390) */
     int32_t n_batch_max;    /* most tokens one decode call may carry; 0 = 512 */
-    int32_t kv_type;        /* 0 or MESH_F16 (f16 K and V, the tier of launch.rs:585-589) */
+    int32_t kv_type;        /* K cache rows: 0 or MESH_F16, MESH_Q8_0, MESH_Q4_0            (--cache-type-k, launch.rs:639-644) */
+    int32_t kv_type_v;      /* V cache rows: 0 = MESH_F16 when kv_type is f16, else MESH_Q4_0 (--cache-type-v).  The pairs of
+                               KvCacheQuant::for_model_size (launch.rs:568-591) are supported: f16/f16, q8_0/q4_0, q4_0/q4_0 */
 } mesh_stage_opts;
 
 typedef struct mesh_batch {

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmeshstage.so")
 
 # ggml type ids (include/mesh_stage.h: mesh_dtype)
-F32, F16, Q5_0, Q8_0, Q4_K, Q6_K = 0, 1, 6, 8, 12, 14
+F32, F16, Q4_0, Q5_0, Q8_0, Q4_K, Q6_K = 0, 1, 2, 6, 8, 12, 14
 
 OK, ERR_INVALID, ERR_DEVICE, ERR_NOMEM, ERR_IO, ERR_FORMAT, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
 
@@ -61,7 +61,7 @@ class TensorInfo(ctypes.Structure):
 class StageOpts(ctypes.Structure):
     """mesh_stage_opts"""
     _fields_ = [("device", ctypes.c_char_p), ("n_ctx", ctypes.c_int32), ("n_seq_max", ctypes.c_int32),
-                ("n_batch_max", ctypes.c_int32), ("kv_type", ctypes.c_int32)]
+                ("n_batch_max", ctypes.c_int32), ("kv_type", ctypes.c_int32), ("kv_type_v", ctypes.c_int32)]
 
 
 class Batch(ctypes.Structure):
@@ -239,8 +239,10 @@ def gguf_tensor(path, name):
 class Stage:
     """Layers [layer_begin, layer_end) of a GGUF model resident on the GPU (mesh_stage)."""
 
-    def __init__(self, gguf_path, layer_begin, layer_end=-1, n_ctx=0, n_seq_max=0, n_batch_max=0, device=None):
-        opts = StageOpts(device.encode() if device else None, n_ctx, n_seq_max, n_batch_max, 0)
+    def __init__(self, gguf_path, layer_begin, layer_end=-1, n_ctx=0, n_seq_max=0, n_batch_max=0, device=None, kv_types=None):
+        """kv_types: (K, V) cache row types, one of (F16, F16), (Q8_0, Q4_0), (Q4_0, Q4_0); None = f16 / f16."""
+        kt, vt = kv_types if kv_types else (0, 0)
+        opts = StageOpts(device.encode() if device else None, n_ctx, n_seq_max, n_batch_max, kt, vt)
         self._h = ctypes.c_void_p()
         check(lib().mesh_stage_open(os.fsencode(gguf_path), layer_begin, layer_end, ctypes.byref(opts), ctypes.byref(self._h)))
         self.info = ModelInfo()

@@ -1,9 +1,9 @@
-// RoPE + KV append, and GQA attention over the stage-local f16 KV cache (split-KV, online softmax).
+// RoPE + KV append, and GQA attention over the stage-local KV cache (split-KV, online softmax).
 // Stands where the worker's graph runs rope -> kv store -> flash_attn_ext (-fa on, mesh-llm/src/inference/launch.rs:1350-1353;
-// f16 cache is the small-model tier of KvCacheQuant::for_model_size, launch.rs:568-591).
+// cache types per KvCacheQuant::for_model_size, launch.rs:568-591: f16/f16, q8_0/q4_0, q4_0/q4_0).
 //
-// Cache layout per layer: K and V as f16 [n_seq][n_head_kv][n_ctx][head_dim]; one (sequence, kv head) is a
-// contiguous run so a workgroup streams its key range linearly.  The `group` query heads that share a kv head
+// Cache layout per layer: K and V as [n_seq][n_head_kv][n_ctx] rows of head_dim values (kv_cache.hpp); one
+// (sequence, kv head) is a contiguous run so a workgroup streams its key range linearly.  The `group` query heads that share a kv head
 // are processed together, so each K/V byte is read once per token.
 
 #include "attn.hpp"
@@ -12,7 +12,9 @@ namespace mesh {
 
 // ------------------------------------------------------------------------------------------------ rope + append
 // grid (n_head + 2*n_head_kv, T), one wave per head vector.
+constexpr int ROPE_HD_MAX = 256;
 __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvArgs a) {
+    __shared__ float s_vec[ROPE_HD_MAX];         // the finished K / V row before it is stored in the cache type
     const int hh = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int hd = a.head_dim;
     const int pos = a.pos[t], seq = a.seq[t];
@@ -23,11 +25,14 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvArgs a) {
     else if (hh < a.n_head + a.n_kv) { kind = 1; head = hh - a.n_head; vec = const_cast<float *>(a.k) + ((size_t)t * a.n_kv + head) * hd; nw = a.k_norm; }
     else { kind = 2; head = hh - a.n_head - a.n_kv; vec = const_cast<float *>(a.v) + ((size_t)t * a.n_kv + head) * hd; }
 
-    uint16_t *cache = nullptr;
-    if (kind) cache = (kind == 1 ? a.kcache : a.vcache) + (((size_t)seq * a.n_kv + head) * a.n_ctx + pos) * hd;
+    const int ctype = kind == 1 ? a.k_type : a.v_type;
+    uint8_t *row = nullptr;
+    if (kind) row = (kind == 1 ? a.kcache : a.vcache) + (((size_t)seq * a.n_kv + head) * a.n_ctx + pos) * (size_t)kv_row_bytes(ctype, hd);
 
     if (kind == 2) {
-        for (int i = lane; i < hd; i += 64) cache[i] = f32_to_f16_bits(vec[i]);
+        for (int i = lane; i < hd; i += 64) s_vec[i] = vec[i];
+        __syncthreads();
+        kv_store_row(ctype, row, s_vec, hd, lane);
         return;
     }
     // optional per-head RMS norm (qwen3: attn_q_norm / attn_k_norm over head_dim)
@@ -50,20 +55,27 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvArgs a) {
         const float o0 = x0 * cs - x1 * sn;
         const float o1 = x0 * sn + x1 * cs;
         if (kind == 0) { vec[ia] = o0; vec[ib] = o1; }
-        else { cache[ia] = f32_to_f16_bits(o0); cache[ib] = f32_to_f16_bits(o1); }
+        else { s_vec[ia] = o0; s_vec[ib] = o1; }
     }
     // dimensions beyond n_rot are not rotated
     for (int e = a.n_rot + lane; e < hd; e += 64) {
         float x0 = vec[e];
         if (nw) x0 = x0 * nscale * nw[e];
         if (kind == 0) vec[e] = x0;
-        else cache[e] = f32_to_f16_bits(x0);
+        else s_vec[e] = x0;
+    }
+    if (kind == 1) {
+        __syncthreads();
+        kv_store_row(ctype, row, s_vec, hd, lane);
     }
 }
 
 int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
-    if (a.head_dim % 2 || a.n_rot % 2 || a.n_rot > a.head_dim) return fail(MESH_ERR_INVALID, "rope: bad head_dim/n_rot %d/%d", a.head_dim, a.n_rot);
+    if (a.head_dim % 2 || a.n_rot % 2 || a.n_rot > a.head_dim || a.head_dim > ROPE_HD_MAX)
+        return fail(MESH_ERR_INVALID, "rope: bad head_dim/n_rot %d/%d", a.head_dim, a.n_rot);
+    if (!kv_type_supported(a.k_type) || !kv_type_supported(a.v_type) || ((a.k_type != MESH_F16 || a.v_type != MESH_F16) && a.head_dim % 32))
+        return fail(MESH_ERR_UNSUPPORTED, "rope: KV cache types %d/%d with head_dim %d", a.k_type, a.v_type, a.head_dim);
     rope_kv_kernel<<<dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream>>>(a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
@@ -74,19 +86,14 @@ constexpr int ATTN_THREADS = 256;
 constexpr int ATTN_WAVES = ATTN_THREADS / 64;
 constexpr int KPT = 4;                      // keys per thread per pass: 8 x 16-byte loads in flight per lane
 
-__device__ __forceinline__ void unpack8h(const uint4 &v, float (&o)[8]) {
-    o[0] = f16_bits_to_f32((uint16_t)(v.x & 0xFFFF)); o[1] = f16_bits_to_f32((uint16_t)(v.x >> 16));
-    o[2] = f16_bits_to_f32((uint16_t)(v.y & 0xFFFF)); o[3] = f16_bits_to_f32((uint16_t)(v.y >> 16));
-    o[4] = f16_bits_to_f32((uint16_t)(v.z & 0xFFFF)); o[5] = f16_bits_to_f32((uint16_t)(v.z >> 16));
-    o[6] = f16_bits_to_f32((uint16_t)(v.w & 0xFFFF)); o[7] = f16_bits_to_f32((uint16_t)(v.w >> 16));
-}
-
 // grid (n_splits, n_kv * (group/G), T).  HD/8 lanes share one key ("slot"); a thread visits keys
 // j0 + slot + SLOTS*i and keeps one online-softmax state (m, l, acc[8]) per query head.  Per pass all KPT keys'
 // K and V vectors are requested first, then scored, then folded in with a single rescale.  The slots of a
 // workgroup are merged through LDS.  With one split the normalised output is written directly; otherwise each
 // workgroup writes an un-normalised partial plus (max, sum) and attn_combine_kernel merges the splits.
-template <int HD, int G>
+// Quantised rows decode to scale * (u - off) with small integers u (kv_cache.hpp): the offset leaves the inner
+// loops, as off * sum(q) per score and as one running sum of p * scale per head on the value side.
+template <int HD, int G, int KT, int VT>
 __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
     constexpr int LPK = HD / 8;                 // lanes per key
     constexpr int SLOTS = ATTN_THREADS / LPK;   // keys visited side by side
@@ -104,7 +111,8 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
     const int j0 = split * per;
     const int j1 = j0 + per < n_keys ? j0 + per : n_keys;
 
-    float q[G][8], acc[G][8], m[G], l[G];
+    constexpr int KRB = kv_row_bytes(KT, HD), VRB = kv_row_bytes(VT, HD);
+    float q[G][8], acc[G][8], m[G], l[G], qoff[G], voff[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
         const float4 qa = *reinterpret_cast<const float4 *>(a.q + ((size_t)t * a.n_head + h0 + h) * HD + ds);
@@ -116,39 +124,48 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
         for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
         m[h] = -INFINITY;
         l[h] = 0.f;
+        voff[h] = 0.f;
+        qoff[h] = 0.f;
+        if (KT != MESH_F16) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qoff[h] += q[h][i];
+            qoff[h] *= -KvAffine<KT>::off;
+        }
     }
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
     for (int jb = j0; jb < j1; jb += SLOTS * KPT) {
-        uint4 kr[KPT], vr[KPT];
+        KvRaw<KT> kr[KPT];
+        KvRaw<VT> vr[KPT];
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
             const int j = jb + slot + SLOTS * i;
-            kr[i] = make_uint4(0, 0, 0, 0);
-            vr[i] = kr[i];
+            kv_zero<KT>(kr[i]);
+            kv_zero<VT>(vr[i]);
             if (j < j1) {
-                kr[i] = *reinterpret_cast<const uint4 *>(a.kcache + (base + j) * HD + ds);
-                vr[i] = *reinterpret_cast<const uint4 *>(a.vcache + (base + j) * HD + ds);
+                kr[i] = kv_load<KT, HD>(a.kcache + (base + j) * KRB, ds);
+                vr[i] = kv_load<VT, HD>(a.vcache + (base + j) * VRB, ds);
             }
         }
         float sc[KPT][G];
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
             float kf[8];
-            unpack8h(kr[i], kf);
+            const float kd = kv_decode<KT>(kr[i], kf);
             const bool ok = jb + slot + SLOTS * i < j1;
 #pragma unroll
             for (int h = 0; h < G; ++h) {
-                float s = 0.f;
+                float s = qoff[h];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s = fmaf(q[h][e], kf[e], s);
+                if (KT != MESH_F16) s *= kd;
 #pragma unroll
                 for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
                 sc[i][h] = ok ? s : -INFINITY;
             }
         }
-        float vf[KPT][8];
+        float vf[KPT][8], vd[KPT];
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) unpack8h(vr[i], vf[i]);
+        for (int i = 0; i < KPT; ++i) vd[i] = kv_decode<VT>(vr[i], vf[i]);
 #pragma unroll
         for (int h = 0; h < G; ++h) {
             float mn = m[h];
@@ -160,6 +177,12 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < KPT; ++i) { p[i] = exp2f(sc[i][h] - mn); ps += p[i]; }
             l[h] = l[h] * corr + ps;
+            if (VT != MESH_F16) {       // from here on p carries the row scale; the offset term is summed apart
+                float po = 0.f;
+#pragma unroll
+                for (int i = 0; i < KPT; ++i) { p[i] *= vd[i]; po += p[i]; }
+                voff[h] = voff[h] * corr + po * KvAffine<VT>::off;
+            }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 float v = acc[h][e] * corr;
@@ -169,6 +192,12 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
             }
             m[h] = mn;
         }
+    }
+    if (VT != MESH_F16) {
+#pragma unroll
+        for (int h = 0; h < G; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] -= voff[h];
     }
     // merge the slots of this workgroup: every slot state is rescaled to the workgroup's maximum, slots sharing a
     // wave are added with shuffles, the 4 waves meet in LDS
@@ -240,12 +269,12 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(AttnArgs a) {
     a.out[row * a.head_dim + dd] = num / den;
 }
 
-template <int HD>
+template <int HD, int KT, int VT>
 static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     const dim3 block(ATTN_THREADS);
 #define MESH_ATTN_CASE(GG)                                                                          \
     if (a.group == GG) {                                                                            \
-        attn_kernel<HD, GG><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
+        attn_kernel<HD, GG, KT, VT><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
         MESH_LAUNCH_CHECK();                                                                        \
         return MESH_OK;                                                                             \
     }
@@ -256,9 +285,21 @@ static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     if (HD == 64) { MESH_ATTN_CASE(7) }
 #undef MESH_ATTN_CASE
     // any other group size: one query head per workgroup (K/V re-read per head)
-    attn_kernel<HD, 1><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
+    attn_kernel<HD, 1, KT, VT><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
+}
+
+template <int HD>
+static int launch_attn_typed(const AttnArgs &a, int T, hipStream_t stream) {
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) return launch_attn<HD, MESH_F16, MESH_F16>(a, T, stream);
+    if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) return launch_attn<HD, MESH_Q8_0, MESH_Q4_0>(a, T, stream);
+    if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) return launch_attn<HD, MESH_Q4_0, MESH_Q4_0>(a, T, stream);
+    return fail(MESH_ERR_UNSUPPORTED, "attention: KV cache types %d/%d (f16/f16, q8_0/q4_0 and q4_0/q4_0 have kernels)", a.k_type, a.v_type);
+}
+
+bool kv_pair_supported(int k_type, int v_type) {
+    return (k_type == MESH_F16 && v_type == MESH_F16) || (k_type == MESH_Q8_0 && v_type == MESH_Q4_0) || (k_type == MESH_Q4_0 && v_type == MESH_Q4_0);
 }
 
 int attention(const AttnArgs &a, int T, hipStream_t stream) {
@@ -267,11 +308,41 @@ int attention(const AttnArgs &a, int T, hipStream_t stream) {
         return fail(MESH_ERR_INVALID, "attention: bad head layout or split count");
     if (a.n_splits > 1 && (!a.part || !a.ml)) return fail(MESH_ERR_INVALID, "attention: split buffers missing");
     int rc;
-    if (a.head_dim == 128) rc = launch_attn<128>(a, T, stream);
-    else if (a.head_dim == 64) rc = launch_attn<64>(a, T, stream);
+    if (a.head_dim == 128) rc = launch_attn_typed<128>(a, T, stream);
+    else if (a.head_dim == 64) rc = launch_attn_typed<64>(a, T, stream);
     else return fail(MESH_ERR_UNSUPPORTED, "attention: head_dim %d has no kernel (64 and 128 do)", a.head_dim);
     if (rc != MESH_OK || a.n_splits == 1) return rc;
     attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ f16 <-> cache rows
+// grid (n_kv, n_pos), one wave per row
+__global__ __launch_bounds__(64) void kv_import_kernel(int type, uint8_t *cache, const uint16_t *half, int n_kv, int n_ctx, int hd, int seq, int pos0) {
+    __shared__ float s_vec[ROPE_HD_MAX];
+    const int h = blockIdx.x, p = blockIdx.y, lane = threadIdx.x;
+    const uint16_t *src = half + ((size_t)p * n_kv + h) * hd;
+    for (int i = lane; i < hd; i += 64) s_vec[i] = f16_bits_to_f32(src[i]);
+    __syncthreads();
+    kv_store_row(type, cache + (((size_t)seq * n_kv + h) * n_ctx + pos0 + p) * (size_t)kv_row_bytes(type, hd), s_vec, hd, lane);
+}
+__global__ __launch_bounds__(64) void kv_export_kernel(int type, const uint8_t *cache, uint16_t *half, int n_kv, int n_ctx, int hd, int seq, int pos0) {
+    const int h = blockIdx.x, p = blockIdx.y, lane = threadIdx.x;
+    const uint8_t *row = cache + (((size_t)seq * n_kv + h) * n_ctx + pos0 + p) * (size_t)kv_row_bytes(type, hd);
+    uint16_t *dst = half + ((size_t)p * n_kv + h) * hd;
+    for (int i = lane; i < hd; i += 64) dst[i] = f32_to_f16_bits(kv_fetch(type, row, hd, i));
+}
+
+int kv_import(int type, uint8_t *cache, const uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream) {
+    if (!kv_type_supported(type) || head_dim > ROPE_HD_MAX || (type != MESH_F16 && head_dim % 32)) return fail(MESH_ERR_UNSUPPORTED, "kv_import: type %d, head_dim %d", type, head_dim);
+    kv_import_kernel<<<dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream>>>(type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+int kv_export(int type, const uint8_t *cache, uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream) {
+    if (!kv_type_supported(type)) return fail(MESH_ERR_UNSUPPORTED, "kv_export: type %d", type);
+    kv_export_kernel<<<dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream>>>(type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

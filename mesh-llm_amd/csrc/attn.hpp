@@ -1,6 +1,7 @@
 // RoPE + KV append and GQA attention launchers (attn.hip).
 #pragma once
 
+#include "kv_cache.hpp"
 #include "mesh_common.hpp"
 
 namespace mesh {
@@ -12,8 +13,9 @@ struct RopeKvArgs {
     float *q = nullptr;            // [T][n_head][head_dim], rotated in place
     const float *k = nullptr;      // [T][n_kv][head_dim]
     const float *v = nullptr;
-    uint16_t *kcache = nullptr;    // this layer's K: [n_seq][n_kv][n_ctx][head_dim] f16
-    uint16_t *vcache = nullptr;
+    uint8_t *kcache = nullptr;     // this layer's K: [n_seq][n_kv][n_ctx] rows of k_type (kv_cache.hpp)
+    uint8_t *vcache = nullptr;
+    int k_type = MESH_F16, v_type = MESH_F16;
     const int32_t *pos = nullptr;  // device, [T]
     const int32_t *seq = nullptr;  // device, [T]
     const float *inv_freq = nullptr;   // device, [n_rot/2]
@@ -26,7 +28,8 @@ int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream);
 
 struct AttnArgs {
     const float *q = nullptr;      // [T][n_head][head_dim]
-    const uint16_t *kcache = nullptr, *vcache = nullptr;
+    const uint8_t *kcache = nullptr, *vcache = nullptr;    // rows of k_type / v_type
+    int k_type = MESH_F16, v_type = MESH_F16;              // (f16, f16), (q8_0, q4_0) or (q4_0, q4_0)
     const int32_t *pos = nullptr, *seq = nullptr;
     float *part = nullptr;         // [T][n_head][n_splits][head_dim]
     float *ml = nullptr;           // [T][n_head][n_splits][2]
@@ -39,5 +42,11 @@ int attention(const AttnArgs &a, int T, hipStream_t stream);
 // The same for a chunk of T consecutive positions pos0 .. pos0 + T - 1 of one sequence, on the matrix cores
 // (attn_prefill.hip; head_dim 128).  a.pos / a.seq / a.part / a.ml are not used.
 int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t stream);
+bool kv_pair_supported(int k_type, int v_type);
+
+// f16 <-> cache rows for mesh_session_kv_write / _read: `half` is a device buffer [n_pos][n_kv][head_dim] of f16
+// bits, `cache` one layer's K or V rows; positions pos0 .. pos0 + n_pos - 1 of sequence seq.
+int kv_import(int type, uint8_t *cache, const uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream);
+int kv_export(int type, const uint8_t *cache, uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream);
 
 }  // namespace mesh

@@ -1,4 +1,5 @@
-// Causal GQA attention for a prefill chunk on the matrix cores (head_dim 128, f16 KV cache).
+// Causal GQA attention for a prefill chunk on the matrix cores (head_dim 128; f16 or quantised KV cache rows, which
+// are dequantised to f16 on their way into LDS).
 //
 // The chunk is T consecutive positions pos0 .. pos0 + T - 1 of one sequence whose keys and values are already in
 // the cache (rope_kv appended them); token t attends to cache positions [0, pos0 + t].  A workgroup takes 32
@@ -37,7 +38,24 @@ __device__ __forceinline__ uint32_t pf_pack(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// the 8 values a (key, piece) pair contributes to a tile, as packed f16
+template <int TYPE>
+__device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
+    const KvRaw<TYPE> r = kv_load<TYPE, PF_HD>(row, piece * 8);
+    if constexpr (TYPE == MESH_F16) {
+        return r.v;
+    } else {
+        float u[8];
+        const float d = kv_decode<TYPE>(r, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = (u[e] - KvAffine<TYPE>::off) * d;
+        return make_uint4(pf_pack(u[0], u[1]), pf_pack(u[2], u[3]), pf_pack(u[4], u[5]), pf_pack(u[6], u[7]));
+    }
+}
+
+template <int KT, int VT>
 __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw) {
+    constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
     __shared__ __align__(16) _Float16 sK[PF_TILE * PF_KPITCH];
     __shared__ __align__(16) _Float16 sVt[PF_HD * PF_VPITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
@@ -77,8 +95,8 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
             const int key = p >> 4, piece = p & 15;
             int kr = k0 + key;
             kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
-            const uint4 kv = *reinterpret_cast<const uint4 *>(a.kcache + (base + kr) * PF_HD + piece * 8);
-            const uint4 vv = *reinterpret_cast<const uint4 *>(a.vcache + (base + kr) * PF_HD + piece * 8);
+            const uint4 kv = pf_row_piece<KT>(a.kcache + (base + kr) * KRB, piece);
+            const uint4 vv = pf_row_piece<VT>(a.vcache + (base + kr) * VRB, piece);
             *reinterpret_cast<uint4 *>(sK + key * PF_KPITCH + piece * 8) = kv;
             const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
 #pragma unroll
@@ -153,7 +171,11 @@ int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t str
     int hpw = a.group;                       // heads (waves) per workgroup: the largest divisor of the group up to 8
     while (hpw > 8 || a.group % hpw) --hpw;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
-    attn_chunk_kernel<<<grid, dim3((unsigned)(64 * hpw)), 0, stream>>>(a, T, pos0, seq, hpw);
+    const dim3 block((unsigned)(64 * hpw));
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) attn_chunk_kernel<MESH_F16, MESH_F16><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
+    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) attn_chunk_kernel<MESH_Q8_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
+    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) attn_chunk_kernel<MESH_Q4_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
+    else return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: KV cache types %d/%d", a.k_type, a.v_type);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

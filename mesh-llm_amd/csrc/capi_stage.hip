@@ -5,6 +5,7 @@
 #include <vector>
 
 #include "gemv.hpp"
+#include "attn.hpp"
 #include "stage.hpp"
 
 struct mesh_weight {
@@ -213,23 +214,30 @@ static int kv_xfer(mesh_session *s, int layer, int seq_id, int pos0, int n_pos, 
         return fail(MESH_ERR_INVALID, "mesh_session_kv: sequence %d positions [%d,%d) outside the cache", seq_id, pos0, pos0 + n_pos);
     MESH_HIP_TRY(hipSetDevice(st->device));
     MESH_HIP_TRY(hipStreamSynchronize(s->stream));
-    const size_t hd = hp.head_dim, nkv = hp.n_head_kv;
-    std::vector<uint16_t> tmp((size_t)n_pos * hd);
-    for (int which = 0; which < 2; ++which) {
-        uint16_t *cache = (which ? s->vcache : s->kcache) + (size_t)(layer - st->layer_begin) * s->kv_layer_elems;
+    // through a device buffer of f16 rows [n_pos][n_head_kv][head_dim]: the cache rows may be quantised
+    const int hd = (int)hp.head_dim, nkv = (int)hp.n_head_kv;
+    const size_t bytes = (size_t)n_pos * nkv * hd * 2;
+    uint16_t *tmp = nullptr;
+    MESH_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&tmp), bytes));
+    int rc = MESH_OK;
+    for (int which = 0; which < 2 && rc == MESH_OK; ++which) {
+        const size_t lb = which ? s->v_layer_bytes : s->k_layer_bytes;
+        uint8_t *cache = (which ? s->vcache : s->kcache) + (size_t)(layer - st->layer_begin) * lb;
+        const int type = which ? st->v_type : st->k_type;
         uint16_t *host = which ? v : k;
-        for (size_t h = 0; h < nkv; ++h) {
-            uint16_t *dev = cache + (((size_t)seq_id * nkv + h) * (size_t)st->n_ctx + (size_t)pos0) * hd;
-            if (write) {
-                for (int p = 0; p < n_pos; ++p) memcpy(&tmp[(size_t)p * hd], host + ((size_t)p * nkv + h) * hd, hd * 2);
-                MESH_HIP_TRY(hipMemcpy(dev, tmp.data(), tmp.size() * 2, hipMemcpyHostToDevice));
-            } else {
-                MESH_HIP_TRY(hipMemcpy(tmp.data(), dev, tmp.size() * 2, hipMemcpyDeviceToHost));
-                for (int p = 0; p < n_pos; ++p) memcpy(host + ((size_t)p * nkv + h) * hd, &tmp[(size_t)p * hd], hd * 2);
-            }
+        hipError_t e = hipSuccess;
+        if (write) {
+            e = hipMemcpyAsync(tmp, host, bytes, hipMemcpyHostToDevice, s->stream);
+            if (e == hipSuccess) rc = kv_import(type, cache, tmp, nkv, st->n_ctx, hd, seq_id, pos0, n_pos, s->stream);
+        } else {
+            rc = kv_export(type, cache, tmp, nkv, st->n_ctx, hd, seq_id, pos0, n_pos, s->stream);
+            if (rc == MESH_OK) e = hipMemcpyAsync(host, tmp, bytes, hipMemcpyDeviceToHost, s->stream);
         }
+        if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
+        if (e != hipSuccess && rc == MESH_OK) rc = fail(MESH_ERR_DEVICE, "mesh_session_kv: %s", hipGetErrorString(e));
     }
-    return MESH_OK;
+    (void)hipFree(tmp);
+    return rc;
 }
 
 int mesh_session_kv_write(mesh_session *session, int layer, int seq_id, int pos0, int n_pos, const uint16_t *k, const uint16_t *v) {

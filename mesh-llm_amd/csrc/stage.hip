@@ -149,8 +149,10 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
     st->n_ctx = opts && opts->n_ctx > 0 ? opts->n_ctx : 4096;
     st->n_seq_max = opts && opts->n_seq_max > 0 ? opts->n_seq_max : 1;
     st->n_batch_max = opts && opts->n_batch_max > 0 ? opts->n_batch_max : 512;
-    if (opts && opts->kv_type != 0 && opts->kv_type != MESH_F16)
-        return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: KV cache type %d not supported (f16 is)", opts->kv_type);
+    st->k_type = opts && opts->kv_type ? opts->kv_type : MESH_F16;
+    st->v_type = opts && opts->kv_type_v ? opts->kv_type_v : (st->k_type == MESH_F16 ? MESH_F16 : MESH_Q4_0);
+    if (!kv_pair_supported(st->k_type, st->v_type))
+        return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: KV cache types %d/%d not supported (f16/f16, q8_0/q4_0 and q4_0/q4_0 are)", st->k_type, st->v_type);
     if (opts && opts->device && opts->device[0]) {
         if ((rc = mesh_device_select(opts->device)) != MESH_OK) return rc;
     }
@@ -276,6 +278,7 @@ static bool mega_eligible(const mesh_stage *st) {
     const char *env = getenv("MESH_STAGE_PERSISTENT");       // opt-in while it is slower than the per-projection kernels
     if (!env || env[0] != '1') return false;
     if (hp.head_dim != 128 || hp.n_ff == 0 || hp.n_head_kv == 0 || hp.n_head % hp.n_head_kv) return false;
+    if (st->k_type != MESH_F16 || st->v_type != MESH_F16) return false;
     if (!mega_group_supported((int)(hp.n_head / hp.n_head_kv))) return false;
     const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, FF = hp.n_ff;
     if (E % 256 || QD % 256 || FF % 256) return false;
@@ -342,8 +345,8 @@ static int mega_setup(mesh_session *s) {
         dn.part[0] = MegaPart{w(L.w_down), nullptr, L.w_down.type, E, 0, E, m.x, nullptr, MEGA_REPLICAS, xs};
         dn.total_rows = E / TILE_ROWS;
         dn.x = m.ffn; dn.x_rep_stride = fs; dn.ldx = FF; dn.K = FF; dn.norm_w = nullptr; dn.epi = EPI_RESIDUAL;
-        d.kc = s->kcache + il * s->kv_layer_elems;
-        d.vc = s->vcache + il * s->kv_layer_elems;
+        d.kc = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
+        d.vc = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
     }
     // widest batch whose LDS need fits one workgroup
     const int group = (int)(hp.n_head / hp.n_head_kv);
@@ -440,15 +443,17 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const HParams &hp = st->hp;
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
-    s->kv_layer_elems = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx * hp.head_dim;
+    const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
+    s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
+    s->v_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->v_type, (int)hp.head_dim);
     int rc;
     void *p = nullptr;
-    if ((rc = sess_alloc(s.get(), &p, nl * s->kv_layer_elems * 2)) != MESH_OK) return rc;
-    s->kcache = static_cast<uint16_t *>(p);
-    if ((rc = sess_alloc(s.get(), &p, nl * s->kv_layer_elems * 2)) != MESH_OK) return rc;
-    s->vcache = static_cast<uint16_t *>(p);
-    MESH_HIP_TRY(hipMemsetAsync(s->kcache, 0, nl * s->kv_layer_elems * 2, s->stream));
-    MESH_HIP_TRY(hipMemsetAsync(s->vcache, 0, nl * s->kv_layer_elems * 2, s->stream));
+    if ((rc = sess_alloc(s.get(), &p, nl * s->k_layer_bytes)) != MESH_OK) return rc;
+    s->kcache = static_cast<uint8_t *>(p);
+    if ((rc = sess_alloc(s.get(), &p, nl * s->v_layer_bytes)) != MESH_OK) return rc;
+    s->vcache = static_cast<uint8_t *>(p);
+    MESH_HIP_TRY(hipMemsetAsync(s->kcache, 0, nl * s->k_layer_bytes, s->stream));
+    MESH_HIP_TRY(hipMemsetAsync(s->vcache, 0, nl * s->v_layer_bytes, s->stream));
     const size_t QD = (size_t)hp.n_head * hp.head_dim, KD = (size_t)hp.n_head_kv * hp.head_dim;
     const size_t ff = std::max<size_t>(hp.n_ff, (size_t)hp.n_ff_exp * std::max<uint32_t>(hp.n_expert_used, 1));
     auto fbuf = [&](float **dst, size_t n) -> int {
@@ -592,8 +597,9 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     }
     RopeKvArgs ra;
     ra.q = s->q; ra.k = s->k; ra.v = s->v;
-    ra.kcache = s->kcache + il * s->kv_layer_elems;
-    ra.vcache = s->vcache + il * s->kv_layer_elems;
+    ra.kcache = s->kcache + il * s->k_layer_bytes;
+    ra.vcache = s->vcache + il * s->v_layer_bytes;
+    ra.k_type = st->k_type; ra.v_type = st->v_type;
     ra.pos = s->d_pos; ra.seq = s->d_seq; ra.inv_freq = st->rope_inv_freq;
     ra.q_norm = L.q_norm.present() ? static_cast<const float *>(L.q_norm.data) : nullptr;
     ra.k_norm = L.k_norm.present() ? static_cast<const float *>(L.k_norm.data) : nullptr;
@@ -603,7 +609,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     { ProfScope ps(s, MESH_PROF_ROPE); rc = rope_kv(ra, T, stream); }
     if (rc != MESH_OK) return rc;
     AttnArgs aa;
-    aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.pos = s->d_pos; aa.seq = s->d_seq;
+    aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.k_type = st->k_type; aa.v_type = st->v_type; aa.pos = s->d_pos; aa.seq = s->d_seq;
     aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = s->attn;
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
@@ -697,8 +703,9 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
 
         RopeKvArgs ra;
         ra.q = s->q; ra.k = s->k; ra.v = s->v;
-        ra.kcache = s->kcache + il * s->kv_layer_elems;
-        ra.vcache = s->vcache + il * s->kv_layer_elems;
+        ra.kcache = s->kcache + il * s->k_layer_bytes;
+        ra.vcache = s->vcache + il * s->v_layer_bytes;
+        ra.k_type = st->k_type; ra.v_type = st->v_type;
         ra.pos = s->d_pos; ra.seq = s->d_seq; ra.inv_freq = st->rope_inv_freq;
         ra.q_norm = L.q_norm.present() ? static_cast<const float *>(L.q_norm.data) : nullptr;
         ra.k_norm = L.k_norm.present() ? static_cast<const float *>(L.k_norm.data) : nullptr;
@@ -709,7 +716,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         if (rc != MESH_OK) return rc;
 
         AttnArgs aa;
-        aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.pos = s->d_pos; aa.seq = s->d_seq;
+        aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.k_type = st->k_type; aa.v_type = st->v_type; aa.pos = s->d_pos; aa.seq = s->d_seq;
         aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = s->attn;
         aa.scale = 1.0f / sqrtf((float)hp.head_dim);
         aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);

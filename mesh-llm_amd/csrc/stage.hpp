@@ -57,6 +57,7 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
 struct mesh_stage {
     mesh::HParams hp;
     int device = 0;
+    int k_type = MESH_F16, v_type = MESH_F16;          // KV cache row types
     int layer_begin = 0, layer_end = 0;
     int n_ctx = 0, n_seq_max = 1, n_batch_max = 0;
     std::vector<mesh::LayerWeights> layers;
@@ -71,8 +72,8 @@ struct mesh_session {
     mesh_stage *stage = nullptr;
     hipStream_t stream = nullptr;
     // KV cache: per local layer, K and V as f16 [n_seq_max][n_head_kv][n_ctx][head_dim]
-    uint16_t *kcache = nullptr, *vcache = nullptr;
-    size_t kv_layer_elems = 0;
+    uint8_t *kcache = nullptr, *vcache = nullptr;       // rows of the stage's k_type / v_type (kv_cache.hpp)
+    size_t k_layer_bytes = 0, v_layer_bytes = 0;
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs

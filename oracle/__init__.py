@@ -13,7 +13,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libmesh_oracle.so")
 
-F32, F16, Q5_0, Q8_0, Q4_K, Q6_K = 0, 1, 6, 8, 12, 14
+F32, F16, Q4_0, Q5_0, Q8_0, Q4_K, Q6_K = 0, 1, 2, 6, 8, 12, 14
 ROPE_NORM, ROPE_NEOX = 0, 2
 
 _lib = None
@@ -53,6 +53,8 @@ def lib():
         L.mo_rope.argtypes = [vp, i64, i32, i32, i32, vp, f32, i32]
         L.mo_swiglu.argtypes = [vp, vp, vp, i64]
         L.mo_attn_token.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, f32, vp]
+        L.mo_attn_token_f32.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, f32, vp]
+        L.mo_quantize_row_q4_0.argtypes = [vp, vp, i64]
         L.mo_moe_route.argtypes = [vp, vp, i32, i32, i32, vp, vp]
         L.mo_set_threads.argtypes = [i32]
         L.mo_get_threads.restype = i32
@@ -102,6 +104,24 @@ def quantize_q8_0(x):
     y = np.empty(x.size // 32 * 34, dtype=np.uint8)
     lib().mo_quantize_row_q8_0(_p(x), _p(y), x.size)
     return y
+
+
+def quantize_q4_0(x):
+    """f32 array (size % 32 == 0) -> uint8 array of 18-byte blocks."""
+    x = _f32(x)
+    assert x.size % 32 == 0
+    y = np.empty(x.size // 32 * 18, dtype=np.uint8)
+    lib().mo_quantize_row_q4_0(_p(x), _p(y), x.size)
+    return y
+
+
+def kv_round(type_, x):
+    """The values a KV cache of `type_` (F16, Q8_0 or Q4_0) holds for the f32 rows x [..., head_dim], as f32."""
+    x = _f32(x)
+    if type_ == F16:
+        return fp16_to_fp32(fp32_to_fp16(x)).reshape(x.shape)
+    packed = quantize_q8_0(x) if type_ == Q8_0 else quantize_q4_0(x)
+    return dequantize(type_, packed, x.size).reshape(x.shape)
 
 
 def dequantize(type_, data, k):
@@ -155,15 +175,19 @@ def swiglu(gate, up):
 
 
 def attn_token(q, kcache, vcache, n_past, scale):
-    """q: [n_head, hd] f32; kcache/vcache: [n_kv, ctx, hd] uint16 (f16 bits); attends to [0, n_past]."""
+    """q: [n_head, hd] f32; kcache/vcache: [n_kv, ctx, hd], both uint16 (f16 bits) or both float32 (the values a
+    quantised cache holds); attends to [0, n_past]."""
     q = _f32(q)
     n_head, hd = q.shape
-    kcache = np.ascontiguousarray(kcache, dtype=np.uint16)
-    vcache = np.ascontiguousarray(vcache, dtype=np.uint16)
+    as_f32 = kcache.dtype == np.float32
+    assert vcache.dtype == kcache.dtype and kcache.dtype in (np.float32, np.uint16)
+    kcache = np.ascontiguousarray(kcache)
+    vcache = np.ascontiguousarray(vcache)
     n_kv, ctx, hd2 = kcache.shape
     assert hd2 == hd and vcache.shape == kcache.shape and n_past < ctx
     out = np.empty_like(q)
-    lib().mo_attn_token(_p(q), _p(kcache), _p(vcache), n_head, n_kv, hd, ctx, n_past, scale, _p(out))
+    fn = lib().mo_attn_token_f32 if as_f32 else lib().mo_attn_token
+    fn(_p(q), _p(kcache), _p(vcache), n_head, n_kv, hd, ctx, n_past, scale, _p(out))
     return out
 
 

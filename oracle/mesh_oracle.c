@@ -84,6 +84,8 @@ void mo_fp16_to_fp32_row(const uint16_t *x, float *y, int64_t n) {
 
 #define QK8_0 32
 #define QK5_0 32
+#define QK4_0 32
+#define Q4_0_BYTES 18
 #define QK_K 256
 #define Q8_0_BYTES 34
 #define Q5_0_BYTES 22
@@ -93,7 +95,7 @@ void mo_fp16_to_fp32_row(const uint16_t *x, float *y, int64_t n) {
 int64_t mo_block_elems(int type) {
     switch (type) {
         case MO_F32: case MO_F16: return 1;
-        case MO_Q5_0: case MO_Q8_0: return 32;
+        case MO_Q4_0: case MO_Q5_0: case MO_Q8_0: return 32;
         case MO_Q4_K: case MO_Q6_K: return 256;
         default: return -1;
     }
@@ -102,6 +104,7 @@ int64_t mo_block_bytes(int type) {
     switch (type) {
         case MO_F32: return 4;
         case MO_F16: return 2;
+        case MO_Q4_0: return Q4_0_BYTES;
         case MO_Q5_0: return Q5_0_BYTES;
         case MO_Q8_0: return Q8_0_BYTES;
         case MO_Q4_K: return Q4_K_BYTES;
@@ -138,6 +141,47 @@ void mo_quantize_row_q8_0(const float *x, void *vy, int64_t k) {
         for (int j = 0; j < QK8_0; j++) {
             const float x0 = x[i * QK8_0 + j] * id;
             b[2 + j] = (uint8_t)(int8_t)roundf(x0);
+        }
+    }
+}
+
+/* quantize_row_q4_0_ref: block = { fp16 d; uint8 qs[16] }.  max = the element of largest magnitude (the first one on
+ * ties), d = max / -8, id = 1/d from the unrounded d; q = min(15, (int8)(x*id + 8.5f)); byte j holds element j in
+ * its low nibble and element j + 16 in its high nibble. */
+void mo_quantize_row_q4_0(const float *x, void *vy, int64_t k) {
+    uint8_t *y = (uint8_t *)vy;
+    const int64_t nb = k / QK4_0;
+    for (int64_t i = 0; i < nb; i++) {
+        float amax = 0.0f, max = 0.0f;
+        for (int j = 0; j < QK4_0; j++) {
+            const float v = x[i * QK4_0 + j];
+            if (amax < fabsf(v)) { amax = fabsf(v); max = v; }
+        }
+        const float d = max / -8.0f;
+        const float id = d ? 1.0f / d : 0.0f;
+        const uint16_t dh = mo_fp32_to_fp16(d);
+        uint8_t *b = y + i * Q4_0_BYTES;
+        b[0] = (uint8_t)(dh & 0xFF);
+        b[1] = (uint8_t)(dh >> 8);
+        for (int j = 0; j < QK4_0 / 2; j++) {
+            const float x0 = x[i * QK4_0 + j] * id, x1 = x[i * QK4_0 + QK4_0 / 2 + j] * id;
+            int q0 = (int8_t)(x0 + 8.5f), q1 = (int8_t)(x1 + 8.5f);
+            if (q0 > 15) q0 = 15;
+            if (q1 > 15) q1 = 15;
+            b[2 + j] = (uint8_t)(q0 | (q1 << 4));
+        }
+    }
+}
+
+/* dequantize_row_q4_0: y[j] = ((qs[j] & 0xF) - 8) * d, y[j + 16] = ((qs[j] >> 4) - 8) * d */
+static void dequantize_row_q4_0(const uint8_t *x, float *y, int64_t k) {
+    const int64_t nb = k / QK4_0;
+    for (int64_t i = 0; i < nb; i++) {
+        const uint8_t *b = x + i * Q4_0_BYTES;
+        const float d = mo_fp16_to_fp32(rd16(b));
+        for (int j = 0; j < QK4_0 / 2; j++) {
+            y[i * QK4_0 + j] = (float)((b[2 + j] & 0x0F) - 8) * d;
+            y[i * QK4_0 + j + QK4_0 / 2] = (float)((b[2 + j] >> 4) - 8) * d;
         }
     }
 }
@@ -243,6 +287,7 @@ int mo_dequantize_row(int type, const void *vx, float *y, int64_t k) {
         case MO_F32: memcpy(y, x, (size_t)k * 4); return 0;
         case MO_F16: mo_fp16_to_fp32_row((const uint16_t *)vx, y, k); return 0;
         case MO_Q8_0: dequantize_row_q8_0(x, y, k); return 0;
+        case MO_Q4_0: dequantize_row_q4_0(x, y, k); return 0;
         case MO_Q5_0: dequantize_row_q5_0(x, y, k); return 0;
         case MO_Q4_K: dequantize_row_q4_K(x, y, k); return 0;
         case MO_Q6_K: dequantize_row_q6_K(x, y, k); return 0;
@@ -334,9 +379,10 @@ void mo_swiglu(const float *gate, const float *up, float *out, int64_t n) {
     }
 }
 
-/* softmax(q.K^T * scale) . V for one token, float64 throughout; K/V are the f16 cache contents */
-void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcache, int n_head, int n_kv,
-                   int head_dim, int64_t ctx_stride, int64_t n_past, float scale, float *out) {
+/* softmax(q.K^T * scale) . V for one token, float64 throughout.  K/V are the cache contents as values: f16 bits
+ * (kv_f32 = 0) or the f32 values a quantised cache dequantises to (kv_f32 = 1). */
+static void attn_token(const float *q, const void *kcache, const void *vcache, int kv_f32, int n_head, int n_kv,
+                       int head_dim, int64_t ctx_stride, int64_t n_past, float scale, float *out) {
     const int group = n_head / n_kv;
     const int64_t n = n_past + 1;
 #ifdef _OPENMP
@@ -344,15 +390,17 @@ void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcach
 #endif
     for (int h = 0; h < n_head; h++) {
         const int kvh = h / group;
-        const uint16_t *K = kcache + (int64_t)kvh * ctx_stride * head_dim;
-        const uint16_t *V = vcache + (int64_t)kvh * ctx_stride * head_dim;
+        const int64_t off = (int64_t)kvh * ctx_stride * head_dim;
+        const uint16_t *K16 = (const uint16_t *)kcache + off, *V16 = (const uint16_t *)vcache + off;
+        const float *K32 = (const float *)kcache + off, *V32 = (const float *)vcache + off;
         const float *qh = q + (int64_t)h * head_dim;
         double *s = (double *)malloc((size_t)n * sizeof(double));
         double *acc = (double *)calloc((size_t)head_dim, sizeof(double));
         double mx = -INFINITY;
         for (int64_t j = 0; j < n; j++) {
             double d = 0.0;
-            for (int i = 0; i < head_dim; i++) d += (double)qh[i] * (double)mo_fp16_to_fp32(K[j * head_dim + i]);
+            for (int i = 0; i < head_dim; i++)
+                d += (double)qh[i] * (double)(kv_f32 ? K32[j * head_dim + i] : mo_fp16_to_fp32(K16[j * head_dim + i]));
             s[j] = d * (double)scale;
             if (s[j] > mx) mx = s[j];
         }
@@ -360,12 +408,21 @@ void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcach
         for (int64_t j = 0; j < n; j++) { s[j] = exp(s[j] - mx); den += s[j]; }
         for (int64_t j = 0; j < n; j++) {
             const double p = s[j] / den;
-            for (int i = 0; i < head_dim; i++) acc[i] += p * (double)mo_fp16_to_fp32(V[j * head_dim + i]);
+            for (int i = 0; i < head_dim; i++)
+                acc[i] += p * (double)(kv_f32 ? V32[j * head_dim + i] : mo_fp16_to_fp32(V16[j * head_dim + i]));
         }
         for (int i = 0; i < head_dim; i++) out[(int64_t)h * head_dim + i] = (float)acc[i];
         free(s);
         free(acc);
     }
+}
+void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcache, int n_head, int n_kv,
+                   int head_dim, int64_t ctx_stride, int64_t n_past, float scale, float *out) {
+    attn_token(q, kcache, vcache, 0, n_head, n_kv, head_dim, ctx_stride, n_past, scale, out);
+}
+void mo_attn_token_f32(const float *q, const float *kcache, const float *vcache, int n_head, int n_kv,
+                       int head_dim, int64_t ctx_stride, int64_t n_past, float scale, float *out) {
+    attn_token(q, kcache, vcache, 1, n_head, n_kv, head_dim, ctx_stride, n_past, scale, out);
 }
 
 /* MoE gating as llama.cpp's build_moe_ffn runs it for softmax-gated models (qwen3moe), with the expert mask of

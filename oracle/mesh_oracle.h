@@ -32,8 +32,8 @@
 extern "C" {
 #endif
 
-/* ggml type ids used by a Q4_K_M file */
-enum { MO_F32 = 0, MO_F16 = 1, MO_Q5_0 = 6, MO_Q8_0 = 8, MO_Q4_K = 12, MO_Q6_K = 14 };
+/* ggml type ids used by a Q4_K_M file, plus Q4_0 (a KV cache type of mesh-llm/src/inference/launch.rs:568-591) */
+enum { MO_F32 = 0, MO_F16 = 1, MO_Q4_0 = 2, MO_Q5_0 = 6, MO_Q8_0 = 8, MO_Q4_K = 12, MO_Q6_K = 14 };
 /* rope pairings */
 enum { MO_ROPE_NORM = 0, MO_ROPE_NEOX = 2 };
 
@@ -48,6 +48,7 @@ int64_t  mo_block_elems(int type);
 int64_t  mo_block_bytes(int type);
 int64_t  mo_row_bytes(int type, int64_t k);              /* -1 if k is not a whole number of blocks */
 void     mo_quantize_row_q8_0(const float *x, void *y, int64_t k);
+void     mo_quantize_row_q4_0(const float *x, void *y, int64_t k);
 int      mo_dequantize_row(int type, const void *x, float *y, int64_t k);   /* 0 ok, -1 bad type/size */
 
 /* --- operators --- */
@@ -66,6 +67,10 @@ void mo_swiglu(const float *gate, const float *up, float *out, int64_t n);
 void mo_attn_token(const float *q, const uint16_t *kcache, const uint16_t *vcache,
                    int n_head, int n_kv, int head_dim, int64_t ctx_stride, int64_t n_past,
                    float scale, float *out);
+/* the same over caches held as f32 values (what a q8_0 / q4_0 cache dequantises to) */
+void mo_attn_token_f32(const float *q, const float *kcache, const float *vcache,
+                       int n_head, int n_kv, int head_dim, int64_t ctx_stride, int64_t n_past,
+                       float scale, float *out);
 /* MoE router: probs = softmax(logits) over n_expert; top-k ids by (probs + mask), mask 0 / -inf (ties: lower id
  * first); weights = unmasked probs of the selected experts, optionally renormalised to sum 1. */
 void mo_moe_route(const float *logits, const float *mask, int n_expert, int top_k, int norm_w,

@@ -16,13 +16,18 @@ import oracle as O
 class StageOracle:
     """tensors: dict name -> (ggml_type, dims (ne0, ne1[, ne2]), uint8 ndarray) as written to the GGUF file."""
 
-    def __init__(self, cfg, tensors, layer_begin, layer_end, n_ctx, n_seq_max=1, expert_mask=None):
+    def __init__(self, cfg, tensors, layer_begin, layer_end, n_ctx, n_seq_max=1, expert_mask=None, kv_types=None):
+        """kv_types: (K type, V type) of the cache, each F16, Q8_0 or Q4_0 (the tiers of
+        mesh-llm/src/inference/launch.rs:568-591); None = f16 / f16.  A quantised cache is held as the f32 values its
+        blocks dequantise to (rows quantised per 32 elements along head_dim, as ggml stores the cache rows)."""
         self.c = cfg
         self.t = tensors
         self.lb, self.le = layer_begin, layer_end
         self.n_ctx = n_ctx
         hk, hd = cfg["n_head_kv"], cfg["head_dim"]
-        self.k = np.zeros((layer_end - layer_begin, n_seq_max, hk, n_ctx, hd), np.uint16)
+        self.kv_types = tuple(kv_types) if kv_types else (O.F16, O.F16)
+        self.kv_f32 = self.kv_types != (O.F16, O.F16)
+        self.k = np.zeros((layer_end - layer_begin, n_seq_max, hk, n_ctx, hd), np.float32 if self.kv_f32 else np.uint16)
         self.v = np.zeros_like(self.k)
         self.rope_mode = O.ROPE_NORM if cfg["arch"] == "llama" else O.ROPE_NEOX
         self.expert_mask = expert_mask
@@ -102,7 +107,10 @@ class StageOracle:
                 k = self._head_norm(k, p + "attn_k_norm.weight")
             q = O.rope(q, pos, hd, c["rope"], self.rope_mode)
             k = O.rope(k, pos, hd, c["rope"], self.rope_mode)
-            kh, vh = O.fp32_to_fp16(k), O.fp32_to_fp16(v)
+            if self.kv_f32:
+                kh, vh = O.kv_round(self.kv_types[0], k), O.kv_round(self.kv_types[1], v)
+            else:
+                kh, vh = O.fp32_to_fp16(k), O.fp32_to_fp16(v)
             for t in range(T):
                 self.k[li, seq[t], :, pos[t], :] = kh[t]
                 self.v[li, seq[t], :, pos[t], :] = vh[t]

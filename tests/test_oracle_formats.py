@@ -146,3 +146,55 @@ def test_add_and_truncate_equals_round_half_away():
         fast = np.trunc(x + np.copysign(c, x))                                   # float32 add, round to nearest even
         exact = np.copysign(np.floor(np.abs(x).astype(np.float64) + 0.5), x)     # roundf
         assert np.array_equal(fast.astype(np.float64), exact)
+
+
+def test_q4_0_known_answer_block():
+    """Hand-packed block: d = 0.5, byte j = (j) | ((15 - j) << 4): element j is (j - 8) / 2, element j + 16 is
+    (7 - j) / 2.  A swap of the nibbles, of the halves, or a missing -8 fails this."""
+    blk = np.zeros(18, np.uint8)
+    blk[:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    j = np.arange(16)
+    blk[2:] = j | ((15 - j) << 4)
+    y = oracle.dequantize(oracle.Q4_0, blk, 32)
+    assert np.array_equal(y[:16], (j - 8) * 0.5)
+    assert np.array_equal(y[16:], (7 - j) * 0.5)
+    assert oracle.row_bytes(oracle.Q4_0, 128) == 72
+
+
+def test_q4_0_quantise_invariants_and_numpy_restatement():
+    rng = np.random.default_rng(404)
+    x = rng.standard_normal((4000, 32)).astype(np.float32)
+    x[0] = 0.0                                   # all-zero block: d = 0 / -8 = -0.0, every nibble 8
+    x[1, 3], x[1, 20] = 5.0, -5.0                # tie in magnitude: the first element (positive) decides the sign of d
+    x[1, [i for i in range(32) if i not in (3, 20)]] *= 0.1
+    x[2, 7], x[2, 2] = -6.0, 6.0                 # tie the other way round: index 2 (positive) comes first
+    x[2, [i for i in range(32) if i not in (2, 7)]] *= 0.1
+    x[3] *= 1e-6                                 # small values: d is an fp16 subnormal
+    packed = oracle.quantize_q4_0(x).reshape(-1, 18)
+    # independent float32 restatement in numpy
+    idx = np.argmax(np.abs(x), axis=1)           # argmax returns the first maximum
+    mx = x[np.arange(len(x)), idx]
+    d = (mx / np.float32(-8.0)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+    q = np.minimum(15, np.trunc((x * idv[:, None]).astype(np.float32) + np.float32(8.5)).astype(np.int32))
+    want = (q[:, :16] | (q[:, 16:] << 4)).astype(np.uint8)
+    assert np.array_equal(packed[:, 2:], want)
+    assert np.array_equal(packed[:, :2].copy().view(np.float16)[:, 0], d.astype(np.float16))
+    assert np.all(packed[0] == np.r_[np.array([0x00, 0x80], np.uint8), np.full(16, 0x88, np.uint8)])
+    assert d[1] < 0 and d[2] < 0                 # the first of the tied elements is the positive one in both rows
+    # the element of largest magnitude is reproduced as -8 * d; everything else within one step
+    y = oracle.dequantize(oracle.Q4_0, packed.reshape(-1), x.size).reshape(x.shape)
+    dh = d.astype(np.float16).astype(np.float32)
+    assert np.array_equal(y[np.arange(len(x)), idx], np.float32(-8) * dh)
+    assert np.all(np.abs(y - x) <= np.abs(dh)[:, None] * 1.001 + np.abs(x) * 2.0 ** -10)
+
+
+def test_kv_round_is_quantise_then_dequantise():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 2, 64)).astype(np.float32)
+    assert np.array_equal(oracle.kv_round(oracle.F16, x), x.astype(np.float16).astype(np.float32))
+    r8 = oracle.kv_round(oracle.Q8_0, x)
+    assert r8.shape == x.shape and np.array_equal(r8.reshape(-1), oracle.dequantize(oracle.Q8_0, oracle.quantize_q8_0(x), x.size))
+    r4 = oracle.kv_round(oracle.Q4_0, x)
+    assert np.abs(r4 - x).max() < 0.5 and np.abs(r8 - x).max() < 0.03
