@@ -124,6 +124,7 @@ static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStrea
 template <int TYPE, int NU>
 static int launch_dot_nb(int nb, const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
     if (nb == 4) return launch_dot<TYPE, 4, NU>(ka, grid, smem, stream);
+    if (nb == 3) return launch_dot<TYPE, 3, NU>(ka, grid, smem, stream);
     if (nb == 2) return launch_dot<TYPE, 2, NU>(ka, grid, smem, stream);
     return launch_dot<TYPE, 1, NU>(ka, grid, smem, stream);
 }
@@ -207,8 +208,8 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     int t = 0;
     while (t < a.T) {
         const int left = a.T - t;
-        int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
-        while (nb > 1 && dot_smem_bytes(type, nb, a.K, rows_max, KS, NU) > LDS_LIMIT) nb >>= 1;
+        int nb = left >= 4 ? 4 : left;      // 3 columns have a kernel of their own: no second pass over the weights
+        while (nb > 1 && dot_smem_bytes(type, nb, a.K, rows_max, KS, NU) > LDS_LIMIT) --nb;
         GemvKernelArgs kb = ka;
         kb.x = a.x + (size_t)t * a.ldx;
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
@@ -251,14 +252,15 @@ static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream)
     int t = 0;
     while (t < a4.T) {
         const int left = a4.T - t;
-        int nb = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        int nb = left >= 4 ? 4 : left;
         auto need = [&](int n) { return std::max(dot_smem_bytes(MESH_Q4_K, n, a4.K, p4.rows_max, p4.KS, 1), dot_smem_bytes(MESH_Q6_K, n, a6.K, p6.rows_max, p6.KS, 1)); };
-        while (nb > 1 && need(nb) > LDS_LIMIT) nb >>= 1;
+        while (nb > 1 && need(nb) > LDS_LIMIT) --nb;
         GemvKernelArgs k4 = p4.ka, k6 = p6.ka;
         k4.x = k6.x = a4.x + (size_t)t * a4.ldx;
         for (int i = 0; i < a4.n_mat; ++i) k4.y[i] = a4.mat[i].y + (size_t)t * a4.mat[i].ldy;
         for (int i = 0; i < a6.n_mat; ++i) k6.y[i] = a6.mat[i].y + (size_t)t * a6.mat[i].ldy;
         if (nb == 4) rc = launch_dual<4>(k4, k6, p4.grid, p6.grid, need(4), stream);
+        else if (nb == 3) rc = launch_dual<3>(k4, k6, p4.grid, p6.grid, need(3), stream);
         else if (nb == 2) rc = launch_dual<2>(k4, k6, p4.grid, p6.grid, need(2), stream);
         else rc = launch_dual<1>(k4, k6, p4.grid, p6.grid, need(1), stream);
         if (rc != MESH_OK) return rc;

@@ -157,6 +157,12 @@ def test_llama3_8b_shaped_layers_decode_with_long_kv(tmp_path):
     got = ses.decode(x4, pos, seq=seq).view(np.float32).reshape(4, 4096)
     ref = orc.forward(x4, pos, seq=seq)
     assert rel_l2(got, ref) <= 1e-3
+    # three tokens: the 3-column mat-vec kernels
+    x3 = rng.standard_normal((3, 4096)).astype(np.float32)
+    pos, seq = [n_past + 1, n_past + 1, n_past], [0, 1, 3]
+    got = ses.decode(x3, pos, seq=seq).view(np.float32).reshape(3, 4096)
+    ref = orc.forward(x3, pos, seq=seq)
+    assert rel_l2(got, ref) <= 1e-3
     ses.close()
     st.close()
 
@@ -177,7 +183,7 @@ def test_qwen25_32b_shaped_layer_all_decode_paths(tmp_path):
         orc.k[0, s_, :, :n_past] = k.transpose(1, 0, 2)
         orc.v[0, s_, :, :n_past] = v.transpose(1, 0, 2)
     nxt = [n_past] * 16
-    for seqs, tol in (([3], 1e-3), ([0, 5, 9, 12], 1e-3), (list(range(16)), 3e-3), ([1, 2, 3, 4, 6, 7, 8, 10, 11, 13, 15], 3e-3)):
+    for seqs, tol in (([3], 1e-3), ([0, 5, 9, 12], 1e-3), ([2, 6, 14], 1e-3), (list(range(16)), 3e-3), ([1, 2, 3, 4, 6, 7, 8, 10, 11, 13, 15], 3e-3)):
         T = len(seqs)
         pos = [nxt[q] for q in seqs]
         for q in seqs:
