@@ -59,6 +59,13 @@ def time_on_stream(torch, stream, fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall_ms
 
 
+def hbm_probe(m):
+    """Streaming-read bandwidth of this GPU: 512 MiB, 3 warm-up + 20 timed passes, the protocol of the reference's
+    mesh-llm/benchmarks/membench-fingerprint.hip; quoted beside the nominal 8 TB/s."""
+    g = m.hbm_read_probe(512 << 20, 3, 20)
+    return {"p50": round(g[len(g) // 2], 1), "p90": round(g[int(len(g) * 0.9)], 1), "bytes": 512 << 20, "runs": len(g)}
+
+
 # ------------------------------------------------------------------------------------------------ codec
 def run_codec(torch, m, steps, warmup, T=4096, h=4096):
     """Each op cycles through enough distinct buffers (> 256 MiB in total) that no pass is served by the
@@ -116,7 +123,7 @@ def bench_codec(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32->i8+f16", "data": "synthetic",
         "config": {"workload": "codec: pack_q8_0 of hidden state [4096,4096] f32, N(0,1) with 0.1% channels x50"},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "measured_stream_read_GBps": hbm_probe(m)},
         "codec": res,
     }
     if not args.no_cpu:
@@ -248,6 +255,7 @@ def bench_stage(args):
     g_n = b1["kernel_launches_per_step"]["gemv"]
     gemv_gbs = weight_bytes / g_ms / 1e6
     codec = run_codec(torch, m, max(10, args.steps // 2), args.warmup)
+    probe = hbm_probe(m)
     out = {
         "metric": "stage decode tok/s @8B Q4_K_M", "value": b1["tok_s"], "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": b1["ms_per_step"], "higher_is_better": True,
@@ -260,7 +268,8 @@ def bench_stage(args):
                      # HBM bytes per average launch: rocprofv3 FETCH_SIZE (x2.0 calibration) + WRITE_SIZE of the gemv
                      # launches, profiles/stage_decode_llama3_8b_l0_15_hbm_traffic.txt: 1.006 x algorithmic
                      "traffic": int(round(1.006 * weight_bytes / g_n)), "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
-                     "algorithmic_bytes_per_launch": weight_bytes // g_n},
+                     "algorithmic_bytes_per_launch": weight_bytes // g_n,
+                     "measured_stream_read_GBps": probe, "frac_of_measured_p90": round(gemv_gbs / probe["p90"], 4)},
         "stage_frac_hbm": b1["frac_hbm"],
         "decode": {str(k): v for k, v in results.items()},
         "prefill": prefill,

@@ -60,6 +60,12 @@ int mesh_device_count(void);
  * mesh-llm/src/inference/launch.rs:812-823 does). */
 int mesh_device_select(const char *device);
 
+/* Streaming-read bandwidth of the current GPU: `timed_runs` event-timed passes over a zero-filled buffer of `bytes`
+ * (after `warmup_runs` untimed ones), GB/s of each pass into gbps[timed_runs].  The protocol of the reference's GPU
+ * fingerprint benchmark (mesh-llm/benchmarks/membench-fingerprint.hip:24-39,151-160: 512 MiB, 3 + 20 runs, p50 / p90
+ * taken by the caller; its output feeds mesh-llm/src/system/benchmark.rs:11-29). */
+int mesh_hbm_read_probe(size_t bytes, int warmup_runs, int timed_runs, double *gbps);
+
 /* ---- boundary activation codec -------------------------------------------------------------------
  * The inter-stage hidden state [n_tokens, n_embd] f32, packed for transport.  Replaces the raw-f32
  * ggml_backend_tensor_get -> TCP -> ggml_backend_tensor_set hop of push_tensor_to_peer

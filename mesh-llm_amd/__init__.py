@@ -33,6 +33,7 @@ SIGNATURES = {
     "mesh_last_error": (_cp, []),
     "mesh_device_count": (_i32, []),
     "mesh_device_select": (_i32, [_cp]),
+    "mesh_hbm_read_probe": (_i32, [_sz, _i32, _i32, _vp]),
     "mesh_act_packed_size": (_sz, [_i32, _i64, _i64]),
     "mesh_act_pack": (_i32, [_i32, _vp, _vp, _i64]),
     "mesh_act_unpack": (_i32, [_i32, _vp, _vp, _i64]),
@@ -141,6 +142,13 @@ def device_count():
 
 def device_select(name):
     check(lib().mesh_device_select(str(name).encode()))
+
+
+def hbm_read_probe(nbytes=512 << 20, warmup=3, runs=20):
+    """GB/s of `runs` streaming-read passes over a buffer of nbytes (mesh_hbm_read_probe), ascending."""
+    out = (ctypes.c_double * runs)()
+    check(lib().mesh_hbm_read_probe(nbytes, warmup, runs, out))
+    return sorted(out)
 
 
 def act_packed_size(fmt, n_tokens, n_embd):

@@ -49,5 +49,8 @@ def test_errors_are_codes_plus_message_not_exceptions():
     with pytest.raises(m.MeshError) as e:
         m.device_select("Vulkan0")
     assert e.value.code == m.ERR_INVALID
+    with pytest.raises(m.MeshError) as e:
+        m.hbm_read_probe(1024, 0, 1)        # below a megabyte: refused before any device call
+    assert e.value.code == m.ERR_INVALID
     # zero elements is a no-op, not an error, and touches no device
     assert m.act_pack(m.Q8_0, np.zeros(0, np.float32)).size == 0

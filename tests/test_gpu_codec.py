@@ -164,3 +164,11 @@ def test_device_entry_points_reject_bad_arguments():
     m.device_select("ROCm0")
     m.device_select("HIP0")
     assert m.device_count() >= 1
+
+
+def test_hbm_read_probe_reports_plausible_bandwidth():
+    """The streaming-read yardstick (protocol of mesh-llm/benchmarks/membench-fingerprint.hip): 5 timed passes over
+    256 MiB, each between 1 and 10 TB/s on an MI355X."""
+    m = mesh()
+    g = m.hbm_read_probe(256 << 20, 2, 5)
+    assert len(g) == 5 and all(1000.0 < v < 10000.0 for v in g), g
