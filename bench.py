@@ -9,6 +9,11 @@ Workloads
           hidden state resident in HBM, output the q8_0 boundary activation.  A step = one decode call of the
           whole stage at batch 1; value = tokens/s.  Batch 4 and 16 and the boundary codec are reported beside it.
   codec   boundary activation codec alone on [4096, 4096] f32; value = algorithmic GB/s of pack_q8_0.
+  c4      Qwen2.5-32B-shaped stage, layers 0-31 of 64 (hidden 5120, 40/8 heads, FFN 27648, q/k/v biases), 8192-token
+          KV context in the cache tier the reference picks for a 20 GB model (K q8_0 / V q4_0; --kv f16 for the f16
+          tier), decode batch 1/8/32 and a 4096-token prefill.  value = batch-1 tokens/s.
+  c5      Qwen3-30B-A3B-shaped expert shard: all 48 layers, 64 of the 128 experts per layer (top-8 routing, expert FFN
+          768, per-head q/k norms), decode batch 16 at a 4096-token context.  value = tokens/s at batch 16.
 
 Timing uses HIP events recorded on the stream the kernels run on (the session's own stream for the stage).
 The cpu_baseline leg times the CPU oracle (a restatement of ggml's reference routines, NOT llama.cpp) on the
@@ -283,12 +288,119 @@ def bench_stage(args):
     return out
 
 
+# ------------------------------------------------------------------------------------------------ other shapes
+SHAPES = {
+    "c4": dict(model="qwen2.5-32b", layers=32, n_ctx=8192, batches=[1, 8, 32], prefill=4096, n_expert_local=None, kv="q8_0/q4_0",
+               metric="stage decode tok/s @32B Q4_K_M, layers 0-31 of 64"),
+    "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=0, n_expert_local=64, kv="q8_0/q4_0",
+               metric="expert-shard decode tok/s @Qwen3-30B-A3B Q4_K_M, 64 of 128 experts, batch 16"),
+}
+
+
+def bench_shape(args):
+    """The larger BASELINE shapes at full size on one GPU: same timing as the default workload, fewer extras."""
+    import torch
+    import __graft_entry__ as graft
+    import models
+    m = graft.load_package()
+    m.lib()
+    sp = SHAPES[args.workload]
+    cfg = models.CONFIGS[sp["model"]]
+    kv_name = args.kv if args.kv_given else sp["kv"]
+    kv_types = {"f16": (m.F16, m.F16), "q8_0/q4_0": (m.Q8_0, m.Q4_0), "q4_0/q4_0": (m.Q4_0, m.Q4_0)}[kv_name]
+    kv_row = {m.F16: HD_BYTES_F16, m.Q8_0: HD_BYTES_Q8_0, m.Q4_0: HD_BYTES_Q4_0}
+    path = os.path.join(models.tmp_dir(), "mesh_bench_%s.gguf" % args.workload)
+    t0 = time.perf_counter()
+    tensors = models.write_model(path, cfg, range(sp["layers"]), seed=42, fast=True, n_expert_local=sp["n_expert_local"])
+    t_gen = time.perf_counter() - t0
+    expert_bytes = sum(d.nbytes for n, (_, _, d) in tensors.items() if "_exps." in n)
+    del tensors
+    print("[bench] model file written in %.1f s" % t_gen, file=sys.stderr, flush=True)
+    batches = sp["batches"]
+    bmax = max(batches)
+    n_ctx, L = sp["n_ctx"], sp["layers"]
+    t0 = time.perf_counter()
+    st = m.Stage(path, 0, L, n_ctx=n_ctx, n_seq_max=bmax, n_batch_max=max(bmax, 16, sp["prefill"]), kv_types=kv_types)
+    t_load = time.perf_counter() - t0
+    os.unlink(path)
+    ses = st.session()
+    E, HK, HD = cfg["n_embd"], cfg["n_head_kv"], cfg["head_dim"]
+    rng = np.random.Generator(np.random.PCG64(99))
+    kv = (rng.standard_normal((n_ctx - 1, HK, HD)) * 0.1).astype(np.float16).view(np.uint16)
+    t0 = time.perf_counter()
+    for il in range(L):
+        for s in range(bmax):
+            ses.kv_write(il, s, 0, kv, kv)
+    t_kv = time.perf_counter() - t0
+    print("[bench] stage open %.1f s, KV context filled in %.1f s" % (t_load, t_kv), file=sys.stderr, flush=True)
+    kv_bytes_per_seq = L * n_ctx * HK * (kv_row[kv_types[0]] + kv_row[kv_types[1]])
+    stream = torch.cuda.ExternalStream(ses.stream)
+    results = {}
+    for B in batches:
+        print("[bench] decode batch %d" % B, file=sys.stderr, flush=True)
+        x = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
+        out = torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")
+        pos = np.full(B, n_ctx - 1, np.int32)
+        seq = np.arange(B, dtype=np.int32)
+
+        def step(i):
+            ses.decode_dev(x.data_ptr(), pos, out.data_ptr(), out.numel(), seq=seq, in_fmt=m.F32, out_fmt=m.Q8_0)
+
+        ms, wall = time_on_stream(torch, stream, step, args.steps, args.warmup)
+        ses.profile(True)
+        for i in range(3):
+            step(i)
+        prof = ses.profile_read()
+        ses.profile(False)
+        r = {"ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall, 4), "tok_s": round(B * 1e3 / ms, 1),
+             "kernel_ms_per_step": {k: round(v["ms"] / 3, 4) for k, v in prof.items()}}
+        if sp["n_expert_local"]:
+            # bytes a step must read: attention + router + the DISTINCT experts the batch selected (last layer's count)
+            ids = ses.moe_last_ids(B)
+            distinct = int(np.unique(ids).size)
+            r["distinct_experts_last_layer"] = distinct
+            step_bytes = (st.weight_bytes - expert_bytes) + expert_bytes * distinct / sp["n_expert_local"] + kv_bytes_per_seq * B
+        else:
+            step_bytes = st.weight_bytes + kv_bytes_per_seq * B
+        r["algorithmic_GB_per_step"] = round(step_bytes / 1e9, 3)
+        r["GBps"] = round(step_bytes / ms / 1e6, 1)
+        r["frac_hbm"] = round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)
+        results[B] = r
+    prefill = None
+    if sp["prefill"]:
+        T = sp["prefill"]
+        xp = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).cuda()
+        outp = torch.empty(m.act_packed_size(m.Q8_0, T, E), dtype=torch.uint8, device="cuda")
+        ppos = np.arange(T, dtype=np.int32)
+
+        def pstep(i):
+            ses.decode_dev(xp.data_ptr(), ppos, outp.data_ptr(), outp.numel(), in_fmt=m.F32, out_fmt=m.Q8_0)
+
+        pms, _ = time_on_stream(torch, stream, pstep, 2, 1)
+        H, FF = cfg["n_head"], cfg["n_ff"]
+        mm_flop = 2.0 * T * L * (E * H * HD * 2 + E * HK * HD * 2 + 3 * E * FF)
+        prefill = {"tokens": T, "ms": round(pms, 2), "tok_s": round(T * 1e3 / pms, 1), "matmul_TFLOP": round(mm_flop / 1e12, 2),
+                   "matmul_TFLOPs_over_whole_step": round(mm_flop / pms / 1e9, 1)}
+    head = results[batches[0]]
+    out = {"metric": sp["metric"], "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32 activations x q4_K/q6_K weights, %s KV" % kv_name, "data": "synthetic",
+           "config": {"workload": "%s-shaped stage, %d layers, Q4_K_M block-domain random weights, %d-token %s KV context, decode batch %d"
+                                  % (sp["model"], L, n_ctx, kv_name, batches[0]),
+                      "weight_bytes": st.weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
+           "decode": {str(k): v for k, v in results.items()}, "prefill": prefill,
+           "setup_s": {"generate_gguf": round(t_gen, 1), "open_stage": round(t_load, 1), "fill_kv": round(t_kv, 1)}}
+    ses.close()
+    st.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="stage", choices=["stage", "codec"])
+    ap.add_argument("--workload", default="stage", choices=["stage", "codec", "c4", "c5"])
     ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
     ap.add_argument("--kv", default="f16", choices=["f16", "q8_0/q4_0", "q4_0/q4_0"],
                     help="KV cache row types K/V (default f16: the tier the reference picks for an 8B Q4_K_M model)")
@@ -299,7 +411,8 @@ def main():
         print("bench.py measures one GPU's share of the stage path (one GPU per box); --gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
-    out = bench_stage(args) if args.workload == "stage" else bench_codec(args)
+    args.kv_given = any(a == "--kv" or a.startswith("--kv=") for a in sys.argv[1:])
+    out = bench_stage(args) if args.workload == "stage" else bench_codec(args) if args.workload == "codec" else bench_shape(args)
     print(json.dumps(out))
 
 

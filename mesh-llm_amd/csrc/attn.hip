@@ -86,6 +86,21 @@ constexpr int ATTN_THREADS = 256;
 constexpr int ATTN_WAVES = ATTN_THREADS / 64;
 constexpr int KPT = 4;                      // keys per thread per pass: 8 x 16-byte loads in flight per lane
 
+// 2^x by the hardware instruction alone: arguments here are <= 0 (score minus running maximum), and results too small
+// for a normal float may flush to zero, which a softmax weight of that size is anyway.
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Sum over the LPK (8 or 16) consecutive lanes that share a key, result in every one of them: data-parallel-primitive
+// moves inside a row of 16 lanes (swap neighbours, swap pairs, mirror the 8, mirror the 16) instead of LDS permutes.
+template <int LPK>
+__device__ __forceinline__ float slot_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false));    // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false));    // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false));   // row_half_mirror
+    if (LPK == 16) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false));   // row_mirror
+    return v;
+}
+
 // grid (n_splits, n_kv * (group/G), T).  HD/8 lanes share one key ("slot"); a thread visits keys
 // j0 + slot + SLOTS*i and keeps one online-softmax state (m, l, acc[8]) per query head.  Per pass all KPT keys'
 // K and V vectors are requested first, then scored, then folded in with a single rescale.  The slots of a
@@ -158,8 +173,7 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s = fmaf(q[h][e], kf[e], s);
                 if (KT != MESH_F16) s *= kd;
-#pragma unroll
-                for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+                s = slot_sum<LPK>(s);
                 sc[i][h] = ok ? s : -INFINITY;
             }
         }
@@ -172,10 +186,10 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < KPT; ++i) mn = fmaxf(mn, sc[i][h]);
             if (mn == -INFINITY) continue;          // this slot had no key in range yet
-            const float corr = exp2f(m[h] - mn);    // exp2(-inf) = 0 the first time
+            const float corr = exp2_fast(m[h] - mn);    // exp2(-inf) = 0 the first time
             float p[KPT], ps = 0.f;
 #pragma unroll
-            for (int i = 0; i < KPT; ++i) { p[i] = exp2f(sc[i][h] - mn); ps += p[i]; }
+            for (int i = 0; i < KPT; ++i) { p[i] = exp2_fast(sc[i][h] - mn); ps += p[i]; }
             l[h] = l[h] * corr + ps;
             if (VT != MESH_F16) {       // from here on p carries the row scale; the offset term is summed apart
                 float po = 0.f;
