@@ -326,6 +326,10 @@ int attention(const AttnArgs &a, int T, hipStream_t stream) {
     else if (a.head_dim == 64) rc = launch_attn_typed<64>(a, T, stream);
     else return fail(MESH_ERR_UNSUPPORTED, "attention: head_dim %d has no kernel (64 and 128 do)", a.head_dim);
     if (rc != MESH_OK || a.n_splits == 1) return rc;
+    return attention_combine(a, T, stream);
+}
+
+int attention_combine(const AttnArgs &a, int T, hipStream_t stream) {
     attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;

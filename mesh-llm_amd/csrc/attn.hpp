@@ -39,6 +39,12 @@ struct AttnArgs {
 };
 // token t attends to cache positions [0, pos[t]] of sequence seq[t]
 int attention(const AttnArgs &a, int T, hipStream_t stream);
+// merge of the split partials (a.part, a.ml) into a.out; a no-op contract for n_splits == 1 is the caller's business
+int attention_combine(const AttnArgs &a, int T, hipStream_t stream);
+// The same attention with the query heads of a KV head as the columns of matrix-core tiles (attn_mma.hip): per-key
+// cost independent of the group size; Q and the probabilities rounded to f16.  For batches of decode tokens.
+bool attention_mma_supported(const AttnArgs &a);
+int attention_mma(const AttnArgs &a, int T, hipStream_t stream);
 // The same for a chunk of T consecutive positions pos0 .. pos0 + T - 1 of one sequence, on the matrix cores
 // (attn_prefill.hip; head_dim 128).  a.pos / a.seq / a.part / a.ml are not used.
 int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t stream);

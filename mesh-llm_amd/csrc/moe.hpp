@@ -13,6 +13,11 @@ struct MoeRouteArgs {
     int n_expert = 0, top_k = 0, norm_w = 1;
 };
 int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream);
+// Router mat-vec (f32 matrix W [n_expert][E] over the RMS-normalised hidden state) and routing in one launch; a.logits is
+// not read, logits_out (optional) receives [T][n_expert].
+bool moe_router_fused_supported(int E, int n_expert, int top_k);
+int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
+                     float *logits_out, int T, hipStream_t stream);
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 

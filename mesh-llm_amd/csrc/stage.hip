@@ -468,13 +468,15 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
     if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
-    if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && hp.n_ff > 0) {
+    if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens())) {
         const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
-        if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
-        s->ffn16 = static_cast<uint16_t *>(p);
-        if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
+        if (hp.n_ff > 0) {
+            if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
+            s->ffn16 = static_cast<uint16_t *>(p);
+            if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
+        }
     }
     if (hp.n_expert_used > 0 && !st->layers.empty() && st->layers[0].gate_inp.present()) {
         const size_t ne = (size_t)st->layers[0].gate_inp.M, k = hp.n_expert_used;
@@ -507,6 +509,17 @@ static GemvMat mat_of(const DevTensor &w, float *y, int ldy, const DevTensor *bi
     m.W = w.data; m.type = w.type; m.M = (int)w.M; m.y = y; m.ldy = ldy;
     m.bias = bias && bias->present() ? static_cast<const float *>(bias->data) : nullptr;
     return m;
+}
+
+// batches of at least this many tokens take the matrix-core decode attention (its inputs are rounded to f16, like the
+// batched projections around it)
+static int attn_mma_min_tokens() {
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("MESH_ATTN_MMA_MIN_TOKENS");
+        v = e ? std::max(1, atoi(e)) : 5;
+    }
+    return v;
 }
 
 static int attn_splits_for(int T, int n_kv, int max_keys) {
@@ -552,11 +565,17 @@ int profile_collect(mesh_session *s) {
     return MESH_OK;
 }
 
-static bool layer_is_kquant_dense(const LayerWeights &L) {
-    const DevTensor *w[] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down};
+static bool layer_attn_is_kquant(const LayerWeights &L) {
+    const DevTensor *w[] = {&L.wq, &L.wk, &L.wv, &L.wo};
     for (const DevTensor *t : w)
         if (!t->present() || !t->tiled) return false;
     return true;
+}
+static bool layer_is_kquant_dense(const LayerWeights &L) {
+    const DevTensor *w[] = {&L.w_gate, &L.w_up, &L.w_down};
+    for (const DevTensor *t : w)
+        if (!t->present() || !t->tiled) return false;
+    return layer_attn_is_kquant(L);
 }
 
 static GemmArgs gemm_of(const DevTensor &w, const uint16_t *x16, int ldx, int T, float *y, int ldy, const DevTensor *bias) {
@@ -570,7 +589,8 @@ static GemmArgs gemm_of(const DevTensor &w, const uint16_t *x16, int ldx, int T,
 // One layer over many tokens: norms and activations are materialised in f16 and every projection is an MFMA GEMM.
 // One dense K-quant layer over f16 activations on the matrix cores: `skinny` selects the batched-decode GEMM (few
 // tokens, weight-streaming bound) instead of the large-tile prefill GEMM.
-static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, int T, int max_keys, bool skinny) {
+// attn_only: stop after the attention block (x += Wo . attention); the caller runs the feed-forward part.
+static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, int T, int max_keys, bool skinny, bool attn_only) {
     mesh_stage *st = s->stage;
     const HParams &hp = st->hp;
     hipStream_t stream = s->stream;
@@ -618,6 +638,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     {
         ProfScope ps(s, MESH_PROF_ATTN);
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
+        else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) rc = attention_mma(aa, T, stream);
         else rc = attention(aa, T, stream);
     }
     if (rc != MESH_OK) return rc;
@@ -638,6 +659,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         go.residual = s->x; go.ldres = E;
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
+    if (attn_only) return MESH_OK;
     if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
@@ -686,10 +708,18 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0 &&
                                 L.w_gate.type == L.w_up.type;
             if (skinny || T >= PREFILL_MIN_TOKENS) {
-                if ((rc = run_layer_prefill(s, L, il, T, max_keys, skinny)) != MESH_OK) return rc;
+                if ((rc = run_layer_prefill(s, L, il, T, max_keys, skinny, false)) != MESH_OK) return rc;
                 continue;
             }
         }
+        // a mixture-of-experts layer with many tokens: its attention block on the matrix cores, experts below
+        bool attn_done = false;
+        if (!L.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_attn_is_kquant(L) &&
+            hp.n_embd % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0) {
+            if ((rc = run_layer_prefill(s, L, il, T, max_keys, T < PREFILL_MIN_TOKENS, true)) != MESH_OK) return rc;
+            attn_done = true;
+        }
+        if (!attn_done) {
         // q, k, v = W{q,k,v} . rms_norm(x)
         GemvArgs qa;
         qa.n_mat = 3;
@@ -722,7 +752,10 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
         aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
         aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys);
-        { ProfScope ps(s, MESH_PROF_ATTN); rc = attention(aa, T, stream); }
+        {
+            ProfScope ps(s, MESH_PROF_ATTN);
+            rc = T >= attn_mma_min_tokens() && attention_mma_supported(aa) ? attention_mma(aa, T, stream) : attention(aa, T, stream);
+        }
         if (rc != MESH_OK) return rc;
 
         // x += Wo . attn
@@ -733,21 +766,29 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
         { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(oa, stream); }
         if (rc != MESH_OK) return rc;
+        }
 
         if (!L.w_gate.present()) {
             // mixture of experts: router -> top-k -> per-(token, slot) expert FFN -> weighted sum into x
             const int ne = (int)L.gate_inp.M, k = (int)hp.n_expert_used, ffe = (int)hp.n_ff_exp;
-            GemvArgs ra2;
-            ra2.n_mat = 1;
-            ra2.mat[0] = mat_of(L.gate_inp, s->moe_logits, ne, nullptr);
-            ra2.x = s->x; ra2.ldx = E; ra2.K = E; ra2.T = T;
-            ra2.norm_w = static_cast<const float *>(L.ffn_norm.data); ra2.eps = hp.rms_eps;
-            { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ra2, stream); }
-            if (rc != MESH_OK) return rc;
             MoeRouteArgs mr;
             mr.logits = s->moe_logits; mr.mask = s->expert_mask_on ? s->expert_mask : nullptr;
             mr.ids = s->moe_ids; mr.weights = s->moe_w; mr.n_expert = ne; mr.top_k = k; mr.norm_w = 1;
-            if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
+            if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
+                // the router matrix is small and f32: logits and routing in one launch
+                ProfScope ps(s, MESH_PROF_GEMV);
+                if ((rc = moe_router_fused(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
+                                           static_cast<const float *>(L.gate_inp.data), E, s->moe_logits, T, stream)) != MESH_OK) return rc;
+            } else {
+                GemvArgs ra2;
+                ra2.n_mat = 1;
+                ra2.mat[0] = mat_of(L.gate_inp, s->moe_logits, ne, nullptr);
+                ra2.x = s->x; ra2.ldx = E; ra2.K = E; ra2.T = T;
+                ra2.norm_w = static_cast<const float *>(L.ffn_norm.data); ra2.eps = hp.rms_eps;
+                { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ra2, stream); }
+                if (rc != MESH_OK) return rc;
+                if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
+            }
             GemvArgs ea;
             ea.n_mat = 2;
             ea.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);
