@@ -23,6 +23,7 @@
 namespace mesh {
 
 constexpr int MMA_THREADS = 256, MMA_WAVES = 4, MMA_KEYS = 16;
+constexpr float MMA_RESCALE_STEP = 8.f;  // log2 units
 constexpr int MMA_VPITCH = 20;          // halfs per dim row of the transposed V tile (16 keys + padding, 8-byte aligned)
 
 typedef _Float16 mm_h8 __attribute__((ext_vector_type(8)));
@@ -37,18 +38,39 @@ __device__ __forceinline__ uint32_t mm_pack(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-// the 8 values [ds, ds + 8) of a cache row as packed f16 (quantised rows are dequantised, then rounded to f16)
-template <int TYPE, int HD>
-__device__ __forceinline__ uint4 mm_row_piece(const uint8_t *row, int ds) {
-    const KvRaw<TYPE> r = kv_load<TYPE, HD>(row, ds);
+// Bytes / nibbles -> f16 without conversions: 0x6400 | u is the half 1024 + u, so one packed subtraction of
+// 1024 + offset leaves the signed quant exactly, and one packed multiply by the block scale (an f16 in the cache)
+// gives d * q rounded to f16 -- the same value as the f32 product rounded once.
+__device__ __forceinline__ uint32_t mm_scale_pair(uint32_t biased, _Float16 bias, mm_h2 d2) {
+    const mm_h2 v = (__builtin_bit_cast(mm_h2, biased) - mm_h2{bias, bias}) * d2;
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// the 8 values a lane fetched from a cache row as packed f16 (quantised rows are dequantised in f16, exactly as above)
+template <int TYPE>
+__device__ __forceinline__ uint4 mm_piece_f16(const KvRaw<TYPE> &r) {
     if constexpr (TYPE == MESH_F16) {
         return r.v;
     } else {
-        float u[8];
-        const float d = kv_decode<TYPE>(r, u);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) u[e] = (u[e] - KvAffine<TYPE>::off) * d;
-        return make_uint4(mm_pack(u[0], u[1]), mm_pack(u[2], u[3]), mm_pack(u[4], u[5]), mm_pack(u[6], u[7]));
+        const _Float16 d = __builtin_bit_cast(_Float16, r.d);
+        const mm_h2 d2 = {d, d};
+        if constexpr (TYPE == MESH_Q8_0) {
+            const uint32_t a = r.v.x ^ 0x80808080u, b = r.v.y ^ 0x80808080u;       // int8 -> biased uint8
+            const _Float16 bias = (_Float16)(1024.f + 128.f);
+            return make_uint4(mm_scale_pair(__builtin_amdgcn_perm(0x64646464u, a, 0x04010400u), bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(0x64646464u, a, 0x04030402u), bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(0x64646464u, b, 0x04010400u), bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(0x64646464u, b, 0x04030402u), bias, d2));
+        } else {
+            // byte i of the word holds elements 2i (low nibble) and 2i + 1 (high nibble)
+            const uint32_t lo = r.v & 0x0F0F0F0Fu, hi = (r.v >> 4) & 0x0F0F0F0Fu;
+            const _Float16 bias = (_Float16)(1024.f + 8.f);
+            // pair k = elements (2k, 2k + 1) = (byte k of lo, byte k of hi); selector bytes 0-3 address hi, 4-7 address lo
+            return make_uint4(mm_scale_pair(__builtin_amdgcn_perm(lo, hi, 0x0c000c04u) | 0x64006400u, bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(lo, hi, 0x0c010c05u) | 0x64006400u, bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(lo, hi, 0x0c020c06u) | 0x64006400u, bias, d2),
+                              mm_scale_pair(__builtin_amdgcn_perm(lo, hi, 0x0c030c07u) | 0x64006400u, bias, d2));
+        }
     }
 }
 
@@ -100,16 +122,28 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
 
     _Float16 *sV = reinterpret_cast<_Float16 *>(s_raw) + wave * HD * MMA_VPITCH;
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
-    for (int kb = j0 + wave * MMA_KEYS; kb < j1; kb += MMA_WAVES * MMA_KEYS) {
-        // rows past the range are clamped to its last key and masked below
+    // what a lane fetches of a 16-key block: its key row c, dims 32*cc + 8*g .. + 8 of K and of V; rows past the range
+    // are clamped to its last key (and masked below), so the fetch of the block after the last one is harmless
+    KvRaw<KT> kraw[NC];
+    KvRaw<VT> vraw[NC];
+    auto fetch = [&](int kb) {
         int kr = kb + c;
         kr = kr < j1 ? kr : j1 - 1;
         const uint8_t *krow = a.kcache + (base + kr) * KRB, *vrow = a.vcache + (base + kr) * VRB;
+#pragma unroll
+        for (int cc = 0; cc < NC; ++cc) kraw[cc] = kv_load<KT, HD>(krow, 32 * cc + 8 * g);
+#pragma unroll
+        for (int cc = 0; cc < NC; ++cc) vraw[cc] = kv_load<VT, HD>(vrow, 32 * cc + 8 * g);
+    };
+    const int kb0 = j0 + wave * MMA_KEYS;
+    if (kb0 < j1) fetch(kb0);
+    for (int kb = kb0; kb < j1; kb += MMA_WAVES * MMA_KEYS) {
         uint4 kf[NC], vf[NC];
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) kf[cc] = mm_row_piece<KT, HD>(krow, 32 * cc + 8 * g);
+        for (int cc = 0; cc < NC; ++cc) kf[cc] = mm_piece_f16<KT>(kraw[cc]);
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) vf[cc] = mm_row_piece<VT, HD>(vrow, 32 * cc + 8 * g);
+        for (int cc = 0; cc < NC; ++cc) vf[cc] = mm_piece_f16<VT>(vraw[cc]);
+        fetch(kb + MMA_WAVES * MMA_KEYS);      // the next block's rows travel while this one is worked on
 
         // S^T = K . Q^T : register i is key kb + 4*g + i for head c
         mm_f4 s = {0.f, 0.f, 0.f, 0.f};
@@ -134,19 +168,25 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx);               // the first key of a block is always in range: finite
-        const float corr = __builtin_amdgcn_exp2f(m - m_new);
+        // The reference point m of the exponentials only moves when a score exceeds it by more than 2^RESCALE_STEP
+        // (probabilities then stay below that factor, harmless in f16 / f32), and then for the whole wave at once:
+        // the rescale of the 32 accumulator registers becomes rare instead of once per block.
+        if (__builtin_amdgcn_ballot_w64(mx > m + MMA_RESCALE_STEP) != 0) {      // first block: m = -inf
+            const float m_new = fmaxf(m, mx);
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);               // exp2(-inf) = 0 on the first block
+            l *= corr;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[db][i] *= corr;
+            m = m_new;
+        }
         float p[4], ps = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { p[i] = __builtin_amdgcn_exp2f(s[i] - m_new); ps += p[i]; }
+        for (int i = 0; i < 4; ++i) { p[i] = __builtin_amdgcn_exp2f(s[i] - m); ps += p[i]; }
         ps += __shfl_xor(ps, 16);
         ps += __shfl_xor(ps, 32);
-        l = l * corr + ps;
-        m = m_new;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[db][i] *= corr;
+        l += ps;
         const mm_u2 pu = {mm_pack(p[0], p[1]), mm_pack(p[2], p[3])};
         const mm_h4 pf = __builtin_bit_cast(mm_h4, pu);      // P^T operand: head column c, keys 4*g + j
 
