@@ -511,13 +511,14 @@ static GemvMat mat_of(const DevTensor &w, float *y, int ldy, const DevTensor *bi
     return m;
 }
 
-// batches of at least this many tokens take the matrix-core decode attention (its inputs are rounded to f16, like the
-// batched projections around it)
+// Batches of at least this many tokens take the matrix-core decode attention (Q and the probabilities rounded to f16;
+// faster at every batch size, so the default is 1).  MESH_ATTN_MMA_MIN_TOKENS raises it for callers that want the
+// all-f32 vector-ALU kernel at small batches.
 static int attn_mma_min_tokens() {
     static int v = -1;
     if (v < 0) {
         const char *e = getenv("MESH_ATTN_MMA_MIN_TOKENS");
-        v = e ? std::max(1, atoi(e)) : 5;
+        v = e ? std::max(1, atoi(e)) : 1;
     }
     return v;
 }
