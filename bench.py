@@ -204,6 +204,16 @@ def bench_stage(args):
             ses.kv_write(il, s, 0, kv, kv)
     kv_bytes_per_seq = STAGE_LAYERS * N_CTX * HK * (kv_row[kv_types[0]] + kv_row[kv_types[1]])
     stream = torch.cuda.ExternalStream(ses.stream)
+    # Burn-in, outside every timed region: the first ~10-20 thousand kernel launches of a process contain a one-time
+    # stall of ~35 ms (seen at a fixed launch count whatever kernel is running), which would otherwise land in
+    # whichever batch size happens to be measured at that moment.
+    for B in batches:
+        xb = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
+        ob = torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")
+        for _ in range(args.burn_in):
+            ses.decode_dev(xb.data_ptr(), np.full(B, N_CTX - 1, np.int32), ob.data_ptr(), ob.numel(), seq=np.arange(B, dtype=np.int32),
+                           in_fmt=m.F32, out_fmt=m.Q8_0)
+    stream.synchronize()
     results = {}
     for B in batches:
         x = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
@@ -404,6 +414,7 @@ def main():
     ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
     ap.add_argument("--kv", default="f16", choices=["f16", "q8_0/q4_0", "q4_0/q4_0"],
                     help="KV cache row types K/V (default f16: the tier the reference picks for an 8B Q4_K_M model)")
+    ap.add_argument("--burn-in", type=int, default=80, help="untimed decode steps per batch size before anything is timed")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", dest="prefill", action="store_false", help="skip the 2048-token prefill measurement")
     args = ap.parse_args()

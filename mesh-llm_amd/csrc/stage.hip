@@ -524,7 +524,9 @@ static int attn_mma_min_tokens() {
 }
 
 static int attn_splits_for(int T, int n_kv, int max_keys) {
-    int s = 512 / std::max(1, T * n_kv);
+    // one workgroup per compute unit (256 on gfx950) measured best from batch 1 to 16 with the matrix-core kernel
+    constexpr int target = 256;
+    int s = target / std::max(1, T * n_kv);
     s = std::min(s, (max_keys + 63) / 64);
     return std::max(1, std::min(s, ATTN_SPLITS_MAX));
 }
