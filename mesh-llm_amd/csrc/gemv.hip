@@ -51,6 +51,8 @@ struct GemvKernelArgs {
     const int32_t *expert_ids;
     size_t expert_stride;
     int x_div;
+    GemvRope rope;         // rope.pos / rope.seq already point at the launch's first column
+    int kind[3];
 };
 
 // Phase timestamps for tuning builds (-DMESH_GEMV_TRACE); compiled out of the product.
@@ -160,6 +162,7 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
         ka.bias[i] = a.mat[i].bias;
         ka.M[i] = a.mat[i].M;
         ka.ldy[i] = a.mat[i].ldy;
+        ka.kind[i] = a.kind[i];
         if (!(NU == 2 && i == 1)) total_rows += (a.mat[i].M + TILE_ROWS - 1) / TILE_ROWS;
     }
     const int n_mat_k = NU == 2 ? 1 : a.n_mat;      // boundaries the kernel searches
@@ -171,6 +174,7 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
     ka.eps = a.eps;
     ka.ldres = a.ldres;
     ka.epi = a.epi;
+    ka.rope = a.rope;
     const int KS = nsb < GEMV_WAVES ? nsb : GEMV_WAVES;
     ka.ks = KS;
     // tile-rows per workgroup: spread over the CUs, bounded by the LDS partial buffer
@@ -211,6 +215,7 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
         int nb = left >= 4 ? 4 : left;      // 3 columns have a kernel of their own: no second pass over the weights
         while (nb > 1 && dot_smem_bytes(type, nb, a.K, rows_max, KS, NU) > LDS_LIMIT) --nb;
         GemvKernelArgs kb = ka;
+        if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
         kb.x = a.x + (size_t)t * a.ldx;
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
         for (int i = 0; i < a.n_mat; ++i)
@@ -256,6 +261,7 @@ static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream)
         auto need = [&](int n) { return std::max(dot_smem_bytes(MESH_Q4_K, n, a4.K, p4.rows_max, p4.KS, 1), dot_smem_bytes(MESH_Q6_K, n, a6.K, p6.rows_max, p6.KS, 1)); };
         while (nb > 1 && need(nb) > LDS_LIMIT) --nb;
         GemvKernelArgs k4 = p4.ka, k6 = p6.ka;
+        if (k4.rope.pos) { k4.rope.pos += t; k4.rope.seq += t; k6.rope.pos += t; k6.rope.seq += t; }
         k4.x = k6.x = a4.x + (size_t)t * a4.ldx;
         for (int i = 0; i < a4.n_mat; ++i) k4.y[i] = a4.mat[i].y + (size_t)t * a4.mat[i].ldy;
         for (int i = 0; i < a6.n_mat; ++i) k6.y[i] = a6.mat[i].y + (size_t)t * a6.mat[i].ldy;
@@ -269,7 +275,15 @@ static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream)
     return MESH_OK;
 }
 
+bool gemv_can_fuse_rope(const GemvArgs &a) {
+    if (!a.rope.pos || a.epi != EPI_STORE || a.expert_ids || a.rope.head_dim % 2 || a.rope.n_rot % 2) return false;
+    for (int i = 0; i < a.n_mat; ++i)
+        if (a.mat[i].type != MESH_Q4_K && a.mat[i].type != MESH_Q6_K) return false;
+    return true;
+}
+
 int gemv(const GemvArgs &a, hipStream_t stream) {
+    if (a.rope.pos && !gemv_can_fuse_rope(a)) return fail(MESH_ERR_INVALID, "gemv: rope epilogue asked for a launch that cannot carry it");
     if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.K <= 0 || a.T < 0)
         return fail(MESH_ERR_INVALID, "gemv: bad arguments (n_mat %d, K %d, T %d)", a.n_mat, a.K, a.T);
     if (a.epi == EPI_SWIGLU && a.n_mat != 2) return fail(MESH_ERR_INVALID, "gemv: swiglu needs exactly gate and up");
@@ -298,8 +312,8 @@ int gemv(const GemvArgs &a, hipStream_t stream) {
         a4.n_mat = a6.n_mat = 0;
         bool kq_only = a.epi == EPI_STORE && !a.expert_ids;
         for (int i = 0; i < a.n_mat && kq_only; ++i) {
-            if (a.mat[i].type == MESH_Q4_K) a4.mat[a4.n_mat++] = a.mat[i];
-            else if (a.mat[i].type == MESH_Q6_K) a6.mat[a6.n_mat++] = a.mat[i];
+            if (a.mat[i].type == MESH_Q4_K) { a4.kind[a4.n_mat] = a.kind[i]; a4.mat[a4.n_mat++] = a.mat[i]; }
+            else if (a.mat[i].type == MESH_Q6_K) { a6.kind[a6.n_mat] = a.kind[i]; a6.mat[a6.n_mat++] = a.mat[i]; }
             else kq_only = false;
         }
         if (kq_only && a4.n_mat > 0 && a6.n_mat > 0) return gemv_dual(a4, a6, stream);

@@ -46,6 +46,17 @@ struct GemvMat {
     const float *bias = nullptr;
 };
 
+// RoPE + KV append in the epilogue of a q/k/v launch (NORM pairing: a pair's two rows are neighbours, so they live in
+// one 16-row tile): q rows are rotated before they are stored, k rows are rotated and stored as f16 in the K cache
+// at the token's position, v rows go to the V cache.  Same arithmetic, hence the same bits, as rope_kv_kernel.
+enum { GEMV_KIND_PLAIN = 0, GEMV_KIND_Q = 1, GEMV_KIND_K = 2, GEMV_KIND_V = 3 };
+struct GemvRope {
+    const int32_t *pos = nullptr, *seq = nullptr;      // device, [T]; pos == nullptr: no fusion
+    const float *inv_freq = nullptr;
+    uint16_t *kcache = nullptr, *vcache = nullptr;     // this layer's f16 rows [n_seq][n_kv][n_ctx][head_dim]
+    int head_dim = 0, n_rot = 0, n_kv = 0, n_ctx = 0;
+};
+
 struct GemvArgs {
     GemvMat mat[3];
     int n_mat = 1;             // matrices sharing x (q, k, v); for EPI_SWIGLU exactly 2, written through mat[0].y
@@ -64,7 +75,12 @@ struct GemvArgs {
     const int32_t *expert_ids = nullptr;
     int n_pairs = 0;
     int x_div = 1;
+    // Fused RoPE / KV append: kind[i] says what matrix i produces (tiled K-quant matrices, EPI_STORE, no experts only)
+    GemvRope rope;
+    int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
 };
+// whether gemv() will honour a.rope for this argument set (otherwise the caller runs rope_kv itself)
+bool gemv_can_fuse_rope(const GemvArgs &a);
 
 int gemv(const GemvArgs &a, hipStream_t stream);
 

@@ -443,6 +443,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const HParams &hp = st->hp;
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
+    if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
     s->v_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->v_type, (int)hp.head_dim);
@@ -731,6 +732,18 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = s->x; qa.ldx = E; qa.K = E; qa.T = T;
         qa.norm_w = static_cast<const float *>(L.attn_norm.data); qa.eps = hp.rms_eps;
+        // neighbouring-pair RoPE into an f16 cache without per-head norms: rotation and KV append ride in the
+        // projection's epilogue (the same arithmetic as rope_kv_kernel), one launch fewer per layer
+        bool rope_fused = false;
+        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() && !L.k_norm.present()) {
+            qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;
+            qa.rope.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
+            qa.rope.vcache = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
+            qa.rope.head_dim = (int)hp.head_dim; qa.rope.n_rot = (int)hp.n_rot; qa.rope.n_kv = (int)hp.n_head_kv; qa.rope.n_ctx = st->n_ctx;
+            qa.kind[0] = GEMV_KIND_Q; qa.kind[1] = GEMV_KIND_K; qa.kind[2] = GEMV_KIND_V;
+            rope_fused = gemv_can_fuse_rope(qa);
+            if (!rope_fused) qa.rope = GemvRope{};
+        }
         { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(qa, stream); }
         if (rc != MESH_OK) return rc;
 
@@ -745,8 +758,10 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         ra.eps = hp.rms_eps;
         ra.n_head = (int)hp.n_head; ra.n_kv = (int)hp.n_head_kv; ra.head_dim = (int)hp.head_dim;
         ra.n_rot = (int)hp.n_rot; ra.rope_mode = (int)hp.rope_mode; ra.n_ctx = st->n_ctx;
-        { ProfScope ps(s, MESH_PROF_ROPE); rc = rope_kv(ra, T, stream); }
-        if (rc != MESH_OK) return rc;
+        if (!rope_fused) {
+            ProfScope ps(s, MESH_PROF_ROPE);
+            if ((rc = rope_kv(ra, T, stream)) != MESH_OK) return rc;
+        }
 
         AttnArgs aa;
         aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.k_type = st->k_type; aa.v_type = st->v_type; aa.pos = s->d_pos; aa.seq = s->d_seq;

@@ -73,6 +73,7 @@ struct mesh_session {
     hipStream_t stream = nullptr;
     // KV cache: per local layer, K and V as f16 [n_seq_max][n_head_kv][n_ctx][head_dim]
     uint8_t *kcache = nullptr, *vcache = nullptr;       // rows of the stage's k_type / v_type (kv_cache.hpp)
+    bool rope_in_gemv = true;        // MESH_GEMV_ROPE=0 at session creation keeps RoPE / KV append in their own kernel
     size_t k_layer_bytes = 0, v_layer_bytes = 0;
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;

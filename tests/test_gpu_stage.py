@@ -341,3 +341,35 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         assert rel_l2(got, ref) <= 3e-3, T
         assert rel_l2(got, alt) <= 3e-3, T
     ses.close(); ses4.close(); st.close()
+
+
+def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
+    """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
+    1-4 tokens; with MESH_GEMV_ROPE=0 the separate kernel does them.  Outputs and cache contents must agree bit
+    for bit (the arithmetic is the same), through the single-type and the mixed q4_K/q6_K launch, and partial rotation."""
+    for name, layers in (("llama3-8b", [3, 4]), ("tiny-llama", [0, 1])):
+        m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=64, n_seq=4, n_batch=4)
+        E = cfg["n_embd"]
+        rng = np.random.Generator(np.random.PCG64(3))
+        xs = [rng.standard_normal((T, E)).astype(np.float32) for T in (1, 2, 3, 4, 1)]
+        runs = []
+        for flag in ("1", "0"):
+            monkeypatch.setenv("MESH_GEMV_ROPE", flag)
+            ses = st.session()
+            outs, nxt = [], [0, 0, 0, 0]
+            for x in xs:
+                T = x.shape[0]
+                seqs = list(range(T))
+                pos = [nxt[q] for q in seqs]
+                for q in seqs:
+                    nxt[q] += 1
+                outs.append(ses.decode(x, pos, seq=seqs).copy())
+            kv = [ses.kv_read(il, q, 0, 5) for il in layers for q in range(4)]
+            runs.append((outs, kv))
+            ses.close()
+        for a, b in zip(runs[0][0], runs[1][0]):
+            assert np.array_equal(a, b)
+        for (ka, va), (kb, vb) in zip(runs[0][1], runs[1][1]):
+            assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+            assert ka.any() and va.any()
+        st.close()
