@@ -186,6 +186,10 @@ int mesh_session_synchronize(mesh_session *session);
  * session creation turns that kernel on).  -1 for a null session.  No counterpart in the reference; it lets tests and
  * benchmarks tell which path produced a result. */
 int64_t mesh_session_persistent_steps(const mesh_session *session);
+/* Number of decode steps of this session whose layer launches were replayed from a captured HIP graph (batches of up to
+ * 32 tokens, from the third call with the same token count and KV split count on; environment MESH_STAGE_GRAPHS=1 at
+ * session creation turns graphs on: they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
+int64_t mesh_session_graph_replays(const mesh_session *session);
 
 /* Per-kernel-class timing of a session, measured with HIP events recorded on the session's stream around each
  * launch.  Off by default (it adds two event records per launch).  Kinds index the arrays below. */

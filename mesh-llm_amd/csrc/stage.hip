@@ -444,6 +444,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
+    if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
     s->v_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->v_type, (int)hp.head_dim);
@@ -865,6 +866,47 @@ static int validate_batch(const mesh_session *s, const mesh_batch *b, int *max_k
     return MESH_OK;
 }
 
+// run_layers, replayed from a captured graph for decode-sized batches.  The launches depend on T, on the KV split count
+// (a function of the deepest position) and on whether an expert mask is set; everything else they read is device
+// memory at fixed addresses (hidden state, positions, caches).  The first use of a key runs eagerly (which also
+// finishes every lazy initialisation), the second is captured, later ones are replays.
+constexpr int GRAPH_MAX_TOKENS = 32;
+constexpr size_t GRAPH_MAX_ENTRIES = 96;
+static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
+    if (!s->graphs_on || s->profile || T > GRAPH_MAX_TOKENS) return run_layers(s, T, max_keys);
+    const mesh_stage *st = s->stage;
+    const int n_splits = attn_splits_for(T, (int)st->hp.n_head_kv, max_keys);
+    const uint64_t key = (uint64_t)T | ((uint64_t)n_splits << 8) | ((uint64_t)(s->expert_mask_on ? 1 : 0) << 20);
+    auto it = s->graphs.find(key);
+    if (it == s->graphs.end()) {
+        if (s->graphs.size() >= GRAPH_MAX_ENTRIES) return run_layers(s, T, max_keys);
+        it = s->graphs.emplace(key, mesh_session::LayerGraph{}).first;
+    }
+    mesh_session::LayerGraph &e = it->second;
+    if (!e.exec) {
+        if (e.uses++ == 0) return run_layers(s, T, max_keys);
+        if (hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+            (void)hipGetLastError();
+            s->graphs_on = false;
+            return run_layers(s, T, max_keys);
+        }
+        const int rc = run_layers(s, T, max_keys);           // records, does not execute
+        hipGraph_t g = nullptr;
+        hipError_t err = hipStreamEndCapture(s->stream, &g);
+        if (rc == MESH_OK && err == hipSuccess && g) err = hipGraphInstantiate(&e.exec, g, nullptr, nullptr, 0);
+        if (g) (void)hipGraphDestroy(g);
+        if (rc != MESH_OK || err != hipSuccess || !e.exec) {
+            (void)hipGetLastError();
+            e.exec = nullptr;
+            s->graphs_on = false;
+            return rc != MESH_OK ? rc : run_layers(s, T, max_keys);      // nothing has run yet
+        }
+    }
+    MESH_HIP_TRY(hipGraphLaunch(e.exec, s->stream));
+    ++s->graph_replays;
+    return MESH_OK;
+}
+
 int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int in_fmt, void *d_out, int out_fmt,
                      size_t out_cap, size_t *out_len) {
     if (!s || !d_in || !d_out) return fail(MESH_ERR_INVALID, "mesh_stage_decode: null argument");
@@ -918,7 +960,7 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
     }
     { ProfScope ps(s, MESH_PROF_CODEC); rc = act_unpack_dev(in_fmt, d_in, s->x, (int64_t)T * hp.n_embd, stream); }
     if (rc != MESH_OK) return rc;
-    if ((rc = run_layers(s, T, max_keys)) != MESH_OK) return rc;
+    if ((rc = run_layers_graphed(s, T, max_keys)) != MESH_OK) return rc;
     if (logits_out) {
         GemvArgs la;
         la.n_mat = 1;
@@ -988,6 +1030,8 @@ mesh_session::~mesh_session() {
     for (hipEvent_t e : prof_events) (void)hipEventDestroy(e);
     for (void *p : allocations) (void)hipFree(p);
     if (mega.pool && stage) mesh::mega_pool_release(mega.pool, mega.pool_bytes, stage->device);
+    for (auto &kv : graphs)
+        if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
     if (h_meta) (void)hipHostFree(h_meta);
     if (h_io) (void)hipHostFree(h_io);
     if (stream) (void)hipStreamDestroy(stream);

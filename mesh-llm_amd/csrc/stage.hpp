@@ -2,6 +2,7 @@
 #pragma once
 
 #include <memory>
+#include <unordered_map>
 #include <string>
 #include <vector>
 
@@ -114,6 +115,13 @@ struct mesh_session {
     std::vector<void *> allocations;
     // optional per-kernel-class timing (HIP events on `stream` around every launch group)
     bool profile = false;
+    // Captured launch sequences of run_layers, one per (token count, KV split count, expert mask) seen: a decode step
+    // is ~80 dependent launches; replaying them as a graph takes the host out of their submission (about 0.3 ms of CPU
+    // per step).  Off by default: on the measured system the stream is GPU-bound and the step time does not change.
+    struct LayerGraph { hipGraphExec_t exec = nullptr; int uses = 0; };
+    std::unordered_map<uint64_t, LayerGraph> graphs;
+    int64_t graph_replays = 0;
+    bool graphs_on = false;          // MESH_STAGE_GRAPHS=1 at session creation turns them on; a failed capture turns them off
     std::vector<hipEvent_t> prof_events;      // pairs (begin, end)
     std::vector<int> prof_kinds;
     size_t prof_used = 0;

@@ -373,3 +373,38 @@ def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
             assert np.array_equal(ka, kb) and np.array_equal(va, vb)
             assert ka.any() and va.any()
         st.close()
+
+
+@pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-moe", [0, 1])])
+def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers):
+    """Decode-sized batches replay their layer launches from a captured graph (first use of a shape eager, second
+    captured, then replays).  Every replay must give the bits the eager launches give: two sessions, graphs on and
+    off, walk the same sequence of steps -- repeated shapes, other shapes and host synchronisations in between, KV
+    depth growing past a change of the split count."""
+    m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=6, n_batch=8)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(17))
+    plan = [1, 1, 1, 4, 1, 4, 6, 1, 4, 6, 6, 1] + [1] * 70 + [4, 4, 1, 6]
+    xs = [rng.standard_normal((T, E)).astype(np.float32) for T in plan]
+    runs = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("MESH_STAGE_GRAPHS", flag)
+        ses = st.session()
+        nxt = [0] * 6
+        outs = []
+        for x in xs:
+            T = x.shape[0]
+            seqs = list(range(T))
+            pos = [nxt[q] for q in seqs]
+            for q in seqs:
+                nxt[q] += 1
+            outs.append(ses.decode(x, pos, seq=seqs).copy())      # the host-pointer entry synchronises after every call
+        runs.append((outs, [ses.kv_read(layers[0], q, 0, 8) for q in range(6)]))
+        # shapes seen at least twice were captured and replayed; with graphs off nothing is
+        assert (ses.graph_replays > 40) if flag == "1" else (ses.graph_replays == 0), ses.graph_replays
+        ses.close()
+    for i, (a, b) in enumerate(zip(runs[0][0], runs[1][0])):
+        assert np.array_equal(a, b), "step %d (T=%d)" % (i, plan[i])
+    for (ka, va), (kb, vb) in zip(runs[0][1], runs[1][1]):
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+    st.close()
