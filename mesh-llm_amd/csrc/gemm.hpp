@@ -33,6 +33,9 @@ struct SkinnyArgs {
     const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y
     int ldres = 0;
     _Float16 *y16 = nullptr;         // optional f16 copy of matrix 0's output in the k8-major layout (feeds the next GEMM)
+    // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
+    GemvRope rope;
+    int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
 };
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion

@@ -61,6 +61,8 @@ struct SkinnyKernelArgs {
     _Float16 *y16;                // optional f16 copy of the output (matrix 0): k8-major block with M16 rows as its k
     int M16;
     int ks;                       // waves along K
+    GemvRope rope;                // rope.pos / rope.seq point at the launch's first column
+    int kind[3];
 };
 
 // four bytes (values < 64) -> four f16 holding 1024 + value
@@ -312,6 +314,28 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
             if (NU == 2) s1 += red[((((size_t)k2 * rows_here + j) * NU + 1) * 16 + r) * 16 + t];
         }
         if (a.bias[mi]) s0 += a.bias[mi][row];
+        if (NU == 1 && a.rope.pos && a.kind[mi] != GEMV_KIND_PLAIN) {
+            // q / k / v row of a token (see gemv.hpp): rotate q and k with the neighbouring row, k and v go to the cache
+            const int kind = a.kind[mi], hd = a.rope.head_dim;
+            const int head = row / hd, dd = row - head * hd;
+            const int pos = a.rope.pos[t];
+            float val = s0;
+            if (kind != GEMV_KIND_V && dd < a.rope.n_rot) {
+                float sp = 0.f;
+                for (int k2 = 0; k2 < KS; ++k2) sp += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + (r ^ 1)) * 16 + t];
+                if (a.bias[mi]) sp += a.bias[mi][row ^ 1];
+                float sn, cs;
+                sincosf((float)pos * a.rope.inv_freq[dd >> 1], &sn, &cs);
+                val = (dd & 1) ? sp * sn + s0 * cs : s0 * cs - sp * sn;
+            }
+            if (kind == GEMV_KIND_Q) {
+                a.y[mi][(size_t)t * a.ldy[mi] + row] = val;
+            } else {
+                uint16_t *cache = kind == GEMV_KIND_K ? a.rope.kcache : a.rope.vcache;
+                cache[(((size_t)a.rope.seq[t] * a.rope.n_kv + head) * a.rope.n_ctx + pos) * hd + dd] = f32_to_f16_bits(val);
+            }
+            continue;
+        }
         float out;
         if (NU == 2) {
             if (a.bias[1]) s1 += a.bias[1][row];
@@ -372,12 +396,14 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
         ka.bias[i] = a.mat[i].bias;
         ka.M[i] = a.mat[i].M;
         ka.ldy[i] = a.mat[i].ldy;
+        ka.kind[i] = a.kind[i];
         if (!(NU == 2 && i == 1)) total_rows += (a.mat[i].M + TILE_ROWS - 1) / TILE_ROWS;
     }
     const int n_bound = NU == 2 ? 1 : a.n_mat;          // matrix boundaries the kernel searches
     for (int i = n_bound; i < 4; ++i) ka.tile_begin[i] = total_rows;
     ka.K = a.K;
     ka.ldres = a.ldres; ka.epi = a.epi;
+    ka.rope = a.rope;
     ka.M16 = a.mat[0].M;
     const int KS = nsb < SK_WAVES ? nsb : SK_WAVES, RS = SK_WAVES / KS;
     ka.ks = KS;
@@ -395,6 +421,7 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     for (int t = 0; t < a.T; t += SK_NT) {
         SkinnyKernelArgs kb = ka;
         kb.T = std::min(SK_NT, a.T - t);
+        if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
         kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
         kb.y16 = a.y16 ? a.y16 + (size_t)t * a.mat[0].M : nullptr;
@@ -469,6 +496,7 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
     if (a.epi == EPI_SWIGLU && (a.n_mat != 2 || a.mat[0].M != a.mat[1].M || a.mat[0].type != a.mat[1].type))
         return fail(MESH_ERR_INVALID, "gemm_skinny: SwiGLU needs a gate and an up matrix of equal shape and type");
     if (a.epi == EPI_RESIDUAL && !a.residual) return fail(MESH_ERR_INVALID, "gemm_skinny: residual epilogue without residual");
+    if (a.rope.pos && (a.epi != EPI_STORE || a.rope.head_dim % 2 || a.rope.n_rot % 2)) return fail(MESH_ERR_INVALID, "gemm_skinny: rope epilogue needs a plain store");
     for (int i = 0; i < a.n_mat; ++i) {
         if (!a.mat[i].W || a.mat[i].M <= 0 || !type_is_tiled(a.mat[i].type)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d is not a tiled K-quant", i);
         if (!a.mat[i].y && !(i == 1 && a.epi == EPI_SWIGLU) && !(i == 0 && a.y16)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d has no output", i);
@@ -483,7 +511,7 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
         while (j < a.n_mat && a.mat[j].type == a.mat[i].type) ++j;
         SkinnyArgs sub = a;
         sub.n_mat = j - i;
-        for (int k2 = 0; k2 < sub.n_mat; ++k2) sub.mat[k2] = a.mat[i + k2];
+        for (int k2 = 0; k2 < sub.n_mat; ++k2) { sub.mat[k2] = a.mat[i + k2]; sub.kind[k2] = a.kind[i + k2]; }
         sub.y16 = i == 0 ? a.y16 : nullptr;
         int rc = skinny_one_type(sub, stream);
         if (rc != MESH_OK) return rc;

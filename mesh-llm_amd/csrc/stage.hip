@@ -602,6 +602,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
+    bool rope_fused = false;
     if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
@@ -612,6 +613,15 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = xn; qa.K = E; qa.T = T;
+        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+            !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
+            qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;
+            qa.rope.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
+            qa.rope.vcache = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
+            qa.rope.head_dim = (int)hp.head_dim; qa.rope.n_rot = (int)hp.n_rot; qa.rope.n_kv = (int)hp.n_head_kv; qa.rope.n_ctx = st->n_ctx;
+            qa.kind[0] = GEMV_KIND_Q; qa.kind[1] = GEMV_KIND_K; qa.kind[2] = GEMV_KIND_V;
+            rope_fused = true;
+        }
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
     } else {
@@ -631,8 +641,10 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     ra.eps = hp.rms_eps;
     ra.n_head = (int)hp.n_head; ra.n_kv = (int)hp.n_head_kv; ra.head_dim = (int)hp.head_dim;
     ra.n_rot = (int)hp.n_rot; ra.rope_mode = (int)hp.rope_mode; ra.n_ctx = st->n_ctx;
-    { ProfScope ps(s, MESH_PROF_ROPE); rc = rope_kv(ra, T, stream); }
-    if (rc != MESH_OK) return rc;
+    if (!rope_fused) {
+        ProfScope ps(s, MESH_PROF_ROPE);
+        if ((rc = rope_kv(ra, T, stream)) != MESH_OK) return rc;
+    }
     AttnArgs aa;
     aa.q = s->q; aa.kcache = ra.kcache; aa.vcache = ra.vcache; aa.k_type = st->k_type; aa.v_type = st->v_type; aa.pos = s->d_pos; aa.seq = s->d_seq;
     aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = s->attn;

@@ -345,18 +345,19 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
 
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
     """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
-    1-4 tokens; with MESH_GEMV_ROPE=0 the separate kernel does them.  Outputs and cache contents must agree bit
-    for bit (the arithmetic is the same), through the single-type and the mixed q4_K/q6_K launch, and partial rotation."""
+    1-4 tokens (mat-vec kernels) and of 5+ tokens (batched MFMA GEMM); with MESH_GEMV_ROPE=0 the separate kernel does
+    them.  Outputs and cache contents must agree bit for bit (the arithmetic is the same), through the single-type
+    and the mixed q4_K/q6_K launches."""
     for name, layers in (("llama3-8b", [3, 4]), ("tiny-llama", [0, 1])):
-        m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=64, n_seq=4, n_batch=4)
+        m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=64, n_seq=9, n_batch=16)
         E = cfg["n_embd"]
         rng = np.random.Generator(np.random.PCG64(3))
-        xs = [rng.standard_normal((T, E)).astype(np.float32) for T in (1, 2, 3, 4, 1)]
+        xs = [rng.standard_normal((T, E)).astype(np.float32) for T in (1, 2, 3, 4, 1, 6, 9, 5)]
         runs = []
         for flag in ("1", "0"):
             monkeypatch.setenv("MESH_GEMV_ROPE", flag)
             ses = st.session()
-            outs, nxt = [], [0, 0, 0, 0]
+            outs, nxt = [], [0] * 9
             for x in xs:
                 T = x.shape[0]
                 seqs = list(range(T))
@@ -364,7 +365,7 @@ def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
                 for q in seqs:
                     nxt[q] += 1
                 outs.append(ses.decode(x, pos, seq=seqs).copy())
-            kv = [ses.kv_read(il, q, 0, 5) for il in layers for q in range(4)]
+            kv = [ses.kv_read(il, q, 0, 8) for il in layers for q in range(9)]
             runs.append((outs, kv))
             ses.close()
         for a, b in zip(runs[0][0], runs[1][0]):
