@@ -280,7 +280,12 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(AttnArgs a) {
         num = fmaf(pp[(size_t)s2 * a.head_dim], w, num);
         den = fmaf(s_l[s2], w, den);
     }
-    a.out[row * a.head_dim + dd] = num / den;
+    if (a.out16_k8) {
+        const size_t kk = (size_t)h * a.head_dim + dd, KK = (size_t)a.n_head * a.head_dim;
+        a.out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(num / den);
+    } else {
+        a.out[row * a.head_dim + dd] = num / den;
+    }
 }
 
 template <int HD, int KT, int VT>

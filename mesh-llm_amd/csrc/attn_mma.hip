@@ -225,7 +225,12 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
         }
         const size_t row = (size_t)t * a.n_head + (size_t)kvh * G + h;
         if (single) {
-            a.out[row * HD + dd] = sum / ll;
+            if (a.out16_k8) {
+                const size_t kk = ((size_t)kvh * G + h) * HD + dd, KK = (size_t)a.n_head * HD;
+                a.out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(sum / ll);
+            } else {
+                a.out[row * HD + dd] = sum / ll;
+            }
         } else {
             a.part[(row * a.n_splits + split) * HD + dd] = sum;
             if (dd == 0) {

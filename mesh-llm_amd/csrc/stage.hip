@@ -474,6 +474,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
         const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
+        MESH_HIP_TRY(hipMemsetAsync(p, 0, B16 * std::max<size_t>(hp.n_embd, QD) * 2, s->stream));     // unused token columns stay finite
         if (hp.n_ff > 0) {
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
@@ -602,7 +603,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
-    bool rope_fused = false;
+    bool rope_fused = false, attn_is_k8 = false;
     if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
@@ -655,11 +656,14 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     {
         ProfScope ps(s, MESH_PROF_ATTN);
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
-        else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) rc = attention_mma(aa, T, stream);
-        else rc = attention(aa, T, stream);
+        else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
+            if (skinny) { aa.out16_k8 = xn; attn_is_k8 = true; }     // straight into the output projection's input layout
+            rc = attention_mma(aa, T, stream);
+        } else rc = attention(aa, T, stream);
     }
     if (rc != MESH_OK) return rc;
-    if (skinny) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
+    if (attn_is_k8) rc = MESH_OK;
+    else if (skinny) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
     else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
