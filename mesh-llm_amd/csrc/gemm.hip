@@ -23,7 +23,7 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int GM = 128, GN = 128, GK = 64;     // workgroup tile: weight rows x tokens x k-step
 constexpr int LDS_LD = GK + 8;                 // f16 elements per LDS row (16-byte pad against bank conflicts)
-constexpr int GEMM_THREADS = 256;
+constexpr int GEMM_THREADS = 512;              // 4 matrix-core waves + 4 staging waves
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
@@ -113,19 +113,74 @@ template <> struct RawSub<MESH_Q6_K> {
     }
 };
 
-// Software pipeline: while the matrix cores work on LDS stage kc & 1, the staging threads hold the raw weight
-// bytes and activations of step kc + 1 in registers (loads in flight), then dequantise them into the other stage.
+// Role split: waves 0-3 only multiply (each a 64 x 64 corner of the tile out of LDS stage kc & 1), waves 4-7 only
+// stage (fetch the raw weight bytes and activations of step kc + 2, dequantise step kc + 1 into the other LDS
+// stage).  A SIMD then holds one wave of each kind per workgroup, and the dequantisation (vector ALU) of one runs
+// while the MFMAs (matrix core) of the other execute -- in one wave doing both, the ~110 dequant instructions of
+// a step only start once its 16 MFMAs have been issued, and the four waves move in lockstep between barriers.
 template <int TYPE>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     extern __shared__ __align__(16) _Float16 gemm_smem[];
     _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
     _Float16 *Xs = gemm_smem + 2 * GM * LDS_LD;                // [2][GN][LDS_LD]
     constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = blockIdx.x * GM, t0 = blockIdx.y * GN;
     const int nsb = a.K / QK_K, n_steps = a.K / GK;
-    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;     // wave's 64 x 64 corner of the tile
 
+    if (wave >= 4) {
+        // ---- staging waves: thread s (0..255): weights -- row s/2, sub-block half s%2; activations -- token s/2, 32 elements s%2
+        const int st = tid - 256;
+        const int srow = st >> 1, sh = st & 1;
+        const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
+        const bool wlive = wrow < a.M_pad;
+        const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
+        const int tok = t0 + srow;
+        const bool xlive = tok < a.T;
+        const _Float16 *xrow = a.X + (size_t)(xlive ? tok : 0) * a.ldx + 32 * sh;
+        RawSub<TYPE> rw[2];
+        uint4 rx[2][4];
+        auto fetch = [&](int kc, RawSub<TYPE> &w, uint4 (&x)[4]) {
+            w.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
+            const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[i] = s4[i];
+        };
+        auto stage = [&](int kc, int buf, const RawSub<TYPE> &w, const uint4 (&x)[4]) {
+            _Float16 *wdst = Ws + (buf * GM + srow) * LDS_LD + 32 * sh;
+            if (wlive) {
+                w.store(kc & 3, sh, wdst);
+            } else {
+                uint4 *d4 = reinterpret_cast<uint4 *>(wdst);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
+            }
+            uint4 *x4 = reinterpret_cast<uint4 *>(Xs + (buf * GN + srow) * LDS_LD + 32 * sh);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x4[i] = xlive ? x[i] : make_uint4(0, 0, 0, 0);
+        };
+        fetch(0, rw[0], rx[0]);
+        fetch(n_steps > 1 ? 1 : 0, rw[1], rx[1]);
+        stage(0, 0, rw[0], rx[0]);
+        __syncthreads();
+        // step kc (its slot parity = kc & 1): the slot of step kc was staged already -> refill it with step kc + 2;
+        // then dequantise step kc + 1 (the other slot) into the LDS stage the multiplying waves are not reading
+        for (int kc0 = 0; kc0 < n_steps; kc0 += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int kc = kc0 + u;
+                if (kc >= n_steps) break;
+                fetch(kc + 2 < n_steps ? kc + 2 : n_steps - 1, rw[u], rx[u]);
+                if (kc + 1 < n_steps) stage(kc + 1, u ^ 1, rw[u ^ 1], rx[u ^ 1]);
+                __syncthreads();
+            }
+        }
+        return;
+    }
+
+    // ---- multiplying waves
+    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;     // wave's 64 x 64 corner of the tile
     float16v acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -133,45 +188,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    // staging roles: weights -- row tid/2, sub-block half tid%2; activations -- token tid/2, 32 elements tid%2
-    const int srow = tid >> 1, sh = tid & 1;
-    const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
-    const bool wlive = wrow < a.M_pad;
-    const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
-    const int tok = t0 + srow;
-    const bool xlive = tok < a.T;
-    const _Float16 *xrow = a.X + (size_t)(xlive ? tok : 0) * a.ldx + 32 * sh;
-
-    RawSub<TYPE> rw;
-    uint4 rx[4];
-    auto fetch = [&](int kc) {
-        rw.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
-        const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rx[i] = s4[i];
-    };
-    auto stage = [&](int kc, int buf) {
-        _Float16 *wdst = Ws + (buf * GM + srow) * LDS_LD + 32 * sh;
-        if (wlive) {
-            rw.store(kc & 3, sh, wdst);
-        } else {
-            uint4 *d4 = reinterpret_cast<uint4 *>(wdst);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
-        }
-        uint4 *x4 = reinterpret_cast<uint4 *>(Xs + (buf * GN + srow) * LDS_LD + 32 * sh);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) x4[i] = xlive ? rx[i] : make_uint4(0, 0, 0, 0);
-    };
-
-    fetch(0);
-    stage(0, 0);
     __syncthreads();
     for (int kc = 0; kc < n_steps; ++kc) {
         const int buf = kc & 1;
-        const bool more = kc + 1 < n_steps;
-        if (more) fetch(kc + 1);
         const _Float16 *Wb = Ws + buf * GM * LDS_LD, *Xb = Xs + buf * GN * LDS_LD;
 #pragma unroll
         for (int ks = 0; ks < GK / 16; ++ks) {
@@ -186,7 +205,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
-        if (more) stage(kc + 1, buf ^ 1);
         __syncthreads();
     }
 
