@@ -302,7 +302,7 @@ def bench_stage(args):
 SHAPES = {
     "c4": dict(model="qwen2.5-32b", layers=32, n_ctx=8192, batches=[1, 8, 32], prefill=4096, n_expert_local=None, kv="q8_0/q4_0",
                metric="stage decode tok/s @32B Q4_K_M, layers 0-31 of 64"),
-    "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=0, n_expert_local=64, kv="q8_0/q4_0",
+    "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=1024, n_expert_local=64, kv="q8_0/q4_0",
                metric="expert-shard decode tok/s @Qwen3-30B-A3B Q4_K_M, 64 of 128 experts, batch 16"),
 }
 
@@ -387,7 +387,8 @@ def bench_shape(args):
             ses.decode_dev(xp.data_ptr(), ppos, outp.data_ptr(), outp.numel(), in_fmt=m.F32, out_fmt=m.Q8_0)
 
         pms, _ = time_on_stream(torch, stream, pstep, 2, 1)
-        H, FF = cfg["n_head"], cfg["n_ff"]
+        H = cfg["n_head"]
+        FF = cfg["n_ff_exp"] * cfg["n_expert_used"] if cfg.get("n_expert") else cfg["n_ff"]      # FFN rows a token passes through
         mm_flop = 2.0 * T * L * (E * H * HD * 2 + E * HK * HD * 2 + 3 * E * FF)
         prefill = {"tokens": T, "ms": round(pms, 2), "tok_s": round(T * 1e3 / pms, 1), "matmul_TFLOP": round(mm_flop / 1e12, 2),
                    "matmul_TFLOPs_over_whole_step": round(mm_flop / pms / 1e9, 1)}

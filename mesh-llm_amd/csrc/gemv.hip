@@ -51,6 +51,8 @@ struct GemvKernelArgs {
     const int32_t *expert_ids;
     size_t expert_stride;
     int x_div;
+    // pairs grouped by expert: blockIdx.y = work item (gemv.hpp: MOE_ITEM_INTS int32 each); items past *n_items do nothing
+    const int32_t *items, *n_items;
     GemvRope rope;         // rope.pos / rope.seq already point at the launch's first column
     int kind[3];
 };
@@ -58,13 +60,16 @@ struct GemvKernelArgs {
 // Phase timestamps for tuning builds (-DMESH_GEMV_TRACE); compiled out of the product.
 #ifdef MESH_GEMV_TRACE
 __device__ long long *g_gemv_trace = nullptr;
-extern "C" int mesh_debug_set_gemv_trace(long long *p) {
+__device__ int g_gemv_trace_sel = -1;      // -1: every launch; else only kernels with (GROUPED ? 1 : 0) | (NU == 2 ? 2 : 0) | (expert_ids ? 4 : 0) == sel
+extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
+    if (hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace_sel), &sel, sizeof sel) != hipSuccess) return -2;
     return hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace), &p, sizeof p) == hipSuccess ? 0 : -2;
 }
 #define GEMV_MARK(k)                                                                              \
     do {                                                                                          \
-        if (g_gemv_trace && (threadIdx.x & 63) == 0)                                              \
-            g_gemv_trace[((size_t)blockIdx.x * GEMV_WAVES + (threadIdx.x >> 6)) * 8 + (k)] = wall_clock64(); \
+        if (g_gemv_trace && (threadIdx.x & 63) == 0 &&                                            \
+            (g_gemv_trace_sel < 0 || g_gemv_trace_sel == ((GROUPED ? 1 : 0) | (NU == 2 ? 2 : 0) | (a.expert_ids ? 4 : 0))))    \
+            g_gemv_trace[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * WAVES + (threadIdx.x >> 6)) * 8 + (k)] = wall_clock64(); \
     } while (0)
 #else
 #define GEMV_MARK(k) do { } while (0)
@@ -81,7 +86,35 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p) {
 template <int TYPE, int NB, int NU>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernelArgs a) {
     const int bid = blockIdx.x, nblk = gridDim.x;
+    constexpr bool GROUPED = false;
+    constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
 #include "gemv_body.inc"
+}
+
+// Expert matrices over pairs grouped by expert: the workgroup runs the body with as many columns as its item has pairs.
+// Workgroups of GROUPED_THREADS: two share a compute unit, so that one streams tiles while the other is between its
+// dependent start-up loads (work item -> expert -> activations) or in its epilogue.
+constexpr int GROUPED_THREADS = 512;
+template <int TYPE, int NU>
+__global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const GemvKernelArgs a) {
+    if ((int)blockIdx.y >= a.n_items[0]) return;
+    const int bid = blockIdx.x, nblk = gridDim.x;
+    constexpr bool GROUPED = true;
+    constexpr int THREADS = GROUPED_THREADS, WAVES = GROUPED_THREADS / 64;
+    const int n = __builtin_amdgcn_readfirstlane(a.items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
+    if (n == 4) {
+        constexpr int NB = 4;
+#include "gemv_body.inc"
+    } else if (n == 3) {
+        constexpr int NB = 3;
+#include "gemv_body.inc"
+    } else if (n == 2) {
+        constexpr int NB = 2;
+#include "gemv_body.inc"
+    } else if (n == 1) {
+        constexpr int NB = 1;
+#include "gemv_body.inc"
+    }
 }
 
 // q/k/v groups whose matrices are of both K-quant types (attn_v in q6_K on the "more bits" layers of a Q4_K_M
@@ -89,6 +122,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
 template <int NB>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const GemvKernelArgs a4, const GemvKernelArgs a6, int n4) {
     constexpr int NU = 1;
+    constexpr bool GROUPED = false;
+    constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
     if ((int)blockIdx.x < n4) {
         const GemvKernelArgs &a = a4;
         constexpr int TYPE = MESH_Q4_K;
@@ -105,9 +140,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const GemvKerne
 constexpr size_t LDS_LIMIT = 160 * 1024;
 constexpr int MAX_ROWS_X_KS = 64;       // bound on (tile-rows per workgroup) x KS, sizes the LDS partial buffer
 
-static size_t dot_smem_bytes(int type, int NB, int K, int rows_here, int KS, int NU) {
+static size_t dot_smem_bytes(int type, int NB, int K, int rows_here, int KS, int NU, int waves = GEMV_WAVES) {
     return (size_t)NB * (2 * (size_t)K + (size_t)(K / 32) * 8 + (type == MESH_Q6_K ? (size_t)(K / 16) * 4 : 0)) +
-           sizeof(float) * ((size_t)KS * rows_here * NU * 16 * NB + GEMV_WAVES * NB);
+           sizeof(float) * ((size_t)KS * rows_here * NU * 16 * NB + waves * NB);
 }
 
 template <int TYPE, int NB, int NU>
@@ -119,6 +154,19 @@ static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStrea
         attr_set = true;
     }
     gemv_dot_kernel<TYPE, NB, NU><<<grid, dim3(GEMV_THREADS), smem, stream>>>(ka);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+template <int TYPE, int NU>
+static int launch_grouped(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_grouped_kernel<TYPE, NU>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
+        attr_set = true;
+    }
+    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -147,7 +195,7 @@ struct KquantPlan {
     GemvKernelArgs ka;
     int type, NU, KS, grid, rows_max;
 };
-static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
+static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p, int waves = GEMV_WAVES) {
     const int type = a.mat[0].type;
     const int nsb = a.K / QK_K, NU = a.epi == EPI_SWIGLU ? 2 : 1;
     const size_t row_stride = (size_t)nsb * (type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES);
@@ -175,7 +223,13 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
     ka.ldres = a.ldres;
     ka.epi = a.epi;
     ka.rope = a.rope;
-    const int KS = nsb < GEMV_WAVES ? nsb : GEMV_WAVES;
+    int KS = nsb < waves ? nsb : waves;
+    if (waves != GEMV_WAVES) {
+        // half-size workgroups: every wave gets work only if KS divides the waves, evenly only if it divides the row too
+        KS = 1;
+        for (int d = waves; d > 1; d >>= 1)
+            if (d <= nsb && nsb % d == 0) { KS = d; break; }
+    }
     ka.ks = KS;
     // tile-rows per workgroup: spread over the CUs, bounded by the LDS partial buffer
     int rows_per_wg = (total_rows + ncu - 1) / ncu;
@@ -189,10 +243,14 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p) {
 
 // All matrices of `a` are tiled K-quants of one type.
 static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
-    const int n_pairs = a.expert_ids ? a.n_pairs : 1;
+    const int n_pairs = a.expert_ids ? (a.items ? a.max_items : a.n_pairs) : 1;       // workgroup columns of the grid
     if (a.expert_ids && (a.n_pairs <= 0 || a.x_div <= 0 || a.epi == EPI_RESIDUAL)) return fail(MESH_ERR_INVALID, "gemv: bad expert-indirection arguments");
+    if (a.items && (!a.expert_ids || !a.n_items || a.max_items <= 0)) return fail(MESH_ERR_INVALID, "gemv: bad grouped-expert arguments");
     KquantPlan plan;
-    int rc0 = plan_kquant(a, std::max(1, n_compute_units() / n_pairs), plan);
+    // (grouped launches: workgroups of half the size, twice as many per item)
+    static const int oversub = getenv("MESH_GROUPED_OVERSUB") ? std::max(1, atoi(getenv("MESH_GROUPED_OVERSUB"))) : 8;
+    int rc0 = a.items ? plan_kquant(a, std::max(1, oversub * n_compute_units() / n_pairs), plan, GROUPED_THREADS / 64)
+                      : plan_kquant(a, std::max(1, n_compute_units() / n_pairs), plan);
     if (rc0 != MESH_OK) return rc0;
     GemvKernelArgs &ka = plan.ka;
     const int type = plan.type, NU = plan.NU, KS = plan.KS, grid = plan.grid, rows_max = plan.rows_max;
@@ -200,6 +258,18 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
         ka.expert_ids = a.expert_ids;
         ka.expert_stride = (size_t)tiled_bytes(type, a.mat[0].M, a.K);
         ka.x_div = a.x_div;
+    }
+    if (a.items) {
+        // pairs of one expert share a pass over its weights, up to MOE_ITEM_PAIRS columns per workgroup
+        int nb = MOE_ITEM_PAIRS;
+        if (dot_smem_bytes(type, nb, a.K, rows_max, KS, NU, GROUPED_THREADS / 64) > LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemv: row length %d does not fit LDS with %d columns", a.K, nb);
+        ka.x = a.x;
+        ka.items = a.items;
+        ka.n_items = a.n_items;
+        const size_t smem = dot_smem_bytes(type, nb, a.K, rows_max, KS, NU, GROUPED_THREADS / 64);
+        const dim3 g((unsigned)grid, (unsigned)a.max_items);
+        if (type == MESH_Q4_K) return NU == 2 ? launch_grouped<MESH_Q4_K, 2>(ka, g, smem, stream) : launch_grouped<MESH_Q4_K, 1>(ka, g, smem, stream);
+        return NU == 2 ? launch_grouped<MESH_Q6_K, 2>(ka, g, smem, stream) : launch_grouped<MESH_Q6_K, 1>(ka, g, smem, stream);
     }
     if (a.expert_ids) {
         // every pair is its own single-column product

@@ -49,6 +49,15 @@ struct GemvMat {
 // RoPE + KV append in the epilogue of a q/k/v launch (NORM pairing: a pair's two rows are neighbours, so they live in
 // one 16-row tile): q rows are rotated before they are stored, k rows are rotated and stored as f16 in the K cache
 // at the token's position, v rows go to the V cache.  Same arithmetic, hence the same bits, as rope_kv_kernel.
+// A work item of a grouped expert launch: MOE_ITEM_INTS int32 = {expert, n, pair[0..n), unused...}, 1 <= n <= MOE_ITEM_PAIRS.
+constexpr int MOE_ITEM_PAIRS = 4, MOE_ITEM_INTS = 8;
+// upper bound on the items n_pairs pairs over n_expert experts can form (sum over experts of ceil(count / 4))
+inline int moe_max_items(int n_pairs, int n_expert) {
+    const int used = n_pairs < n_expert ? n_pairs : n_expert;
+    const int bound = used + n_pairs / MOE_ITEM_PAIRS;
+    return bound < n_pairs ? bound : n_pairs;
+}
+
 enum { GEMV_KIND_PLAIN = 0, GEMV_KIND_Q = 1, GEMV_KIND_K = 2, GEMV_KIND_V = 3 };
 struct GemvRope {
     const int32_t *pos = nullptr, *seq = nullptr;      // device, [T]; pos == nullptr: no fusion
@@ -75,6 +84,12 @@ struct GemvArgs {
     const int32_t *expert_ids = nullptr;
     int n_pairs = 0;
     int x_div = 1;
+    // Pairs grouped by expert (moe_group): when items is set as well, the launch walks the item list instead, so
+    // that the pairs of an item (up to MOE_ITEM_PAIRS, all of one expert) share one pass over that expert's weights.
+    // items / n_items are device memory, max_items bounds *n_items (the launch's grid is sized by it).
+    const int32_t *items = nullptr;
+    const int32_t *n_items = nullptr;
+    int max_items = 0;
     // Fused RoPE / KV append: kind[i] says what matrix i produces (tiled K-quant matrices, EPI_STORE, no experts only)
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};

@@ -77,6 +77,20 @@ __device__ __forceinline__ void x_fetch(XRegs<NB> &X, const float *__restrict__ 
     }
 }
 
+// the same with every column at its own offset (in elements) from x
+template <int NB>
+__device__ __forceinline__ void x_fetch_at(XRegs<NB> &X, const float *__restrict__ x, const size_t (&off)[NB], int g, bool live) {
+#pragma unroll
+    for (int t = 0; t < NB; ++t) {
+        X.a[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        X.b[t] = X.a[t];
+        if (live) {
+            X.a[t] = *reinterpret_cast<const float4 *>(x + off[t] + g * 8);
+            X.b[t] = *reinterpret_cast<const float4 *>(x + off[t] + g * 8 + 4);
+        }
+    }
+}
+
 template <int NB, bool NEED_I16>
 __device__ __forceinline__ void x_quantise(const XRegs<NB> &X, int K, const XStage &S, int g, bool live, float (&ss)[NB]) {
     const int lane = threadIdx.x & 63;

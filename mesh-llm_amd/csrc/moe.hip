@@ -5,6 +5,7 @@
 // for selection only; the weights are the unmasked probabilities of the selected experts, renormalised to sum 1.
 
 #include "moe.hpp"
+#include "gemv.hpp"
 
 namespace mesh {
 
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(MoeRouteArgs a) {
 // Router logits and routing in one launch, one workgroup per token: every wave holds the token's normalised hidden
 // state in registers (E / 64 values per lane) and takes every fourth expert row of the f32 router matrix; the
 // logits meet in LDS and the first wave routes.  logits[t] = W . (x[t] * rsqrt(mean(x^2) + eps) * norm_w).
-constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64, ROUTER_EPL_MAX = 64;     // hidden sizes up to 4096
+constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64;
 template <int NV>      // float4 groups per lane = E / 256
 __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(MoeRouteArgs a, const float *__restrict__ x, int ldx,
                                                                           const float *__restrict__ norm_w, float eps,
@@ -169,6 +170,83 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream) {
     if (a.n_expert < 1 || a.n_expert > 64 * ROUTE_MAX_PER_LANE || a.top_k < 1 || a.top_k > 64 || a.top_k > a.n_expert)
         return fail(MESH_ERR_UNSUPPORTED, "moe: %d experts / top-%d outside what the router kernel handles", a.n_expert, a.top_k);
     moe_route_kernel<<<dim3((unsigned)T), dim3(64), 0, stream>>>(a);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// Pairs -> per-expert work items, one workgroup.  The pair list sits in LDS; a wave takes every 16th expert and finds
+// its pairs with ballots over the list (64 pairs per step), first to count, then -- after a prefix sum over the
+// experts' item counts -- to write each pair into its item.
+constexpr int GROUP_THREADS = 1024, GROUP_WAVES = GROUP_THREADS / 64;
+__global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs, int n_expert,
+                                                                  int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
+    extern __shared__ int32_t g_lds[];
+    int32_t *s_ids = g_lds, *s_cnt = g_lds + n_pairs, *s_base = s_cnt + n_expert;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int p = tid; p < n_pairs; p += GROUP_THREADS) s_ids[p] = ids[p];
+    __syncthreads();
+    for (int e = wave; e < n_expert; e += GROUP_WAVES) {
+        int c = 0;
+        for (int p0 = 0; p0 < n_pairs; p0 += 64) {
+            const int p = p0 + lane;
+            c += __popcll(__ballot(p < n_pairs && s_ids[p] == e));
+        }
+        if (lane == 0) s_cnt[e] = c;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // exclusive prefix of items per expert: each lane sums a run of experts, the runs are scanned across the wave
+        const int per = (n_expert + 63) / 64, e0 = lane * per;
+        int mine = 0;
+        for (int e = e0; e < e0 + per && e < n_expert; ++e) mine += (s_cnt[e] + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+        int incl = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o);
+            if (lane >= o) incl += v;
+        }
+        int run = incl - mine;
+        for (int e = e0; e < e0 + per && e < n_expert; ++e) {
+            s_base[e] = run;
+            run += (s_cnt[e] + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+        }
+        if (lane == 63) n_items[0] = incl;
+    }
+    __syncthreads();
+    for (int e = wave; e < n_expert; e += GROUP_WAVES) {
+        const int cnt = s_cnt[e], base = s_base[e];
+        int seen = 0;
+        for (int p0 = 0; p0 < n_pairs && seen < cnt; p0 += 64) {
+            const int p = p0 + lane;
+            const bool hit = p < n_pairs && s_ids[p] == e;
+            const unsigned long long m = __ballot(hit);
+            if (hit) {
+                const int r = seen + __popcll(m & ((1ull << lane) - 1ull));
+                items[(size_t)(base + r / MOE_ITEM_PAIRS) * MOE_ITEM_INTS + 2 + r % MOE_ITEM_PAIRS] = p;
+            }
+            seen += __popcll(m);
+        }
+        const int n_it = (cnt + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+        for (int i = lane; i < n_it; i += 64) {
+            items[(size_t)(base + i) * MOE_ITEM_INTS + 0] = e;
+            items[(size_t)(base + i) * MOE_ITEM_INTS + 1] = i + 1 < n_it ? MOE_ITEM_PAIRS : cnt - i * MOE_ITEM_PAIRS;
+        }
+    }
+}
+
+bool moe_group_supported(int n_pairs, int n_expert) {
+    return n_pairs >= 1 && n_expert >= 1 && ((size_t)n_pairs + 2 * (size_t)n_expert) * sizeof(int32_t) <= 128 * 1024;
+}
+
+int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, hipStream_t stream) {
+    if (!moe_group_supported(n_pairs, n_expert)) return fail(MESH_ERR_UNSUPPORTED, "moe: %d pairs over %d experts do not fit the grouping kernel", n_pairs, n_expert);
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(moe_group_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+        attr_set = true;
+    }
+    const size_t smem = ((size_t)n_pairs + 2 * (size_t)n_expert) * sizeof(int32_t);
+    moe_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(ids, n_pairs, n_expert, items, n_items);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

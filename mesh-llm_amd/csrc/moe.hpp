@@ -18,6 +18,11 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream);
 bool moe_router_fused_supported(int E, int n_expert, int top_k);
 int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
                      float *logits_out, int T, hipStream_t stream);
+// Groups the n_pairs (token, slot) pairs of ids by expert into work items for the expert mat-vec launches (gemv.hpp:
+// MOE_ITEM_INTS int32 per item = {expert, n, pair[0..n)}, n <= MOE_ITEM_PAIRS pairs of that expert, in ascending pair
+// order; experts in ascending order).  *n_items receives the count.  The order is a function of ids alone.
+bool moe_group_supported(int n_pairs, int n_expert);
+int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, hipStream_t stream);
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 

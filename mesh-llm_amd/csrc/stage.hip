@@ -444,6 +444,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
+    if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
     if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
@@ -488,6 +489,11 @@ int session_new(mesh_stage *st, mesh_session **out) {
             return rc;
         if ((rc = sess_alloc(s.get(), &p, B * k * sizeof(int32_t))) != MESH_OK) return rc;
         s->moe_ids = static_cast<int32_t *>(p);
+        const size_t items = (size_t)moe_max_items((int)(B * k), (int)ne);
+        if ((rc = sess_alloc(s.get(), &p, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t))) != MESH_OK) return rc;
+        s->moe_items = static_cast<int32_t *>(p);
+        s->moe_n_items = s->moe_items + items * MOE_ITEM_INTS;
+        MESH_HIP_TRY(hipMemsetAsync(s->moe_items, 0, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t), s->stream));
         MESH_HIP_TRY(hipMemsetAsync(s->expert_mask, 0, ne * sizeof(float), s->stream));
     }
     if ((rc = sess_alloc(s.get(), &p, 3 * B * sizeof(int32_t))) != MESH_OK) return rc;
@@ -824,6 +830,9 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                 if (rc != MESH_OK) return rc;
                 if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
             }
+            // pairs of one expert share a pass over its weights
+            const bool grouped = s->moe_grouped && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
+            if (grouped && (rc = moe_group(s->moe_ids, T * k, ne, s->moe_items, s->moe_n_items, stream)) != MESH_OK) return rc;
             GemvArgs ea;
             ea.n_mat = 2;
             ea.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);
@@ -832,6 +841,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             ea.norm_w = static_cast<const float *>(L.ffn_norm.data); ea.eps = hp.rms_eps;
             ea.epi = EPI_SWIGLU;
             ea.expert_ids = s->moe_ids; ea.n_pairs = T * k; ea.x_div = k;
+            if (grouped) { ea.items = s->moe_items; ea.n_items = s->moe_n_items; ea.max_items = moe_max_items(T * k, ne); }
             { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ea, stream); }
             if (rc != MESH_OK) return rc;
             GemvArgs xa;
@@ -839,6 +849,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             xa.mat[0] = mat_of(L.down_exps, s->moe_out, E, nullptr);
             xa.x = s->ffn; xa.ldx = ffe; xa.K = ffe; xa.T = 1;
             xa.expert_ids = s->moe_ids; xa.n_pairs = T * k; xa.x_div = 1;
+            if (grouped) { xa.items = s->moe_items; xa.n_items = s->moe_n_items; xa.max_items = ea.max_items; }
             { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(xa, stream); }
             if (rc != MESH_OK) return rc;
             if ((rc = moe_combine(s->x, s->moe_out, s->moe_w, T, E, k, stream)) != MESH_OK) return rc;

@@ -85,6 +85,8 @@ struct mesh_session {
     float *moe_logits = nullptr, *moe_w = nullptr, *moe_out = nullptr, *expert_mask = nullptr;
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
+    int32_t *moe_items = nullptr, *moe_n_items = nullptr;      // (token, slot) pairs grouped by expert, see moe_group
+    bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)
     unsigned meta_counter = 0;

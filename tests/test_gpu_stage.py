@@ -241,6 +241,32 @@ def test_moe_stage_matches_oracle_with_and_without_mask(tmp_path):
     ses.close(); ses2.close(); st.close()
 
 
+def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path, monkeypatch):
+    """The expert launches walk (token, slot) pairs grouped by expert, up to four pairs of an expert per pass over its
+    weights; MESH_MOE_GROUP=0 runs every pair as its own product.  A column's arithmetic does not depend on its
+    neighbours, so both must give the same bits, whatever the group sizes (8 experts, top-2: 1 to 40 tokens make
+    groups of every size 1..4 and experts with more than one group)."""
+    m, cfg, tensors, st = _open(tmp_path, "tiny-moe", range(0, 2), 0, 2, n_ctx=64, n_batch=64)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(77))
+    ses = st.session()
+    monkeypatch.setenv("MESH_MOE_GROUP", "0")
+    ses0 = st.session()
+    monkeypatch.delenv("MESH_MOE_GROUP")
+    orc = StageOracle(cfg, tensors, 0, 2, 64)
+    pos0 = 0
+    for T in (1, 2, 5, 23, 3, 30):
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        pos = np.arange(pos0, pos0 + T)
+        a = ses.decode(x, pos).view(np.float32).reshape(T, E)
+        b = ses0.decode(x, pos).view(np.float32).reshape(T, E)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), T
+        assert np.array_equal(ses.moe_last_ids(T), ses0.moe_last_ids(T))
+        assert rel_l2(a, orc.forward(x, pos)) <= 1e-3
+        pos0 += T
+    ses.close(); ses0.close(); st.close()
+
+
 def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
     """One real-shape MoE layer of a 64-expert shard (of 128), decode batch 16, top-8 routing."""
     m = mesh()
