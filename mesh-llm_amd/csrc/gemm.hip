@@ -16,6 +16,8 @@
 
 #include "gemm.hpp"
 
+#include <type_traits>
+
 namespace mesh {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -72,6 +74,20 @@ template <> struct RawSub<MESH_Q4_K> {
             d4[i] = o;
         }
     }
+    // this thread's part of a GEMM-layout chunk (gemm.hpp); s = 2 * row + h
+    __device__ __forceinline__ void pack(int c, int h, uint8_t *chunk, int s) const {
+        const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+        const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
+        const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
+        const int sh = (c & 1) * 16 + h * 8;
+        const half2v sm = {(_Float16)(d * (float)((scw >> sh) & 0xFFu)), (_Float16)(-dmin * (float)((mnw >> sh) & 0xFFu))};
+        const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        uint32_t n[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) n[j] = ((w[2 * j] >> (4 * h)) & 0x0F0F0F0Fu) | (((w[2 * j + 1] >> (4 * h)) & 0x0F0F0F0Fu) << 4);
+        *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(n[0], n[1], n[2], n[3]);
+        *reinterpret_cast<uint32_t *>(chunk + 4096 + s * 4) = __builtin_bit_cast(uint32_t, sm);
+    }
 };
 
 // q6_K: row r, k-chunk c: half n = c/2, elements 128n + 32*t4 + l with t4 = 2*(c%2) + h, l = 0..31
@@ -111,6 +127,81 @@ template <> struct RawSub<MESH_Q6_K> {
             d4[i] = o;
         }
     }
+    __device__ __forceinline__ void pack(int c, int h, uint8_t *chunk, int s) const {
+        const int t4 = 2 * (c & 1) + h;
+        const float df = f16_bits_to_f32((uint16_t)d);
+        const half2v s01 = {(_Float16)(df * (float)(int8_t)(sc & 0xFFu)), (_Float16)(df * (float)(int8_t)(sc >> 8))};
+        const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
+        const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        uint32_t q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t nib = (t4 & 2) ? (lw[j] >> 4) & 0x0F0F0F0Fu : lw[j] & 0x0F0F0F0Fu;
+            q[j] = nib | (((hw[j] >> (2 * t4)) & 0x03030303u) << 4);
+        }
+        uint32_t n[4], hb2[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            n[j] = (q[2 * j] & 0x0F0F0F0Fu) | ((q[2 * j + 1] & 0x0F0F0F0Fu) << 4);
+            hb2[j >> 1] |= (((q[2 * j] >> 4) & 0x03030303u) | (((q[2 * j + 1] >> 4) & 0x03030303u) << 2)) << (4 * (j & 1));
+        }
+        *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(n[0], n[1], n[2], n[3]);
+        *reinterpret_cast<uint2 *>(chunk + 4096 + s * 8) = make_uint2(hb2[0], hb2[1]);
+        *reinterpret_cast<uint32_t *>(chunk + 6144 + s * 4) = __builtin_bit_cast(uint32_t, s01);
+    }
+};
+
+// The same (row, sub-block) out of the GEMM layout: two or three loads at the thread's own slot of the chunk.
+template <int TYPE> struct PackedSub;
+template <> struct PackedSub<MESH_Q4_K> {
+    static constexpr int CHUNK = 5120;
+    uint4 q;
+    uint32_t sm;
+    __device__ __forceinline__ void load(const uint8_t *__restrict__ chunk, int s) {
+        q = *reinterpret_cast<const uint4 *>(chunk + s * 16);
+        sm = *reinterpret_cast<const uint32_t *>(chunk + 4096 + s * 4);
+    }
+    __device__ __forceinline__ void store(_Float16 *dst) const {
+        const half2v s = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm, sm, 0x01000100u));
+        const half2v mn = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm, sm, 0x03020302u));
+        const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint4 o;
+            dequant4(w[j] & 0x0F0F0F0Fu, off, s, mn, o.x, o.y);
+            dequant4((w[j] >> 4) & 0x0F0F0F0Fu, off, s, mn, o.z, o.w);
+            d4[j] = o;
+        }
+    }
+};
+template <> struct PackedSub<MESH_Q6_K> {
+    static constexpr int CHUNK = 7168;
+    uint4 q;
+    uint2 hb;
+    uint32_t sc;
+    __device__ __forceinline__ void load(const uint8_t *__restrict__ chunk, int s) {
+        q = *reinterpret_cast<const uint4 *>(chunk + s * 16);
+        hb = *reinterpret_cast<const uint2 *>(chunk + 4096 + s * 8);
+        sc = *reinterpret_cast<const uint32_t *>(chunk + 6144 + s * 4);
+    }
+    __device__ __forceinline__ void store(_Float16 *dst) const {
+        const half2v s0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc, sc, 0x01000100u));
+        const half2v s1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc, sc, 0x03020302u));
+        const half2v off = {(_Float16)1056.f, (_Float16)1056.f}, zero = {(_Float16)0.f, (_Float16)0.f};
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t hs = (j < 2 ? hb.x : hb.y) >> (4 * (j & 1));
+            const half2v s = j < 2 ? s0 : s1;
+            uint4 o;
+            dequant4((w[j] & 0x0F0F0F0Fu) | ((hs & 0x03030303u) << 4), off, s, zero, o.x, o.y);
+            dequant4(((w[j] >> 4) & 0x0F0F0F0Fu) | (((hs >> 2) & 0x03030303u) << 4), off, s, zero, o.z, o.w);
+            d4[j] = o;
+        }
+    }
 };
 
 // Role split: waves 0-3 only multiply (each a 64 x 64 corner of the tile out of LDS stage kc & 1), waves 4-7 only
@@ -118,7 +209,12 @@ template <> struct RawSub<MESH_Q6_K> {
 // stage).  A SIMD then holds one wave of each kind per workgroup, and the dequantisation (vector ALU) of one runs
 // while the MFMAs (matrix core) of the other execute -- in one wave doing both, the ~110 dequant instructions of
 // a step only start once its 16 MFMAs have been issued, and the four waves move in lockstep between barriers.
-template <int TYPE>
+// PACKED: the weights come from the GEMM layout (a.Wp) instead of the mat-vec tiles (a.W).
+// XDIRECT: the activations are k8-major (gemm.hpp) and never enter LDS: a matrix-core wave's B fragment of 32 tokens x
+// 16 k is four contiguous 256-byte pieces of that layout, so each lane fetches its 16 bytes straight from memory (L2),
+// four k16 steps ahead, into a ring of registers.  That halves the LDS reads per MFMA and leaves the staging waves only
+// the weights.
+template <int TYPE, bool PACKED, bool XDIRECT>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     extern __shared__ __align__(16) _Float16 gemm_smem[];
     _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
@@ -134,31 +230,40 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         const int st = tid - 256;
         const int srow = st >> 1, sh = st & 1;
         const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
-        const bool wlive = wrow < a.M_pad;
-        const uint8_t *wtile_row = static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
+        const bool wlive = PACKED || wrow < a.M_pad;                 // (the GEMM layout holds its zero rows)
+        const uint8_t *wtile_row = PACKED ? static_cast<const uint8_t *>(a.Wp) + (size_t)blockIdx.x * n_steps * PackedSub<TYPE>::CHUNK
+                                          : static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
+        using Sub = typename std::conditional<PACKED, PackedSub<TYPE>, RawSub<TYPE>>::type;
         const int tok = t0 + srow;
         const bool xlive = tok < a.T;
-        const _Float16 *xrow = a.X + (size_t)(xlive ? tok : 0) * a.ldx + 32 * sh;
-        RawSub<TYPE> rw[2];
+        const _Float16 *xrow = XDIRECT ? a.X : a.X + (size_t)(xlive ? tok : 0) * a.ldx + 32 * sh;
+        Sub rw[2];
         uint4 rx[2][4];
-        auto fetch = [&](int kc, RawSub<TYPE> &w, uint4 (&x)[4]) {
-            w.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
-            const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+        auto fetch = [&](int kc, Sub &w, uint4 (&x)[4]) {
+            if constexpr (PACKED) w.load(wtile_row + (size_t)kc * PackedSub<TYPE>::CHUNK, st);
+            else w.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
+            if constexpr (!XDIRECT) {
+                const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) x[i] = s4[i];
+                for (int i = 0; i < 4; ++i) x[i] = s4[i];
+            }
         };
-        auto stage = [&](int kc, int buf, const RawSub<TYPE> &w, const uint4 (&x)[4]) {
+        auto stage = [&](int kc, int buf, const Sub &w, const uint4 (&x)[4]) {
             _Float16 *wdst = Ws + (buf * GM + srow) * LDS_LD + 32 * sh;
-            if (wlive) {
+            if constexpr (PACKED) {
+                w.store(wdst);
+            } else if (wlive) {
                 w.store(kc & 3, sh, wdst);
             } else {
                 uint4 *d4 = reinterpret_cast<uint4 *>(wdst);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
             }
-            uint4 *x4 = reinterpret_cast<uint4 *>(Xs + (buf * GN + srow) * LDS_LD + 32 * sh);
+            if constexpr (!XDIRECT) {
+                uint4 *x4 = reinterpret_cast<uint4 *>(Xs + (buf * GN + srow) * LDS_LD + 32 * sh);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) x4[i] = xlive ? x[i] : make_uint4(0, 0, 0, 0);
+                for (int i = 0; i < 4; ++i) x4[i] = xlive ? x[i] : make_uint4(0, 0, 0, 0);
+            }
         };
         fetch(0, rw[0], rx[0]);
         fetch(n_steps > 1 ? 1 : 0, rw[1], rx[1]);
@@ -188,6 +293,43 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    if constexpr (XDIRECT) {
+        // lane's slot in the fragments of its two 32-token groups: token (lane & 31), k8 group (lane >> 5) of a k16 step;
+        // consecutive k16 steps are 256 halfs apart.  Token blocks past the batch re-read the last one (never stored).
+        const int n_blk = (a.T + 15) >> 4, n_g = n_steps * (GK / 16);
+        const _Float16 *bp[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int tok = t0 + wn + 32 * i + (lane & 31);
+            const int blk = (tok >> 4) < n_blk ? (tok >> 4) : n_blk - 1;
+            bp[i] = a.X + (size_t)blk * 16 * a.K + ((lane >> 5) * 16 + (tok & 15)) * 8;
+        }
+        half8 ring[GK / 16][2];
+#pragma unroll
+        for (int ks = 0; ks < GK / 16; ++ks)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)(ks < n_g ? ks : n_g - 1) * 256);
+        __syncthreads();
+        for (int kc = 0; kc < n_steps; ++kc) {
+            const _Float16 *Wb = Ws + (kc & 1) * GM * LDS_LD;
+#pragma unroll
+            for (int ks = 0; ks < GK / 16; ++ks) {
+                half8 af[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    af[i] = *reinterpret_cast<const half8 *>(Wb + (wm + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], ring[ks][j], acc[i][j], 0, 0, 0);
+                int gn = (kc + 1) * (GK / 16) + ks;
+                gn = gn < n_g ? gn : n_g - 1;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)gn * 256);
+            }
+            __syncthreads();
+        }
+    } else {
     __syncthreads();
     for (int kc = 0; kc < n_steps; ++kc) {
         const int buf = kc & 1;
@@ -206,6 +348,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
+    }
     }
 
     // D[m][t]: lane holds column t = lane%32 and rows 8*(e/4) + 4*(lane/32) + e%4 -> four consecutive m per store
@@ -233,6 +376,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         }
 }
 
+template <int TYPE, bool PACKED, bool XDIRECT>
+static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
+    // two stages of the weight slab, and of the activation slab unless the activations bypass LDS: 73 728 / 36 864 B
+    constexpr size_t smem = sizeof(_Float16) * 2 * (GM + (XDIRECT ? 0 : GN)) * LDS_LD;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    gemm_kq_kernel<TYPE, PACKED, XDIRECT><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
 int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     if (!a.W || !a.X || !a.Y || a.M <= 0 || a.K <= 0 || a.T <= 0) return fail(MESH_ERR_INVALID, "gemm: null pointer or empty shape");
     if (a.K % QK_K || a.M % 4 || a.ldx % 8 || a.ldy % 4 || (a.residual && a.ldres % 4))
@@ -241,16 +398,50 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     GemmArgs k = a;
     k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
     const dim3 grid((unsigned)((a.M + GM - 1) / GM), (unsigned)((a.T + GN - 1) / GN));
-    constexpr size_t smem = sizeof(_Float16) * 2 * (GM + GN) * LDS_LD;        // two stages of both slabs: 73 728 B
-    static bool attr_set = false;
-    if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<MESH_Q4_K>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<MESH_Q6_K>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
+    if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
+    const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
+    if (a.x_k8) {
+        if (packed) return q4 ? launch_gemm<MESH_Q4_K, true, true>(k, grid, stream) : launch_gemm<MESH_Q6_K, true, true>(k, grid, stream);
+        return q4 ? launch_gemm<MESH_Q4_K, false, true>(k, grid, stream) : launch_gemm<MESH_Q6_K, false, true>(k, grid, stream);
     }
-    if (a.type == MESH_Q4_K) gemm_kq_kernel<MESH_Q4_K><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
-    else if (a.type == MESH_Q6_K) gemm_kq_kernel<MESH_Q6_K><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
-    else return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
+    if (packed) return q4 ? launch_gemm<MESH_Q4_K, true, false>(k, grid, stream) : launch_gemm<MESH_Q6_K, true, false>(k, grid, stream);
+    return q4 ? launch_gemm<MESH_Q4_K, false, false>(k, grid, stream) : launch_gemm<MESH_Q6_K, false, false>(k, grid, stream);
+}
+
+// ---- GEMM layout ----------------------------------------------------------------------------------------------
+// One workgroup writes one chunk: thread s re-reads its (row, sub-block) from the mat-vec tiles the way the staging
+// thread of the unpacked kernel does, and writes it in the packed form.
+template <int TYPE>
+__global__ __launch_bounds__(256) void gemm_pack_kernel(const uint8_t *__restrict__ tiled, uint8_t *__restrict__ packed, int M_pad, int nsb) {
+    constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
+    constexpr int CH = PackedSub<TYPE>::CHUNK;
+    const int kc = blockIdx.x, mb = blockIdx.y, n_steps = gridDim.x, s = threadIdx.x;
+    const int wrow = mb * GM + (s >> 1), h = s & 1;
+    uint8_t *chunk = packed + ((size_t)mb * n_steps + kc) * CH;
+    if (wrow >= M_pad) {
+        *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(0, 0, 0, 0);
+        if (TYPE == MESH_Q6_K) *reinterpret_cast<uint2 *>(chunk + 4096 + s * 8) = make_uint2(0, 0);
+        *reinterpret_cast<uint32_t *>(chunk + (TYPE == MESH_Q6_K ? 6144 : 4096) + s * 4) = 0u;
+        return;
+    }
+    RawSub<TYPE> r;
+    r.load(tiled + ((size_t)(wrow >> 4) * nsb + (kc >> 2)) * TB, wrow & 15, kc & 3, h);
+    r.pack(kc & 3, h, chunk, s);
+}
+
+size_t gemm_packed_bytes(int type, int64_t M, int64_t K) {
+    if ((type != MESH_Q4_K && type != MESH_Q6_K) || M <= 0 || K <= 0 || K % QK_K) return 0;
+    const size_t chunk = type == MESH_Q4_K ? PackedSub<MESH_Q4_K>::CHUNK : PackedSub<MESH_Q6_K>::CHUNK;
+    return (size_t)((M + GM - 1) / GM) * (size_t)(K / GK) * chunk;
+}
+
+int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, hipStream_t stream) {
+    if (!tiled || !packed || gemm_packed_bytes(type, M, K) == 0) return fail(MESH_ERR_INVALID, "gemm_pack: bad arguments (type %d, M %lld, K %lld)", type, (long long)M, (long long)K);
+    const dim3 grid((unsigned)(K / GK), (unsigned)((M + GM - 1) / GM));
+    const int M_pad = (int)((M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS), nsb = (int)(K / QK_K);
+    if (grid.y > 65535u) return fail(MESH_ERR_UNSUPPORTED, "gemm_pack: %lld rows are too many", (long long)M);
+    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), static_cast<uint8_t *>(packed), M_pad, nsb);
+    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), static_cast<uint8_t *>(packed), M_pad, nsb);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -7,11 +7,13 @@ namespace mesh {
 
 struct GemmArgs {
     const void *W = nullptr;         // tiled q4_K / q6_K matrix [M][K]
+    const void *Wp = nullptr;        // optional: the same matrix in the GEMM layout (gemm_pack); used instead of W when set
     int type = -1;
     int M = 0, K = 0, T = 0;
     int M_pad = 0;                   // filled in by gemm_kquant
-    const _Float16 *X = nullptr;     // [T][ldx] f16 activations
+    const _Float16 *X = nullptr;     // [T][ldx] f16 activations; or, with x_k8, the k8-major layout of the skinny GEMM (below)
     int ldx = 0;
+    bool x_k8 = false;               // X is k8-major: the matrix-core waves fetch their operand fragments from it directly
     float *Y = nullptr;              // [T][ldy] f32
     int ldy = 0;
     const float *bias = nullptr;     // [M] or null
@@ -19,6 +21,20 @@ struct GemmArgs {
     int ldres = 0;
 };
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
+
+// GEMM layout of a K-quant matrix: a second copy for the prefill GEMM, arranged by the workgroup tile that consumes it.
+// One chunk per (128-row block, 64-element k-step), chunks of a row block consecutive in k.  A chunk holds, for each of
+// the 256 (row, 32-element sub-block) pairs s = 2 * row + half, what the staging thread s needs, at s * stride of
+// each section, so that every load of a staging wave covers one contiguous kilobyte:
+//   q4_K (5120 B): [256 x 16 B quants: dword j = elements 8j..8j+3 in the low nibbles, 8j+4..8j+7 in the high ones]
+//                  [256 x (f16 d*scale, f16 -dmin*min)]
+//   q6_K (7168 B): [256 x 16 B low nibbles, same order][256 x 8 B upper two bits: byte b of dword j/2 holds, from
+//                  bit 4*(j%2), the bits of element 8j+b and, two bits up, of element 8j+4+b]
+//                  [256 x (f16 d*scale of elements 0..15, f16 d*scale of elements 16..31)]
+// The f16 products are the ones the kernel would otherwise compute from the block headers, so both layouts give the
+// same bits.  Rows beyond M are zero.
+size_t gemm_packed_bytes(int type, int64_t M, int64_t K);
+int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, hipStream_t stream);
 
 // Skinny GEMM for a batch of decode steps (gemm_skinny.hip): up to three tiled K-quant matrices sharing the f16
 // activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel.  Activations are in the
@@ -41,6 +57,7 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream);
 int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream);
+int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream);
 
 int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream);
 int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream);

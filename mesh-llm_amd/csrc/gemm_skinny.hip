@@ -484,6 +484,37 @@ int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Flo
     return MESH_OK;
 }
 
+// out (k8-major) = f16( silu(gate) * up ): one workgroup per token, padding tokens of the last block write zeros
+__global__ __launch_bounds__(256) void swiglu_k8_kernel(const float *__restrict__ g, const float *__restrict__ u, int T, int n,
+                                                        _Float16 *__restrict__ y) {
+    const int t = blockIdx.x, tid = threadIdx.x;
+    _Float16 *yb = y + (size_t)(t >> 4) * 16 * n + (size_t)(t & 15) * 8;
+    if (t >= T) {
+        for (int i = tid * 8; i < n; i += 2048) *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = make_uint4(0, 0, 0, 0);
+        return;
+    }
+    const float *gt = g + (size_t)t * n, *ut = u + (size_t)t * n;
+    for (int i = tid * 8; i < n; i += 2048) {
+        const float4 a0 = *reinterpret_cast<const float4 *>(gt + i), a1 = *reinterpret_cast<const float4 *>(gt + i + 4);
+        const float4 b0 = *reinterpret_cast<const float4 *>(ut + i), b1 = *reinterpret_cast<const float4 *>(ut + i + 4);
+        auto f = [](float a, float b) { return a / (1.0f + expf(-a)) * b; };
+        uint4 o;
+        o.x = sk_pack_h2(f(a0.x, b0.x), f(a0.y, b0.y));
+        o.y = sk_pack_h2(f(a0.z, b0.z), f(a0.w, b0.w));
+        o.z = sk_pack_h2(f(a1.x, b1.x), f(a1.y, b1.y));
+        o.w = sk_pack_h2(f(a1.z, b1.z), f(a1.w, b1.w));
+        *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = o;
+    }
+}
+
+int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (n % 8) return fail(MESH_ERR_INVALID, "swiglu_f16_k8: row length %d not a multiple of 8", n);
+    swiglu_k8_kernel<<<dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream>>>(gate, up, T, n, y);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
 int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream) {
     return rmsnorm_f16_k8(x, nullptr, 0.f, T, n, y, stream);
 }

@@ -64,6 +64,8 @@ int hparams_from_gguf(const GgufFile &g, HParams &hp) {
     return MESH_OK;
 }
 
+static int gemm_min_tokens();
+
 // ------------------------------------------------------------------------------------------------ loading
 namespace {
 
@@ -72,6 +74,7 @@ struct Loader {
     mesh_stage &st;
     void *staging = nullptr;
     size_t staging_bytes = 0;
+    bool gemm_layout = false;      // also keep K-quant projection matrices in the prefill GEMM's layout
 
     ~Loader() { if (staging) (void)hipFree(staging); }
 
@@ -125,6 +128,12 @@ struct Loader {
                               static_cast<uint8_t *>(out.data) + e * per_e, M, K, nullptr);
             if (rc != MESH_OK) return rc;
         }
+        if (gemm_layout && E == 1 && &out != &st.output && gemm_packed_bytes(out.type, M, K) > 0) {
+            const size_t pb = gemm_packed_bytes(out.type, M, K);
+            if ((rc = dev_alloc(&out.gemm, pb)) != MESH_OK) return rc;
+            if ((rc = gemm_pack(out.type, out.data, out.gemm, M, K, nullptr)) != MESH_OK) return rc;
+            st.gemm_layout_bytes += pb;
+        }
         MESH_HIP_TRY(hipDeviceSynchronize());
         return MESH_OK;
     }
@@ -162,6 +171,12 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
         return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: head_dim %u has no attention kernel (64 and 128 do)", hp.head_dim);
 
     Loader ld{g, *st};
+    // stages that can be handed prefill-sized calls keep a GEMM-layout copy of their projections (MESH_GEMM_LAYOUT=0:
+    // no copy, the GEMM reads the mat-vec tiles)
+    {
+        const char *e = getenv("MESH_GEMM_LAYOUT");
+        ld.gemm_layout = st->n_batch_max >= gemm_min_tokens() && !(e && e[0] == '0');
+    }
     const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, KD = (int64_t)hp.n_head_kv * hp.head_dim;
     const bool moe = hp.arch == "qwen3moe";
     st->layers.resize((size_t)(layer_end - layer_begin));
@@ -445,6 +460,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
+    if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
     if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
@@ -592,7 +608,7 @@ static bool layer_is_kquant_dense(const LayerWeights &L) {
 
 static GemmArgs gemm_of(const DevTensor &w, const uint16_t *x16, int ldx, int T, float *y, int ldy, const DevTensor *bias) {
     GemmArgs g;
-    g.W = w.data; g.type = w.type; g.M = (int)w.M; g.K = (int)w.K; g.T = T;
+    g.W = w.data; g.Wp = w.gemm; g.type = w.type; g.M = (int)w.M; g.K = (int)w.K; g.T = T;
     g.X = reinterpret_cast<const _Float16 *>(x16); g.ldx = ldx; g.Y = y; g.ldy = ldy;
     g.bias = bias && bias->present() ? static_cast<const float *>(bias->data) : nullptr;
     return g;
@@ -610,7 +626,9 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
     bool rope_fused = false, attn_is_k8 = false;
-    if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
+    const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
+    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; return g; };
+    if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
@@ -633,9 +651,9 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
     } else {
         ProfScope ps(s, MESH_PROF_GEMV);
-        if ((rc = gemm_kquant(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq), stream)) != MESH_OK) return rc;
-        if ((rc = gemm_kquant(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk), stream)) != MESH_OK) return rc;
-        if ((rc = gemm_kquant(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq)), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk)), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv)), stream)) != MESH_OK) return rc;
     }
     RopeKvArgs ra;
     ra.q = s->q; ra.k = s->k; ra.v = s->v;
@@ -669,7 +687,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     }
     if (rc != MESH_OK) return rc;
     if (attn_is_k8) rc = MESH_OK;
-    else if (skinny) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
+    else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
     else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
@@ -682,12 +700,12 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_skinny(oa, stream)) != MESH_OK) return rc;
     } else {
         ProfScope ps(s, MESH_PROF_GEMV);
-        GemmArgs go = gemm_of(L.wo, s->xn16, QD, T, s->x, E, nullptr);
+        GemmArgs go = gemm_k8(gemm_of(L.wo, s->xn16, QD, T, s->x, E, nullptr));
         go.residual = s->x; go.ldres = E;
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
     if (attn_only) return MESH_OK;
-    if (skinny) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
+    if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
@@ -709,13 +727,15 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     }
     {
         ProfScope ps(s, MESH_PROF_GEMV);
-        if ((rc = gemm_kquant(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr), stream)) != MESH_OK) return rc;
-        if ((rc = gemm_kquant(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr)), stream)) != MESH_OK) return rc;
+        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr)), stream)) != MESH_OK) return rc;
     }
-    if ((rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream)) != MESH_OK) return rc;
+    if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
+    else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
+    if (rc != MESH_OK) return rc;
     {
         ProfScope ps(s, MESH_PROF_GEMV);
-        GemmArgs gd = gemm_of(L.w_down, s->ffn16, FF, T, s->x, E, nullptr);
+        GemmArgs gd = gemm_k8(gemm_of(L.w_down, s->ffn16, FF, T, s->x, E, nullptr));
         gd.residual = s->x; gd.ldres = E;
         if ((rc = gemm_kquant(gd, stream)) != MESH_OK) return rc;
     }

@@ -28,6 +28,7 @@ int hparams_from_gguf(const GgufFile &g, HParams &hp);
 // (same byte count as the GGUF tensor); everything else keeps the GGUF row-major layout.
 struct DevTensor {
     void *data = nullptr;
+    void *gemm = nullptr;   // K-quant projections of stages that can take prefill-sized calls: second copy in the GEMM layout (gemm.hpp)
     int type = -1;
     int64_t K = 0;       // row length (ggml ne[0])
     int64_t M = 0;       // rows (ggml ne[1]); for 1-D tensors M = 1
@@ -64,6 +65,7 @@ struct mesh_stage {
     std::vector<mesh::LayerWeights> layers;
     mesh::DevTensor tok_embd, output_norm, output;
     std::vector<void *> allocations;
+    size_t gemm_layout_bytes = 0; // extra HBM held by the GEMM-layout copies
     size_t weight_bytes = 0;      // GGUF bytes of everything resident (the algorithmic weight traffic of one decode step)
     float *rope_inv_freq = nullptr;   // [n_rot/2] f32, theta_scale^i by the f32 recurrence ggml uses
     ~mesh_stage();
@@ -86,6 +88,7 @@ struct mesh_session {
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
     int32_t *moe_items = nullptr, *moe_n_items = nullptr;      // (token, slot) pairs grouped by expert, see moe_group
+    bool gemm_x_k8 = true;           // MESH_GEMM_XDIRECT=0 at session creation: the prefill GEMM stages row-major activations through LDS
     bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)

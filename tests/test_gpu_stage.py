@@ -290,6 +290,43 @@ def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
     ses.close(); st.close()
 
 
+@pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2])])
+def test_prefill_gemm_layout_copy_gives_the_same_bits(tmp_path, monkeypatch, name, layers):
+    """Stages that can take prefill-sized calls keep a second copy of their projections arranged for the GEMM's
+    staging threads, with the per-sub-block f16 scale products precomputed; MESH_GEMM_LAYOUT=0 makes the GEMM read the
+    mat-vec tiles instead.  Same arithmetic on the same values: the outputs must be bit-identical (q4_K and q6_K
+    matrices, row counts that are and are not multiples of the 128-row tile)."""
+    m = mesh()
+    cfg = models.CONFIGS[name]
+    path = os.path.join(str(tmp_path), name + ".gguf")
+    models.write_model(path, cfg, layers, seed=5)
+    lb, le = layers[0], layers[-1] + 1
+    st1 = m.Stage(path, lb, le, n_ctx=256, n_seq_max=1, n_batch_max=208)
+    monkeypatch.setenv("MESH_GEMM_LAYOUT", "0")
+    st0 = m.Stage(path, lb, le, n_ctx=256, n_seq_max=1, n_batch_max=208)
+    monkeypatch.delenv("MESH_GEMM_LAYOUT")
+    os.unlink(path)
+    E = cfg["n_embd"]
+    T = 200
+    x = np.random.Generator(np.random.PCG64(3)).standard_normal((T, E)).astype(np.float32)
+    s1, s0 = st1.session(), st0.session()
+    a = s1.decode(x, np.arange(T)).view(np.uint32)
+    b = s0.decode(x, np.arange(T)).view(np.uint32)
+    assert np.array_equal(a, b)
+    # the matrix-core waves take their activation fragments straight from the k8-major layout; MESH_GEMM_XDIRECT=0
+    # stages row-major activations through LDS instead.  The GEMM's products and their order are the same, but the
+    # f16 activations come from different producer kernels (whose f32 sums may be contracted differently), so a few
+    # values differ by an f16 rounding step
+    monkeypatch.setenv("MESH_GEMM_XDIRECT", "0")
+    s2, s3 = st1.session(), st0.session()
+    monkeypatch.delenv("MESH_GEMM_XDIRECT")
+    c = s2.decode(x, np.arange(T)).view(np.uint32)
+    assert np.array_equal(s3.decode(x, np.arange(T)).view(np.uint32), c)
+    assert rel_l2(c.view(np.float32), a.view(np.float32)) <= 1e-3
+    for o in (s0, s1, s2, s3, st1, st0):
+        o.close()
+
+
 def test_prefill_mfma_path_matches_oracle_and_decode_path(tmp_path):
     """Calls with >= 192 tokens take the large-tile MFMA GEMM (f16 activations, f32 accumulate): compare it with the
     oracle and with the same tokens fed 16 at a time (skinny GEMM), then keep decoding on top of the prefilled cache."""
