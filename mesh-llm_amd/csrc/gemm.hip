@@ -352,6 +352,58 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     }
 
     // D[m][t]: lane holds column t = lane%32 and rows 8*(e/4) + 4*(lane/32) + e%4 -> four consecutive m per store
+    if (a.y16_k8) {
+        // SwiGLU pair: the waves of the upper half of the tile hold the up rows of the gate rows in the lower half, at
+        // the same (register, lane).  They hand them over through LDS (free by now: the staging waves have left, and
+        // the barrier makes sure every matrix-core wave has read its last fragments).
+        float *xch = reinterpret_cast<float *>(gemm_smem);         // [token half][64 registers][64 lanes]
+        __syncthreads();
+        if (wm) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) xch[(((wn >> 6) * 4 + i * 2 + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+        }
+        __syncthreads();
+        if (wm) return;
+        const int t_pad = (a.T + 15) & ~15;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int t = t0 + wn + 32 * j + (lane & 31);
+                if (t >= t_pad) continue;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const int m = (int)blockIdx.x * (GM / 2) + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                    if (m >= a.M) continue;
+                    float o[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float g = acc[i][j][4 * e4 + c], u = xch[(((wn >> 6) * 4 + i * 2 + j) * 16 + 4 * e4 + c) * 64 + lane];
+                        o[c] = t < a.T ? g / (1.0f + expf(-g)) * u : 0.f;       // padding columns of the last token block hold zeros
+                    }
+                    *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
+                        make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
+                }
+            }
+        return;
+    }
+    float *Y = a.Y;
+    const float *bias = a.bias;
+    int M = a.M, ldy = a.ldy, mb0 = m0;
+    if (a.n_seg > 1) {
+        // (selected, not indexed: a dynamically indexed kernel-argument array would be spilled to scratch)
+        const int bx = blockIdx.x;
+        const int sg = (bx >= a.seg_begin[1] ? 1 : 0) + (a.n_seg > 2 && bx >= a.seg_begin[2] ? 1 : 0);
+        Y = sg == 0 ? a.seg_Y[0] : sg == 1 ? a.seg_Y[1] : a.seg_Y[2];
+        bias = sg == 0 ? a.seg_bias[0] : sg == 1 ? a.seg_bias[1] : a.seg_bias[2];
+        M = sg == 0 ? a.seg_M[0] : sg == 1 ? a.seg_M[1] : a.seg_M[2];
+        ldy = sg == 0 ? a.seg_ldy[0] : sg == 1 ? a.seg_ldy[1] : a.seg_ldy[2];
+        mb0 = (bx - (sg == 0 ? 0 : sg == 1 ? a.seg_begin[1] : a.seg_begin[2])) * GM;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -360,18 +412,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
             if (t >= a.T) continue;
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
-                const int m = m0 + wm + 32 * i + 8 * e4 + 4 * (lane >> 5);
-                if (m >= a.M) continue;      // M is a multiple of 4 for every projection
+                const int m = mb0 + wm + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                if (m >= M) continue;      // M is a multiple of 4 for every projection
                 float4 o = make_float4(acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]);
-                if (a.bias) {
-                    const float4 b = *reinterpret_cast<const float4 *>(a.bias + m);
+                if (bias) {
+                    const float4 b = *reinterpret_cast<const float4 *>(bias + m);
                     o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w;
                 }
                 if (a.residual) {
                     const float4 r = *reinterpret_cast<const float4 *>(a.residual + (size_t)t * a.ldres + m);
                     o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
                 }
-                *reinterpret_cast<float4 *>(a.Y + (size_t)t * a.ldy + m) = o;
+                *reinterpret_cast<float4 *>(Y + (size_t)t * ldy + m) = o;
             }
         }
 }
@@ -391,13 +443,21 @@ static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
 }
 
 int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
-    if (!a.W || !a.X || !a.Y || a.M <= 0 || a.K <= 0 || a.T <= 0) return fail(MESH_ERR_INVALID, "gemm: null pointer or empty shape");
+    if (!a.X || a.M <= 0 || a.K <= 0 || a.T <= 0) return fail(MESH_ERR_INVALID, "gemm: null pointer or empty shape");
+    if (a.y16_k8 || a.n_seg > 1) {
+        if (!a.Wp || (a.y16_k8 && (a.n_seg > 1 || a.bias || a.residual)) || a.n_seg > 3)
+            return fail(MESH_ERR_INVALID, "gemm: multi-matrix and SwiGLU launches need the GEMM layout (and no bias / residual for SwiGLU)");
+        for (int i = 0; i < a.n_seg && !a.y16_k8; ++i)
+            if (!a.seg_Y[i] || a.seg_M[i] <= 0 || a.seg_M[i] % 4 || a.seg_ldy[i] % 4 || (i + 1 < a.n_seg && a.seg_M[i] % GM) || (a.residual))
+                return fail(MESH_ERR_INVALID, "gemm: bad matrix %d of a multi-matrix launch", i);
+    } else if (!a.W || !a.Y) return fail(MESH_ERR_INVALID, "gemm: null pointer");
     if (a.K % QK_K || a.M % 4 || a.ldx % 8 || a.ldy % 4 || (a.residual && a.ldres % 4))
         return fail(MESH_ERR_INVALID, "gemm: shape M=%d K=%d not supported (K %% 256, M %% 4)", a.M, a.K);
     if ((reinterpret_cast<uintptr_t>(a.X) | reinterpret_cast<uintptr_t>(a.Y)) & 15) return fail(MESH_ERR_INVALID, "gemm: X and Y must be 16-byte aligned");
     GemmArgs k = a;
     k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
-    const dim3 grid((unsigned)((a.M + GM - 1) / GM), (unsigned)((a.T + GN - 1) / GN));
+    const int row_blocks = a.y16_k8 ? (a.M + GM / 2 - 1) / (GM / 2) : (a.M + GM - 1) / GM;
+    const dim3 grid((unsigned)row_blocks, (unsigned)((a.T + GN - 1) / GN));
     if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
     if (a.x_k8) {
@@ -411,12 +471,19 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
 // ---- GEMM layout ----------------------------------------------------------------------------------------------
 // One workgroup writes one chunk: thread s re-reads its (row, sub-block) from the mat-vec tiles the way the staging
 // thread of the unpacked kernel does, and writes it in the packed form.
+// tiled2 set: a gate / up pair -- the chunk's rows 0..63 are rows [64 mb, 64 mb + 64) of `tiled`, rows 64..127 those of tiled2.
 template <int TYPE>
-__global__ __launch_bounds__(256) void gemm_pack_kernel(const uint8_t *__restrict__ tiled, uint8_t *__restrict__ packed, int M_pad, int nsb) {
+__global__ __launch_bounds__(256) void gemm_pack_kernel(const uint8_t *__restrict__ tiled, const uint8_t *__restrict__ tiled2,
+                                                        uint8_t *__restrict__ packed, int M_pad, int nsb) {
     constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
     constexpr int CH = PackedSub<TYPE>::CHUNK;
     const int kc = blockIdx.x, mb = blockIdx.y, n_steps = gridDim.x, s = threadIdx.x;
-    const int wrow = mb * GM + (s >> 1), h = s & 1;
+    const int h = s & 1;
+    int wrow = mb * GM + (s >> 1);
+    if (tiled2) {
+        wrow = mb * (GM / 2) + ((s >> 1) & (GM / 2 - 1));
+        if ((s >> 1) >= GM / 2) tiled = tiled2;
+    }
     uint8_t *chunk = packed + ((size_t)mb * n_steps + kc) * CH;
     if (wrow >= M_pad) {
         *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(0, 0, 0, 0);
@@ -440,8 +507,27 @@ int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, h
     const dim3 grid((unsigned)(K / GK), (unsigned)((M + GM - 1) / GM));
     const int M_pad = (int)((M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS), nsb = (int)(K / QK_K);
     if (grid.y > 65535u) return fail(MESH_ERR_UNSUPPORTED, "gemm_pack: %lld rows are too many", (long long)M);
-    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), static_cast<uint8_t *>(packed), M_pad, nsb);
-    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), static_cast<uint8_t *>(packed), M_pad, nsb);
+    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
+    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+size_t gemm_packed_pair_bytes(int type, int64_t M, int64_t K) {
+    if ((type != MESH_Q4_K && type != MESH_Q6_K) || M <= 0 || K <= 0 || K % QK_K) return 0;
+    const size_t chunk = type == MESH_Q4_K ? PackedSub<MESH_Q4_K>::CHUNK : PackedSub<MESH_Q6_K>::CHUNK;
+    return (size_t)((M + GM / 2 - 1) / (GM / 2)) * (size_t)(K / GK) * chunk;
+}
+
+int gemm_pack_pair(int type, const void *gate_tiled, const void *up_tiled, void *packed, int64_t M, int64_t K, hipStream_t stream) {
+    if (!gate_tiled || !up_tiled || !packed || gemm_packed_pair_bytes(type, M, K) == 0)
+        return fail(MESH_ERR_INVALID, "gemm_pack_pair: bad arguments (type %d, M %lld, K %lld)", type, (long long)M, (long long)K);
+    const dim3 grid((unsigned)(K / GK), (unsigned)((M + GM / 2 - 1) / (GM / 2)));
+    const int M_pad = (int)((M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS), nsb = (int)(K / QK_K);
+    if (grid.y > 65535u) return fail(MESH_ERR_UNSUPPORTED, "gemm_pack_pair: %lld rows are too many", (long long)M);
+    const uint8_t *g = static_cast<const uint8_t *>(gate_tiled), *u = static_cast<const uint8_t *>(up_tiled);
+    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
+    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -19,6 +19,16 @@ struct GemmArgs {
     const float *bias = nullptr;     // [M] or null
     const float *residual = nullptr; // [T][ldres] or null; may alias Y
     int ldres = 0;
+    // Several matrices sharing X in one launch (GEMM layout only: Wp holds their row blocks back to back, every matrix
+    // but the last a whole number of 128-row blocks): matrix i starts at row block seg_begin[i] and has its own output,
+    // bias and row count; M is the total.  n_seg == 1: the fields above describe the one matrix.
+    int n_seg = 1;
+    int seg_begin[3] = {0, 0, 0}, seg_M[3] = {0, 0, 0}, seg_ldy[3] = {0, 0, 0};
+    float *seg_Y[3] = {nullptr, nullptr, nullptr};
+    const float *seg_bias[3] = {nullptr, nullptr, nullptr};
+    // SwiGLU pair: Wp is a gate/up pair packed by gemm_pack_pair (every row block 64 gate rows, then the same 64 up
+    // rows), M their common row count; the launch writes f16(silu(gate) * up) in the k8-major layout to y16_k8 (Y unused).
+    _Float16 *y16_k8 = nullptr;
 };
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
 
@@ -35,6 +45,9 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream);
 // same bits.  Rows beyond M are zero.
 size_t gemm_packed_bytes(int type, int64_t M, int64_t K);
 int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, hipStream_t stream);
+// gate / up pair for the SwiGLU launch: row block b = gate rows [64b, 64b + 64) followed by up rows [64b, 64b + 64)
+size_t gemm_packed_pair_bytes(int type, int64_t M, int64_t K);
+int gemm_pack_pair(int type, const void *gate_tiled, const void *up_tiled, void *packed, int64_t M, int64_t K, hipStream_t stream);
 
 // Skinny GEMM for a batch of decode steps (gemm_skinny.hip): up to three tiled K-quant matrices sharing the f16
 // activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel.  Activations are in the

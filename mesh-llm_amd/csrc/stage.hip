@@ -128,13 +128,57 @@ struct Loader {
                               static_cast<uint8_t *>(out.data) + e * per_e, M, K, nullptr);
             if (rc != MESH_OK) return rc;
         }
-        if (gemm_layout && E == 1 && &out != &st.output && gemm_packed_bytes(out.type, M, K) > 0) {
-            const size_t pb = gemm_packed_bytes(out.type, M, K);
-            if ((rc = dev_alloc(&out.gemm, pb)) != MESH_OK) return rc;
-            if ((rc = gemm_pack(out.type, out.data, out.gemm, M, K, nullptr)) != MESH_OK) return rc;
-            st.gemm_layout_bytes += pb;
-        }
         MESH_HIP_TRY(hipDeviceSynchronize());
+        return MESH_OK;
+    }
+
+    static bool packable(const DevTensor &t) { return t.present() && t.tiled && t.E == 1 && gemm_packed_bytes(t.type, t.M, t.K) > 0; }
+    // GEMM-layout copies of n matrices back to back in one buffer (every matrix but the last must be a whole number
+    // of 128-row blocks for the buffer to serve one launch; the caller checks that before relying on it)
+    int pack_group(DevTensor *const *ts, int n) {
+        size_t total = 0;
+        for (int i = 0; i < n; ++i) total += gemm_packed_bytes(ts[i]->type, ts[i]->M, ts[i]->K);
+        void *buf = nullptr;
+        int rc;
+        if ((rc = dev_alloc(&buf, total)) != MESH_OK) return rc;
+        size_t off = 0;
+        for (int i = 0; i < n; ++i) {
+            ts[i]->gemm = static_cast<uint8_t *>(buf) + off;
+            if ((rc = gemm_pack(ts[i]->type, ts[i]->data, ts[i]->gemm, ts[i]->M, ts[i]->K, nullptr)) != MESH_OK) return rc;
+            off += gemm_packed_bytes(ts[i]->type, ts[i]->M, ts[i]->K);
+        }
+        st.gemm_layout_bytes += total;
+        MESH_HIP_TRY(hipDeviceSynchronize());
+        return MESH_OK;
+    }
+    // the dense projections of a layer
+    int pack_layer(LayerWeights &L) {
+        if (!gemm_layout) return MESH_OK;
+        int rc;
+        auto same = [](const DevTensor &a, const DevTensor &b) { return a.type == b.type && a.K == b.K; };
+        DevTensor *q = &L.wq, *k = &L.wk, *v = &L.wv, *o = &L.wo, *g = &L.w_gate, *u = &L.w_up, *d = &L.w_down;
+        if (packable(*q) && packable(*k) && same(*q, *k) && q->M % 128 == 0) {
+            const bool three = packable(*v) && same(*q, *v) && k->M % 128 == 0;
+            DevTensor *grp[3] = {q, k, v};
+            if ((rc = pack_group(grp, three ? 3 : 2)) != MESH_OK) return rc;
+            L.qkv_fused = three ? 3 : 2;
+            if (!three && packable(*v) && (rc = pack_group(&v, 1)) != MESH_OK) return rc;
+        } else {
+            for (DevTensor *t : {q, k, v})
+                if (packable(*t) && (rc = pack_group(&t, 1)) != MESH_OK) return rc;
+        }
+        for (DevTensor *t : {o, d})
+            if (packable(*t) && (rc = pack_group(&t, 1)) != MESH_OK) return rc;
+        if (packable(*g) && packable(*u) && same(*g, *u) && g->M == u->M) {
+            const size_t pb = gemm_packed_pair_bytes(g->type, g->M, g->K);
+            if ((rc = dev_alloc(&L.gate_up_gemm, pb)) != MESH_OK) return rc;
+            if ((rc = gemm_pack_pair(g->type, g->data, u->data, L.gate_up_gemm, g->M, g->K, nullptr)) != MESH_OK) return rc;
+            st.gemm_layout_bytes += pb;
+            MESH_HIP_TRY(hipDeviceSynchronize());
+        } else {
+            for (DevTensor *t : {g, u})
+                if (packable(*t) && (rc = pack_group(&t, 1)) != MESH_OK) return rc;
+        }
         return MESH_OK;
     }
 };
@@ -195,12 +239,14 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
             (rc = ld.load(p + "attn_k_norm.weight", L.k_norm, hp.head_dim, 1, 1, false, false, true)) ||
             (rc = ld.load(p + "ffn_norm.weight", L.ffn_norm, E, 1, 1, true, false, true)))
             return rc;
+        if (moe && (rc = ld.pack_layer(L)) != MESH_OK) return rc;       // (its attention projections)
         if (!moe) {
             if (hp.n_ff == 0) return fail(MESH_ERR_FORMAT, "gguf: feed_forward_length missing");
             if ((rc = ld.load(p + "ffn_gate.weight", L.w_gate, E, hp.n_ff, 1, true, true, false)) ||
                 (rc = ld.load(p + "ffn_up.weight", L.w_up, E, hp.n_ff, 1, true, true, false)) ||
                 (rc = ld.load(p + "ffn_down.weight", L.w_down, hp.n_ff, E, 1, true, true, false)))
                 return rc;
+            if ((rc = ld.pack_layer(L)) != MESH_OK) return rc;
         } else {
             const GgufTensorInfo *gi = g.find(p + "ffn_gate_inp.weight");
             if (!gi) return fail(MESH_ERR_FORMAT, "gguf: tensor '%sffn_gate_inp.weight' not found", p.c_str());
@@ -461,6 +507,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
     if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
+    if (const char *e = getenv("MESH_GEMM_FUSED")) s->gemm_fused = e[0] != '0';
     if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
@@ -651,9 +698,26 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
     } else {
         ProfScope ps(s, MESH_PROF_GEMV);
+        if (L.qkv_fused >= 2 && s->gemm_fused) {
+            // q, k (and v when it is of the same K-quant type) as one launch over their back-to-back GEMM-layout copies
+            const DevTensor *w[3] = {&L.wq, &L.wk, &L.wv}, *b[3] = {&L.bq, &L.bk, &L.bv};
+            float *y[3] = {s->q, s->k, s->v};
+            GemmArgs g = gemm_k8(gemm_of(L.wq, s->xn16, E, T, s->q, QD, nullptr));
+            g.n_seg = L.qkv_fused;
+            g.M = 0;
+            for (int i = 0; i < g.n_seg; ++i) {
+                g.seg_begin[i] = g.M / 128;
+                g.seg_M[i] = (int)w[i]->M; g.seg_ldy[i] = (int)w[i]->M; g.seg_Y[i] = y[i];
+                g.seg_bias[i] = b[i]->present() ? static_cast<const float *>(b[i]->data) : nullptr;
+                g.M += (int)w[i]->M;
+            }
+            if ((rc = gemm_kquant(g, stream)) != MESH_OK) return rc;
+            if (L.qkv_fused == 2 && (rc = gemm_kquant(gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv)), stream)) != MESH_OK) return rc;
+        } else {
         if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq)), stream)) != MESH_OK) return rc;
         if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk)), stream)) != MESH_OK) return rc;
         if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv)), stream)) != MESH_OK) return rc;
+        }
     }
     RopeKvArgs ra;
     ra.q = s->q; ra.k = s->k; ra.v = s->v;
@@ -725,14 +789,24 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_skinny(ga, stream)) != MESH_OK) return rc;
         return gemm_skinny(da, stream);
     }
-    {
+    if (L.gate_up_gemm && k8 && s->gemm_fused) {
+        // gate and up as one launch whose epilogue writes f16(silu(gate) * up) straight into the down projection's input
         ProfScope ps(s, MESH_PROF_GEMV);
-        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr)), stream)) != MESH_OK) return rc;
-        if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr)), stream)) != MESH_OK) return rc;
+        GemmArgs g = gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, nullptr, FF, nullptr));
+        g.Wp = L.gate_up_gemm;
+        g.y16_k8 = f16ffn;
+        if ((rc = gemm_kquant(g, stream)) != MESH_OK) return rc;
+    } else {
+        // (without the pair copy each matrix may still have its own GEMM-layout copy, or none)
+        {
+            ProfScope ps(s, MESH_PROF_GEMV);
+            if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr)), stream)) != MESH_OK) return rc;
+            if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr)), stream)) != MESH_OK) return rc;
+        }
+        if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
+        else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
+        if (rc != MESH_OK) return rc;
     }
-    if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
-    else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
-    if (rc != MESH_OK) return rc;
     {
         ProfScope ps(s, MESH_PROF_GEMV);
         GemmArgs gd = gemm_k8(gemm_of(L.w_down, s->ffn16, FF, T, s->x, E, nullptr));

@@ -42,6 +42,11 @@ struct LayerWeights {
     DevTensor attn_norm, wq, wk, wv, wo, bq, bk, bv, q_norm, k_norm;
     DevTensor ffn_norm, w_gate, w_up, w_down;
     DevTensor gate_inp, gate_exps, up_exps, down_exps;   // MoE
+    // GEMM-layout copies (gemm.hpp) beyond the per-tensor ones: wq / wk (/ wv) of one K-quant type sit back to back in
+    // one buffer (qkv_fused = 2 or 3 matrices; their .gemm pointers point into it), and gate / up of one type are
+    // packed as a SwiGLU pair.
+    int qkv_fused = 0;
+    void *gate_up_gemm = nullptr;
 };
 
 }  // namespace mesh
@@ -88,6 +93,7 @@ struct mesh_session {
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
     int32_t *moe_items = nullptr, *moe_n_items = nullptr;      // (token, slot) pairs grouped by expert, see moe_group
+    bool gemm_fused = true;          // MESH_GEMM_FUSED=0 at session creation: q / k / v and gate / up as separate prefill GEMM launches
     bool gemm_x_k8 = true;           // MESH_GEMM_XDIRECT=0 at session creation: the prefill GEMM stages row-major activations through LDS
     bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
