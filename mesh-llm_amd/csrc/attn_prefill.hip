@@ -27,6 +27,7 @@ constexpr int PF_HD = 128;
 constexpr int PF_TILE = 32;                 // queries per workgroup and keys per step
 constexpr int PF_KPITCH = PF_HD + 8;        // halfs per key row of the K tile in LDS (bank-conflict padding)
 constexpr int PF_VPITCH = PF_TILE + 4;      // halfs per dim row of the transposed V tile
+constexpr float PF_RESCALE_STEP = 8.f;      // the softmax reference moves only when the running maximum exceeds it by this (log2)
 
 typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 pf_h2 __attribute__((ext_vector_type(2)));
@@ -114,28 +115,38 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
             const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + qcol * PF_KPITCH + kc * 16 + 8 * half);
             s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s, 0, 0, 0);
         }
-        // register i of the result is key k0 + 8 * (i / 4) + 4 * half + i % 4 for query qcol
-        float mx = -INFINITY;
+        // register i of the result is key k0 + 8 * (i / 4) + 4 * half + i % 4 for query qcol.  Only a tile that reaches
+        // past the first query's position has anything to mask (a dead query column has q = 0 and is never stored).
+        if (k0 + PF_TILE - 1 > pos0 + qt * PF_TILE) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int key = k0 + 8 * (i >> 2) + 4 * half + (i & 3);
-            s[i] = (q_live && key <= pos_q) ? s[i] : -INFINITY;
-            mx = fmaxf(mx, s[i]);
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + 8 * (i >> 2) + 4 * half + (i & 3);
+                s[i] = key <= pos_q ? s[i] : -INFINITY;
+            }
         }
+        float mx = s[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;       // a query that has seen no key yet
-        const float corr = exp2f(m - m_use);                        // exp2(-inf) = 0 while nothing is accumulated
+        // m is the reference the exponentials are taken against.  It follows the running maximum only when that has
+        // moved by more than PF_RESCALE_STEP (log2 units), so that most steps skip the rescale of the 64 accumulator
+        // registers; in between p <= 2^PF_RESCALE_STEP, which f16 holds comfortably.  (Key 0 is visible to every
+        // query, so after the first tile m is finite for every live column.)
+        if (__builtin_amdgcn_ballot_w64(mx > m + PF_RESCALE_STEP) != 0ull) {
+            const float m_new = mx > m + PF_RESCALE_STEP ? mx : m;
+            const float corr = exp2f(m - m_new);                    // exp2(-inf) = 0 while nothing is accumulated; 1 for lanes that stay
+            l *= corr;
+            m = m_new;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+        }
         float p[16], ps = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { p[i] = exp2f(s[i] - m_use); ps += p[i]; }
+        for (int i = 0; i < 16; ++i) { p[i] = exp2f(s[i] - m); ps += p[i]; }
         ps += __shfl_xor(ps, 32);
-        l = l * corr + ps;
-        m = m_new;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+        l += ps;
         // P^T as the B operand: the lane's own registers, 8 per MFMA
         const pf_u4 pu1 = {pf_pack(p[0], p[1]), pf_pack(p[2], p[3]), pf_pack(p[4], p[5]), pf_pack(p[6], p[7])};
         const pf_u4 pu2 = {pf_pack(p[8], p[9]), pf_pack(p[10], p[11]), pf_pack(p[12], p[13]), pf_pack(p[14], p[15])};
