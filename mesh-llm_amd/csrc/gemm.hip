@@ -326,6 +326,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
                 gn = gn < n_g ? gn : n_g - 1;
 #pragma unroll
                 for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)gn * 256);
+                // keep each refill where it is written: left to itself the scheduler sinks all eight loads to the end
+                // of the step, where the next step's first MFMA waits for them at full memory latency
+                __builtin_amdgcn_sched_barrier(0);
             }
             __syncthreads();
         }
