@@ -92,9 +92,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernel
 }
 
 // Expert matrices over pairs grouped by expert: the workgroup runs the body with as many columns as its item has pairs.
-// Workgroups of GROUPED_THREADS: two share a compute unit, so that one streams tiles while the other is between its
-// dependent start-up loads (work item -> expert -> activations) or in its epilogue.
-constexpr int GROUPED_THREADS = 512;
+// Workgroups of GROUPED_THREADS: four share a compute unit, so that some stream tiles while others are between their
+// dependent start-up loads (work item -> expert -> activations) or in their epilogue.
+constexpr int GROUPED_THREADS = 256;
 template <int TYPE, int NU>
 __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const GemvKernelArgs a) {
     if ((int)blockIdx.y >= a.n_items[0]) return;
@@ -247,7 +247,7 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     if (a.expert_ids && (a.n_pairs <= 0 || a.x_div <= 0 || a.epi == EPI_RESIDUAL)) return fail(MESH_ERR_INVALID, "gemv: bad expert-indirection arguments");
     if (a.items && (!a.expert_ids || !a.n_items || a.max_items <= 0)) return fail(MESH_ERR_INVALID, "gemv: bad grouped-expert arguments");
     KquantPlan plan;
-    // (grouped launches: workgroups of half the size, twice as many per item)
+    // (grouped launches: workgroups of a quarter of the size, several times as many per item)
     static const int oversub = getenv("MESH_GROUPED_OVERSUB") ? std::max(1, atoi(getenv("MESH_GROUPED_OVERSUB"))) : 8;
     int rc0 = a.items ? plan_kquant(a, std::max(1, oversub * n_compute_units() / n_pairs), plan, GROUPED_THREADS / 64)
                       : plan_kquant(a, std::max(1, n_compute_units() / n_pairs), plan);
