@@ -88,6 +88,8 @@ __global__ __launch_bounds__(64) void moe_route_kernel(MoeRouteArgs a) {
 // Router logits and routing in one launch, one workgroup per token: every wave holds the token's normalised hidden
 // state in registers (E / 64 values per lane) and takes every fourth expert row of the f32 router matrix; the
 // logits meet in LDS and the first wave routes.  logits[t] = W . (x[t] * rsqrt(mean(x^2) + eps) * norm_w).
+// With gridDim.y > 1 the experts are split over blockIdx.y and the kernel only writes logits_out (routing follows in
+// moe_route_group_kernel): small batches then have enough workgroups to pull the router matrix through quickly.
 constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64;
 template <int NV>      // float4 groups per lane = E / 256
 __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(MoeRouteArgs a, const float *__restrict__ x, int ldx,
@@ -115,9 +117,11 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(MoeRou
         xr[i].z = xr[i].z * scale * w.z; xr[i].w = xr[i].w * scale * w.w;
     }
     // two expert rows per step, all of their loads in flight together
-    for (int e0 = wave; e0 < a.n_expert; e0 += 2 * ROUTER_WAVES) {
+    const int per = (a.n_expert + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int e_lo = (int)blockIdx.y * per, e_hi = e_lo + per < a.n_expert ? e_lo + per : a.n_expert;
+    for (int e0 = e_lo + wave; e0 < e_hi; e0 += 2 * ROUTER_WAVES) {
         const int e1 = e0 + ROUTER_WAVES;
-        const bool has1 = e1 < a.n_expert;
+        const bool has1 = e1 < e_hi;
         const float *w0 = W + (size_t)e0 * E, *w1 = W + (size_t)(has1 ? e1 : e0) * E;
         float4 r0[NV], r1[NV];
 #pragma unroll
@@ -142,6 +146,7 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(MoeRou
             }
         }
     }
+    if (gridDim.y > 1) return;
     __syncthreads();
     if (wave == 0) route_wave_any(s_logits, a, t, lane);
 }
@@ -178,10 +183,10 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream) {
 // its pairs with ballots over the list (64 pairs per step), first to count, then -- after a prefix sum over the
 // experts' item counts -- to write each pair into its item.
 constexpr int GROUP_THREADS = 1024, GROUP_WAVES = GROUP_THREADS / 64;
-__global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs, int n_expert,
-                                                                  int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
-    extern __shared__ int32_t g_lds[];
-    int32_t *s_ids = g_lds, *s_cnt = g_lds + n_pairs, *s_base = s_cnt + n_expert;
+// (whole workgroup; lds: n_pairs + 2 * n_expert ints)
+__device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int n_pairs, int n_expert, int32_t *__restrict__ items,
+                                            int32_t *__restrict__ n_items, int32_t *lds) {
+    int32_t *s_ids = lds, *s_cnt = lds + n_pairs, *s_base = s_cnt + n_expert;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (int p = tid; p < n_pairs; p += GROUP_THREADS) s_ids[p] = ids[p];
     __syncthreads();
@@ -232,6 +237,51 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t 
             items[(size_t)(base + i) * MOE_ITEM_INTS + 1] = i + 1 < n_it ? MOE_ITEM_PAIRS : cnt - i * MOE_ITEM_PAIRS;
         }
     }
+}
+
+__global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs, int n_expert,
+                                                                  int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
+    extern __shared__ int32_t g_lds[];
+    group_pairs(ids, n_pairs, n_expert, items, n_items, g_lds);
+}
+
+// Routing of a small batch and the grouping of its pairs in one single-workgroup launch: wave w routes tokens w,
+// w + 16, ... from their logits, then the workgroup groups the pairs it has just written (the barrier in between
+// also makes those writes visible to the whole workgroup).
+__global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(MoeRouteArgs a, int T, int32_t *__restrict__ items,
+                                                                        int32_t *__restrict__ n_items) {
+    extern __shared__ int32_t g_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(a.logits + (size_t)t * a.n_expert, a, t, lane);
+    __syncthreads();
+    group_pairs(a.ids, T * a.top_k, a.n_expert, items, n_items, g_lds);
+}
+
+int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
+                     float *logits, int T, int32_t *items, int32_t *n_items, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (!moe_router_group_supported(E, a.n_expert, a.top_k, T) || !logits)
+        return fail(MESH_ERR_UNSUPPORTED, "moe: split router for hidden size %d / %d experts / %d tokens", E, a.n_expert, T);
+    const int split = (a.n_expert + ROUTER_WAVES - 1) / ROUTER_WAVES;      // one expert row per wave
+    const dim3 grid((unsigned)T, (unsigned)split), block(ROUTER_THREADS);
+    MoeRouteArgs la = a;
+    switch (E / 256) {
+        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
+        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
+        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
+        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
+        default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
+    }
+    MESH_LAUNCH_CHECK();
+    la.logits = logits;
+    const size_t smem = ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
+    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(la, T, items, n_items);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+bool moe_router_group_supported(int E, int n_expert, int top_k, int T) {
+    return moe_router_fused_supported(E, n_expert, top_k) && n_expert > ROUTER_WAVES && T >= 1 && T <= 64 &&
+           ((size_t)T * top_k + 2 * (size_t)n_expert) * sizeof(int32_t) <= 48 * 1024;
 }
 
 bool moe_group_supported(int n_pairs, int n_expert) {

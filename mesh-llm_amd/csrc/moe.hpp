@@ -23,6 +23,12 @@ int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float
 // order; experts in ascending order).  *n_items receives the count.  The order is a function of ids alone.
 bool moe_group_supported(int n_pairs, int n_expert);
 int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, hipStream_t stream);
+// Small batches (T <= 64): router logits with the experts split over several workgroups per token, then routing and
+// grouping in one single-workgroup launch.  Same results as moe_router_fused followed by moe_group; `logits`
+// ([T][n_expert]) is required.
+bool moe_router_group_supported(int E, int n_expert, int top_k, int T);
+int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
+                     float *logits, int T, int32_t *items, int32_t *n_items, hipStream_t stream);
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 

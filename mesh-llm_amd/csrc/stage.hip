@@ -909,7 +909,16 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             MoeRouteArgs mr;
             mr.logits = s->moe_logits; mr.mask = s->expert_mask_on ? s->expert_mask : nullptr;
             mr.ids = s->moe_ids; mr.weights = s->moe_w; mr.n_expert = ne; mr.top_k = k; mr.norm_w = 1;
-            if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
+            const bool want_groups = s->moe_grouped && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
+            bool grouped_done = false;
+            if (want_groups && L.gate_inp.type == MESH_F32 && moe_router_group_supported(E, ne, k, T)) {
+                // a batch of decode steps: logits over many workgroups, then routing and grouping in one launch
+                ProfScope ps(s, MESH_PROF_GEMV);
+                if ((rc = moe_router_group(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
+                                           static_cast<const float *>(L.gate_inp.data), E, s->moe_logits, T, s->moe_items, s->moe_n_items,
+                                           stream)) != MESH_OK) return rc;
+                grouped_done = true;
+            } else if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
                 // the router matrix is small and f32: logits and routing in one launch
                 ProfScope ps(s, MESH_PROF_GEMV);
                 if ((rc = moe_router_fused(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
@@ -925,8 +934,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                 if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
             }
             // pairs of one expert share a pass over its weights
-            const bool grouped = s->moe_grouped && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
-            if (grouped && (rc = moe_group(s->moe_ids, T * k, ne, s->moe_items, s->moe_n_items, stream)) != MESH_OK) return rc;
+            const bool grouped = want_groups;
+            if (grouped && !grouped_done && (rc = moe_group(s->moe_ids, T * k, ne, s->moe_items, s->moe_n_items, stream)) != MESH_OK) return rc;
             GemvArgs ea;
             ea.n_mat = 2;
             ea.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);
