@@ -54,6 +54,10 @@ def test_mul_mat_vs_oracle(type_, M, K):
     w.close()
 
 
+def cfg_layers(name):
+    return models.CONFIGS[name]["n_layer"]
+
+
 def _open(tmp_path, name, layers, lb, le, n_ctx=64, n_seq=2, n_batch=16, seed=5, **kw):
     m = mesh()
     cfg = models.CONFIGS[name]
@@ -290,7 +294,27 @@ def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
     ses.close(); st.close()
 
 
-@pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2])])
+@pytest.mark.parametrize("name,T", [("tiny-llama", 192), ("tiny-llama", 257), ("tiny-qwen2", 256), ("tiny-qwen3", 300), ("tiny-g7", 193)])
+def test_prefill_gemm_token_counts_and_head_layouts(tmp_path, name, T):
+    """Prefill-sized calls at and around the 128-token tile edges, over the small models: head_dim 64 and 128, K / V
+    projections of 128 and 256 rows (q and k fused with and without v), q/k norms, biases, odd head groups."""
+    m, cfg, tensors, st = _open(tmp_path, name, range(cfg_layers(name)), 0, cfg_layers(name), n_ctx=320, n_seq=1, n_batch=304)
+    E = cfg["n_embd"]
+    x = np.random.Generator(np.random.PCG64(T)).standard_normal((T, E)).astype(np.float32)
+    ses = st.session()
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
+    orc = StageOracle(cfg, tensors, 0, cfg_layers(name), 320, n_seq_max=1)
+    ref = orc.forward(x, np.arange(T))
+    assert rel_l2(got, ref) <= 3e-3
+    assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 1e-2
+    # one more token on top of the prefilled cache, through the mat-vec path
+    x1 = np.random.Generator(np.random.PCG64(1)).standard_normal((1, E)).astype(np.float32)
+    got1 = ses.decode(x1, [T]).view(np.float32)
+    assert rel_l2(got1, orc.forward(x1, [T])) <= 3e-3
+    ses.close(); st.close()
+
+
+@pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-llama", [0, 1])])
 def test_prefill_gemm_variants_agree(tmp_path, monkeypatch, name, layers):
     """Stages that can take prefill-sized calls keep a second copy of their projections arranged for the GEMM's
     staging threads, with the per-sub-block f16 scale products precomputed; MESH_GEMM_LAYOUT=0 makes the GEMM read the
