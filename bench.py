@@ -377,7 +377,7 @@ def bench_shape(args):
         r["frac_hbm"] = round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)
         results[B] = r
     prefill = None
-    if sp["prefill"]:
+    if sp["prefill"] and args.prefill:
         T = sp["prefill"]
         xp = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).cuda()
         outp = torch.empty(m.act_packed_size(m.Q8_0, T, E), dtype=torch.uint8, device="cuda")
