@@ -124,26 +124,37 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
     // what a lane fetches of a 16-key block: its key row c, dims 32*cc + 8*g .. + 8 of K and of V; rows past the range
     // are clamped to its last key (and masked below), so the fetch of the block after the last one is harmless
-    KvRaw<KT> kraw[NC];
-    KvRaw<VT> vraw[NC];
-    auto fetch = [&](int kb) {
+    // Blocks in flight per wave: quantised rows are 2.5 - 3.5 times smaller than f16 rows, so one block ahead leaves
+    // too few bytes in flight to cover the memory latency; they run two ahead (20 more registers).
+    constexpr int DEPTH = (KT == MESH_F16 && VT == MESH_F16) ? 1 : 2;
+    constexpr int STEP = MMA_WAVES * MMA_KEYS;
+    KvRaw<KT> kraw[DEPTH][NC];
+    KvRaw<VT> vraw[DEPTH][NC];
+    auto fetch = [&](KvRaw<KT> (&kr_)[NC], KvRaw<VT> (&vr_)[NC], int kb) {
         int kr = kb + c;
         kr = kr < j1 ? kr : j1 - 1;
         const uint8_t *krow = a.kcache + (base + kr) * KRB, *vrow = a.vcache + (base + kr) * VRB;
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) kraw[cc] = kv_load<KT, HD>(krow, 32 * cc + 8 * g);
+        for (int cc = 0; cc < NC; ++cc) kr_[cc] = kv_load<KT, HD>(krow, 32 * cc + 8 * g);
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) vraw[cc] = kv_load<VT, HD>(vrow, 32 * cc + 8 * g);
+        for (int cc = 0; cc < NC; ++cc) vr_[cc] = kv_load<VT, HD>(vrow, 32 * cc + 8 * g);
     };
     const int kb0 = j0 + wave * MMA_KEYS;
-    if (kb0 < j1) fetch(kb0);
-    for (int kb = kb0; kb < j1; kb += MMA_WAVES * MMA_KEYS) {
+    if (kb0 < j1) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) fetch(kraw[d], vraw[d], kb0 + d * STEP);
+    }
+    for (int kbb = kb0; kbb < j1; kbb += DEPTH * STEP) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int kb = kbb + d * STEP;
+        if (kb >= j1) break;
         uint4 kf[NC], vf[NC];
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) kf[cc] = mm_piece_f16<KT>(kraw[cc]);
+        for (int cc = 0; cc < NC; ++cc) kf[cc] = mm_piece_f16<KT>(kraw[d][cc]);
 #pragma unroll
-        for (int cc = 0; cc < NC; ++cc) vf[cc] = mm_piece_f16<VT>(vraw[cc]);
-        fetch(kb + MMA_WAVES * MMA_KEYS);      // the next block's rows travel while this one is worked on
+        for (int cc = 0; cc < NC; ++cc) vf[cc] = mm_piece_f16<VT>(vraw[d][cc]);
+        fetch(kraw[d], vraw[d], kb + DEPTH * STEP);      // rows of a later block travel while this one is worked on
 
         // S^T = K . Q^T : register i is key kb + 4*g + i for head c
         mm_f4 s = {0.f, 0.f, 0.f, 0.f};
@@ -198,6 +209,7 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
             o[db] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mm_h4, vv), pf, o[db], 0, 0, 0);
         }
         mm_wave_lds_sync();        // the tile is rewritten by the next block
+      }
     }
 
     // merge the waves: o[db][i] is dim 16*db + 4*g + i of head c
