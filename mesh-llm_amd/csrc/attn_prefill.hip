@@ -162,7 +162,24 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         }
         __syncthreads();        // the tiles are overwritten by the next step
     }
-    if (q_live) {
+    if (a.out16_k8) {
+        // f16, in the k8-major layout the output projection's GEMM reads (gemm.hpp); the padding columns of the last
+        // block of 16 tokens are written as zeros
+        const int t_pad = (T + 15) & ~15;
+        if (tq < t_pad) {
+            const float inv = q_live ? 1.0f / l : 0.f;
+            const size_t KK = (size_t)a.n_head * PF_HD;
+            _Float16 *ob = a.out16_k8 + (size_t)(tq >> 4) * 16 * KK + (size_t)(tq & 15) * 8;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const size_t kk = (size_t)h * PF_HD + db * 32 + 8 * i4 + 4 * half;
+                    *reinterpret_cast<uint2 *>(ob + (kk >> 3) * 128 + (kk & 7)) =
+                        make_uint2(pf_pack(o[db][4 * i4] * inv, o[db][4 * i4 + 1] * inv), pf_pack(o[db][4 * i4 + 2] * inv, o[db][4 * i4 + 3] * inv));
+                }
+        }
+    } else if (q_live) {
         const float inv = 1.0f / l;
         float *op = a.out + ((size_t)tq * a.n_head + h) * PF_HD;
 #pragma unroll

@@ -743,7 +743,10 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;     // a batch of decode steps still splits the long KV
     {
         ProfScope ps(s, MESH_PROF_ATTN);
-        if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
+        if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) {
+            if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }          // straight into the output projection's input layout
+            rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
+        }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
             if (skinny) { aa.out16_k8 = xn; attn_is_k8 = true; }     // straight into the output projection's input layout
             rc = attention_mma(aa, T, stream);
