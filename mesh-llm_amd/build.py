@@ -15,6 +15,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # never let the compiler emit packed-FP32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # leading scalar kernel arguments arrive in SGPRs at wave start instead of through a scalar load (kernels whose
+    # start-up chain matters list those arguments first)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 

@@ -260,31 +260,33 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
 
 // Merge of the KV splits: grid (n_head, T), head_dim threads.  Split statistics go through LDS so every thread
 // sees them with broadcast reads and the partial rows are fetched with independent loads.
-__global__ __launch_bounds__(128) void attn_combine_kernel(AttnArgs a) {
+// (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
+__global__ __launch_bounds__(128) void attn_combine_kernel(const float *p_part, const float *p_ml, float *p_out, _Float16 *p_out16_k8,
+                                                           int p_n_splits, int p_n_head, int p_head_dim) {
     __shared__ float s_m[ATTN_SPLITS_CAP], s_l[ATTN_SPLITS_CAP];
     const int h = blockIdx.x, t = blockIdx.y, dd = threadIdx.x;
-    const size_t row = (size_t)t * a.n_head + h;
-    for (int s2 = dd; s2 < a.n_splits; s2 += blockDim.x) {
-        s_m[s2] = a.ml[(row * a.n_splits + s2) * 2 + 0];
-        s_l[s2] = a.ml[(row * a.n_splits + s2) * 2 + 1];
+    const size_t row = (size_t)t * p_n_head + h;
+    for (int s2 = dd; s2 < p_n_splits; s2 += blockDim.x) {
+        s_m[s2] = p_ml[(row * p_n_splits + s2) * 2 + 0];
+        s_l[s2] = p_ml[(row * p_n_splits + s2) * 2 + 1];
     }
     __syncthreads();
     float mh = -INFINITY;
-    for (int s2 = 0; s2 < a.n_splits; ++s2) mh = fmaxf(mh, s_m[s2]);
+    for (int s2 = 0; s2 < p_n_splits; ++s2) mh = fmaxf(mh, s_m[s2]);
     float num = 0.f, den = 0.f;
-    const float *pp = a.part + row * a.n_splits * a.head_dim + dd;
+    const float *pp = p_part + row * p_n_splits * p_head_dim + dd;
 #pragma unroll 8
-    for (int s2 = 0; s2 < a.n_splits; ++s2) {
+    for (int s2 = 0; s2 < p_n_splits; ++s2) {
         const float ms = s_m[s2];
         const float w = ms == -INFINITY ? 0.f : exp2f(ms - mh);      // maxima are in log2 units
-        num = fmaf(pp[(size_t)s2 * a.head_dim], w, num);
+        num = fmaf(pp[(size_t)s2 * p_head_dim], w, num);
         den = fmaf(s_l[s2], w, den);
     }
-    if (a.out16_k8) {
-        const size_t kk = (size_t)h * a.head_dim + dd, KK = (size_t)a.n_head * a.head_dim;
-        a.out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(num / den);
+    if (p_out16_k8) {
+        const size_t kk = (size_t)h * p_head_dim + dd, KK = (size_t)p_n_head * p_head_dim;
+        p_out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(num / den);
     } else {
-        a.out[row * a.head_dim + dd] = num / den;
+        p_out[row * p_head_dim + dd] = num / den;
     }
 }
 
@@ -335,7 +337,7 @@ int attention(const AttnArgs &a, int T, hipStream_t stream) {
 }
 
 int attention_combine(const AttnArgs &a, int T, hipStream_t stream) {
-    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a);
+    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a.part, a.ml, a.out, a.out16_k8, a.n_splits, a.n_head, a.head_dim);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

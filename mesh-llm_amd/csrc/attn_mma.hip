@@ -81,8 +81,13 @@ __device__ __forceinline__ void mm_wave_lds_sync() {
 }
 
 // grid (n_splits, n_kv, T), 256 threads.  group <= 16.
+// (the arguments on the way to the first K / V loads come first, as scalars, so that they are preloaded into SGPRs:
+// see gemv.hip)
 template <int HD, int KT, int VT>
-__global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(const float *p_q, const int32_t *p_pos, const int32_t *p_seq,
+                                                               const uint8_t *p_kcache, const uint8_t *p_vcache, int p_n_splits,
+                                                               int p_n_ctx, int p_n_kv, int p_group, int p_n_head, float p_scale,
+                                                               const AttnArgs a) {
     constexpr int NC = HD / 32;             // 32-dim chunks of the score product
     constexpr int NDB = HD / 16;            // 16-dim blocks of the output
     constexpr int KRB = kv_row_bytes(KT, HD), VRB = kv_row_bytes(VT, HD);
@@ -96,18 +101,18 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
     const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;         // head column / key row of a tile, lane group
-    const int G = a.group;
-    const int seq = a.seq[t];
-    const int n_keys = a.pos[t] + 1;
-    const int per = (n_keys + a.n_splits - 1) / a.n_splits;
+    const int G = p_group;
+    const int seq = p_seq[t];
+    const int n_keys = p_pos[t] + 1;
+    const int per = (n_keys + p_n_splits - 1) / p_n_splits;
     const int j0 = split * per;
     const int j1 = j0 + per < n_keys ? j0 + per : n_keys;
 
     // Q^T operand: head column c, dims 32*cc + 8*g + j, in log2 units
     mm_h8 qf[NC];
     {
-        const float qs = c < G ? a.scale * 1.44269504088896341f : 0.f;
-        const float *qp = a.q + ((size_t)t * a.n_head + (size_t)kvh * G + (c < G ? c : 0)) * HD + 8 * g;
+        const float qs = c < G ? p_scale * 1.44269504088896341f : 0.f;
+        const float *qp = p_q + ((size_t)t * p_n_head + (size_t)kvh * G + (c < G ? c : 0)) * HD + 8 * g;
 #pragma unroll
         for (int cc = 0; cc < NC; ++cc) {
             const float4 v0 = *reinterpret_cast<const float4 *>(qp + 32 * cc), v1 = *reinterpret_cast<const float4 *>(qp + 32 * cc + 4);
@@ -121,7 +126,7 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
     float m = -INFINITY, l = 0.f;
 
     _Float16 *sV = reinterpret_cast<_Float16 *>(s_raw) + wave * HD * MMA_VPITCH;
-    const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
+    const size_t base = ((size_t)seq * p_n_kv + kvh) * p_n_ctx;
     // what a lane fetches of a 16-key block: its key row c, dims 32*cc + 8*g .. + 8 of K and of V; rows past the range
     // are clamped to its last key (and masked below), so the fetch of the block after the last one is harmless
     // Blocks in flight per wave: quantised rows are 2.5 - 3.5 times smaller than f16 rows, so one block ahead leaves
@@ -133,7 +138,7 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
     auto fetch = [&](KvRaw<KT> (&kr_)[NC], KvRaw<VT> (&vr_)[NC], int kb) {
         int kr = kb + c;
         kr = kr < j1 ? kr : j1 - 1;
-        const uint8_t *krow = a.kcache + (base + kr) * KRB, *vrow = a.vcache + (base + kr) * VRB;
+        const uint8_t *krow = p_kcache + (base + kr) * KRB, *vrow = p_vcache + (base + kr) * VRB;
 #pragma unroll
         for (int cc = 0; cc < NC; ++cc) kr_[cc] = kv_load<KT, HD>(krow, 32 * cc + 8 * g);
 #pragma unroll
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) s_o[(wave * HD + 16 * db + 4 * g + i) * 16 + c] = o[db][i];
     __syncthreads();
-    const bool single = a.n_splits == 1;
+    const bool single = p_n_splits == 1;
     for (int idx = tid; idx < G * HD; idx += MMA_THREADS) {
         const int h = idx / HD, dd = idx % HD;
         float mh = -INFINITY;
@@ -235,19 +240,19 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
             sum = fmaf(s_o[(w * HD + dd) * 16 + h], wgt, sum);
             ll = fmaf(s_l[w][h], wgt, ll);
         }
-        const size_t row = (size_t)t * a.n_head + (size_t)kvh * G + h;
+        const size_t row = (size_t)t * p_n_head + (size_t)kvh * G + h;
         if (single) {
             if (a.out16_k8) {
-                const size_t kk = ((size_t)kvh * G + h) * HD + dd, KK = (size_t)a.n_head * HD;
+                const size_t kk = ((size_t)kvh * G + h) * HD + dd, KK = (size_t)p_n_head * HD;
                 a.out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(sum / ll);
             } else {
                 a.out[row * HD + dd] = sum / ll;
             }
         } else {
-            a.part[(row * a.n_splits + split) * HD + dd] = sum;
+            a.part[(row * p_n_splits + split) * HD + dd] = sum;
             if (dd == 0) {
-                a.ml[(row * a.n_splits + split) * 2 + 0] = mh;
-                a.ml[(row * a.n_splits + split) * 2 + 1] = ll;
+                a.ml[(row * p_n_splits + split) * 2 + 0] = mh;
+                a.ml[(row * p_n_splits + split) * 2 + 1] = ll;
             }
         }
     }
@@ -256,9 +261,9 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(AttnArgs a) {
 template <int HD>
 static int launch_mma(const AttnArgs &a, int T, hipStream_t stream) {
     const dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block(MMA_THREADS);
-    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) attn_mma_kernel<HD, MESH_F16, MESH_F16><<<grid, block, 0, stream>>>(a);
-    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q8_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a);
-    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q4_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a);
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) attn_mma_kernel<HD, MESH_F16, MESH_F16><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
+    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q8_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
+    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q4_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
     else return fail(MESH_ERR_UNSUPPORTED, "attention_mma: KV cache types %d/%d", a.k_type, a.v_type);
     MESH_LAUNCH_CHECK();
     return MESH_OK;

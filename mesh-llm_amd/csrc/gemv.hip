@@ -76,6 +76,14 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
 #endif
 
 
+// the body's hot fields straight from the argument block
+#define GEMV_HOT_FROM_ARGS(a)                                                                                  \
+    const float *const h_x = (a).x, *const h_norm_w = (a).norm_w;                                              \
+    const int32_t *const h_expert_ids = (a).expert_ids;                                                        \
+    const uint8_t *const h_wbase0 = (a).wbase[0];                                                              \
+    const int h_K = (a).K, h_ldx = (a).ldx, h_ks = (a).ks, h_rows = (a).tile_begin[3], h_begin1 = (a).tile_begin[1], \
+              h_begin2 = (a).tile_begin[2];
+
 // ------------------------------------------------------------------------------------------------ kernel
 // Work decomposition.  A workgroup owns `rows_here` consecutive tile-rows (16 output rows each) of the launch's
 // matrices (all of one K-quant type) and stages the activations once.  Its 16 waves are arranged KS x RS: wave
@@ -83,8 +91,19 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
 // fused gate/up pair).  A wave walks its tiles as one flat list with the next tile always in flight; at the end of
 // each (tile-row, matrix) segment the lanes' sums are reduced over the 4 lanes of a row and parked in LDS, where the
 // KS partials of a row meet after one barrier.
+// The arguments every wave needs before it can issue its first loads come first and as scalars: the build asks for
+// kernel-argument preloading (-amdgpu-kernarg-preload-count), which delivers the leading scalar arguments in SGPRs at
+// wave start instead of through a scalar load that misses every cache (the argument block was just written by the
+// host).  The struct carries the same fields; the preloaded copies replace them.
 template <int TYPE, int NB, int NU>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const GemvKernelArgs a) {
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x, const int32_t *p_expert_ids, const float *p_norm_w,
+                                                                const uint8_t *p_wbase0, int p_K, int p_ldx, int p_ks, int p_rows,
+                                                                int p_begin1, int p_begin2, const GemvKernelArgs a_in) {
+    const GemvKernelArgs &a = a_in;
+    const float *const h_x = p_x, *const h_norm_w = p_norm_w;
+    const int32_t *const h_expert_ids = p_expert_ids;
+    const uint8_t *const h_wbase0 = p_wbase0;
+    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_begin1, h_begin2 = p_begin2;
     const int bid = blockIdx.x, nblk = gridDim.x;
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
@@ -104,15 +123,19 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const Gem
     const int n = __builtin_amdgcn_readfirstlane(a.items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
     if (n == 4) {
         constexpr int NB = 4;
+        GEMV_HOT_FROM_ARGS(a)
 #include "gemv_body.inc"
     } else if (n == 3) {
         constexpr int NB = 3;
+        GEMV_HOT_FROM_ARGS(a)
 #include "gemv_body.inc"
     } else if (n == 2) {
         constexpr int NB = 2;
+        GEMV_HOT_FROM_ARGS(a)
 #include "gemv_body.inc"
     } else if (n == 1) {
         constexpr int NB = 1;
+        GEMV_HOT_FROM_ARGS(a)
 #include "gemv_body.inc"
     }
 }
@@ -120,7 +143,9 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const Gem
 // q/k/v groups whose matrices are of both K-quant types (attn_v in q6_K on the "more bits" layers of a Q4_K_M
 // file): one launch, the first n4 workgroups run the q4_K matrices, the rest the q6_K ones.
 template <int NB>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const GemvKernelArgs a4, const GemvKernelArgs a6, int n4) {
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_x, const float *p_norm_w, const uint8_t *p_w4, const uint8_t *p_w6,
+                                                                 int p_K, int p_ldx, int n4, int p_ks4, int p_ks6, int p_rows4, int p_rows6,
+                                                                 const GemvKernelArgs a4, const GemvKernelArgs a6) {
     constexpr int NU = 1;
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
@@ -128,11 +153,19 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const GemvKerne
         const GemvKernelArgs &a = a4;
         constexpr int TYPE = MESH_Q4_K;
         const int bid = blockIdx.x, nblk = n4;
+        const float *const h_x = p_x, *const h_norm_w = p_norm_w;
+        const int32_t *const h_expert_ids = nullptr;
+        const uint8_t *const h_wbase0 = p_w4;
+        const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks4, h_rows = p_rows4, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
 #include "gemv_body.inc"
     } else {
         const GemvKernelArgs &a = a6;
         constexpr int TYPE = MESH_Q6_K;
         const int bid = (int)blockIdx.x - n4, nblk = (int)gridDim.x - n4;
+        const float *const h_x = p_x, *const h_norm_w = p_norm_w;
+        const int32_t *const h_expert_ids = nullptr;
+        const uint8_t *const h_wbase0 = p_w6;
+        const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks6, h_rows = p_rows6, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
 #include "gemv_body.inc"
     }
 }
@@ -153,7 +186,8 @@ static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStrea
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dot_kernel<TYPE, NB, NU><<<grid, dim3(GEMV_THREADS), smem, stream>>>(ka);
+    gemv_dot_kernel<TYPE, NB, NU><<<grid, dim3(GEMV_THREADS), smem, stream>>>(ka.x, ka.expert_ids, ka.norm_w, ka.wbase[0], ka.K, ka.ldx, ka.ks,
+                                                                              ka.tile_begin[3], ka.tile_begin[1], ka.tile_begin[2], ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -308,7 +342,8 @@ static int launch_dual(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int n
         MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dual_kernel<NB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dual_kernel<NB><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(k4, k6, n4);
+    gemv_dual_kernel<NB><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(k4.x, k4.norm_w, k4.wbase[0], k6.wbase[0], k4.K, k4.ldx, n4, k4.ks,
+                                                                                          k6.ks, k4.tile_begin[3], k6.tile_begin[3], k4, k6);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
