@@ -197,19 +197,20 @@ __device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_la
 }
 
 template <int TYPE, int NU, int SEGS>
-__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKernelArgs a) {
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, int p_K, int p_ks, int p_rows, const SkinnyKernelArgs a) {
+    // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
     extern __shared__ __align__(16) uint8_t smem[];
     float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
     constexpr int TB = TileRegs<TYPE>::BYTES;
     constexpr int SK_DEPTH = TYPE == MESH_Q4_K ? SK_DEPTH_Q4 : SK_DEPTH_Q6;
-    const int K = a.K, nsb = K / QK_K;
+    const int K = p_K, nsb = K / QK_K;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: tile addresses become SGPR base + lane offset
     const int m = lane & 15, g = lane >> 4;
     const int src_lane4 = 4 * (4 * m + g);                // byte address, for ds_bpermute, of the lane that loaded row m, quarter g
-    const int KS = a.ks, RS = SK_WAVES / KS;
+    const int KS = p_ks, RS = SK_WAVES / KS;
     const int ks = wave % KS, rs = wave / KS;
-    const int total_rows = a.tile_begin[3];
+    const int total_rows = p_rows;
     const int tr0 = (int)(((long long)blockIdx.x * total_rows) / gridDim.x);
     const int tr1 = (int)(((long long)(blockIdx.x + 1) * total_rows) / gridDim.x);
     const int rows_here = tr1 - tr0;
@@ -258,8 +259,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
     if (total > 0) {
 #pragma unroll
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
-        B[0].load(a.x, lane_off, ks);
-        B[1].load(a.x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
+        B[0].load(p_x, lane_off, ks);
+        B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
         if (n_i <= 2 && total <= SK_DEPTH) {
             // short walk: everything it needs is already in flight
 #pragma unroll
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const SkinnyKer
                     // refill this slot with the tile DEPTH positions ahead
                     load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
                     // last segment of a super-block: its activation buffer is free for the one after next
-                    if (seg == SEGS - 1) B[r % 2].load(a.x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
+                    if (seg == SEGS - 1) B[r % 2].load(p_x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
                     __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
                 }
             }
@@ -358,7 +359,7 @@ static int launch_skinny(const SkinnyKernelArgs &ka, int grid, size_t smem, hipS
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka);
+    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka.x, ka.K, ka.ks, ka.tile_begin[3], ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -79,7 +79,7 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
 // the body's hot fields straight from the argument block
 #define GEMV_HOT_FROM_ARGS(a)                                                                                  \
     const float *const h_x = (a).x, *const h_norm_w = (a).norm_w;                                              \
-    const int32_t *const h_expert_ids = (a).expert_ids;                                                        \
+    const int32_t *const h_expert_ids = (a).expert_ids, *const h_items = (a).items;                            \
     const uint8_t *const h_wbase0 = (a).wbase[0];                                                              \
     const int h_K = (a).K, h_ldx = (a).ldx, h_ks = (a).ks, h_rows = (a).tile_begin[3], h_begin1 = (a).tile_begin[1], \
               h_begin2 = (a).tile_begin[2];
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
                                                                 int p_begin1, int p_begin2, const GemvKernelArgs a_in) {
     const GemvKernelArgs &a = a_in;
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-    const int32_t *const h_expert_ids = p_expert_ids;
+    const int32_t *const h_expert_ids = p_expert_ids, *const h_items = nullptr;
     const uint8_t *const h_wbase0 = p_wbase0;
     const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_begin1, h_begin2 = p_begin2;
     const int bid = blockIdx.x, nblk = gridDim.x;
@@ -115,27 +115,35 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
 // dependent start-up loads (work item -> expert -> activations) or in their epilogue.
 constexpr int GROUPED_THREADS = 256;
 template <int TYPE, int NU>
-__global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const GemvKernelArgs a) {
-    if ((int)blockIdx.y >= a.n_items[0]) return;
+__global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int32_t *p_items, const int32_t *p_n_items, const float *p_x,
+                                                                       const float *p_norm_w, const uint8_t *p_wbase0, int p_K, int p_ldx,
+                                                                       int p_ks, int p_rows, const GemvKernelArgs a) {
+    // (leading scalar arguments: preloaded into SGPRs, see gemv_dot_kernel)
+    if ((int)blockIdx.y >= p_n_items[0]) return;
     const int bid = blockIdx.x, nblk = gridDim.x;
     constexpr bool GROUPED = true;
     constexpr int THREADS = GROUPED_THREADS, WAVES = GROUPED_THREADS / 64;
-    const int n = __builtin_amdgcn_readfirstlane(a.items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
+    const int n = __builtin_amdgcn_readfirstlane(p_items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
+#define GEMV_HOT_GROUPED                                                                                   \
+    const float *const h_x = p_x, *const h_norm_w = p_norm_w;                                              \
+    const int32_t *const h_expert_ids = nullptr, *const h_items = p_items;                                 \
+    const uint8_t *const h_wbase0 = p_wbase0;                                                              \
+    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows;
     if (n == 4) {
         constexpr int NB = 4;
-        GEMV_HOT_FROM_ARGS(a)
+        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 3) {
         constexpr int NB = 3;
-        GEMV_HOT_FROM_ARGS(a)
+        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 2) {
         constexpr int NB = 2;
-        GEMV_HOT_FROM_ARGS(a)
+        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 1) {
         constexpr int NB = 1;
-        GEMV_HOT_FROM_ARGS(a)
+        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     }
 }
@@ -154,7 +162,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
         constexpr int TYPE = MESH_Q4_K;
         const int bid = blockIdx.x, nblk = n4;
         const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-        const int32_t *const h_expert_ids = nullptr;
+        const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
         const uint8_t *const h_wbase0 = p_w4;
         const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks4, h_rows = p_rows4, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
 #include "gemv_body.inc"
@@ -163,7 +171,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
         constexpr int TYPE = MESH_Q6_K;
         const int bid = (int)blockIdx.x - n4, nblk = (int)gridDim.x - n4;
         const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-        const int32_t *const h_expert_ids = nullptr;
+        const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
         const uint8_t *const h_wbase0 = p_w6;
         const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks6, h_rows = p_rows6, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
 #include "gemv_body.inc"
@@ -200,7 +208,8 @@ static int launch_grouped(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipS
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(ka);
+    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(ka.items, ka.n_items, ka.x, ka.norm_w, ka.wbase[0], ka.K, ka.ldx, ka.ks,
+                                                                                 ka.tile_begin[3], ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
