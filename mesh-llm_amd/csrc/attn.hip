@@ -13,21 +13,23 @@ namespace mesh {
 // ------------------------------------------------------------------------------------------------ rope + append
 // grid (n_head + 2*n_head_kv, T), one wave per head vector.
 constexpr int ROPE_HD_MAX = 256;
-__global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvArgs a) {
+// (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
+__global__ __launch_bounds__(64) void rope_kv_kernel(const int32_t *p_pos, const int32_t *p_seq, float *p_q, const float *p_k, const float *p_v,
+                                                     int p_n_head, int p_n_kv, int p_head_dim, const RopeKvArgs a) {
     __shared__ float s_vec[ROPE_HD_MAX];         // the finished K / V row before it is stored in the cache type
     const int hh = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
-    const int hd = a.head_dim;
-    const int pos = a.pos[t], seq = a.seq[t];
+    const int hd = p_head_dim;
+    const int pos = p_pos[t], seq = p_seq[t];
     float *vec;
     const float *nw = nullptr;
     int kind, head;
-    if (hh < a.n_head) { kind = 0; head = hh; vec = a.q + ((size_t)t * a.n_head + head) * hd; nw = a.q_norm; }
-    else if (hh < a.n_head + a.n_kv) { kind = 1; head = hh - a.n_head; vec = const_cast<float *>(a.k) + ((size_t)t * a.n_kv + head) * hd; nw = a.k_norm; }
-    else { kind = 2; head = hh - a.n_head - a.n_kv; vec = const_cast<float *>(a.v) + ((size_t)t * a.n_kv + head) * hd; }
+    if (hh < p_n_head) { kind = 0; head = hh; vec = p_q + ((size_t)t * p_n_head + head) * hd; nw = a.q_norm; }
+    else if (hh < p_n_head + p_n_kv) { kind = 1; head = hh - p_n_head; vec = const_cast<float *>(p_k) + ((size_t)t * p_n_kv + head) * hd; nw = a.k_norm; }
+    else { kind = 2; head = hh - p_n_head - p_n_kv; vec = const_cast<float *>(p_v) + ((size_t)t * p_n_kv + head) * hd; }
 
     const int ctype = kind == 1 ? a.k_type : a.v_type;
     uint8_t *row = nullptr;
-    if (kind) row = (kind == 1 ? a.kcache : a.vcache) + (((size_t)seq * a.n_kv + head) * a.n_ctx + pos) * (size_t)kv_row_bytes(ctype, hd);
+    if (kind) row = (kind == 1 ? a.kcache : a.vcache) + (((size_t)seq * p_n_kv + head) * a.n_ctx + pos) * (size_t)kv_row_bytes(ctype, hd);
 
     if (kind == 2) {
         for (int i = lane; i < hd; i += 64) s_vec[i] = vec[i];
@@ -76,7 +78,7 @@ int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream) {
         return fail(MESH_ERR_INVALID, "rope: bad head_dim/n_rot %d/%d", a.head_dim, a.n_rot);
     if (!kv_type_supported(a.k_type) || !kv_type_supported(a.v_type) || ((a.k_type != MESH_F16 || a.v_type != MESH_F16) && a.head_dim % 32))
         return fail(MESH_ERR_UNSUPPORTED, "rope: KV cache types %d/%d with head_dim %d", a.k_type, a.v_type, a.head_dim);
-    rope_kv_kernel<<<dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream>>>(a);
+    rope_kv_kernel<<<dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream>>>(a.pos, a.seq, a.q, a.k, a.v, a.n_head, a.n_kv, a.head_dim, a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -92,9 +92,10 @@ __global__ __launch_bounds__(64) void moe_route_kernel(MoeRouteArgs a) {
 // moe_route_group_kernel): small batches then have enough workgroups to pull the router matrix through quickly.
 constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64;
 template <int NV>      // float4 groups per lane = E / 256
-__global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(MoeRouteArgs a, const float *__restrict__ x, int ldx,
-                                                                          const float *__restrict__ norm_w, float eps,
-                                                                          const float *__restrict__ W, float *__restrict__ logits_out) {
+// (scalar arguments first: preloaded into SGPRs, see gemv.hip)
+__global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+                                                                          const float *__restrict__ W, float *__restrict__ logits_out,
+                                                                          int ldx, float eps, const MoeRouteArgs a) {
     constexpr int E = NV * 256;
     __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -157,10 +158,10 @@ int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float
     if (!moe_router_fused_supported(E, a.n_expert, a.top_k)) return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d / %d experts", E, a.n_expert);
     const dim3 grid((unsigned)T), block(ROUTER_THREADS);
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(a, x, ldx, norm_w, eps, W, logits_out); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(a, x, ldx, norm_w, eps, W, logits_out); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(a, x, ldx, norm_w, eps, W, logits_out); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(a, x, ldx, norm_w, eps, W, logits_out); break;
+        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
+        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
+        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
+        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
@@ -248,8 +249,8 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t 
 // Routing of a small batch and the grouping of its pairs in one single-workgroup launch: wave w routes tokens w,
 // w + 16, ... from their logits, then the workgroup groups the pairs it has just written (the barrier in between
 // also makes those writes visible to the whole workgroup).
-__global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(MoeRouteArgs a, int T, int32_t *__restrict__ items,
-                                                                        int32_t *__restrict__ n_items) {
+__global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(int T, int32_t *__restrict__ items, int32_t *__restrict__ n_items,
+                                                                        const MoeRouteArgs a) {
     extern __shared__ int32_t g_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(a.logits + (size_t)t * a.n_expert, a, t, lane);
@@ -266,16 +267,16 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
     const dim3 grid((unsigned)T, (unsigned)split), block(ROUTER_THREADS);
     MoeRouteArgs la = a;
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(la, x, ldx, norm_w, eps, W, logits); break;
+        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
+        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
+        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
+        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
     la.logits = logits;
     const size_t smem = ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
-    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(la, T, items, n_items);
+    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(T, items, n_items, la);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
