@@ -76,13 +76,16 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
 #endif
 
 
+// rows per workgroup by division (kernels that do not get them from the host)
+#define GEMV_HOT_SPLIT const int h_q = (int)((unsigned)h_rows / (unsigned)nblk), h_r = h_rows - h_q * nblk;
 // the body's hot fields straight from the argument block
 #define GEMV_HOT_FROM_ARGS(a)                                                                                  \
     const float *const h_x = (a).x, *const h_norm_w = (a).norm_w;                                              \
     const int32_t *const h_expert_ids = (a).expert_ids, *const h_items = (a).items;                            \
-    const uint8_t *const h_wbase0 = (a).wbase[0];                                                              \
+    const uint8_t *const h_wbase0 = (a).wbase[0], *const h_wbase1 = (a).wbase[1], *const h_wbase2 = (a).wbase[2]; \
     const int h_K = (a).K, h_ldx = (a).ldx, h_ks = (a).ks, h_rows = (a).tile_begin[3], h_begin1 = (a).tile_begin[1], \
-              h_begin2 = (a).tile_begin[2];
+              h_begin2 = (a).tile_begin[2];                                                                    \
+    GEMV_HOT_SPLIT
 
 // ------------------------------------------------------------------------------------------------ kernel
 // Work decomposition.  A workgroup owns `rows_here` consecutive tile-rows (16 output rows each) of the launch's
@@ -95,16 +98,23 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
 // kernel-argument preloading (-amdgpu-kernarg-preload-count), which delivers the leading scalar arguments in SGPRs at
 // wave start instead of through a scalar load that misses every cache (the argument block was just written by the
 // host).  The struct carries the same fields; the preloaded copies replace them.
-template <int TYPE, int NB, int NU>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x, const int32_t *p_expert_ids, const float *p_norm_w,
-                                                                const uint8_t *p_wbase0, int p_K, int p_ldx, int p_ks, int p_rows,
-                                                                int p_begin1, int p_begin2, const GemvKernelArgs a_in) {
+// Fourteen dwords can be preloaded: the small integers travel packed (p_ldx_grid = ldx | gridDim.x << 16, p_rows_q =
+// total tile-rows | tile-rows per workgroup << 16, p_begins = first tile-row of matrix 1 | of matrix 2 << 16,
+// p_r_nsb_ks = workgroups with one tile-row more | K / 256 << 16 | waves along K << 24), and whether the launch uses the per-pair expert
+// indirection is a template parameter, so that the dense kernel does not wait for a pointer only to find it null.
+template <int TYPE, int NB, int NU, bool EXPERT>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x, const float *p_norm_w, const uint8_t *p_wbase0,
+                                                                const uint8_t *p_wbase1, const uint8_t *p_wbase2, unsigned p_ldx_grid,
+                                                                unsigned p_rows_q, unsigned p_begins, unsigned p_r_nsb_ks,
+                                                                const GemvKernelArgs a_in) {
     const GemvKernelArgs &a = a_in;
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-    const int32_t *const h_expert_ids = p_expert_ids, *const h_items = nullptr;
-    const uint8_t *const h_wbase0 = p_wbase0;
-    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_begin1, h_begin2 = p_begin2;
-    const int bid = blockIdx.x, nblk = gridDim.x;
+    const int32_t *const h_expert_ids = EXPERT ? a.expert_ids : nullptr, *const h_items = nullptr;
+    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = p_wbase1, *const h_wbase2 = p_wbase2;
+    const int h_K = (int)((p_r_nsb_ks >> 16) & 0xFFu) * QK_K, h_ldx = (int)(p_ldx_grid & 0xFFFFu), h_ks = (int)(p_r_nsb_ks >> 24),
+              h_rows = (int)(p_rows_q & 0xFFFFu), h_begin1 = (int)(p_begins & 0xFFFFu), h_begin2 = (int)(p_begins >> 16),
+              h_q = (int)(p_rows_q >> 16), h_r = (int)(p_r_nsb_ks & 0xFFFFu);
+    const int bid = blockIdx.x, nblk = (int)(p_ldx_grid >> 16);        // (gridDim.x would be one more load from the argument block)
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
 #include "gemv_body.inc"
@@ -127,8 +137,9 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int
 #define GEMV_HOT_GROUPED                                                                                   \
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;                                              \
     const int32_t *const h_expert_ids = nullptr, *const h_items = p_items;                                 \
-    const uint8_t *const h_wbase0 = p_wbase0;                                                              \
-    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows;
+    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2]; \
+    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows; \
+    GEMV_HOT_SPLIT
     if (n == 4) {
         constexpr int NB = 4;
         GEMV_HOT_GROUPED
@@ -163,8 +174,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
         const int bid = blockIdx.x, nblk = n4;
         const float *const h_x = p_x, *const h_norm_w = p_norm_w;
         const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
-        const uint8_t *const h_wbase0 = p_w4;
+        const uint8_t *const h_wbase0 = p_w4, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2];
         const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks4, h_rows = p_rows4, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
+        GEMV_HOT_SPLIT
 #include "gemv_body.inc"
     } else {
         const GemvKernelArgs &a = a6;
@@ -172,8 +184,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
         const int bid = (int)blockIdx.x - n4, nblk = (int)gridDim.x - n4;
         const float *const h_x = p_x, *const h_norm_w = p_norm_w;
         const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
-        const uint8_t *const h_wbase0 = p_w6;
+        const uint8_t *const h_wbase0 = p_w6, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2];
         const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks6, h_rows = p_rows6, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
+        GEMV_HOT_SPLIT
 #include "gemv_body.inc"
     }
 }
@@ -186,16 +199,21 @@ static size_t dot_smem_bytes(int type, int NB, int K, int rows_here, int KS, int
            sizeof(float) * ((size_t)KS * rows_here * NU * 16 * NB + waves * NB);
 }
 
-template <int TYPE, int NB, int NU>
+template <int TYPE, int NB, int NU, bool EXPERT = false>
 static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
+    if (ka.tile_begin[3] > 0xFFFF || ka.ldx > 0xFFFF || grid.x > 0xFFFFu || ka.K / QK_K > 0xFF)
+        return fail(MESH_ERR_UNSUPPORTED, "gemv: %d tile-rows / activation stride %d / %u workgroups / row length %d in one launch",
+                    ka.tile_begin[3], ka.ldx, grid.x, ka.K);
+    const unsigned rows = (unsigned)ka.tile_begin[3], q = rows / grid.x, r = rows % grid.x;
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dot_kernel<TYPE, NB, NU>),
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dot_kernel<TYPE, NB, NU, EXPERT>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dot_kernel<TYPE, NB, NU><<<grid, dim3(GEMV_THREADS), smem, stream>>>(ka.x, ka.expert_ids, ka.norm_w, ka.wbase[0], ka.K, ka.ldx, ka.ks,
-                                                                              ka.tile_begin[3], ka.tile_begin[1], ka.tile_begin[2], ka);
+    gemv_dot_kernel<TYPE, NB, NU, EXPERT><<<grid, dim3(GEMV_THREADS), smem, stream>>>(
+        ka.x, ka.norm_w, ka.wbase[0], ka.wbase[1], ka.wbase[2], (unsigned)ka.ldx | (grid.x << 16), rows | (q << 16),
+        (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), r | ((unsigned)(ka.K / QK_K) << 16) | ((unsigned)ka.ks << 24), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -266,7 +284,8 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p, int waves = GE
     ka.ldres = a.ldres;
     ka.epi = a.epi;
     ka.rope = a.rope;
-    int KS = nsb < waves ? nsb : waves;
+    int KS = 1;
+    while (KS * 2 <= nsb && KS * 2 <= waves) KS *= 2;      // a power of two: the kernel splits its waves with shifts
     if (waves != GEMV_WAVES) {
         // half-size workgroups: every wave gets work only if KS divides the waves, evenly only if it divides the row too
         KS = 1;
@@ -280,6 +299,7 @@ static int plan_kquant(const GemvArgs &a, int ncu, KquantPlan &p, int waves = GE
     p.grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
     p.rows_max = (total_rows + p.grid - 1) / p.grid;
     p.type = type; p.NU = NU; p.KS = KS;
+    if (total_rows > 0xFFFF || p.grid > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemv: %d tile-rows over %d workgroups in one launch", total_rows, p.grid);
     if (dot_smem_bytes(type, 1, a.K, p.rows_max, KS, NU) > LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemv: row length %d does not fit LDS", a.K);
     return MESH_OK;
 }
@@ -319,8 +339,8 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
         ka.x = a.x;
         const size_t smem = dot_smem_bytes(type, 1, a.K, rows_max, KS, NU);
         const dim3 g((unsigned)grid, (unsigned)n_pairs);
-        if (type == MESH_Q4_K) return NU == 2 ? launch_dot_nb<MESH_Q4_K, 2>(1, ka, g, smem, stream) : launch_dot_nb<MESH_Q4_K, 1>(1, ka, g, smem, stream);
-        return NU == 2 ? launch_dot_nb<MESH_Q6_K, 2>(1, ka, g, smem, stream) : launch_dot_nb<MESH_Q6_K, 1>(1, ka, g, smem, stream);
+        if (type == MESH_Q4_K) return NU == 2 ? launch_dot<MESH_Q4_K, 1, 2, true>(ka, g, smem, stream) : launch_dot<MESH_Q4_K, 1, 1, true>(ka, g, smem, stream);
+        return NU == 2 ? launch_dot<MESH_Q6_K, 1, 2, true>(ka, g, smem, stream) : launch_dot<MESH_Q6_K, 1, 1, true>(ka, g, smem, stream);
     }
     int t = 0;
     while (t < a.T) {
