@@ -161,31 +161,36 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int
 
 // q/k/v groups whose matrices are of both K-quant types (attn_v in q6_K on the "more bits" layers of a Q4_K_M
 // file): one launch, the first n4 workgroups run the q4_K matrices, the rest the q6_K ones.
-template <int NB>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_x, const float *p_norm_w, const uint8_t *p_w4, const uint8_t *p_w6,
-                                                                 int p_K, int p_ldx, int n4, int p_ks4, int p_ks6, int p_rows4, int p_rows6,
-                                                                 const GemvKernelArgs a4, const GemvKernelArgs a6) {
+// Preloaded (see gemv_dot_kernel): the activations, both bases of the q4_K part, the first base of the q6_K part and
+// the packed integers p_ldx_n4 = ldx | n4 << 16, p_rows = tile-rows of the q4_K part | of the q6_K part << 16,
+// p_begin_grid = first tile-row of the q4_K part's second matrix | gridDim.x << 16, p_nsb_ks = K / 256 | waves along K
+// << 8.  SIMPLE: the q4_K part has at most two matrices and the q6_K part one (q, k | v, the usual case), so nothing
+// else is needed before the first weight load; otherwise the remaining bases and boundaries come from the structs.
+template <int NB, bool SIMPLE>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_x, const float *p_norm_w, const uint8_t *p_w4, const uint8_t *p_w4b,
+                                                                 const uint8_t *p_w6, unsigned p_ldx_n4, unsigned p_rows, unsigned p_begin_grid,
+                                                                 unsigned p_nsb_ks, const GemvKernelArgs a4, const GemvKernelArgs a6) {
     constexpr int NU = 1;
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
+    const int n4 = (int)(p_ldx_n4 >> 16);
+    const float *const h_x = p_x, *const h_norm_w = p_norm_w;
+    const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
+    const int h_K = (int)(p_nsb_ks & 0xFFu) * QK_K, h_ldx = (int)(p_ldx_n4 & 0xFFFFu), h_ks = (int)(p_nsb_ks >> 8);
     if ((int)blockIdx.x < n4) {
         const GemvKernelArgs &a = a4;
         constexpr int TYPE = MESH_Q4_K;
         const int bid = blockIdx.x, nblk = n4;
-        const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-        const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
-        const uint8_t *const h_wbase0 = p_w4, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2];
-        const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks4, h_rows = p_rows4, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
+        const int h_rows = (int)(p_rows & 0xFFFFu), h_begin1 = (int)(p_begin_grid & 0xFFFFu), h_begin2 = SIMPLE ? h_rows : a.tile_begin[2];
+        const uint8_t *const h_wbase0 = p_w4, *const h_wbase1 = p_w4b, *const h_wbase2 = SIMPLE ? p_w4b : a.wbase[2];
         GEMV_HOT_SPLIT
 #include "gemv_body.inc"
     } else {
         const GemvKernelArgs &a = a6;
         constexpr int TYPE = MESH_Q6_K;
-        const int bid = (int)blockIdx.x - n4, nblk = (int)gridDim.x - n4;
-        const float *const h_x = p_x, *const h_norm_w = p_norm_w;
-        const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
-        const uint8_t *const h_wbase0 = p_w6, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2];
-        const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks6, h_rows = p_rows6, h_begin1 = a.tile_begin[1], h_begin2 = a.tile_begin[2];
+        const int bid = (int)blockIdx.x - n4, nblk = (int)(p_begin_grid >> 16) - n4;
+        const int h_rows = (int)(p_rows >> 16), h_begin1 = SIMPLE ? h_rows : a.tile_begin[1], h_begin2 = SIMPLE ? h_rows : a.tile_begin[2];
+        const uint8_t *const h_wbase0 = p_w6, *const h_wbase1 = SIMPLE ? p_w6 : a.wbase[1], *const h_wbase2 = SIMPLE ? p_w6 : a.wbase[2];
         GEMV_HOT_SPLIT
 #include "gemv_body.inc"
     }
@@ -364,19 +369,27 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     return MESH_OK;
 }
 
-template <int NB>
-static int launch_dual(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int n4, int n6, size_t smem, hipStream_t stream) {
+template <int NB, bool SIMPLE>
+static int launch_dual2(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int n4, int n6, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dual_kernel<NB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dual_kernel<NB, SIMPLE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dual_kernel<NB><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(k4.x, k4.norm_w, k4.wbase[0], k6.wbase[0], k4.K, k4.ldx, n4, k4.ks,
-                                                                                          k6.ks, k4.tile_begin[3], k6.tile_begin[3], k4, k6);
+    gemv_dual_kernel<NB, SIMPLE><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(
+        k4.x, k4.norm_w, k4.wbase[0], k4.wbase[1], k6.wbase[0], (unsigned)k4.ldx | ((unsigned)n4 << 16),
+        (unsigned)k4.tile_begin[3] | ((unsigned)k6.tile_begin[3] << 16), (unsigned)k4.tile_begin[1] | ((unsigned)(n4 + n6) << 16),
+        (unsigned)(k4.K / QK_K) | ((unsigned)k4.ks << 8), k4, k6);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
-
+template <int NB>
+static int launch_dual(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int n4, int n6, size_t smem, hipStream_t stream) {
+    if (k4.ldx > 0xFFFF || k4.K / QK_K > 0xFF || k4.ks != k6.ks || n4 + n6 > 0xFFFF || k4.tile_begin[3] > 0xFFFF || k6.tile_begin[3] > 0xFFFF)
+        return fail(MESH_ERR_UNSUPPORTED, "gemv: two-type launch outside its packed argument ranges");
+    const bool simple = k4.n_mat <= 2 && k6.n_mat == 1;
+    return simple ? launch_dual2<NB, true>(k4, k6, n4, n6, smem, stream) : launch_dual2<NB, false>(k4, k6, n4, n6, smem, stream);
+}
 // a4: the q4_K matrices of a group, a6: its q6_K matrices; same activations, plain store epilogue
 static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream) {
     const int ncu = n_compute_units();
