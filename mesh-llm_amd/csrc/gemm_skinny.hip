@@ -197,7 +197,9 @@ __device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_la
 }
 
 template <int TYPE, int NU, int SEGS>
-__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, int p_K, int p_ks, int p_rows, const SkinnyKernelArgs a) {
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+                                                                 int p_ks, int p_rows, unsigned p_begins, const SkinnyKernelArgs a) {
+    const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
     // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
     extern __shared__ __align__(16) uint8_t smem[];
     float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
@@ -223,10 +225,10 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     auto tile_ptr = [&](int ii, int seg) -> const uint8_t * {
         const int tr = tr0 + rs + RS * (seg / NU);
         int mi = seg % NU;
-        if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
-        // (selected, not indexed: a dynamically indexed kernel-argument array is fetched with a load, and waiting for
-        // that address would drain every tile load in flight)
-        const uint8_t *wb = mi == 0 ? a.wbase[0] : mi == 1 ? a.wbase[1] : a.wbase[2];
+        if (NU == 1) mi = (tr >= p_begin1 ? 1 : 0) + (tr >= p_begin2 ? 1 : 0);
+        // (offsets added under conditions: an indexed kernel-argument array is fetched with a load, and a three-way
+        // select of preloaded pointers becomes a table in scratch memory)
+        const uint8_t *wb = p_w0 + (mi >= 1 ? p_w1 - p_w0 : (ptrdiff_t)0) + (mi >= 2 ? p_w2 - p_w1 : (ptrdiff_t)0);
         return wb + (size_t)tr * row_stride + (size_t)(ks + KS * ii) * TB;
     };
     // flat tile index f = ii * SEGS + seg, invalid segments included as bubbles; a wave without a valid first
@@ -359,7 +361,8 @@ static int launch_skinny(const SkinnyKernelArgs &ka, int grid, size_t smem, hipS
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka.x, ka.K, ka.ks, ka.tile_begin[3], ka);
+    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka.x, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks,
+                                                                                                 ka.tile_begin[3], (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -417,6 +420,7 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     const int rows_max = (total_rows + grid - 1) / grid;
     const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
     if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d segments per wave", segs);
+    if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d tile-rows in one launch", total_rows);
     const size_t smem = sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
     if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: reduction buffer of %zu bytes does not fit LDS", smem);
     for (int t = 0; t < a.T; t += SK_NT) {
