@@ -84,7 +84,8 @@ extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
     const int32_t *const h_expert_ids = (a).expert_ids, *const h_items = (a).items;                            \
     const uint8_t *const h_wbase0 = (a).wbase[0], *const h_wbase1 = (a).wbase[1], *const h_wbase2 = (a).wbase[2]; \
     const int h_K = (a).K, h_ldx = (a).ldx, h_ks = (a).ks, h_rows = (a).tile_begin[3], h_begin1 = (a).tile_begin[1], \
-              h_begin2 = (a).tile_begin[2];                                                                    \
+              h_begin2 = (a).tile_begin[2], h_x_div = (a).x_div;                                               \
+    const size_t h_expert_stride = (a).expert_stride;                                                          \
     GEMV_HOT_SPLIT
 
 // ------------------------------------------------------------------------------------------------ kernel
@@ -113,7 +114,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
     const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = p_wbase1, *const h_wbase2 = p_wbase2;
     const int h_K = (int)((p_r_nsb_ks >> 16) & 0xFFu) * QK_K, h_ldx = (int)(p_ldx_grid & 0xFFFFu), h_ks = (int)(p_r_nsb_ks >> 24),
               h_rows = (int)(p_rows_q & 0xFFFFu), h_begin1 = (int)(p_begins & 0xFFFFu), h_begin2 = (int)(p_begins >> 16),
-              h_q = (int)(p_rows_q >> 16), h_r = (int)(p_r_nsb_ks & 0xFFFFu);
+              h_q = (int)(p_rows_q >> 16), h_r = (int)(p_r_nsb_ks & 0xFFFFu), h_x_div = EXPERT ? a.x_div : 1;
+    const size_t h_expert_stride = EXPERT ? a.expert_stride : 0;
     const int bid = blockIdx.x, nblk = (int)(p_ldx_grid >> 16);        // (gridDim.x would be one more load from the argument block)
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
@@ -126,9 +128,14 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
 constexpr int GROUPED_THREADS = 256;
 template <int TYPE, int NU>
 __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int32_t *p_items, const int32_t *p_n_items, const float *p_x,
-                                                                       const float *p_norm_w, const uint8_t *p_wbase0, int p_K, int p_ldx,
-                                                                       int p_ks, int p_rows, const GemvKernelArgs a) {
-    // (leading scalar arguments: preloaded into SGPRs, see gemv_dot_kernel)
+                                                                       const float *p_norm_w, const uint8_t *p_wbase0, unsigned p_nsb_ks_rows,
+                                                                       unsigned p_ldx_xdiv, unsigned p_expert_stride, int p_w1_delta,
+                                                                       const GemvKernelArgs a) {
+    // (leading scalar arguments, preloaded into SGPRs, see gemv_dot_kernel: p_nsb_ks_rows = K / 256 | waves along K << 8 |
+    // tile-rows << 16, p_ldx_xdiv = ldx | x_div << 16, the expert stride in bytes, and the second matrix's base as a
+    // distance from the first in units of 256 bytes)
+    const int p_K = (int)(p_nsb_ks_rows & 0xFFu) * QK_K, p_ks = (int)((p_nsb_ks_rows >> 8) & 0xFFu), p_rows = (int)(p_nsb_ks_rows >> 16);
+    const int p_ldx = (int)(p_ldx_xdiv & 0xFFFFu);
     if ((int)blockIdx.y >= p_n_items[0]) return;
     const int bid = blockIdx.x, nblk = gridDim.x;
     constexpr bool GROUPED = true;
@@ -137,8 +144,10 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int
 #define GEMV_HOT_GROUPED                                                                                   \
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;                                              \
     const int32_t *const h_expert_ids = nullptr, *const h_items = p_items;                                 \
-    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = a.wbase[1], *const h_wbase2 = a.wbase[2]; \
-    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows; \
+    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = p_wbase0 + (ptrdiff_t)p_w1_delta * 256, *const h_wbase2 = h_wbase1; \
+    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows, \
+              h_x_div = (int)(p_ldx_xdiv >> 16);                                                           \
+    const size_t h_expert_stride = p_expert_stride;                                                        \
     GEMV_HOT_SPLIT
     if (n == 4) {
         constexpr int NB = 4;
@@ -176,7 +185,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
     const int n4 = (int)(p_ldx_n4 >> 16);
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;
     const int32_t *const h_expert_ids = nullptr, *const h_items = nullptr;
-    const int h_K = (int)(p_nsb_ks & 0xFFu) * QK_K, h_ldx = (int)(p_ldx_n4 & 0xFFFFu), h_ks = (int)(p_nsb_ks >> 8);
+    const int h_K = (int)(p_nsb_ks & 0xFFu) * QK_K, h_ldx = (int)(p_ldx_n4 & 0xFFFFu), h_ks = (int)(p_nsb_ks >> 8), h_x_div = 1;
+    const size_t h_expert_stride = 0;
     if ((int)blockIdx.x < n4) {
         const GemvKernelArgs &a = a4;
         constexpr int TYPE = MESH_Q4_K;
@@ -231,8 +241,13 @@ static int launch_grouped(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipS
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(ka.items, ka.n_items, ka.x, ka.norm_w, ka.wbase[0], ka.K, ka.ldx, ka.ks,
-                                                                                 ka.tile_begin[3], ka);
+    const ptrdiff_t w1d = ka.wbase[1] ? ka.wbase[1] - ka.wbase[0] : 0;
+    if (ka.K / QK_K > 0xFF || ka.tile_begin[3] > 0xFFFF || ka.ldx > 0xFFFF || ka.x_div > 0xFFFF || ka.expert_stride > 0xFFFFFFFFull || (w1d & 255) ||
+        w1d / 256 > INT32_MAX || w1d / 256 < INT32_MIN)
+        return fail(MESH_ERR_UNSUPPORTED, "gemv: grouped expert launch outside its packed argument ranges");
+    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(
+        ka.items, ka.n_items, ka.x, ka.norm_w, ka.wbase[0], (unsigned)(ka.K / QK_K) | ((unsigned)ka.ks << 8) | ((unsigned)ka.tile_begin[3] << 16),
+        (unsigned)ka.ldx | ((unsigned)ka.x_div << 16), (unsigned)ka.expert_stride, (int)(w1d / 256), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
