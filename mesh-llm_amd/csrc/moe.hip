@@ -95,7 +95,7 @@ template <int NV>      // float4 groups per lane = E / 256
 // (scalar arguments first: preloaded into SGPRs, see gemv.hip)
 __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
                                                                           const float *__restrict__ W, float *__restrict__ logits_out,
-                                                                          int ldx, float eps, const MoeRouteArgs a) {
+                                                                          int ldx, float eps, int p_n_expert, const MoeRouteArgs a) {
     constexpr int E = NV * 256;
     __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -118,8 +118,8 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(const 
         xr[i].z = xr[i].z * scale * w.z; xr[i].w = xr[i].w * scale * w.w;
     }
     // two expert rows per step, all of their loads in flight together
-    const int per = (a.n_expert + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int e_lo = (int)blockIdx.y * per, e_hi = e_lo + per < a.n_expert ? e_lo + per : a.n_expert;
+    const int per = (p_n_expert + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int e_lo = (int)blockIdx.y * per, e_hi = e_lo + per < p_n_expert ? e_lo + per : p_n_expert;
     for (int e0 = e_lo + wave; e0 < e_hi; e0 += 2 * ROUTER_WAVES) {
         const int e1 = e0 + ROUTER_WAVES;
         const bool has1 = e1 < e_hi;
@@ -140,10 +140,10 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(const 
         for (int o = 32; o > 0; o >>= 1) { a0 += __shfl_xor(a0, o); a1 += __shfl_xor(a1, o); }
         if (lane == 0) {
             s_logits[e0] = a0;
-            if (logits_out) logits_out[(size_t)t * a.n_expert + e0] = a0;
+            if (logits_out) logits_out[(size_t)t * p_n_expert + e0] = a0;
             if (has1) {
                 s_logits[e1] = a1;
-                if (logits_out) logits_out[(size_t)t * a.n_expert + e1] = a1;
+                if (logits_out) logits_out[(size_t)t * p_n_expert + e1] = a1;
             }
         }
     }
@@ -158,10 +158,10 @@ int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float
     if (!moe_router_fused_supported(E, a.n_expert, a.top_k)) return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d / %d experts", E, a.n_expert);
     const dim3 grid((unsigned)T), block(ROUTER_THREADS);
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a); break;
+        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
@@ -249,13 +249,17 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t 
 // Routing of a small batch and the grouping of its pairs in one single-workgroup launch: wave w routes tokens w,
 // w + 16, ... from their logits, then the workgroup groups the pairs it has just written (the barrier in between
 // also makes those writes visible to the whole workgroup).
-__global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(int T, int32_t *__restrict__ items, int32_t *__restrict__ n_items,
-                                                                        const MoeRouteArgs a) {
+// (the routing arguments as leading scalars: preloaded into SGPRs, see gemv.hip)
+__global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(const float *p_logits, const float *p_mask, int32_t *p_ids, float *p_weights,
+                                                                        int T, int p_n_expert, int p_top_k, int p_norm_w,
+                                                                        int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
     extern __shared__ int32_t g_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(a.logits + (size_t)t * a.n_expert, a, t, lane);
+    MoeRouteArgs a;
+    a.logits = p_logits; a.mask = p_mask; a.ids = p_ids; a.weights = p_weights; a.n_expert = p_n_expert; a.top_k = p_top_k; a.norm_w = p_norm_w;
+    for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(p_logits + (size_t)t * p_n_expert, a, t, lane);
     __syncthreads();
-    group_pairs(a.ids, T * a.top_k, a.n_expert, items, n_items, g_lds);
+    group_pairs(p_ids, T * p_top_k, p_n_expert, items, n_items, g_lds);
 }
 
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
@@ -267,16 +271,17 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
     const dim3 grid((unsigned)T, (unsigned)split), block(ROUTER_THREADS);
     MoeRouteArgs la = a;
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la); break;
+        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
     la.logits = logits;
     const size_t smem = ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
-    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(T, items, n_items, la);
+    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(la.logits, la.mask, la.ids, la.weights, T, la.n_expert, la.top_k, la.norm_w,
+                                                                           items, n_items);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
