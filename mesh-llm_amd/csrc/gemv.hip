@@ -116,7 +116,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
               h_rows = (int)(p_rows_q & 0xFFFFu), h_begin1 = (int)(p_begins & 0xFFFFu), h_begin2 = (int)(p_begins >> 16),
               h_q = (int)(p_rows_q >> 16), h_r = (int)(p_r_nsb_ks & 0xFFFFu), h_x_div = EXPERT ? a.x_div : 1;
     const size_t h_expert_stride = EXPERT ? a.expert_stride : 0;
-    const int bid = blockIdx.x, nblk = (int)(p_ldx_grid >> 16);        // (gridDim.x would be one more load from the argument block)
+    (void)h_rows;
+    const int bid = blockIdx.x;      // (the workgroup count is folded into h_q / h_r: gridDim.x would be one more load from the argument block)
     constexpr bool GROUPED = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
 #include "gemv_body.inc"
@@ -141,29 +142,23 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int
     constexpr bool GROUPED = true;
     constexpr int THREADS = GROUPED_THREADS, WAVES = GROUPED_THREADS / 64;
     const int n = __builtin_amdgcn_readfirstlane(p_items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
-#define GEMV_HOT_GROUPED                                                                                   \
-    const float *const h_x = p_x, *const h_norm_w = p_norm_w;                                              \
-    const int32_t *const h_expert_ids = nullptr, *const h_items = p_items;                                 \
-    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = p_wbase0 + (ptrdiff_t)p_w1_delta * 256, *const h_wbase2 = h_wbase1; \
-    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows, \
-              h_x_div = (int)(p_ldx_xdiv >> 16);                                                           \
-    const size_t h_expert_stride = p_expert_stride;                                                        \
+    const float *const h_x = p_x, *const h_norm_w = p_norm_w;
+    const int32_t *const h_expert_ids = nullptr, *const h_items = p_items;
+    const uint8_t *const h_wbase0 = p_wbase0, *const h_wbase1 = p_wbase0 + (ptrdiff_t)p_w1_delta * 256, *const h_wbase2 = h_wbase1;
+    const int h_K = p_K, h_ldx = p_ldx, h_ks = p_ks, h_rows = p_rows, h_begin1 = p_rows, h_begin2 = p_rows, h_x_div = (int)(p_ldx_xdiv >> 16);
+    const size_t h_expert_stride = p_expert_stride;
     GEMV_HOT_SPLIT
     if (n == 4) {
         constexpr int NB = 4;
-        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 3) {
         constexpr int NB = 3;
-        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 2) {
         constexpr int NB = 2;
-        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     } else if (n == 1) {
         constexpr int NB = 1;
-        GEMV_HOT_GROUPED
 #include "gemv_body.inc"
     }
 }
