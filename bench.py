@@ -142,6 +142,7 @@ STAGE_LAYERS = 16
 # bytes of one head_dim-128 cache row: f16, q8_0 (32 x 34-byte blocks' worth: 128 quants + 4 scales), q4_0 (64 + 8)
 HD_BYTES_F16, HD_BYTES_Q8_0, HD_BYTES_Q4_0 = 256, 136, 72
 PREFILL_T = 2048
+BURN_IN_SECONDS = 2.0
 
 
 def build_stage_model(models, path):
@@ -204,16 +205,22 @@ def bench_stage(args):
             ses.kv_write(il, s, 0, kv, kv)
     kv_bytes_per_seq = STAGE_LAYERS * N_CTX * HK * (kv_row[kv_types[0]] + kv_row[kv_types[1]])
     stream = torch.cuda.ExternalStream(ses.stream)
-    # Burn-in, outside every timed region: the first ~10-20 thousand kernel launches of a process contain a one-time
-    # stall of ~35 ms (seen at a fixed launch count whatever kernel is running), which would otherwise land in
-    # whichever batch size happens to be measured at that moment.
-    for B in batches:
-        xb = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
-        ob = torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")
-        for _ in range(args.burn_in):
-            ses.decode_dev(xb.data_ptr(), np.full(B, N_CTX - 1, np.int32), ob.data_ptr(), ob.numel(), seq=np.arange(B, dtype=np.int32),
-                           in_fmt=m.F32, out_fmt=m.Q8_0)
-    stream.synchronize()
+    # Burn-in, outside every timed region: the first second or so of a process's decode work contains a one-time
+    # stall of ~35 ms (whatever kernel is running; its position follows elapsed time rather than the launch count),
+    # which would otherwise land in whichever batch size happens to be measured at that moment.  Every batch size
+    # runs --burn-in steps, and the whole burn-in lasts at least BURN_IN_SECONDS.
+    burn = [(B, torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda(),
+             torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")) for B in batches]
+    t_burn = time.perf_counter()
+    rounds = 0
+    while rounds < 1 or (args.burn_in > 0 and time.perf_counter() - t_burn < BURN_IN_SECONDS):
+        for B, xb, ob in burn:
+            for _ in range(args.burn_in):
+                ses.decode_dev(xb.data_ptr(), np.full(B, N_CTX - 1, np.int32), ob.data_ptr(), ob.numel(), seq=np.arange(B, dtype=np.int32),
+                               in_fmt=m.F32, out_fmt=m.Q8_0)
+        stream.synchronize()
+        rounds += 1
+    del burn
     results = {}
     for B in batches:
         x = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
@@ -345,6 +352,17 @@ def bench_shape(args):
     print("[bench] stage open %.1f s, KV context filled in %.1f s" % (t_load, t_kv), file=sys.stderr, flush=True)
     kv_bytes_per_seq = L * n_ctx * HK * (kv_row[kv_types[0]] + kv_row[kv_types[1]])
     stream = torch.cuda.ExternalStream(ses.stream)
+    if args.burn_in > 0:
+        # untimed decode work for BURN_IN_SECONDS: the one-time ~35 ms stall early in a process's life (see bench_stage)
+        B0 = batches[0]
+        xb = torch.from_numpy(rng.standard_normal((B0, E)).astype(np.float32)).cuda()
+        ob = torch.empty(m.act_packed_size(m.Q8_0, B0, E), dtype=torch.uint8, device="cuda")
+        t_burn = time.perf_counter()
+        while time.perf_counter() - t_burn < BURN_IN_SECONDS:
+            for _ in range(20):
+                ses.decode_dev(xb.data_ptr(), np.full(B0, n_ctx - 1, np.int32), ob.data_ptr(), ob.numel(), seq=np.arange(B0, dtype=np.int32),
+                               in_fmt=m.F32, out_fmt=m.Q8_0)
+            stream.synchronize()
     results = {}
     for B in batches:
         print("[bench] decode batch %d" % B, file=sys.stderr, flush=True)
