@@ -41,6 +41,21 @@ constexpr int SK_NT = 16;                 // activation columns per launch (one 
 constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
 
+// Phase timestamps for tuning builds (-DMESH_GEMV_TRACE); compiled out of the product.
+#ifdef MESH_GEMV_TRACE
+__device__ long long *g_skinny_trace = nullptr;
+extern "C" int mesh_debug_set_skinny_trace(long long *p) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_skinny_trace), &p, sizeof p) == hipSuccess ? 0 : -2;
+}
+#define SK_MARK(k)                                                                                 \
+    do {                                                                                           \
+        if (g_skinny_trace && (threadIdx.x & 63) == 0)                                             \
+            g_skinny_trace[((size_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (k)] = wall_clock64(); \
+    } while (0)
+#else
+#define SK_MARK(k) do { } while (0)
+#endif
+
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -198,7 +213,10 @@ __device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_la
 
 template <int TYPE, int NU, int SEGS>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
-                                                                 int p_ks, int p_rows, unsigned p_begins, const SkinnyKernelArgs a) {
+                                                                 int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
+                                                                 const SkinnyKernelArgs a) {
+    // (p_begins = first tile-row of matrix 1 | of matrix 2 << 16; p_split = tile-rows per workgroup | workgroups with one
+    // more << 16, computed on the host: no division and no grid-size load stand before the first weight load)
     const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
     // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
     extern __shared__ __align__(16) uint8_t smem[];
@@ -210,13 +228,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: tile addresses become SGPR base + lane offset
     const int m = lane & 15, g = lane >> 4;
     const int src_lane4 = 4 * (4 * m + g);                // byte address, for ds_bpermute, of the lane that loaded row m, quarter g
-    const int KS = p_ks, RS = SK_WAVES / KS;
-    const int ks = wave % KS, rs = wave / KS;
-    const int total_rows = p_rows;
-    const int tr0 = (int)(((long long)blockIdx.x * total_rows) / gridDim.x);
-    const int tr1 = (int)(((long long)(blockIdx.x + 1) * total_rows) / gridDim.x);
-    const int rows_here = tr1 - tr0;
-    const int n_i = rs < RS ? (nsb - ks + KS - 1) / KS : 0;         // super-blocks of this wave (ks < KS <= nsb)
+    const int KS = p_ks, LK = __builtin_ctz((unsigned)KS), RS = SK_WAVES >> LK;      // KS is a power of two
+    const int ks = wave & (KS - 1), rs = wave >> LK;
+    (void)p_rows;
+    const int sq = (int)(p_split & 0xFFFFu), sr = (int)(p_split >> 16), bx = blockIdx.x;
+    const int tr0 = bx * sq + (bx < sr ? bx : sr);
+    const int rows_here = sq + (bx < sr ? 1 : 0);
+    const int n_i = rs < RS ? (nsb - ks + KS - 1) >> LK : 0;        // super-blocks of this wave (ks < KS <= nsb)
     const size_t row_stride = (size_t)nsb * TB;
     // B fragments: lane (n = m, g) supplies column n, quarter g (columns beyond T hold zeros)
     const int lane_off = (TYPE == MESH_Q4_K ? 64 * g : 128 * (g >> 1) + 16 * (g & 1)) * 16 + m * 8;
@@ -258,11 +276,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         for (int t = 0; t < 8; ++t)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
     };
+    SK_MARK(0);
     if (total > 0) {
 #pragma unroll
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
         B[0].load(p_x, lane_off, ks);
         B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
+        SK_MARK(1);
         if (n_i <= 2 && total <= SK_DEPTH) {
             // short walk: everything it needs is already in flight
 #pragma unroll
@@ -288,6 +308,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         }
     }
 
+    SK_MARK(2);
     // partial sums of this wave: D[seg] holds rows 4g..4g+3, column m of segment seg
 #pragma unroll
     for (int seg = 0; seg < SEGS; ++seg) {
@@ -299,6 +320,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     }
     __syncthreads();
 
+    SK_MARK(3);
     // outputs of this workgroup: rows_here x 16 rows x T columns
     for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
@@ -351,6 +373,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         if (a.y[mi]) a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
         if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)out;
     }
+    SK_MARK(4);
 }
 
 template <int TYPE, int NU, int SEGS>
@@ -362,7 +385,8 @@ static int launch_skinny(const SkinnyKernelArgs &ka, int grid, size_t smem, hipS
         attr_set = true;
     }
     gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka.x, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks,
-                                                                                                 ka.tile_begin[3], (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), ka);
+                                                                                                 ka.tile_begin[3], (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16),
+                                                                                                 (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -409,7 +433,9 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     ka.ldres = a.ldres; ka.epi = a.epi;
     ka.rope = a.rope;
     ka.M16 = a.mat[0].M;
-    const int KS = nsb < SK_WAVES ? nsb : SK_WAVES, RS = SK_WAVES / KS;
+    int KS = 1;
+    while (KS * 2 <= nsb && KS * 2 <= SK_WAVES) KS *= 2;      // a power of two: the kernel splits its waves with shifts
+    const int RS = SK_WAVES / KS;
     ka.ks = KS;
     // tile-rows per workgroup: spread over the CUs, bounded by the segments a wave can hold
     const int rows_cap = std::max(1, SK_SEGS_MAX / NU) * RS;
