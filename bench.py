@@ -185,7 +185,7 @@ def bench_stage(args):
     tmp = models.tmp_dir()
     path = os.path.join(tmp, "mesh_bench_llama3_8b_l0_15.gguf")
     cfg, tensors, t_gen = build_stage_model(models, path)
-    batches = sorted(set(int(b) for b in args.batches.split(",")))
+    batches = sorted(set(int(b) for b in (args.batches or "1,4,16").split(",")))
     bmax = max(batches)
     t0 = time.perf_counter()
     kv_types = {"f16": (m.F16, m.F16), "q8_0/q4_0": (m.Q8_0, m.Q4_0), "q4_0/q4_0": (m.Q4_0, m.Q4_0)}[args.kv]
@@ -333,7 +333,7 @@ def bench_shape(args):
     expert_bytes = sum(d.nbytes for n, (_, _, d) in tensors.items() if "_exps." in n)
     del tensors
     print("[bench] model file written in %.1f s" % t_gen, file=sys.stderr, flush=True)
-    batches = sp["batches"]
+    batches = sorted(set(int(b) for b in args.batches.split(","))) if args.batches else sp["batches"]
     bmax = max(batches)
     n_ctx, L = sp["n_ctx"], sp["layers"]
     t0 = time.perf_counter()
@@ -430,7 +430,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="stage", choices=["stage", "codec", "c4", "c5"])
-    ap.add_argument("--batches", default="1,4,16", help="decode batch sizes; the first is the headline value")
+    ap.add_argument("--batches", default=None, help="decode batch sizes; the first is the headline value (default 1,4,16 for the stage workload, the shape's own list for c4 / c5)")
     ap.add_argument("--kv", default="f16", choices=["f16", "q8_0/q4_0", "q4_0/q4_0"],
                     help="KV cache row types K/V (default f16: the tier the reference picks for an 8B Q4_K_M model)")
     ap.add_argument("--burn-in", type=int, default=80, help="untimed decode steps per batch size before anything is timed")

@@ -490,7 +490,7 @@ static int skinny_min_tokens() {
     static int v = 0;
     if (!v) {
         const char *e = getenv("MESH_SKINNY_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 5;
+        v = e && atoi(e) > 0 ? atoi(e) : 4;
     }
     return v;
 }

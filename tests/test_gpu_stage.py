@@ -137,7 +137,7 @@ def test_stage_boundary_formats(tmp_path, fmt_name):
 
 
 def test_llama3_8b_shaped_layers_decode_with_long_kv(tmp_path):
-    """Two real-shape layers (one with Q6_K attn_v/ffn_down, one all Q4_K), batch 1 and 4 at KV depth 300+."""
+    """Two real-shape layers (one with Q6_K attn_v/ffn_down, one all Q4_K), batch 1, 4 and 3 at KV depth 300+."""
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=512, n_seq=4, n_batch=8)
     assert tensors["blk.3.ffn_down.weight"][0] == models.Q6_K and tensors["blk.4.ffn_down.weight"][0] == models.Q4_K
@@ -160,7 +160,7 @@ def test_llama3_8b_shaped_layers_decode_with_long_kv(tmp_path):
     pos, seq = [n_past, n_past, n_past + 1, n_past], [0, 1, 2, 3]
     got = ses.decode(x4, pos, seq=seq).view(np.float32).reshape(4, 4096)
     ref = orc.forward(x4, pos, seq=seq)
-    assert rel_l2(got, ref) <= 1e-3
+    assert rel_l2(got, ref) <= 3e-3        # four tokens: the batched MFMA GEMM (f16 activations)
     # three tokens: the 3-column mat-vec kernels
     x3 = rng.standard_normal((3, 4096)).astype(np.float32)
     pos, seq = [n_past + 1, n_past + 1, n_past], [0, 1, 3]
@@ -173,7 +173,7 @@ def test_llama3_8b_shaped_layers_decode_with_long_kv(tmp_path):
 
 def test_qwen25_32b_shaped_layer_all_decode_paths(tmp_path):
     """One real-shape Qwen2.5-32B layer (hidden 5120 = 20 super-blocks, 40 heads / 8 KV heads = 5 per group, FFN 27648, q/k/v
-    bias, NEOX rope): batch 1 and 4 on the mat-vec kernel, 16 and a ragged 11 on the skinny MFMA GEMM, at KV depth 100."""
+    bias, NEOX rope): batch 1 on the mat-vec kernel, 4, 16 and a ragged 11 on the skinny MFMA GEMM, at KV depth 100."""
     name = "qwen2.5-32b"
     m, cfg, tensors, st = _open(tmp_path, name, [7], 7, 8, n_ctx=128, n_seq=16, n_batch=16)
     ses = st.session()
@@ -187,7 +187,7 @@ def test_qwen25_32b_shaped_layer_all_decode_paths(tmp_path):
         orc.k[0, s_, :, :n_past] = k.transpose(1, 0, 2)
         orc.v[0, s_, :, :n_past] = v.transpose(1, 0, 2)
     nxt = [n_past] * 16
-    for seqs, tol in (([3], 1e-3), ([0, 5, 9, 12], 1e-3), ([2, 6, 14], 1e-3), (list(range(16)), 3e-3), ([1, 2, 3, 4, 6, 7, 8, 10, 11, 13, 15], 3e-3)):
+    for seqs, tol in (([3], 1e-3), ([0, 5, 9, 12], 3e-3), ([2, 6, 14], 1e-3), (list(range(16)), 3e-3), ([1, 2, 3, 4, 6, 7, 8, 10, 11, 13, 15], 3e-3)):
         T = len(seqs)
         pos = [nxt[q] for q in seqs]
         for q in seqs:
@@ -406,9 +406,9 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
 
 
 def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
-    """Decode batches of 5..191 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
+    """Decode batches of 4..191 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
     (one with q6_K attn_v / ffn_down, so q/k/v split into two launches), 16 sequences at KV depth 300, full and ragged
-    batches; against the oracle and against the same steps fed four at a time through the mat-vec kernel."""
+    batches; against the oracle and against the same steps fed three at a time through the mat-vec kernel."""
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=512, n_seq=16, n_batch=16)
     ses, ses4 = st.session(), st.session()
@@ -432,7 +432,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         x = rng.standard_normal((T, 4096)).astype(np.float32)
         got = ses.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
         ref = orc.forward(x, pos, seq=seqs)
-        alt = np.concatenate([ses4.decode(x[i:i + 4], pos[i:i + 4], seq=seqs[i:i + 4]).view(np.float32) for i in range(0, T, 4)]).reshape(T, 4096)
+        alt = np.concatenate([ses4.decode(x[i:i + 3], pos[i:i + 3], seq=seqs[i:i + 3]).view(np.float32) for i in range(0, T, 3)]).reshape(T, 4096)
         assert rel_l2(got, ref) <= 3e-3, T
         assert rel_l2(got, alt) <= 3e-3, T
     ses.close(); ses4.close(); st.close()
@@ -440,7 +440,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
 
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
     """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
-    1-4 tokens (mat-vec kernels) and of 5+ tokens (batched MFMA GEMM); with MESH_GEMV_ROPE=0 the separate kernel does
+    1-3 tokens (mat-vec kernels) and of 4+ tokens (batched MFMA GEMM); with MESH_GEMV_ROPE=0 the separate kernel does
     them.  Outputs and cache contents must agree bit for bit (the arithmetic is the same), through the single-type
     and the mixed q4_K/q6_K launches."""
     for name, layers in (("llama3-8b", [3, 4]), ("tiny-llama", [0, 1])):
