@@ -16,6 +16,7 @@
 
 #include "gemm.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace mesh {
@@ -214,7 +215,7 @@ template <> struct PackedSub<MESH_Q6_K> {
 // 16 k is four contiguous 256-byte pieces of that layout, so each lane fetches its 16 bytes straight from memory (L2),
 // four k16 steps ahead, into a ring of registers.  That halves the LDS reads per MFMA and leaves the staging waves only
 // the weights.
-template <int TYPE, bool PACKED, bool XDIRECT>
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     extern __shared__ __align__(16) _Float16 gemm_smem[];
     _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
@@ -223,7 +224,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = blockIdx.x * GM, t0 = blockIdx.y * GN;
-    const int nsb = a.K / QK_K, n_steps = a.K / GK;
+    const int nsb = a.K / QK_K, n_all = a.K / GK;
+    // k-steps [k0, k0 + n_steps) of this workgroup: all of them, or slice blockIdx.z of a split launch
+    // (a template parameter: the unsplit kernel must not carry the offsets, they cost it 6%)
+    const int k0 = SPLIT ? (int)blockIdx.z * a.k_per_split : 0;
+    const int n_steps = SPLIT ? (n_all - k0 < a.k_per_split ? n_all - k0 : a.k_per_split) : n_all;
 
     if (wave >= 4) {
         // ---- staging waves: thread s (0..255): weights -- row s/2, sub-block half s%2; activations -- token s/2, 32 elements s%2
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         const int srow = st >> 1, sh = st & 1;
         const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
         const bool wlive = PACKED || wrow < a.M_pad;                 // (the GEMM layout holds its zero rows)
-        const uint8_t *wtile_row = PACKED ? static_cast<const uint8_t *>(a.Wp) + (size_t)blockIdx.x * n_steps * PackedSub<TYPE>::CHUNK
+        const uint8_t *wtile_row = PACKED ? static_cast<const uint8_t *>(a.Wp) + ((size_t)blockIdx.x * n_all + k0) * PackedSub<TYPE>::CHUNK
                                           : static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
         using Sub = typename std::conditional<PACKED, PackedSub<TYPE>, RawSub<TYPE>>::type;
         const int tok = t0 + srow;
@@ -241,9 +246,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         uint4 rx[2][4];
         auto fetch = [&](int kc, Sub &w, uint4 (&x)[4]) {
             if constexpr (PACKED) w.load(wtile_row + (size_t)kc * PackedSub<TYPE>::CHUNK, st);
-            else w.load(wtile_row + (size_t)(kc >> 2) * TB, wrow & 15, kc & 3, sh);
+            else w.load(wtile_row + (size_t)((k0 + kc) >> 2) * TB, wrow & 15, (k0 + kc) & 3, sh);
             if constexpr (!XDIRECT) {
-                const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)kc * GK);
+                const uint4 *s4 = reinterpret_cast<const uint4 *>(xrow + (size_t)(k0 + kc) * GK);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) x[i] = s4[i];
             }
@@ -253,7 +258,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
             if constexpr (PACKED) {
                 w.store(wdst);
             } else if (wlive) {
-                w.store(kc & 3, sh, wdst);
+                w.store((k0 + kc) & 3, sh, wdst);
             } else {
                 uint4 *d4 = reinterpret_cast<uint4 *>(wdst);
 #pragma unroll
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     if constexpr (XDIRECT) {
         // lane's slot in the fragments of its two 32-token groups: token (lane & 31), k8 group (lane >> 5) of a k16 step;
         // consecutive k16 steps are 256 halfs apart.  Token blocks past the batch re-read the last one (never stored).
-        const int n_blk = (a.T + 15) >> 4, n_g = n_steps * (GK / 16);
+        const int n_blk = (a.T + 15) >> 4, n_g = n_all * (GK / 16), g0 = k0 * (GK / 16);
         const _Float16 *bp[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
 #pragma unroll
         for (int ks = 0; ks < GK / 16; ++ks)
 #pragma unroll
-            for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)(ks < n_g ? ks : n_g - 1) * 256);
+            for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)(g0 + ks < n_g ? g0 + ks : n_g - 1) * 256);
         __syncthreads();
         for (int kc = 0; kc < n_steps; ++kc) {
             const _Float16 *Wb = Ws + (kc & 1) * GM * LDS_LD;
@@ -322,7 +327,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
                     for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], ring[ks][j], acc[i][j], 0, 0, 0);
-                int gn = (kc + 1) * (GK / 16) + ks;
+                int gn = g0 + (kc + 1) * (GK / 16) + ks;
                 gn = gn < n_g ? gn : n_g - 1;
 #pragma unroll
                 for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)gn * 256);
@@ -355,6 +360,23 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     }
 
     // D[m][t]: lane holds column t = lane%32 and rows 8*(e/4) + 4*(lane/32) + e%4 -> four consecutive m per store
+    if constexpr (SPLIT) {
+        // slice of a split launch: the raw sums go to part[slice][token][row of the launch]
+        const size_t ld = (size_t)gridDim.x * GM;
+        float *P = a.part + (size_t)blockIdx.z * a.T * ld + m0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int t = t0 + wn + 32 * j + (lane & 31);
+                if (t >= a.T) continue;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4)
+                    *reinterpret_cast<float4 *>(P + (size_t)t * ld + wm + 32 * i + 8 * e4 + 4 * (lane >> 5)) =
+                        make_float4(acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]);
+            }
+        return;
+    }
     if (a.y16_k8) {
         // SwiGLU pair: the waves of the upper half of the tile hold the up rows of the gate rows in the lower half, at
         // the same (register, lane).  They hand them over through LDS (free by now: the staging waves have left, and
@@ -431,18 +453,98 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         }
 }
 
-template <int TYPE, bool PACKED, bool XDIRECT>
-static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
+// Second kernel of a split launch: adds the slices of part[slice][token][row] in slice order and applies the epilogue
+// of the unsplit kernel.  One thread per (token, four consecutive rows); rows run fastest, so partial reads and output
+// writes are contiguous.
+__global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, int row_blocks) {
+    const size_t ld = (size_t)row_blocks * GM;
+    const int t_pad = a.y16_k8 ? (a.T + 15) & ~15 : a.T;
+    const int per_block = a.y16_k8 ? GM / 8 : GM / 4;          // threads per row block: 64 gate rows or 128 rows, four each
+    const size_t n = (size_t)t_pad * row_blocks * per_block;
+    for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (size_t)gridDim.x * 256) {
+        const int q = (int)(idx % per_block), bx = (int)((idx / per_block) % row_blocks), t = (int)(idx / ((size_t)per_block * row_blocks));
+        auto sum4 = [&](size_t row) {
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int z = 0; z < a.ksplit; ++z) {
+                const float4 p = *reinterpret_cast<const float4 *>(a.part + ((size_t)z * a.T + t) * ld + row);
+                o.x += p.x; o.y += p.y; o.z += p.z; o.w += p.w;
+            }
+            return o;
+        };
+        if (a.y16_k8) {
+            const int m = bx * (GM / 2) + 4 * q;
+            if (m >= a.M) continue;
+            float o[4] = {0.f, 0.f, 0.f, 0.f};                 // padding columns of the last token block hold zeros
+            if (t < a.T) {
+                const float4 g = sum4((size_t)bx * GM + 4 * q), u = sum4((size_t)bx * GM + GM / 2 + 4 * q);
+                o[0] = g.x / (1.0f + expf(-g.x)) * u.x; o[1] = g.y / (1.0f + expf(-g.y)) * u.y;
+                o[2] = g.z / (1.0f + expf(-g.z)) * u.z; o[3] = g.w / (1.0f + expf(-g.w)) * u.w;
+            }
+            *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
+                make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
+            continue;
+        }
+        float *Y = a.Y;
+        const float *bias = a.bias;
+        int M = a.M, ldy = a.ldy, mb0 = bx * GM;
+        if (a.n_seg > 1) {
+            const int sg = (bx >= a.seg_begin[1] ? 1 : 0) + (a.n_seg > 2 && bx >= a.seg_begin[2] ? 1 : 0);
+            Y = sg == 0 ? a.seg_Y[0] : sg == 1 ? a.seg_Y[1] : a.seg_Y[2];
+            bias = sg == 0 ? a.seg_bias[0] : sg == 1 ? a.seg_bias[1] : a.seg_bias[2];
+            M = sg == 0 ? a.seg_M[0] : sg == 1 ? a.seg_M[1] : a.seg_M[2];
+            ldy = sg == 0 ? a.seg_ldy[0] : sg == 1 ? a.seg_ldy[1] : a.seg_ldy[2];
+            mb0 = (bx - (sg == 0 ? 0 : sg == 1 ? a.seg_begin[1] : a.seg_begin[2])) * GM;
+        }
+        const int m = mb0 + 4 * q;
+        if (m >= M) continue;
+        float4 o = sum4((size_t)bx * GM + 4 * q);
+        if (bias) {
+            const float4 b = *reinterpret_cast<const float4 *>(bias + m);
+            o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w;
+        }
+        if (a.residual) {
+            const float4 r = *reinterpret_cast<const float4 *>(a.residual + (size_t)t * a.ldres + m);
+            o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
+        }
+        *reinterpret_cast<float4 *>(Y + (size_t)t * ldy + m) = o;
+    }
+}
+
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT>
+static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) {
     // two stages of the weight slab, and of the activation slab unless the activations bypass LDS: 73 728 / 36 864 B
     constexpr size_t smem = sizeof(_Float16) * 2 * (GM + (XDIRECT ? 0 : GN)) * LDS_LD;
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    gemm_kq_kernel<TYPE, PACKED, XDIRECT><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
+    gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
     MESH_LAUNCH_CHECK();
+    if (SPLIT) {
+        const int t_pad = k.y16_k8 ? (k.T + 15) & ~15 : k.T;
+        const size_t n = (size_t)t_pad * grid.x * (k.y16_k8 ? GM / 8 : GM / 4);
+        const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
+        gemm_splitk_epilogue_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(k, (int)grid.x);
+        MESH_LAUNCH_CHECK();
+    }
     return MESH_OK;
+}
+
+static int gemm_n_cu() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+template <int TYPE, bool PACKED, bool XDIRECT>
+static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
+    return k.ksplit > 1 ? launch_gemm_kernel<TYPE, PACKED, XDIRECT, true>(k, grid, stream) : launch_gemm_kernel<TYPE, PACKED, XDIRECT, false>(k, grid, stream);
 }
 
 int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
@@ -460,7 +562,23 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     GemmArgs k = a;
     k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
     const int row_blocks = a.y16_k8 ? (a.M + GM / 2 - 1) / (GM / 2) : (a.M + GM - 1) / GM;
-    const dim3 grid((unsigned)row_blocks, (unsigned)((a.T + GN - 1) / GN));
+    dim3 grid((unsigned)row_blocks, (unsigned)((a.T + GN - 1) / GN));
+    // A launch of fewer workgroups than CUs walks all of K in each of them while the rest of the chip idles: split K
+    // over blockIdx.z (slices of at least 8 k-steps, at most one workgroup per CU in total, partial tiles within the
+    // scratch the caller gave).
+    k.ksplit = 1;
+    k.k_per_split = a.K / GK;
+    if (a.part) {
+        const int n_all = a.K / GK, wgs = (int)(grid.x * grid.y), ncu = gemm_n_cu();
+        int ks = 1;
+        while (ks < 16 && wgs * ks * 2 <= ncu && n_all / (ks * 2) >= 8 &&
+               (size_t)(ks * 2) * a.T * row_blocks * GM * sizeof(float) <= a.part_bytes) ks *= 2;
+        if (ks > 1) {
+            k.k_per_split = (n_all + ks - 1) / ks;
+            k.ksplit = (n_all + k.k_per_split - 1) / k.k_per_split;      // no empty slice
+            grid.z = (unsigned)k.ksplit;
+        }
+    }
     if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
     if (a.x_k8) {

@@ -29,6 +29,13 @@ struct GemmArgs {
     // SwiGLU pair: Wp is a gate/up pair packed by gemm_pack_pair (every row block 64 gate rows, then the same 64 up
     // rows), M their common row count; the launch writes f16(silu(gate) * up) in the k8-major layout to y16_k8 (Y unused).
     _Float16 *y16_k8 = nullptr;
+    // Optional scratch for launches too narrow to fill the chip (few row blocks x token blocks): K is then split over
+    // blockIdx.z, every slice writes its f32 partial tile to `part` ([slice][token][row of the launch]) and a second
+    // kernel adds the slices in slice order and applies the epilogue.  Null: never split.  ksplit / k_per_split are
+    // filled in by gemm_kquant.
+    float *part = nullptr;
+    size_t part_bytes = 0;
+    int ksplit = 1, k_per_split = 0;
 };
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
 

@@ -480,7 +480,7 @@ static int gemm_min_tokens() {
     static int v = 0;
     if (!v) {
         const char *e = getenv("MESH_GEMM_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 65;
+        v = e && atoi(e) > 0 ? atoi(e) : 32;
     }
     return v;
 }
@@ -543,6 +543,13 @@ int session_new(mesh_stage *st, mesh_session **out) {
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
             if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
+        }
+        const char *sk = getenv("MESH_GEMM_SPLITK");
+        if (B >= (size_t)PREFILL_MIN_TOKENS && !(sk && sk[0] == '0')) {
+            // a split launch holds at most one 128 x 128 f32 tile per CU: 16.8 MB on 256 CUs
+            s->gemm_part_bytes = (size_t)32 << 20;
+            if ((rc = sess_alloc(s.get(), &p, s->gemm_part_bytes)) != MESH_OK) return rc;
+            s->gemm_part = static_cast<float *>(p);
         }
     }
     if (hp.n_expert_used > 0 && !st->layers.empty() && st->layers[0].gate_inp.present()) {
@@ -674,7 +681,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     int rc;
     bool rope_fused = false, attn_is_k8 = false;
     const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
-    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; return g; };
+    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; return g; };
     if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;

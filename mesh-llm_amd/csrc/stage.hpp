@@ -88,6 +88,8 @@ struct mesh_session {
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
     uint16_t *xn16 = nullptr, *ffn16 = nullptr;
+    float *gemm_part = nullptr;          // partial tiles of large-tile GEMM launches that split K (gemm.hpp)
+    size_t gemm_part_bytes = 0;
     float *ffn_up = nullptr;
     float *moe_logits = nullptr, *moe_w = nullptr, *moe_out = nullptr, *expert_mask = nullptr;
     bool expert_mask_on = false;

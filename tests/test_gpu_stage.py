@@ -360,12 +360,12 @@ def test_prefill_gemm_variants_agree(tmp_path, monkeypatch, name, layers):
 
 
 def test_prefill_mfma_path_matches_oracle_and_decode_path(tmp_path):
-    """Calls with >= 65 tokens take the large-tile MFMA GEMM (f16 activations, f32 accumulate): compare it with the
+    """Calls with >= 32 tokens take the large-tile MFMA GEMM (f16 activations, f32 accumulate): compare it with the
     oracle and with the same tokens fed 16 at a time (skinny GEMM), then keep decoding on top of the prefilled cache."""
     m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [3, 4], 3, 5, n_ctx=256, n_seq=2, n_batch=208)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(41))
-    T = 200                                     # at least 65 tokens take the large-tile GEMM; not a multiple of its 128-token tile
+    T = 200                                     # at least 32 tokens take the large-tile GEMM; not a multiple of its 128-token tile
     x = rng.standard_normal((T, E)).astype(np.float32)
     ses = st.session()
     got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
@@ -394,8 +394,9 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
     orc = StageOracle(cfg, tensors, 0, 3, 512, n_seq_max=2)
     ses = st.session()
     # large-tile GEMM + chunk attention from position 0, a second chunk on top of the first (ragged: 200 = 6 * 32 + 8),
-    # then the skinny GEMM (three 16-column passes, ragged) on the other sequence
-    for T, pos0, seq in ((200, 0, 0), (200, 200, 0), (47, 0, 1)):
+    # then the skinny GEMM (two 16-column passes, ragged) on the other sequence and a 47-token call on top of it (large-tile
+    # GEMM again, K split over workgroups: few row blocks x one token block)
+    for T, pos0, seq in ((200, 0, 0), (200, 200, 0), (27, 0, 1), (47, 27, 1)):
         x = rng.standard_normal((T, E)).astype(np.float32)
         sq = np.full(T, seq, np.int32)
         pos = np.arange(pos0, pos0 + T)
@@ -406,7 +407,7 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
 
 
 def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
-    """Decode batches of 4..64 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
+    """Decode batches of 4..31 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
     (one with q6_K attn_v / ffn_down, so q/k/v split into two launches), 16 sequences at KV depth 300, full and ragged
     batches; against the oracle and against the same steps fed three at a time through the mat-vec kernel."""
     name = "llama3-8b"
@@ -438,13 +439,18 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
     ses.close(); ses4.close(); st.close()
 
 
-def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
-    """From 65 tokens a call takes the large-tile MFMA GEMM whatever its shape: here 70 single-token sequences at ragged
-    positions (not a prefill chunk, so the split-KV decode attention runs behind the GEMM's q/k/v).  Real-shape
-    layers, against the oracle and against the same tokens fed 16 at a time (skinny GEMM)."""
+def test_wide_decode_batch_takes_large_tile_gemm(tmp_path, monkeypatch):
+    """From 32 tokens a call takes the large-tile MFMA GEMM whatever its shape: here 70 single-token sequences at ragged
+    positions (not a prefill chunk, so the split-KV decode attention runs behind the GEMM's q/k/v).  One token block
+    and 32..224 row blocks per projection: the launches split K over workgroups and add the slices in a second
+    kernel.  Real-shape layers, against the oracle, against the same tokens fed 16 at a time (skinny GEMM) and against
+    the unsplit launches (MESH_GEMM_SPLITK=0: same products, another summation order)."""
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=64, n_seq=70, n_batch=70)
     ses, ses16 = st.session(), st.session()
+    monkeypatch.setenv("MESH_GEMM_SPLITK", "0")
+    ses_whole = st.session()
+    monkeypatch.delenv("MESH_GEMM_SPLITK")
     orc = StageOracle(cfg, tensors, 3, 5, 64, n_seq_max=70)
     rng = np.random.Generator(np.random.PCG64(21))
     depth = [int(d) for d in rng.integers(1, 40, size=70)]
@@ -452,7 +458,7 @@ def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
         for s in range(70):
             k = (rng.standard_normal((depth[s], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
             v = (rng.standard_normal((depth[s], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
-            for x_ in (ses, ses16):
+            for x_ in (ses, ses16, ses_whole):
                 x_.kv_write(il, s, 0, k, v)
             orc.k[il - 3, s, :, :depth[s]] = k.transpose(1, 0, 2)
             orc.v[il - 3, s, :, :depth[s]] = v.transpose(1, 0, 2)
@@ -461,15 +467,17 @@ def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
     got = ses.decode(x, depth, seq=seqs).view(np.float32).reshape(70, 4096)
     ref = orc.forward(x, depth, seq=seqs)
     alt = np.concatenate([ses16.decode(x[i:i + 16], depth[i:i + 16], seq=seqs[i:i + 16]).view(np.float32) for i in range(0, 70, 16)]).reshape(70, 4096)
+    whole = ses_whole.decode(x, depth, seq=seqs).view(np.float32).reshape(70, 4096)
     assert rel_l2(got, ref) <= 3e-3
     assert rel_l2(got, alt) <= 3e-3
+    assert rel_l2(got, whole) <= 1e-3 and rel_l2(whole, ref) <= 3e-3
     # the appended K / V rows are the same f16 values on both paths up to one rounding step of the f16 activations
     for s in (0, 33, 69):
         ka, va = ses.kv_read(4, s, depth[s], 1)
         kb, vb = ses16.kv_read(4, s, depth[s], 1)
         assert rel_l2(ka.view(np.float16).astype(np.float32), kb.view(np.float16).astype(np.float32)) <= 3e-3
         assert rel_l2(va.view(np.float16).astype(np.float32), vb.view(np.float16).astype(np.float32)) <= 3e-3
-    ses.close(); ses16.close(); st.close()
+    ses.close(); ses16.close(); ses_whole.close(); st.close()
 
 
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
