@@ -484,6 +484,44 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
         return;
     }
     const float *xt = x + (size_t)t * n;
+    constexpr int RC = 4;                                   // rows of up to 2048 * RC elements stay in registers: one read
+    if (w && n <= 2048 * RC) {
+        float4 v[RC][2], g[RC][2];
+#pragma unroll
+        for (int j = 0; j < RC; ++j) {
+            const int i = tid * 8 + j * 2048;
+            const bool live = i < n;
+            v[j][0] = live ? *reinterpret_cast<const float4 *>(xt + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            v[j][1] = live ? *reinterpret_cast<const float4 *>(xt + i + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < RC; ++j) {
+            const int i = tid * 8 + j * 2048;
+            const bool live = i < n;
+            g[j][0] = live ? *reinterpret_cast<const float4 *>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            g[j][1] = live ? *reinterpret_cast<const float4 *>(w + i + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < RC; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) ss += (v[j][h].x * v[j][h].x + v[j][h].y * v[j][h].y) + (v[j][h].z * v[j][h].z + v[j][h].w * v[j][h].w);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        const float sc = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)n + eps);
+#pragma unroll
+        for (int j = 0; j < RC; ++j) {
+            const int i = tid * 8 + j * 2048;
+            if (i >= n) continue;
+            const float4 v0 = v[j][0], v1 = v[j][1], g0 = g[j][0], g1 = g[j][1];
+            *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) =
+                make_uint4(sk_pack_h2(v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(v0.z * sc * g0.z, v0.w * sc * g0.w),
+                           sk_pack_h2(v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(v1.z * sc * g1.z, v1.w * sc * g1.w));
+        }
+        return;
+    }
     float scale = 1.f;
     if (w) {
         float ss = 0.f;
