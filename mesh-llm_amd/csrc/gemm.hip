@@ -464,10 +464,18 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
     for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (size_t)gridDim.x * 256) {
         const int q = (int)(idx % per_block), bx = (int)((idx / per_block) % row_blocks), t = (int)(idx / ((size_t)per_block * row_blocks));
         auto sum4 = [&](size_t row) {
+            // four slices in flight at a time (indices past the end re-read the last slice and are not added)
             float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int z = 0; z < a.ksplit; ++z) {
-                const float4 p = *reinterpret_cast<const float4 *>(a.part + ((size_t)z * a.T + t) * ld + row);
-                o.x += p.x; o.y += p.y; o.z += p.z; o.w += p.w;
+            for (int z0 = 0; z0 < a.ksplit; z0 += 4) {
+                float4 p[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int z = z0 + u < a.ksplit ? z0 + u : a.ksplit - 1;
+                    p[u] = *reinterpret_cast<const float4 *>(a.part + ((size_t)z * a.T + t) * ld + row);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (z0 + u < a.ksplit) { o.x += p[u].x; o.y += p[u].y; o.z += p[u].z; o.w += p[u].w; }
             }
             return o;
         };
