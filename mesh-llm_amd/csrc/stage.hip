@@ -480,7 +480,7 @@ static int gemm_min_tokens() {
     static int v = 0;
     if (!v) {
         const char *e = getenv("MESH_GEMM_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 32;
+        v = e && atoi(e) > 0 ? atoi(e) : 17;
     }
     return v;
 }

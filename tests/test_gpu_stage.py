@@ -360,12 +360,12 @@ def test_prefill_gemm_variants_agree(tmp_path, monkeypatch, name, layers):
 
 
 def test_prefill_mfma_path_matches_oracle_and_decode_path(tmp_path):
-    """Calls with >= 32 tokens take the large-tile MFMA GEMM (f16 activations, f32 accumulate): compare it with the
+    """Calls with >= 17 tokens take the large-tile MFMA GEMM (f16 activations, f32 accumulate): compare it with the
     oracle and with the same tokens fed 16 at a time (skinny GEMM), then keep decoding on top of the prefilled cache."""
     m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [3, 4], 3, 5, n_ctx=256, n_seq=2, n_batch=208)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(41))
-    T = 200                                     # at least 32 tokens take the large-tile GEMM; not a multiple of its 128-token tile
+    T = 200                                     # at least 17 tokens take the large-tile GEMM; not a multiple of its 128-token tile
     x = rng.standard_normal((T, E)).astype(np.float32)
     ses = st.session()
     got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
@@ -394,9 +394,9 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
     orc = StageOracle(cfg, tensors, 0, 3, 512, n_seq_max=2)
     ses = st.session()
     # large-tile GEMM + chunk attention from position 0, a second chunk on top of the first (ragged: 200 = 6 * 32 + 8),
-    # then the skinny GEMM (two 16-column passes, ragged) on the other sequence and a 47-token call on top of it (large-tile
-    # GEMM again, K split over workgroups: few row blocks x one token block)
-    for T, pos0, seq in ((200, 0, 0), (200, 200, 0), (27, 0, 1), (47, 27, 1)):
+    # then the skinny GEMM (one ragged 16-column pass) on the other sequence and calls of 27 and 47 tokens on top of it
+    # (large-tile GEMM again, K split over workgroups: few row blocks x one token block)
+    for T, pos0, seq in ((200, 0, 0), (200, 200, 0), (13, 0, 1), (27, 13, 1), (47, 40, 1)):
         x = rng.standard_normal((T, E)).astype(np.float32)
         sq = np.full(T, seq, np.int32)
         pos = np.arange(pos0, pos0 + T)
@@ -407,7 +407,7 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
 
 
 def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
-    """Decode batches of 4..31 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
+    """Decode batches of 4..16 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
     (one with q6_K attn_v / ffn_down, so q/k/v split into two launches), 16 sequences at KV depth 300, full and ragged
     batches; against the oracle and against the same steps fed three at a time through the mat-vec kernel."""
     name = "llama3-8b"
@@ -440,7 +440,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
 
 
 def test_wide_decode_batch_takes_large_tile_gemm(tmp_path, monkeypatch):
-    """From 32 tokens a call takes the large-tile MFMA GEMM whatever its shape: here 70 single-token sequences at ragged
+    """From 17 tokens a call takes the large-tile MFMA GEMM whatever its shape: here 70 single-token sequences at ragged
     positions (not a prefill chunk, so the split-KV decode attention runs behind the GEMM's q/k/v).  One token block
     and 32..224 row blocks per projection: the launches split K over workgroups and add the slices in a second
     kernel.  Real-shape layers, against the oracle, against the same tokens fed 16 at a time (skinny GEMM) and against
@@ -519,16 +519,17 @@ def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers)
     captured, then replays).  Every replay must give the bits the eager launches give: two sessions, graphs on and
     off, walk the same sequence of steps -- repeated shapes, other shapes and host synchronisations in between, KV
     depth growing past a change of the split count."""
-    m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=6, n_batch=8)
+    m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=20, n_batch=24)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(17))
-    plan = [1, 1, 1, 4, 1, 4, 6, 1, 4, 6, 6, 1] + [1] * 70 + [4, 4, 1, 6]
+    # (20 tokens: the large-tile GEMM with K split over workgroups, two kernels per projection, inside a graph)
+    plan = [1, 1, 1, 4, 1, 4, 6, 1, 4, 6, 6, 1, 20, 1, 20] + [1] * 70 + [4, 4, 1, 6, 20]
     xs = [rng.standard_normal((T, E)).astype(np.float32) for T in plan]
     runs = []
     for flag in ("1", "0"):
         monkeypatch.setenv("MESH_STAGE_GRAPHS", flag)
         ses = st.session()
-        nxt = [0] * 6
+        nxt = [0] * 20
         outs = []
         for x in xs:
             T = x.shape[0]
