@@ -215,7 +215,7 @@ template <> struct PackedSub<MESH_Q6_K> {
 // 16 k is four contiguous 256-byte pieces of that layout, so each lane fetches its 16 bytes straight from memory (L2),
 // four k16 steps ahead, into a ring of registers.  That halves the LDS reads per MFMA and leaves the staging waves only
 // the weights.
-template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT>
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     extern __shared__ __align__(16) _Float16 gemm_smem[];
     _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
@@ -290,10 +290,14 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
     }
 
     // ---- multiplying waves
-    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;     // wave's 64 x 64 corner of the tile
-    float16v acc[2][2];
+    // wave's corner of the tile: 64 rows x 64 tokens; NARROW (calls of at most 64 tokens, whose upper token half would
+    // be padding): 32 rows x the lower 64 tokens, so all four waves multiply real columns
+    static_assert(!NARROW || XDIRECT, "the narrow tile reads its activations from the k8-major layout");
+    constexpr int MI = NARROW ? 1 : 2;
+    const int wm = NARROW ? wave * 32 : (wave & 1) * 64, wn = NARROW ? 0 : (wave >> 1) * 64;
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -319,12 +323,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
             const _Float16 *Wb = Ws + (kc & 1) * GM * LDS_LD;
 #pragma unroll
             for (int ks = 0; ks < GK / 16; ++ks) {
-                half8 af[2];
+                half8 af[MI];
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < MI; ++i)
                     af[i] = *reinterpret_cast<const half8 *>(Wb + (wm + 32 * i + (lane & 31)) * LDS_LD + 16 * ks + 8 * (lane >> 5));
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < MI; ++i)
 #pragma unroll
                     for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], ring[ks][j], acc[i][j], 0, 0, 0);
                 int gn = g0 + (kc + 1) * (GK / 16) + ks;
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
             }
             __syncthreads();
         }
-    } else {
+    } else if constexpr (!NARROW) {
     __syncthreads();
     for (int kc = 0; kc < n_steps; ++kc) {
         const int buf = kc & 1;
@@ -365,7 +369,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         const size_t ld = (size_t)gridDim.x * GM;
         float *P = a.part + (size_t)blockIdx.z * a.T * ld + m0;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int t = t0 + wn + 32 * j + (lane & 31);
@@ -381,33 +385,37 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         // SwiGLU pair: the waves of the upper half of the tile hold the up rows of the gate rows in the lower half, at
         // the same (register, lane).  They hand them over through LDS (free by now: the staging waves have left, and
         // the barrier makes sure every matrix-core wave has read its last fragments).
-        float *xch = reinterpret_cast<float *>(gemm_smem);         // [token half][64 registers][64 lanes]
+        // (NARROW: waves 2 and 3 hold the up rows of the gate rows of waves 0 and 1)
+        float *xch = reinterpret_cast<float *>(gemm_smem);         // [pair of waves][64 registers][64 lanes]
+        const bool is_up = NARROW ? wave >= 2 : wm != 0;
+        const int pair = NARROW ? (wave & 1) * 2 : (wn >> 6) * 4;  // first 16-register group of this pair of waves
+        const int gm = NARROW ? (wave & 1) * 32 : 0;               // gate rows of this wave inside the block's 64
         __syncthreads();
-        if (wm) {
+        if (is_up) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) xch[(((wn >> 6) * 4 + i * 2 + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+                    for (int e = 0; e < 16; ++e) xch[((pair + i * 2 + j) * 16 + e) * 64 + lane] = acc[i][j][e];
         }
         __syncthreads();
-        if (wm) return;
+        if (is_up) return;
         const int t_pad = (a.T + 15) & ~15;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int t = t0 + wn + 32 * j + (lane & 31);
                 if (t >= t_pad) continue;
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
-                    const int m = (int)blockIdx.x * (GM / 2) + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                    const int m = (int)blockIdx.x * (GM / 2) + gm + 32 * i + 8 * e4 + 4 * (lane >> 5);
                     if (m >= a.M) continue;
                     float o[4];
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const float g = acc[i][j][4 * e4 + c], u = xch[(((wn >> 6) * 4 + i * 2 + j) * 16 + 4 * e4 + c) * 64 + lane];
+                        const float g = acc[i][j][4 * e4 + c], u = xch[((pair + i * 2 + j) * 16 + 4 * e4 + c) * 64 + lane];
                         o[c] = t < a.T ? g / (1.0f + expf(-g)) * u : 0.f;       // padding columns of the last token block hold zeros
                     }
                     *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
@@ -430,7 +438,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         mb0 = (bx - (sg == 0 ? 0 : sg == 1 ? a.seg_begin[1] : a.seg_begin[2])) * GM;
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int t = t0 + wn + 32 * j + (lane & 31);
@@ -518,16 +526,16 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
     }
 }
 
-template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT>
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW>
 static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) {
     // two stages of the weight slab, and of the activation slab unless the activations bypass LDS: 73 728 / 36 864 B
     constexpr size_t smem = sizeof(_Float16) * 2 * (GM + (XDIRECT ? 0 : GN)) * LDS_LD;
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
+    gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
     MESH_LAUNCH_CHECK();
     if (SPLIT) {
         const int t_pad = k.y16_k8 ? (k.T + 15) & ~15 : k.T;
@@ -537,6 +545,13 @@ static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) 
         MESH_LAUNCH_CHECK();
     }
     return MESH_OK;
+}
+
+// MESH_GEMM_NARROW=0: calls of at most 64 tokens use the 128-token tile like the others (for comparison)
+static bool gemm_narrow_on() {
+    static int v = -1;
+    if (v < 0) { const char *e = getenv("MESH_GEMM_NARROW"); v = !(e && e[0] == '0'); }
+    return v != 0;
 }
 
 static int gemm_n_cu() {
@@ -552,7 +567,12 @@ static int gemm_n_cu() {
 
 template <int TYPE, bool PACKED, bool XDIRECT>
 static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
-    return k.ksplit > 1 ? launch_gemm_kernel<TYPE, PACKED, XDIRECT, true>(k, grid, stream) : launch_gemm_kernel<TYPE, PACKED, XDIRECT, false>(k, grid, stream);
+    // calls of at most 64 tokens on the production layout (GEMM-layout weights, k8-major activations): narrow tile
+    if constexpr (PACKED && XDIRECT) {
+        if (k.T <= GN / 2 && gemm_narrow_on())
+            return k.ksplit > 1 ? launch_gemm_kernel<TYPE, true, true, true, true>(k, grid, stream) : launch_gemm_kernel<TYPE, true, true, false, true>(k, grid, stream);
+    }
+    return k.ksplit > 1 ? launch_gemm_kernel<TYPE, PACKED, XDIRECT, true, false>(k, grid, stream) : launch_gemm_kernel<TYPE, PACKED, XDIRECT, false, false>(k, grid, stream);
 }
 
 int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
