@@ -755,7 +755,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
             rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
         }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
-            if (skinny) { aa.out16_k8 = xn; attn_is_k8 = true; }     // straight into the output projection's input layout
+            if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }         // straight into the output projection's input layout
             rc = attention_mma(aa, T, stream);
         } else rc = attention(aa, T, stream);
     }
