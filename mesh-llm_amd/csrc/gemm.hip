@@ -502,9 +502,10 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
         }
         float *Y = a.Y;
         const float *bias = a.bias;
-        int M = a.M, ldy = a.ldy, mb0 = bx * GM;
+        int M = a.M, ldy = a.ldy, mb0 = bx * GM, kind = a.kind[0];
         if (a.n_seg > 1) {
             const int sg = (bx >= a.seg_begin[1] ? 1 : 0) + (a.n_seg > 2 && bx >= a.seg_begin[2] ? 1 : 0);
+            kind = sg == 0 ? a.kind[0] : sg == 1 ? a.kind[1] : a.kind[2];
             Y = sg == 0 ? a.seg_Y[0] : sg == 1 ? a.seg_Y[1] : a.seg_Y[2];
             bias = sg == 0 ? a.seg_bias[0] : sg == 1 ? a.seg_bias[1] : a.seg_bias[2];
             M = sg == 0 ? a.seg_M[0] : sg == 1 ? a.seg_M[1] : a.seg_M[2];
@@ -517,6 +518,32 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
         if (bias) {
             const float4 b = *reinterpret_cast<const float4 *>(bias + m);
             o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w;
+        }
+        if (a.rope.pos && kind != GEMV_KIND_PLAIN) {
+            // rows m..m+3 of a q / k / v projection: two neighbouring pairs of one head (head_dim % 4 == 0)
+            const int hd = a.rope.head_dim, head = m / hd, dd = m - head * hd, pos = a.rope.pos[t];
+            if (kind != GEMV_KIND_V) {
+                if (dd < a.rope.n_rot) {
+                    float sn, cs;
+                    sincosf((float)pos * a.rope.inv_freq[dd >> 1], &sn, &cs);
+                    const float x0 = o.x, x1 = o.y;
+                    o.x = x0 * cs - x1 * sn; o.y = x0 * sn + x1 * cs;
+                }
+                if (dd + 2 < a.rope.n_rot) {
+                    float sn, cs;
+                    sincosf((float)pos * a.rope.inv_freq[(dd >> 1) + 1], &sn, &cs);
+                    const float x0 = o.z, x1 = o.w;
+                    o.z = x0 * cs - x1 * sn; o.w = x0 * sn + x1 * cs;
+                }
+            }
+            if (kind == GEMV_KIND_Q) {
+                *reinterpret_cast<float4 *>(Y + (size_t)t * ldy + m) = o;
+            } else {
+                uint16_t *cache = kind == GEMV_KIND_K ? a.rope.kcache : a.rope.vcache;
+                *reinterpret_cast<uint2 *>(cache + (((size_t)a.rope.seq[t] * a.rope.n_kv + head) * a.rope.n_ctx + pos) * hd + dd) =
+                    make_uint2(pack_h2(o.x, o.y), pack_h2(o.z, o.w));
+            }
+            continue;
         }
         if (a.residual) {
             const float4 r = *reinterpret_cast<const float4 *>(a.residual + (size_t)t * a.ldres + m);
@@ -575,6 +602,27 @@ static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
     return k.ksplit > 1 ? launch_gemm_kernel<TYPE, PACKED, XDIRECT, true, false>(k, grid, stream) : launch_gemm_kernel<TYPE, PACKED, XDIRECT, false, false>(k, grid, stream);
 }
 
+// slices of K for a launch of row_blocks x t_blocks workgroups (1: not split); *k_per_split = k-steps per slice
+static int split_plan(const GemmArgs &a, int row_blocks, int t_blocks, int *k_per_split) {
+    const int n_all = a.K / GK;
+    *k_per_split = n_all;
+    if (!a.part) return 1;
+    const int wgs = row_blocks * t_blocks, ncu = gemm_n_cu();
+    int ks = 1;
+    while (ks < 16 && wgs * ks * 2 <= ncu && n_all / (ks * 2) >= 8 &&
+           (size_t)(ks * 2) * a.T * row_blocks * GM * sizeof(float) <= a.part_bytes) ks *= 2;
+    if (ks <= 1) return 1;
+    *k_per_split = (n_all + ks - 1) / ks;
+    return (n_all + *k_per_split - 1) / *k_per_split;      // no empty slice
+}
+
+int gemm_split_count(const GemmArgs &a) {
+    if (a.M <= 0 || a.K <= 0 || a.T <= 0) return 1;
+    const int row_blocks = a.y16_k8 ? (a.M + GM / 2 - 1) / (GM / 2) : (a.M + GM - 1) / GM;
+    int kps;
+    return split_plan(a, row_blocks, (a.T + GN - 1) / GN, &kps);
+}
+
 int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     if (!a.X || a.M <= 0 || a.K <= 0 || a.T <= 0) return fail(MESH_ERR_INVALID, "gemm: null pointer or empty shape");
     if (a.y16_k8 || a.n_seg > 1) {
@@ -594,19 +642,12 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     // A launch of fewer workgroups than CUs walks all of K in each of them while the rest of the chip idles: split K
     // over blockIdx.z (slices of at least 8 k-steps, at most one workgroup per CU in total, partial tiles within the
     // scratch the caller gave).
-    k.ksplit = 1;
     k.k_per_split = a.K / GK;
-    if (a.part) {
-        const int n_all = a.K / GK, wgs = (int)(grid.x * grid.y), ncu = gemm_n_cu();
-        int ks = 1;
-        while (ks < 16 && wgs * ks * 2 <= ncu && n_all / (ks * 2) >= 8 &&
-               (size_t)(ks * 2) * a.T * row_blocks * GM * sizeof(float) <= a.part_bytes) ks *= 2;
-        if (ks > 1) {
-            k.k_per_split = (n_all + ks - 1) / ks;
-            k.ksplit = (n_all + k.k_per_split - 1) / k.k_per_split;      // no empty slice
-            grid.z = (unsigned)k.ksplit;
-        }
-    }
+    k.ksplit = split_plan(a, row_blocks, (int)grid.y, &k.k_per_split);
+    grid.z = (unsigned)k.ksplit;
+    if (a.rope.pos && k.ksplit <= 1) return fail(MESH_ERR_INVALID, "gemm: RoPE / KV append needs a split launch");
+    if (a.rope.pos && (a.y16_k8 || a.residual || a.rope.head_dim % 4 || a.rope.n_rot % 2))
+        return fail(MESH_ERR_INVALID, "gemm: RoPE / KV append on a launch it does not fit");
     if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
     if (a.x_k8) {

@@ -36,8 +36,15 @@ struct GemmArgs {
     float *part = nullptr;
     size_t part_bytes = 0;
     int ksplit = 1, k_per_split = 0;
+    // Optional, split launches only (ask gemm_split_count first): matrix i is the q / k / v projection of a layer
+    // (kind[i], GEMV_KIND_*); the second kernel rotates q and k rows (neighbouring-pair RoPE) and appends k and v to
+    // the f16 KV cache instead of storing them to their outputs, like the projection epilogues of the decode kernels.
+    GemvRope rope;
+    int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
 };
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
+// Number of K slices gemm_kquant will use for this launch (1: not split).
+int gemm_split_count(const GemmArgs &a);
 
 // GEMM layout of a K-quant matrix: a second copy for the prefill GEMM, arranged by the workgroup tile that consumes it.
 // One chunk per (128-row block, 64-element k-step), chunks of a row block consecutive in k.  A chunk holds, for each of

@@ -718,8 +718,23 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
                 g.seg_bias[i] = b[i]->present() ? static_cast<const float *>(b[i]->data) : nullptr;
                 g.M += (int)w[i]->M;
             }
+            GemmArgs gv = gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv));
+            // RoPE and the KV append ride in the second kernel of split launches (both launches must be split)
+            if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+                !L.k_norm.present() && hp.head_dim % 4 == 0 && hp.n_rot % 2 == 0 && gemm_split_count(g) > 1 &&
+                (L.qkv_fused == 3 || gemm_split_count(gv) > 1)) {
+                GemvRope r;
+                r.pos = s->d_pos; r.seq = s->d_seq; r.inv_freq = st->rope_inv_freq;
+                r.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
+                r.vcache = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
+                r.head_dim = (int)hp.head_dim; r.n_rot = (int)hp.n_rot; r.n_kv = (int)hp.n_head_kv; r.n_ctx = st->n_ctx;
+                g.rope = r; gv.rope = r;
+                g.kind[0] = GEMV_KIND_Q; g.kind[1] = GEMV_KIND_K; g.kind[2] = GEMV_KIND_V;
+                gv.kind[0] = GEMV_KIND_V;
+                rope_fused = true;
+            }
             if ((rc = gemm_kquant(g, stream)) != MESH_OK) return rc;
-            if (L.qkv_fused == 2 && (rc = gemm_kquant(gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv)), stream)) != MESH_OK) return rc;
+            if (L.qkv_fused == 2 && (rc = gemm_kquant(gv, stream)) != MESH_OK) return rc;
         } else {
         if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wq, s->xn16, E, T, s->q, QD, &L.bq)), stream)) != MESH_OK) return rc;
         if ((rc = gemm_kquant(gemm_k8(gemm_of(L.wk, s->xn16, E, T, s->k, KD, &L.bk)), stream)) != MESH_OK) return rc;
