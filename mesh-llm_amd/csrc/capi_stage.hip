@@ -29,7 +29,11 @@ int mesh_weight_upload(int type, const void *host_data, int64_t n_rows, int64_t 
     w->t.tiled = type_is_tiled(type);
     w->t.bytes = w->t.tiled ? (size_t)tiled_bytes(type, n_rows, row_len) : w->gguf_bytes;
     hipError_t e = hipMalloc(&w->t.data, w->t.bytes);
-    if (e != hipSuccess) { delete w; return fail(MESH_ERR_NOMEM, "mesh_weight_upload: hipMalloc(%zu) failed: %s", w->t.bytes, hipGetErrorString(e)); }
+    if (e != hipSuccess) {
+        const size_t wanted = w->t.bytes;
+        delete w;
+        return fail(MESH_ERR_NOMEM, "mesh_weight_upload: hipMalloc(%zu) failed: %s", wanted, hipGetErrorString(e));
+    }
     int rc = MESH_OK;
     if (!w->t.tiled) {
         e = hipMemcpy(w->t.data, host_data, w->gguf_bytes, hipMemcpyHostToDevice);

@@ -9,7 +9,7 @@
 
 namespace mesh {
 
-constexpr int ROUTE_MAX_PER_LANE = 8;      // up to 512 experts
+constexpr int ROUTE_MAX_PER_LANE = MOE_EXPERTS_MAX / 64;
 
 // softmax -> (+mask) -> top-k of one token's logits by one wave; NPL = experts per lane (n_expert <= 64 * NPL)
 template <int NPL>

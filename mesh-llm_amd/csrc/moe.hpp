@@ -5,6 +5,9 @@
 
 namespace mesh {
 
+// most experts one routing wave can rank (64 lanes x 8 candidates each)
+constexpr int MOE_EXPERTS_MAX = 512;
+
 struct MoeRouteArgs {
     const float *logits = nullptr;   // [T][n_expert] router outputs
     const float *mask = nullptr;     // optional [n_expert]: 0 = allowed, -inf = masked out

@@ -57,6 +57,14 @@ int hparams_from_gguf(const GgufFile &g, HParams &hp) {
     g.get_u32(a + ".expert_used_count", hp.n_expert_used);
     g.get_u32(a + ".expert_feed_forward_length", hp.n_ff_exp);
     hp.rope_mode = (a == "llama") ? ROPE_NORM : ROPE_NEOX;
+    // Frequency scaling (linear / yarn keys, or the per-frequency factors tensor of Llama-3.1 files) would change every
+    // rotation angle; no kernel here applies it, so such a file is refused instead of decoded with unscaled angles.
+    {
+        std::string scaling;
+        if (g.get_str(a + ".rope.scaling.type", scaling) && !scaling.empty() && scaling != "none")
+            return fail(MESH_ERR_UNSUPPORTED, "gguf: rope scaling type '%s' is not supported", scaling.c_str());
+        if (g.find("rope_freqs.weight")) return fail(MESH_ERR_UNSUPPORTED, "gguf: rope frequency factors (rope_freqs.weight) are not supported");
+    }
     if (hp.n_layer == 0 || hp.n_embd == 0 || hp.head_dim == 0) return fail(MESH_ERR_FORMAT, "gguf: zero-sized model dimensions");
     if (hp.n_rot > hp.head_dim || hp.n_rot % 2) return fail(MESH_ERR_FORMAT, "gguf: rope dimension count %u does not fit head_dim %u", hp.n_rot, hp.head_dim);
     if (a == "qwen3moe" && (hp.n_expert == 0 || hp.n_expert_used == 0 || hp.n_expert_used > hp.n_expert))
@@ -224,6 +232,7 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
     const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, KD = (int64_t)hp.n_head_kv * hp.head_dim;
     const bool moe = hp.arch == "qwen3moe";
     st->layers.resize((size_t)(layer_end - layer_begin));
+    int64_t n_expert_file = -1;
     for (int il = layer_begin; il < layer_end; ++il) {
         LayerWeights &L = st->layers[(size_t)(il - layer_begin)];
         const std::string p = "blk." + std::to_string(il) + ".";
@@ -253,6 +262,12 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
             const int64_t ne = (int64_t)gi->ne[1];     // experts present in this file (a shard has fewer than the model)
             const int64_t ffe = hp.n_ff_exp;
             if (ffe == 0) return fail(MESH_ERR_FORMAT, "gguf: expert_feed_forward_length missing");
+            // the session sizes its routing buffers by the first layer's count, and one lane of the router holds at
+            // most MOE_EXPERTS_MAX / 64 experts
+            if (n_expert_file < 0) n_expert_file = ne;
+            if (ne != n_expert_file || ne < (int64_t)hp.n_expert_used || ne > MOE_EXPERTS_MAX)
+                return fail(MESH_ERR_FORMAT, "gguf: layer %d routes over %lld experts (first layer %lld, %u used per token, at most %d supported)", il,
+                            (long long)ne, (long long)n_expert_file, hp.n_expert_used, MOE_EXPERTS_MAX);
             if ((rc = ld.load(p + "ffn_gate_inp.weight", L.gate_inp, E, ne, 1, true, false, false)) ||
                 (rc = ld.load(p + "ffn_gate_exps.weight", L.gate_exps, E, ffe, ne, true, true, false)) ||
                 (rc = ld.load(p + "ffn_up_exps.weight", L.up_exps, E, ffe, ne, true, true, false)) ||
@@ -475,6 +490,7 @@ static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
 constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
+constexpr int LOGITS_TOKENS_MAX = 128;        // logits rows the host-pointer entry point stages per call
 // calls with at least this many tokens take the MFMA GEMM path (MESH_GEMM_MIN_TOKENS overrides, for tuning)
 static int gemm_min_tokens() {
     static int v = 0;
@@ -533,7 +549,6 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->v, B * KD)) || (rc = fbuf(&s->attn, B * QD)) || (rc = fbuf(&s->ffn, B * ff)) ||
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
-    if (st->output.present() && (rc = fbuf(&s->logits, B * (size_t)st->output.M)) != MESH_OK) return rc;
     if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens())) {
         const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
@@ -571,11 +586,12 @@ int session_new(mesh_stage *st, mesh_session **out) {
     s->d_seq = s->d_pos + B;
     s->d_tok = s->d_seq + B;
     MESH_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->h_meta), META_SLOTS * 3 * B * sizeof(int32_t), hipHostMallocDefault));
-    // staging for packed in/out of the host-pointer entry point: f32 rows of n_embd (or logits) are the largest
-    const size_t out_row = std::max<size_t>(hp.n_embd, st->output.present() ? (size_t)st->output.M : 0);
-    s->io_stage_bytes = B * out_row * sizeof(float);
-    if ((rc = sess_alloc(s.get(), &s->io_stage, 2 * s->io_stage_bytes)) != MESH_OK) return rc;
-    MESH_HIP_TRY(hipHostMalloc(&s->h_io, 2 * s->io_stage_bytes, hipHostMallocDefault));
+    // staging for packed in/out of the host-pointer entry point: f32 rows of n_embd in; the same or logits rows out
+    // (logits of at most LOGITS_TOKENS_MAX tokens per call: a row of a 152k vocabulary is 0.6 MB)
+    s->io_stage_bytes = B * (size_t)hp.n_embd * sizeof(float);
+    s->io_out_bytes = std::max(s->io_stage_bytes, st->output.present() ? std::min<size_t>(B, LOGITS_TOKENS_MAX) * (size_t)st->output.M * sizeof(float) : 0);
+    if ((rc = sess_alloc(s.get(), &s->io_stage, s->io_stage_bytes + s->io_out_bytes)) != MESH_OK) return rc;
+    MESH_HIP_TRY(hipHostMalloc(&s->h_io, s->io_stage_bytes + s->io_out_bytes, hipHostMallocDefault));
     if ((rc = mega_setup(s.get())) != MESH_OK) return rc;
     MESH_HIP_TRY(hipStreamSynchronize(s->stream));
     *out = s.release();
@@ -1137,6 +1153,8 @@ int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fm
     if (!b || b->n_tokens <= 0) return fail(MESH_ERR_INVALID, "mesh_stage_decode: empty batch");
     if (b->n_tokens > st->n_batch_max) return fail(MESH_ERR_INVALID, "mesh_stage_decode: %d tokens exceed n_batch_max %d", b->n_tokens, st->n_batch_max);
     const int T = b->n_tokens;
+    if (out_fmt == MESH_LOGITS && T > LOGITS_TOKENS_MAX)
+        return fail(MESH_ERR_INVALID, "mesh_stage_decode: logits of %d tokens in one call (at most %d; mesh_stage_decode_dev has no such limit)", T, LOGITS_TOKENS_MAX);
     MESH_HIP_TRY(hipSetDevice(st->device));
     hipStream_t stream = s->stream;
     uint8_t *d_in = static_cast<uint8_t *>(s->io_stage), *d_out = d_in + s->io_stage_bytes;
@@ -1161,7 +1179,7 @@ int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fm
         MESH_HIP_TRY(hipMemcpyAsync(d_in, s->h_io, in_bytes, hipMemcpyHostToDevice, stream));
     }
     size_t len = 0;
-    if ((rc = stage_decode_dev(s, b, d_in, eff_in_fmt, d_out, out_fmt, std::min(out_cap, s->io_stage_bytes), &len)) != MESH_OK) {
+    if ((rc = stage_decode_dev(s, b, d_in, eff_in_fmt, d_out, out_fmt, std::min(out_cap, s->io_out_bytes), &len)) != MESH_OK) {
         if (out_len) *out_len = len;
         return rc;
     }

@@ -84,7 +84,7 @@ struct mesh_session {
     bool rope_in_gemv = true;        // MESH_GEMV_ROPE=0 at session creation keeps RoPE / KV append in their own kernel
     size_t k_layer_bytes = 0, v_layer_bytes = 0;
     // activations (f32), sized for n_batch_max tokens
-    float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *logits = nullptr;
+    float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr;
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
     uint16_t *xn16 = nullptr, *ffn16 = nullptr;
@@ -102,8 +102,9 @@ struct mesh_session {
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)
     unsigned meta_counter = 0;
     void *io_stage = nullptr;       // device staging for packed in/out of the host-pointer entry point
-    size_t io_stage_bytes = 0;
-    void *h_io = nullptr;           // pinned host staging
+    size_t io_stage_bytes = 0;      // input half; the output half (io_out_bytes) follows it
+    size_t io_out_bytes = 0;
+    void *h_io = nullptr;           // pinned host staging, same split
     int attn_splits_max = 0;
     // set per call: the batch is one run of consecutive positions of one sequence (first position, sequence), else -1
     int chunk_pos0 = -1, chunk_seq = -1;
