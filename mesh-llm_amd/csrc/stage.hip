@@ -1045,6 +1045,10 @@ constexpr int GRAPH_MAX_TOKENS = 32;
 constexpr size_t GRAPH_MAX_ENTRIES = 96;
 static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
     if (!s->graphs_on || s->profile || T > GRAPH_MAX_TOKENS) return run_layers(s, T, max_keys);
+    // A prefill chunk (consecutive positions of one sequence, enough tokens for the large-tile GEMM) runs the chunk
+    // attention kernel, whose first position and sequence are launch arguments: a replay would carry the captured
+    // chunk's.  Such calls are always launched eagerly.
+    if (s->chunk_pos0 >= 0 && T >= PREFILL_MIN_TOKENS) return run_layers(s, T, max_keys);
     const mesh_stage *st = s->stage;
     const int n_splits = attn_splits_for(T, (int)st->hp.n_head_kv, max_keys);
     const uint64_t key = (uint64_t)T | ((uint64_t)n_splits << 8) | ((uint64_t)(s->expert_mask_on ? 1 : 0) << 20);

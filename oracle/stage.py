@@ -4,9 +4,11 @@ composed from the pinned primitives of mesh_oracle.c.
 
 TEST INFRASTRUCTURE ONLY.  Parity against llama.cpp's CPU backend is unpinned: activations stay f32 and
 accumulate in f64 here, where ggml rounds them to Q8_K blocks before an integer dot and keeps some f16
-intermediates in flash attention.  What is pinned: every primitive (tests/test_oracle_ops.py), and the
-composition through its invariants (prefill == token-by-token decode, batch invariance, stage split ==
-unsplit model; tests/test_oracle_stage.py).
+intermediates in flash attention.  What is pinned: every primitive (tests/test_oracle_ops.py); the layer
+composition (forward, _moe, logits) against a decoder written separately in torch float64 from the architecture
+definitions, which must also reject deliberately broken compositions (tests/test_oracle_composition.py); and
+its invariants (prefill == token-by-token decode, batch invariance, stage split == unsplit model;
+tests/test_oracle_stage.py).
 """
 import numpy as np
 

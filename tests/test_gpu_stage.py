@@ -519,12 +519,13 @@ def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers)
     captured, then replays).  Every replay must give the bits the eager launches give: two sessions, graphs on and
     off, walk the same sequence of steps -- repeated shapes, other shapes and host synchronisations in between, KV
     depth growing past a change of the split count."""
-    m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=20, n_batch=24)
+    m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=20, n_batch=32)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(17))
     # (20 tokens: the large-tile GEMM with K split over workgroups, two kernels per projection, inside a graph)
     plan = [1, 1, 1, 4, 1, 4, 6, 1, 4, 6, 6, 1, 20, 1, 20] + [1] * 70 + [4, 4, 1, 6, 20]
     xs = [rng.standard_normal((T, E)).astype(np.float32) for T in plan]
+    chunk_xs = [rng.standard_normal((25, E)).astype(np.float32) for _ in range(8)]
     runs = []
     for flag in ("1", "0"):
         monkeypatch.setenv("MESH_STAGE_GRAPHS", flag)
@@ -538,12 +539,26 @@ def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers)
             for q in seqs:
                 nxt[q] += 1
             outs.append(ses.decode(x, pos, seq=seqs).copy())      # the host-pointer entry synchronises after every call
+        # prefill chunks of one sequence, three in a row with the same token count (17..32 tokens: the chunk attention
+        # kernel takes its first position as a launch argument, so these must never be replayed from a capture), with
+        # a 20-sequence decode batch of the same token count in between
+        for T, kind in ((20, "chunk"), (20, "chunk"), (20, "batch"), (20, "chunk"), (25, "chunk"), (25, "chunk"), (20, "batch"), (25, "chunk")):
+            x = chunk_xs[len(outs) - len(xs)]
+            if kind == "chunk":
+                seqs, pos = [19] * T, list(range(nxt[19], nxt[19] + T))
+                nxt[19] += T
+            else:
+                seqs = list(range(T))
+                pos = [nxt[q] for q in seqs]
+                for q in seqs:
+                    nxt[q] += 1
+            outs.append(ses.decode(x[:T], pos, seq=seqs).copy())
         runs.append((outs, [ses.kv_read(layers[0], q, 0, 8) for q in range(6)]))
         # shapes seen at least twice were captured and replayed; with graphs off nothing is
         assert (ses.graph_replays > 40) if flag == "1" else (ses.graph_replays == 0), ses.graph_replays
         ses.close()
     for i, (a, b) in enumerate(zip(runs[0][0], runs[1][0])):
-        assert np.array_equal(a, b), "step %d (T=%d)" % (i, plan[i])
+        assert np.array_equal(a, b), "step %d (T=%d)" % (i, a.size // (4 * E))
     for (ka, va), (kb, vb) in zip(runs[0][1], runs[1][1]):
         assert np.array_equal(ka, kb) and np.array_equal(va, vb)
     st.close()

@@ -53,7 +53,7 @@ def _model(name, seed=3, **kw):
             tensors[n] = (t, d, (x.view(np.float32) * f).view(np.uint8))
         if n.endswith(".bias"):
             t, d, x = tensors[n]
-            tensors[n] = (t, d, (x.view(np.float32) * 50).view(np.uint8))          # sigma 1 instead of 0.02
+            tensors[n] = (t, d, (x.view(np.float32) * 10).view(np.uint8))          # sigma 0.2 instead of 0.02
     return cfg, tensors
 
 
