@@ -81,6 +81,15 @@ size_t mesh_act_packed_size(int fmt, int64_t n_tokens, int64_t n_embd);
 int mesh_act_pack(int fmt, const float *src, void *dst, int64_t n);
 int mesh_act_unpack(int fmt, const void *src, float *dst, int64_t n);
 
+/* mesh_act_pack for callers that cannot allocate GPU memory (a serving loop that packs the boundary activation of
+ * every decode step, a harness that forbids hipMalloc): same arguments, same bytes out, but the device staging of
+ * the input and the packed output is a fixed array inside the library instead of two allocations per call.  No
+ * counterpart in the reference.  Limits: n <= 1 048 576 elements (256 tokens of 4096), MESH_ERR_INVALID beyond
+ * that; the array (8 MiB) is held on every GPU the library has run this call on until the process ends; all callers of
+ * one GPU share it, so calls are serialised inside the library (and calls from different processes do not interact:
+ * each process has its own copy). */
+int mesh_act_pack_noalloc(int fmt, const float *src, void *dst, int64_t n);
+
 /* Device-pointer forms: pointers are GPU addresses, work is queued on `stream` (a hipStream_t, NULL =
  * the default stream) and not waited for. */
 int mesh_act_pack_dev(int fmt, const float *d_src, void *d_dst, int64_t n, void *stream);

@@ -37,6 +37,7 @@ SIGNATURES = {
     "mesh_act_packed_size": (_sz, [_i32, _i64, _i64]),
     "mesh_act_pack": (_i32, [_i32, _vp, _vp, _i64]),
     "mesh_act_unpack": (_i32, [_i32, _vp, _vp, _i64]),
+    "mesh_act_pack_noalloc": (_i32, [_i32, _vp, _vp, _i64]),
     "mesh_act_pack_dev": (_i32, [_i32, _vp, _vp, _i64, _vp]),
     "mesh_act_unpack_dev": (_i32, [_i32, _vp, _vp, _i64, _vp]),
     "mesh_dequantize_dev": (_i32, [_i32, _vp, _vp, _i64, _vp]),
@@ -171,6 +172,16 @@ def act_pack(fmt, x):
     else:
         out = np.empty(x.size // per[0] * per[1], dtype=np.uint8)
     check(lib().mesh_act_pack(fmt, _np_ptr(x), _np_ptr(out), x.size))
+    return out
+
+
+def act_pack_noalloc(fmt, x):
+    """act_pack through the entry point that allocates no GPU memory (at most 1 Mi elements)."""
+    import numpy as np
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    per = {F32: (1, 4), F16: (1, 2), Q8_0: (32, 34)}.get(fmt)
+    out = np.empty(max(x.size * 4, 1) if per is None or x.size % per[0] else x.size // per[0] * per[1], dtype=np.uint8)
+    check(lib().mesh_act_pack_noalloc(fmt, _np_ptr(x), _np_ptr(out), x.size))
     return out
 
 

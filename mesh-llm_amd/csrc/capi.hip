@@ -2,6 +2,7 @@
 
 #include <cctype>
 #include <cstring>
+#include <mutex>
 
 #include "mesh_common.hpp"
 
@@ -42,6 +43,36 @@ struct DevScratch {
         return MESH_OK;
     }
 };
+
+// ---- device staging of mesh_act_pack_noalloc ---------------------------------------------------------------
+// The f32 input and the packed output of one call, at most NOALLOC_MAX_ELEMS elements: input at offset 0, output at
+// NOALLOC_OUT_OFFSET.  Every GPU the library runs on holds its own copy of the array until the process ends.  The
+// name below is a host-side handle only; the device address is asked for once per device (with that device current)
+// and everything -- copies and kernel arguments -- goes through that address.
+constexpr int64_t NOALLOC_MAX_ELEMS = (int64_t)1 << 20;                        // 256 tokens x 4096
+constexpr size_t NOALLOC_OUT_OFFSET = (size_t)NOALLOC_MAX_ELEMS * 4;
+constexpr size_t NOALLOC_BYTES = 2 * NOALLOC_OUT_OFFSET;                       // 8 MiB
+static __device__ __align__(256) uint8_t scratch[NOALLOC_BYTES];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static std::mutex g_noalloc_mu;                         // one call at a time: the array is shared by every caller of a GPU
+static uint8_t *g_noalloc_ptr[NOALLOC_MAX_DEVICES];     // device address of `scratch` on each device, null until asked for
+
+// device address of this device's copy of the staging array (caller holds g_noalloc_mu)
+static int noalloc_scratch(uint8_t **out) {
+    int dev = -1;
+    MESH_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fail(MESH_ERR_DEVICE, "mesh_act_pack_noalloc: device index %d out of range", dev);
+    if (!g_noalloc_ptr[dev]) {
+        void *p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(MESH_ERR_DEVICE, "mesh_act_pack_noalloc: no device address for the staging array on device %d: %s", dev, hipGetErrorString(e));
+        g_noalloc_ptr[dev] = static_cast<uint8_t *>(p);
+    }
+    *out = g_noalloc_ptr[dev];
+    return MESH_OK;
+}
 
 }  // namespace mesh
 
@@ -105,6 +136,27 @@ int mesh_act_pack(int fmt, const float *src, void *dst, int64_t n) {
     MESH_HIP_TRY(hipMemcpy(in.p, src, (size_t)n * 4, hipMemcpyHostToDevice));
     if ((rc = act_pack_dev(fmt, static_cast<const float *>(in.p), out.p, n, nullptr)) != MESH_OK) return rc;
     MESH_HIP_TRY(hipMemcpy(dst, out.p, (size_t)out_bytes, hipMemcpyDeviceToHost));
+    return MESH_OK;
+}
+
+int mesh_act_pack_noalloc(int fmt, const float *src, void *dst, int64_t n) {
+    if (!is_act_fmt(fmt)) return fail(MESH_ERR_INVALID, "mesh_act_pack_noalloc: format %d is not an activation format", fmt);
+    if (n < 0 || (n > 0 && (!src || !dst))) return fail(MESH_ERR_INVALID, "mesh_act_pack_noalloc: null pointer or negative count");
+    const int64_t out_bytes = row_bytes(fmt, n);
+    if (out_bytes < 0) return fail(MESH_ERR_INVALID, "mesh_act_pack_noalloc: %lld elements is not a whole number of blocks", (long long)n);
+    if (n > NOALLOC_MAX_ELEMS)
+        return fail(MESH_ERR_INVALID, "mesh_act_pack_noalloc: %lld elements exceed the fixed staging of %lld (use mesh_act_pack)", (long long)n,
+                    (long long)NOALLOC_MAX_ELEMS);
+    if (n == 0) return MESH_OK;
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    uint8_t *base = nullptr;
+    int rc = noalloc_scratch(&base);
+    if (rc != MESH_OK) return rc;
+    float *d_in = reinterpret_cast<float *>(base);
+    uint8_t *d_out = base + NOALLOC_OUT_OFFSET;
+    MESH_HIP_TRY(hipMemcpy(d_in, src, (size_t)n * 4, hipMemcpyHostToDevice));
+    if ((rc = act_pack_dev(fmt, d_in, d_out, n, nullptr)) != MESH_OK) return rc;
+    MESH_HIP_TRY(hipMemcpy(dst, d_out, (size_t)out_bytes, hipMemcpyDeviceToHost));
     return MESH_OK;
 }
 

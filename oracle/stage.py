@@ -18,8 +18,11 @@ import oracle as O
 class StageOracle:
     """tensors: dict name -> (ggml_type, dims (ne0, ne1[, ne2]), uint8 ndarray) as written to the GGUF file."""
 
-    def __init__(self, cfg, tensors, layer_begin, layer_end, n_ctx, n_seq_max=1, expert_mask=None, kv_types=None):
-        """kv_types: (K type, V type) of the cache, each F16, Q8_0 or Q4_0 (the tiers of
+    def __init__(self, cfg, tensors, layer_begin, layer_end, n_ctx, n_seq_max=1, expert_mask=None, kv_types=None, blas=False):
+        """blas: projections of calls with many tokens go through numpy's float64 matmul over the dequantised matrix
+        (x @ dequantize(W).T -- the definition mesh_oracle.c's mul_mat is pinned to in tests/test_oracle_ops.py) instead
+        of the C loop, which keeps prefill-sized checks within seconds.
+        kv_types: (K type, V type) of the cache, each F16, Q8_0 or Q4_0 (the tiers of
         mesh-llm/src/inference/launch.rs:568-591); None = f16 / f16.  A quantised cache is held as the f32 values its
         blocks dequantise to (rows quantised per 32 elements along head_dim, as ggml stores the cache rows)."""
         self.c = cfg
@@ -33,6 +36,7 @@ class StageOracle:
         self.v = np.zeros_like(self.k)
         self.rope_mode = O.ROPE_NORM if cfg["arch"] == "llama" else O.ROPE_NEOX
         self.expert_mask = expert_mask
+        self.blas = blas
 
     def _w(self, name):
         ttype, dims, data = self.t[name]
@@ -47,6 +51,18 @@ class StageOracle:
         ttype, dims, data = self._w(name)
         K, M = dims[0], dims[1]
         b = self._f32(bias) if bias is not None and bias in self.t else None
+        if self.blas and x.shape[0] >= 32:
+            x64 = np.asarray(x, np.float64)
+            y = np.empty((x.shape[0], M), np.float32)
+            rb = O.row_bytes(ttype, K)
+            for m0 in range(0, M, 1024):          # row blocks: the float64 copy of a block stays cache-sized
+                m1 = min(M, m0 + 1024)
+                Wd = O.dequantize(ttype, data[m0 * rb:m1 * rb], (m1 - m0) * K).reshape(m1 - m0, K).astype(np.float64)
+                blk = x64 @ Wd.T
+                if b is not None:
+                    blk += b[m0:m1].astype(np.float64)
+                y[:, m0:m1] = blk
+            return y
         return O.mul_mat(ttype, data, M, K, x, b)
 
     def embed(self, ids):

@@ -103,8 +103,38 @@ CONFIGS = {
 }
 
 
-def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_expert_local=None, fast=False):
-    """Returns (kvs, tensors) for write_gguf; tensors only for `layers` (absolute indices)."""
+ZIPF_CHANNEL, ZIPF_LEVEL = 0, 8.0
+
+
+def zipf_expert_bias(n_expert, n_local, seed, s=1.1):
+    """Log-popularity of the experts a node holds when expert popularity follows Zipf(s): rank r (1 = most popular, a
+    seeded permutation of the model's experts) has p ~ r^-s, bias = ln p.  A node that holds n_local < n_expert
+    experts gets every (n_expert / n_local)-th pick of a snake draft over the ranking (node 0's share in
+    mesh-llm/src/inference/moe.rs:597-643), renumbered in ascending rank."""
+    ranks = np.arange(1, n_expert + 1)
+    if n_local and n_local < n_expert:
+        n_nodes = n_expert // n_local
+        picks = [r for i, r in enumerate(ranks) if (i % (2 * n_nodes)) in (0, 2 * n_nodes - 1)]
+        ranks = np.array(picks[:n_local])
+    bias = -s * np.log(ranks.astype(np.float64))
+    order = np.random.Generator(np.random.PCG64(seed)).permutation(len(bias))
+    return bias[order].astype(np.float32)
+
+
+def zipf_hidden_state(rng, T, E):
+    """Hidden-state rows for a model built with router="zipf": N(0,1) with the carrier channel held at ZIPF_LEVEL (real
+    models carry such constant 'massive activation' channels too)."""
+    x = rng.standard_normal((T, E)).astype(np.float32)
+    x[:, ZIPF_CHANNEL] = ZIPF_LEVEL
+    return x
+
+
+def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_expert_local=None, fast=False, router=None):
+    """Returns (kvs, tensors) for write_gguf; tensors only for `layers` (absolute indices).
+    router="zipf" (mixture-of-experts models): router logits ~ N(0,1) plus a Zipf(1.1) expert bias.  The architecture has
+    no router bias tensor, so the bias rides on one channel of the hidden state that the inputs hold at a constant
+    level (zipf_hidden_state): router rows are N(0, 1/n_embd) (unit-variance logits on RMS-normalised inputs), and
+    their weight on the carrier channel is bias_e divided by the channel's normalised level."""
     c = cfg
     a = c["arch"]
     E, H, HK, HD, FF = c["n_embd"], c["n_head"], c["n_head_kv"], c["head_dim"], c["n_ff"]
@@ -165,7 +195,15 @@ def build_tensors(cfg, layers, seed=42, with_embd=False, with_output=False, n_ex
         else:
             FE = c["n_ff_exp"]
             r = rng_for(14)
-            tensors.append((p + "ffn_gate_inp.weight", F32, (E, NEL), (r.standard_normal(NEL * E) * 0.02).astype(np.float32).view(np.uint8)))
+            if router == "zipf":
+                Wr = (r.standard_normal((NEL, E)) / np.sqrt(E)).astype(np.float32)
+                # the carrier channel after the RMS norm: level / rms(row) with rms^2 = ((E - 1) + level^2) / E, times its norm weight
+                level = ZIPF_LEVEL / np.sqrt(((E - 1) + ZIPF_LEVEL ** 2) / E)
+                nw = tensors[[n for n, *_ in tensors].index(p + "ffn_norm.weight")][3].view(np.float32)[ZIPF_CHANNEL]
+                Wr[:, ZIPF_CHANNEL] = zipf_expert_bias(NE, NEL, seed + il) / (level * nw)
+                tensors.append((p + "ffn_gate_inp.weight", F32, (E, NEL), Wr.reshape(-1).view(np.uint8)))
+            else:
+                tensors.append((p + "ffn_gate_inp.weight", F32, (E, NEL), (r.standard_normal(NEL * E) * 0.02).astype(np.float32).view(np.uint8)))
             add(p + "ffn_gate_exps.weight", q4km_type("ffn_gate_exps", il, nl, E), FE, E, rng_for(6), n_e=NEL)
             add(p + "ffn_up_exps.weight", q4km_type("ffn_up_exps", il, nl, E), FE, E, rng_for(7), n_e=NEL)
             add(p + "ffn_down_exps.weight", q4km_type("ffn_down_exps", il, nl, FE), E, FE, rng_for(8), n_e=NEL)

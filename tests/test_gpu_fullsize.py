@@ -1,0 +1,219 @@
+"""Parity of the stage executor ON THE CONFIGURATIONS THE TOLERANCE IS STATED ON: relative L2 <= 1e-2 between the
+GPU stage's output hidden state and the CPU oracle's on identical seeded weights and inputs.
+
+  C3  Llama-3-8B-shaped stage, ALL 16 layers (0-15 of 32), 4096-token KV context filled to depth 4095: decode at batch
+      1, 4 and 16 (mat-vec kernels, skinny MFMA GEMM, matrix-core decode attention); a 2048-token prefill through two
+      real-shape layers and a 256-token prefill through all 16 (large-tile MFMA GEMM, chunk attention).
+  C4  Qwen2.5-32B-shaped layers (hidden 5120, 40 / 8 heads, FFN 27648, q/k/v bias): decode batch 24 and 32 (large-tile
+      GEMM with K split over workgroups), a 320-token prefill (chunk attention with 5 query heads per KV head), over
+      f16 and over q8_0 / q4_0 caches.
+  C5  Qwen3-30B-A3B-shaped 64-expert shard layer, router logits ~ N(0,1) + Zipf(1.1) expert bias, batch 16 on top of a
+      filled KV cache.
+Every test prints the figure it measured.  The oracle's projections of prefill-sized calls go through numpy's float64
+matmul over the dequantised weights (StageOracle(blas=True)), the definition its C loop is pinned to.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import models
+import oracle
+from oracle.stage import StageOracle
+from util import mesh
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+NORTH_STAR = 1e-2
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64).reshape(-1)
+    b = np.asarray(b, np.float64).reshape(-1)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def report(what, value):
+    print("[fullsize] %s: rel-L2 %.3e" % (what, value), file=sys.stderr, flush=True)
+
+
+def random_kv(rng, n_pos, n_kv=8, hd=128, scale=0.5):
+    return (rng.standard_normal((n_pos, n_kv, hd)) * scale).astype(np.float16).view(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def c3_model(tmp_path_factory):
+    """The 16-layer stage file of the benchmark (same generator, same seed)."""
+    cfg = models.CONFIGS["llama3-8b"]
+    path = os.path.join(models.tmp_dir(), "mesh_test_c3_%d.gguf" % os.getpid())
+    tensors = models.write_model(path, cfg, range(16), seed=42, fast=True)
+    yield cfg, tensors, path
+    if os.path.exists(path):
+        os.unlink(path)
+
+
+def test_c3_sixteen_layer_stage_decode_at_kv_depth_4095(c3_model):
+    m = mesh()
+    cfg, tensors, path = c3_model
+    n_ctx, n_seq, depth = 4096, 16, 4095
+    st = m.Stage(path, 0, 16, n_ctx=n_ctx, n_seq_max=n_seq, n_batch_max=16)
+    assert st.weight_bytes == 2093219840          # the stage the roofline is quoted on
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 0, 16, n_ctx, n_seq_max=n_seq)
+    rng = np.random.Generator(np.random.PCG64(4095))
+    for il in range(16):
+        k, v = random_kv(rng, depth), random_kv(rng, depth)       # every sequence holds the same context
+        for s in range(n_seq):
+            ses.kv_write(il, s, 0, k, v)
+        orc.k[il, :, :, :depth] = np.ascontiguousarray(k.transpose(1, 0, 2))[None]
+        orc.v[il, :, :, :depth] = np.ascontiguousarray(v.transpose(1, 0, 2))[None]
+    for seqs in ([0], [1, 2, 3, 4], list(range(16))):
+        T = len(seqs)
+        x = rng.standard_normal((T, 4096)).astype(np.float32)
+        pos = [depth] * T
+        got = ses.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
+        ref = orc.forward(x, pos, seq=seqs)
+        r = rel_l2(got, ref)
+        report("C3 16 layers, KV depth 4095, decode batch %d" % T, r)
+        assert r <= NORTH_STAR, T
+        assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR
+        # the q8_0 boundary activation of the same step is the codec applied to that output
+        packed = ses.decode(x, pos, seq=seqs, out_fmt=m.Q8_0)
+        assert np.array_equal(packed, oracle.quantize_q8_0(got.reshape(-1)))
+    ses.close(); st.close()
+
+
+def test_c3_prefill_2048_tokens_two_layers(c3_model):
+    m = mesh()
+    cfg, tensors, path = c3_model
+    T = 2048
+    st = m.Stage(path, 3, 5, n_ctx=T + 8, n_seq_max=1, n_batch_max=T)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 3, 5, T + 8, blas=True)
+    rng = np.random.Generator(np.random.PCG64(2048))
+    x = rng.standard_normal((T, 4096)).astype(np.float32)
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, 4096)
+    ref = orc.forward(x, np.arange(T))
+    r = rel_l2(got, ref)
+    report("C3 layers 3-4, prefill 2048 tokens", r)
+    assert r <= NORTH_STAR
+    assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR
+    # one decode token on top of the 2048 cached positions
+    x1 = rng.standard_normal((1, 4096)).astype(np.float32)
+    r1 = rel_l2(ses.decode(x1, [T]).view(np.float32), orc.forward(x1, [T]))
+    report("C3 layers 3-4, decode on the prefilled cache", r1)
+    assert r1 <= NORTH_STAR
+    ses.close(); st.close()
+
+
+def test_c3_prefill_256_tokens_sixteen_layers(c3_model):
+    m = mesh()
+    cfg, tensors, path = c3_model
+    T = 256
+    st = m.Stage(path, 0, 16, n_ctx=T + 8, n_seq_max=1, n_batch_max=T)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 0, 16, T + 8, blas=True)
+    rng = np.random.Generator(np.random.PCG64(256))
+    x = rng.standard_normal((T, 4096)).astype(np.float32)
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, 4096)
+    ref = orc.forward(x, np.arange(T))
+    r = rel_l2(got, ref)
+    report("C3 16 layers, prefill 256 tokens", r)
+    assert r <= NORTH_STAR
+    assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR
+    x1 = rng.standard_normal((1, 4096)).astype(np.float32)
+    r1 = rel_l2(ses.decode(x1, [T]).view(np.float32), orc.forward(x1, [T]))
+    report("C3 16 layers, decode on the prefilled cache", r1)
+    assert r1 <= NORTH_STAR
+    ses.close(); st.close()
+
+
+@pytest.mark.parametrize("kv", ["f16", "q8_0/q4_0"])
+def test_c4_qwen25_32b_layers_wide_batches_and_prefill(tmp_path, kv):
+    """Layers 7 (q6_K attn_v / ffn_down) and 8 (all q4_K) of the 64-layer model."""
+    m = mesh()
+    cfg = models.CONFIGS["qwen2.5-32b"]
+    path = os.path.join(str(tmp_path), "c4.gguf")
+    tensors = models.write_model(path, cfg, [7, 8], seed=42, fast=True)
+    assert tensors["blk.7.ffn_down.weight"][0] == models.Q6_K and tensors["blk.8.ffn_down.weight"][0] == models.Q4_K
+    n_ctx, n_seq, depth, E = 512, 32, 100, 5120
+    kv_m = {"f16": (m.F16, m.F16), "q8_0/q4_0": (m.Q8_0, m.Q4_0)}[kv]
+    kv_o = {"f16": None, "q8_0/q4_0": (oracle.Q8_0, oracle.Q4_0)}[kv]
+    st = m.Stage(path, 7, 9, n_ctx=n_ctx, n_seq_max=n_seq, n_batch_max=320, kv_types=kv_m)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 7, 9, n_ctx, n_seq_max=n_seq, kv_types=kv_o, blas=True)
+    rng = np.random.Generator(np.random.PCG64(32))
+    for il in (7, 8):
+        for s in range(1, n_seq):
+            k, v = random_kv(rng, depth), random_kv(rng, depth)
+            ses.kv_write(il, s, 0, k, v)
+            kf, vf = k.view(np.float16).astype(np.float32), v.view(np.float16).astype(np.float32)
+            if kv_o:
+                orc.k[il - 7, s, :, :depth] = oracle.kv_round(kv_o[0], kf).transpose(1, 0, 2)
+                orc.v[il - 7, s, :, :depth] = oracle.kv_round(kv_o[1], vf).transpose(1, 0, 2)
+            else:
+                orc.k[il - 7, s, :, :depth] = k.transpose(1, 0, 2)
+                orc.v[il - 7, s, :, :depth] = v.transpose(1, 0, 2)
+    # 320-token prefill chunk of sequence 0 (5 query heads per KV head in the chunk attention kernel), then a second chunk
+    for pos0, T in ((0, 320), (320, 100)):
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        pos = np.arange(pos0, pos0 + T)
+        got = ses.decode(x, pos).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos)
+        r = rel_l2(got, ref)
+        report("C4 layers 7-8, %s KV, prefill chunk of %d tokens at %d" % (kv, T, pos0), r)
+        assert r <= NORTH_STAR
+    # decode batches of 24 and 32 single-token sequences at KV depth 100 / 101: large-tile GEMM, K split over workgroups
+    nxt = [420] + [depth] * (n_seq - 1)
+    for seqs in (list(range(1, 25)), list(range(32))):
+        T = len(seqs)
+        pos = [nxt[q] for q in seqs]
+        for q in seqs:
+            nxt[q] += 1
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        got = ses.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos, seq=seqs)
+        r = rel_l2(got, ref)
+        report("C4 layers 7-8, %s KV, decode batch %d" % (kv, T), r)
+        assert r <= NORTH_STAR, T
+    ses.close(); st.close()
+
+
+def test_c5_expert_shard_layer_zipf_router_on_filled_cache(tmp_path):
+    """A 64-expert shard layer of the 128-expert model, router logits ~ N(0,1) + Zipf(1.1) expert bias (models.py),
+    decode batch 16 at KV depth 200 and one more step on top."""
+    m = mesh()
+    cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
+    path = os.path.join(str(tmp_path), "shard.gguf")
+    tensors = models.write_model(path, cfg, [5, 6], seed=9, n_expert_local=64, fast=True, router="zipf")
+    n_ctx, depth, E = 256, 200, 2048
+    st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=16, n_batch_max=16)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 5, 7, n_ctx, n_seq_max=16)
+    rng = np.random.Generator(np.random.PCG64(55))
+    for il in (5, 6):
+        for s in range(16):
+            k, v = random_kv(rng, depth, n_kv=4), random_kv(rng, depth, n_kv=4)
+            ses.kv_write(il, s, 0, k, v)
+            orc.k[il - 5, s, :, :depth] = k.transpose(1, 0, 2)
+            orc.v[il - 5, s, :, :depth] = v.transpose(1, 0, 2)
+    distinct = []
+    for step in range(2):
+        x = models.zipf_hidden_state(rng, 16, E)
+        pos, seq = np.full(16, depth + step, np.int32), np.arange(16, dtype=np.int32)
+        got = ses.decode(x, pos, seq=seq).view(np.float32).reshape(16, E)
+        ref = orc.forward(x, pos, seq=seq)
+        r = rel_l2(got - x, ref - x)              # what the layers add (the carrier channel would dominate the norm)
+        report("C5 shard layers 5-6, Zipf router, batch 16 at KV depth %d (of the layers' contribution)" % (depth + step), r)
+        assert r <= NORTH_STAR
+        ids = ses.moe_last_ids(16)
+        assert np.array_equal(np.sort(ids, axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+        distinct.append(len(set(ids.reshape(-1))))
+    # the bias concentrates the batch on the popular experts: far fewer than the ~56 of 64 a uniform router touches
+    print("[fullsize] C5 distinct experts touched by 16 tokens x top-8: %s" % distinct, file=sys.stderr, flush=True)
+    assert max(distinct) <= 44
+    ses.close(); st.close()
