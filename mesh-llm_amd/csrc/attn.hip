@@ -7,6 +7,7 @@
 // are processed together, so each K/V byte is read once per token.
 
 #include "attn.hpp"
+#include "q16.hpp"
 
 namespace mesh {
 
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_kernel(AttnArgs a) {
 // sees them with broadcast reads and the partial rows are fetched with independent loads.
 // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
 __global__ __launch_bounds__(128) void attn_combine_kernel(const float *p_part, const float *p_ml, float *p_out, _Float16 *p_out16_k8,
-                                                           int p_n_splits, int p_n_head, int p_head_dim) {
+                                                           uint8_t *p_out_q16, int p_n_splits, int p_n_head, int p_head_dim) {
     __shared__ float s_m[ATTN_SPLITS_CAP], s_l[ATTN_SPLITS_CAP];
     const int h = blockIdx.x, t = blockIdx.y, dd = threadIdx.x;
     const size_t row = (size_t)t * p_n_head + h;
@@ -284,7 +285,9 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float *p_part, 
         num = fmaf(pp[(size_t)s2 * p_head_dim], w, num);
         den = fmaf(s_l[s2], w, den);
     }
-    if (p_out16_k8) {
+    if (p_out_q16) {
+        q16_store_block32(p_out_q16, p_n_head * p_head_dim, t, h * p_head_dim + dd, num / den);
+    } else if (p_out16_k8) {
         const size_t kk = (size_t)h * p_head_dim + dd, KK = (size_t)p_n_head * p_head_dim;
         p_out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(num / den);
     } else {
@@ -339,7 +342,7 @@ int attention(const AttnArgs &a, int T, hipStream_t stream) {
 }
 
 int attention_combine(const AttnArgs &a, int T, hipStream_t stream) {
-    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a.part, a.ml, a.out, a.out16_k8, a.n_splits, a.n_head, a.head_dim);
+    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a.part, a.ml, a.out, a.out16_k8, a.out_q16, a.n_splits, a.n_head, a.head_dim);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

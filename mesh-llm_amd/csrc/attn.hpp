@@ -37,6 +37,8 @@ struct AttnArgs {
     // attention_mma only: when set, the result is written as f16 in the k8-major activation layout of the batched GEMM
     // (gemm.hpp; row length n_head * head_dim) INSTEAD of `out`, so the output projection can read it as it is
     _Float16 *out16_k8 = nullptr;
+    // or, when set, quantised into the q16 activation layout of the skinny GEMM (gemm.hpp), also instead of `out`
+    uint8_t *out_q16 = nullptr;
     float scale = 1.f;
     int n_head = 0, n_kv = 0, group = 1, head_dim = 0, n_ctx = 0, n_splits = 1;
 };

@@ -19,6 +19,7 @@
 // Q and the probabilities are rounded to f16 for the matrix cores; sums are f32.
 
 #include "attn.hpp"
+#include "q16.hpp"
 
 namespace mesh {
 
@@ -242,7 +243,9 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(const float *p_q,
         }
         const size_t row = (size_t)t * p_n_head + (size_t)kvh * G + h;
         if (single) {
-            if (a.out16_k8) {
+            if (a.out_q16) {
+                q16_store_block32(a.out_q16, p_n_head * HD, t, (kvh * G + h) * HD + dd, sum / ll);
+            } else if (a.out16_k8) {
                 const size_t kk = ((size_t)kvh * G + h) * HD + dd, KK = (size_t)p_n_head * HD;
                 a.out16_k8[(size_t)(t / 16) * 16 * KK + ((kk >> 3) * 16 + (t % 16)) * 8 + (kk & 7)] = (_Float16)(sum / ll);
             } else {

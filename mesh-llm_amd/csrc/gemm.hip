@@ -34,13 +34,22 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
-// four bytes (values < 64) -> four f16 holding (value - off) * s + mn, as two packed dwords.  0x6400 | q is the f16
-// 1024 + q exactly; the offset comes off exactly, then one packed fma applies the block scale and minimum.
-__device__ __forceinline__ void dequant4(uint32_t q, half2v off, half2v s, half2v mn, uint32_t &lo, uint32_t &hi) {
-    const half2v a = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04010400u)) - off;
-    const half2v b = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04030402u)) - off;
-    lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(a, s, mn));
-    hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(b, s, mn));
+// four bytes (values < 64) -> four f16 holding ((value - off) * sc) * d + c, as two packed dwords.  0x6400 | q is the f16
+// 1024 + q exactly and the offset comes off exactly; sc is the block's integer scale, so (q - off) * sc is an exact
+// small integer (|.| <= 504 for q4_K with off = 1024 + 8; q6_K's reaches 4064, where integers above 2048 round to even);
+// d is the super-block's f16 scale as stored in the file.  One packed fma then makes the weight with a single
+// rounding: products of ROUNDED per-block scales (f16(d * sc), f16(dmin * m)) carry their rounding error into every
+// weight of the block, three times the error of this form on q4_K.
+__device__ __forceinline__ void dequant4(uint32_t q, half2v off, half2v sc, half2v d, half2v c, uint32_t &lo, uint32_t &hi) {
+    const half2v a = (__builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04010400u)) - off) * sc;
+    const half2v b = (__builtin_bit_cast(half2v, __builtin_amdgcn_perm(0x64646464u, q, 0x04030402u)) - off) * sc;
+    lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(a, d, c));
+    hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(b, d, c));
+}
+// q4_K: w = d sc (q - 8) + c with c = 8 d sc - dmin m (f32, rounded to f16 once).  {sc, c} of a sub-block:
+__device__ __forceinline__ half2v q4k_sc_c(float d, float dmin, uint32_t scb, uint32_t mnb) {
+    const float sc = (float)scb;
+    return half2v{(_Float16)sc, (_Float16)(8.0f * d * sc - dmin * (float)mnb)};
 }
 __device__ __forceinline__ half2v h2_splat(float v) {
     const _Float16 h = (_Float16)v;
@@ -63,15 +72,16 @@ template <> struct RawSub<MESH_Q4_K> {
         const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
         const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
         const int sh = (c & 1) * 16 + h * 8;
-        const half2v s = h2_splat(d * (float)((scw >> sh) & 0xFFu)), mn = h2_splat(-dmin * (float)((mnw >> sh) & 0xFFu));
-        const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
+        const half2v sc_c = q4k_sc_c(d, dmin, (scw >> sh) & 0xFFu, (mnw >> sh) & 0xFFu);
+        const half2v sc = {sc_c[0], sc_c[0]}, cc = {sc_c[1], sc_c[1]}, dd = h2_splat(d);
+        const half2v off = {(_Float16)1032.f, (_Float16)1032.f};
         const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
         uint4 *d4 = reinterpret_cast<uint4 *>(dst);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint4 o;
-            dequant4((w[2 * i] >> (4 * h)) & 0x0F0F0F0Fu, off, s, mn, o.x, o.y);
-            dequant4((w[2 * i + 1] >> (4 * h)) & 0x0F0F0F0Fu, off, s, mn, o.z, o.w);
+            dequant4((w[2 * i] >> (4 * h)) & 0x0F0F0F0Fu, off, sc, dd, cc, o.x, o.y);
+            dequant4((w[2 * i + 1] >> (4 * h)) & 0x0F0F0F0Fu, off, sc, dd, cc, o.z, o.w);
             d4[i] = o;
         }
     }
@@ -81,13 +91,13 @@ template <> struct RawSub<MESH_Q4_K> {
         const uint32_t scw = c < 2 ? (hdr.y & 0x3F3F3F3Fu) : ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u));
         const uint32_t mnw = c < 2 ? (hdr.z & 0x3F3F3F3Fu) : (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u));
         const int sh = (c & 1) * 16 + h * 8;
-        const half2v sm = {(_Float16)(d * (float)((scw >> sh) & 0xFFu)), (_Float16)(-dmin * (float)((mnw >> sh) & 0xFFu))};
+        const half2v sc_c = q4k_sc_c(d, dmin, (scw >> sh) & 0xFFu, (mnw >> sh) & 0xFFu);
         const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
         uint32_t n[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) n[j] = ((w[2 * j] >> (4 * h)) & 0x0F0F0F0Fu) | (((w[2 * j + 1] >> (4 * h)) & 0x0F0F0F0Fu) << 4);
         *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(n[0], n[1], n[2], n[3]);
-        *reinterpret_cast<uint32_t *>(chunk + 4096 + s * 4) = __builtin_bit_cast(uint32_t, sm);
+        *reinterpret_cast<uint2 *>(chunk + 4096 + s * 8) = make_uint2(__builtin_bit_cast(uint32_t, sc_c), hdr.x & 0xFFFFu);
     }
 };
 
@@ -106,8 +116,8 @@ template <> struct RawSub<MESH_Q6_K> {
     }
     __device__ __forceinline__ void store(int c, int h, _Float16 *dst) const {
         const int t4 = 2 * (c & 1) + h;
-        const float df = f16_bits_to_f32((uint16_t)d);
-        const half2v s0 = h2_splat(df * (float)(int8_t)(sc & 0xFFu)), s1 = h2_splat(df * (float)(int8_t)(sc >> 8));
+        const half2v dd = h2_splat(f16_bits_to_f32((uint16_t)d));
+        const half2v s0 = h2_splat((float)(int8_t)(sc & 0xFFu)), s1 = h2_splat((float)(int8_t)(sc >> 8));
         const half2v off = {(_Float16)1056.f, (_Float16)1056.f}, zero = {(_Float16)0.f, (_Float16)0.f};
         const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
         const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
@@ -123,15 +133,14 @@ template <> struct RawSub<MESH_Q6_K> {
             }
             const half2v s = i < 2 ? s0 : s1;       // one scale per 16 elements
             uint4 o;
-            dequant4(q[0], off, s, zero, o.x, o.y);
-            dequant4(q[1], off, s, zero, o.z, o.w);
+            dequant4(q[0], off, s, dd, zero, o.x, o.y);
+            dequant4(q[1], off, s, dd, zero, o.z, o.w);
             d4[i] = o;
         }
     }
     __device__ __forceinline__ void pack(int c, int h, uint8_t *chunk, int s) const {
         const int t4 = 2 * (c & 1) + h;
-        const float df = f16_bits_to_f32((uint16_t)d);
-        const half2v s01 = {(_Float16)(df * (float)(int8_t)(sc & 0xFFu)), (_Float16)(df * (float)(int8_t)(sc >> 8))};
+        const half2v s01 = {(_Float16)(float)(int8_t)(sc & 0xFFu), (_Float16)(float)(int8_t)(sc >> 8)};
         const uint32_t lw[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
         const uint32_t hw[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
         uint32_t q[8];
@@ -148,48 +157,50 @@ template <> struct RawSub<MESH_Q6_K> {
         }
         *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(n[0], n[1], n[2], n[3]);
         *reinterpret_cast<uint2 *>(chunk + 4096 + s * 8) = make_uint2(hb2[0], hb2[1]);
-        *reinterpret_cast<uint32_t *>(chunk + 6144 + s * 4) = __builtin_bit_cast(uint32_t, s01);
+        *reinterpret_cast<uint2 *>(chunk + 6144 + s * 8) = make_uint2(__builtin_bit_cast(uint32_t, s01), d & 0xFFFFu);
     }
 };
 
 // The same (row, sub-block) out of the GEMM layout: two or three loads at the thread's own slot of the chunk.
 template <int TYPE> struct PackedSub;
 template <> struct PackedSub<MESH_Q4_K> {
-    static constexpr int CHUNK = 5120;
+    static constexpr int CHUNK = 6144;
     uint4 q;
-    uint32_t sm;
+    uint2 sm;          // {f16 sc, f16 c}, {f16 d, -}
     __device__ __forceinline__ void load(const uint8_t *__restrict__ chunk, int s) {
         q = *reinterpret_cast<const uint4 *>(chunk + s * 16);
-        sm = *reinterpret_cast<const uint32_t *>(chunk + 4096 + s * 4);
+        sm = *reinterpret_cast<const uint2 *>(chunk + 4096 + s * 8);
     }
     __device__ __forceinline__ void store(_Float16 *dst) const {
-        const half2v s = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm, sm, 0x01000100u));
-        const half2v mn = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm, sm, 0x03020302u));
-        const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
+        const half2v sc = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm.x, sm.x, 0x01000100u));
+        const half2v cc = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm.x, sm.x, 0x03020302u));
+        const half2v dd = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sm.y, sm.y, 0x01000100u));
+        const half2v off = {(_Float16)1032.f, (_Float16)1032.f};
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
         uint4 *d4 = reinterpret_cast<uint4 *>(dst);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint4 o;
-            dequant4(w[j] & 0x0F0F0F0Fu, off, s, mn, o.x, o.y);
-            dequant4((w[j] >> 4) & 0x0F0F0F0Fu, off, s, mn, o.z, o.w);
+            dequant4(w[j] & 0x0F0F0F0Fu, off, sc, dd, cc, o.x, o.y);
+            dequant4((w[j] >> 4) & 0x0F0F0F0Fu, off, sc, dd, cc, o.z, o.w);
             d4[j] = o;
         }
     }
 };
 template <> struct PackedSub<MESH_Q6_K> {
-    static constexpr int CHUNK = 7168;
+    static constexpr int CHUNK = 8192;
     uint4 q;
     uint2 hb;
-    uint32_t sc;
+    uint2 sc;          // {f16 sc of elements 0..15, f16 sc of elements 16..31}, {f16 d, -}
     __device__ __forceinline__ void load(const uint8_t *__restrict__ chunk, int s) {
         q = *reinterpret_cast<const uint4 *>(chunk + s * 16);
         hb = *reinterpret_cast<const uint2 *>(chunk + 4096 + s * 8);
-        sc = *reinterpret_cast<const uint32_t *>(chunk + 6144 + s * 4);
+        sc = *reinterpret_cast<const uint2 *>(chunk + 6144 + s * 8);
     }
     __device__ __forceinline__ void store(_Float16 *dst) const {
-        const half2v s0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc, sc, 0x01000100u));
-        const half2v s1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc, sc, 0x03020302u));
+        const half2v s0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc.x, sc.x, 0x01000100u));
+        const half2v s1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc.x, sc.x, 0x03020302u));
+        const half2v dd = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(sc.y, sc.y, 0x01000100u));
         const half2v off = {(_Float16)1056.f, (_Float16)1056.f}, zero = {(_Float16)0.f, (_Float16)0.f};
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
         uint4 *d4 = reinterpret_cast<uint4 *>(dst);
@@ -198,8 +209,8 @@ template <> struct PackedSub<MESH_Q6_K> {
             const uint32_t hs = (j < 2 ? hb.x : hb.y) >> (4 * (j & 1));
             const half2v s = j < 2 ? s0 : s1;
             uint4 o;
-            dequant4((w[j] & 0x0F0F0F0Fu) | ((hs & 0x03030303u) << 4), off, s, zero, o.x, o.y);
-            dequant4(((w[j] >> 4) & 0x0F0F0F0Fu) | (((hs >> 2) & 0x03030303u) << 4), off, s, zero, o.z, o.w);
+            dequant4((w[j] & 0x0F0F0F0Fu) | ((hs & 0x03030303u) << 4), off, s, dd, zero, o.x, o.y);
+            dequant4(((w[j] >> 4) & 0x0F0F0F0Fu) | (((hs >> 2) & 0x03030303u) << 4), off, s, dd, zero, o.z, o.w);
             d4[j] = o;
         }
     }
@@ -678,7 +689,7 @@ __global__ __launch_bounds__(256) void gemm_pack_kernel(const uint8_t *__restric
     if (wrow >= M_pad) {
         *reinterpret_cast<uint4 *>(chunk + s * 16) = make_uint4(0, 0, 0, 0);
         if (TYPE == MESH_Q6_K) *reinterpret_cast<uint2 *>(chunk + 4096 + s * 8) = make_uint2(0, 0);
-        *reinterpret_cast<uint32_t *>(chunk + (TYPE == MESH_Q6_K ? 6144 : 4096) + s * 4) = 0u;
+        *reinterpret_cast<uint2 *>(chunk + (TYPE == MESH_Q6_K ? 6144 : 4096) + s * 8) = make_uint2(0u, 0u);
         return;
     }
     RawSub<TYPE> r;

@@ -50,37 +50,44 @@ int gemm_split_count(const GemmArgs &a);
 // One chunk per (128-row block, 64-element k-step), chunks of a row block consecutive in k.  A chunk holds, for each of
 // the 256 (row, 32-element sub-block) pairs s = 2 * row + half, what the staging thread s needs, at s * stride of
 // each section, so that every load of a staging wave covers one contiguous kilobyte:
-//   q4_K (5120 B): [256 x 16 B quants: dword j = elements 8j..8j+3 in the low nibbles, 8j+4..8j+7 in the high ones]
-//                  [256 x (f16 d*scale, f16 -dmin*min)]
-//   q6_K (7168 B): [256 x 16 B low nibbles, same order][256 x 8 B upper two bits: byte b of dword j/2 holds, from
+//   q4_K (6144 B): [256 x 16 B quants: dword j = elements 8j..8j+3 in the low nibbles, 8j+4..8j+7 in the high ones]
+//                  [256 x 8 B: f16 sc (the integer block scale), f16 c = 8 d sc - dmin m, f16 d, unused]
+//   q6_K (8192 B): [256 x 16 B low nibbles, same order][256 x 8 B upper two bits: byte b of dword j/2 holds, from
 //                  bit 4*(j%2), the bits of element 8j+b and, two bits up, of element 8j+4+b]
-//                  [256 x (f16 d*scale of elements 0..15, f16 d*scale of elements 16..31)]
-// The f16 products are the ones the kernel would otherwise compute from the block headers, so both layouts give the
-// same bits.  Rows beyond M are zero.
+//                  [256 x 8 B: f16 sc of elements 0..15, f16 sc of elements 16..31, f16 d, unused]
+// The kernel forms a weight as ((q - offset) * sc) * d + c: an exact small integer times the super-block's own f16
+// scale, rounded once.  The fields are the ones the kernel would otherwise derive from the block headers, so both
+// layouts give the same bits.  Rows beyond M are zero.
 size_t gemm_packed_bytes(int type, int64_t M, int64_t K);
 int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, hipStream_t stream);
 // gate / up pair for the SwiGLU launch: row block b = gate rows [64b, 64b + 64) followed by up rows [64b, 64b + 64)
 size_t gemm_packed_pair_bytes(int type, int64_t M, int64_t K);
 int gemm_pack_pair(int type, const void *gate_tiled, const void *up_tiled, void *packed, int64_t M, int64_t K, hipStream_t stream);
 
-// Skinny GEMM for a batch of decode steps (gemm_skinny.hip): up to three tiled K-quant matrices sharing the f16
-// activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel.  Activations are in the
-// "k8-major" layout: blocks of 16 tokens, element (t, k) of block t / 16 at ((k / 8) * 16 + t % 16) * 8 + k % 8 within
-// the block of 16 * K halfs; columns beyond T hold zeros.  rmsnorm_f16_k8 / pack_f16_k8 produce it.
+// Skinny GEMM for a batch of decode steps (gemm_skinny.hip): up to three tiled K-quant matrices sharing the
+// activations, any T (processed 16 columns at a time), epilogues as in the mat-vec kernel, integer dot products on
+// the matrix cores.  Activations come in the "q16" layout quant16_k8 produces: per block of 16 tokens
+// q16_block_bytes(K) bytes holding 16-bit fixed-point values per 32-element block as two int8 planes, the f32 block
+// scales and the f32 block sums (gemm_skinny.hip describes the arrangement); columns beyond T hold zeros.
 struct SkinnyArgs {
     GemvMat mat[3];
-    int n_mat = 1;                   // for EPI_SWIGLU exactly 2 (gate, up), written through mat[0].y and/or y16
-    const _Float16 *x = nullptr;     // k8-major, ceil(T / 16) blocks of 16 * K halfs, 16-byte aligned
+    int n_mat = 1;                   // for EPI_SWIGLU exactly 2 (gate, up), written through mat[0].y
+    const uint8_t *xq = nullptr;     // q16 layout, ceil(T / 16) blocks of q16_block_bytes(K), 16-byte aligned
     int K = 0, T = 0;
     int epi = EPI_STORE;
     const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y
     int ldres = 0;
-    _Float16 *y16 = nullptr;         // optional f16 copy of matrix 0's output in the k8-major layout (feeds the next GEMM)
     // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
 };
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
+// Bytes of one 16-token block of the q16 layout for rows of K elements.
+size_t q16_block_bytes(int K);
+// y (q16 layout) = quantise(rms_norm(x) * w) for T rows of n floats (w == null: quantise(x)); n a multiple of 32
+int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t *y, hipStream_t stream);
+// The "k8-major" f16 layout the large-tile GEMM reads: blocks of 16 tokens, element (t, k) of block t / 16 at
+// ((k / 8) * 16 + t % 16) * 8 + k % 8 within the block of 16 * K halfs; columns beyond T hold zeros.
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream);
 int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream);

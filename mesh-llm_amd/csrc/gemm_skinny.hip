@@ -1,32 +1,36 @@
-// Skinny GEMM for batched decode: Y[T][M] = W[M][K] . X[T][K] with 5 <= T <= a few dozen tokens, W a tiled
-// q4_K / q6_K matrix, X in f16.
+// Skinny GEMM for batched decode: Y[T][M] = W[M][K] . X[T][K] with 4 <= T <= a few dozen tokens, W a tiled
+// q4_K / q6_K matrix, on the integer matrix cores.
 //
 // Between the mat-vec kernel (gemv.hip: one dot4 chain per activation column, so the weights' integer work is
 // repeated per token) and the prefill GEMM (gemm.hip: 128x128 output tiles, far too few workgroups when T is
-// small) sits the batch of decode steps.  Here the weight stream is organised exactly as in the mat-vec kernel --
-// a workgroup owns a few tile-rows (16 rows each), its waves split K and each keeps four weight tiles in flight --
-// but a tile is dequantised in registers to f16 and multiplied with 16 activation columns at once on the matrix
-// cores (v_mfma_f32_16x16x32_f16), so the per-token cost is a fraction of an MFMA instead of a dot4 chain.
+// small) sits the batch of decode steps.  The weight stream is organised exactly as in the mat-vec kernel -- a
+// workgroup owns a few tile-rows (16 rows each), its waves split K and each keeps several weight tiles in flight --
+// and so is the arithmetic: activations are 16-bit fixed point per 32-element block (x ~ d_b * (256 hi + lo), hi and lo
+// int8), the raw 4- / 6-bit quants are the other integer operand, and the block scales meet the integer sums in f32.
+// Only the dot products move from v_dot4 to v_mfma_i32_16x16x32_i8, 16 token columns at a time:
 //
-// Register dequantisation: lane (m = l % 16, g = l / 16) loads what lane 4m + g of the mat-vec kernel loads, i.e.
-// quarter g of row m of the super-block (gemv.hpp).  An MFMA's k-slots of lane group g are then 8 consecutive
-// elements of that quarter; the B operand (activations) is read with the same element indices, so the k-order of
-// the instruction never has to match the order in memory.  Nibbles become f16 through the exponent trick
-// (0x6400 | q is 1024 + q exactly), the offset is removed exactly, and the sub-block scale and minimum are applied
-// with one packed fma, all in f16 (sums are f32, in the MFMA accumulator).
+//   * A operand = activations (rows = 16 tokens), B operand = weights (columns = the 16 rows of a tile), so lane
+//     (m = l % 16, g = l / 16) supplies 8 k-slots of token m and of weight row m, and receives the sums of tokens
+//     4g..4g+3 for ITS OWN weight row m: the sub-block scales a lane applies are those of the row whose header it
+//     holds, and only the activation scales fan out (one 16-byte load of four tokens' block scales per sub-block).
+//   * q4_K: one MFMA pair (hi plane, lo plane) per 32-element sub-block; sum = (I_hi << 8) + I_lo, scaled by
+//     d * sc_s * dx_s[token].  The "- dmin * m_s * sum(x)" term of all 8 sub-blocks is itself a small matrix product
+//     over s and runs on v_mfma_f32_16x16x4_f32 (two per super-block), straight into the f32 accumulator.
+//   * q6_K: scales cover 16 elements, i.e. two lane groups of a 32-element block each, so a block takes two MFMAs per
+//     plane, each with the other scale group's weights zeroed; the -32 offset is folded into the quants (int8 q - 32).
 //
-// Activation layout ("k8-major"): X is not read as [T][K] rows.  Tokens are grouped in blocks of 16 columns, and
-// within a block the 8 consecutive k of every column sit together: element (t, k) of block b = t / 16 is at
-// ((b * K/8 + k/8) * 16 + t % 16) * 8 + k % 8.  The 16 lanes that supply the 16 columns of one MFMA B fragment then
-// read 256 contiguous bytes, where row-major activations would cost one cache line per lane.  The producers
-// (rmsnorm_f16_k8, pack_f16_k8, this kernel's own f16 output) write that layout, zero-filling the unused columns.
-// Weight tiles are loaded with the mat-vec kernel's dense lane mapping and moved to the MFMA lanes with
-// ds_bpermute (register crossbar), again so that a wave's load touches whole cache lines.
+// A tile arrives with the mat-vec kernel's dense lane mapping (whole cache lines per wave instruction) and passes
+// through a wave-private LDS slot to reach the MFMA lanes.
 //
-// Same math as ggml's mul_mat for K-quant weights (ggml_vec_dot_q4_K_q8_K / q6_K in
-// third_party/llama.cpp ggml-cpu/quants.c, reached from rpc_server::graph_compute,
-// patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451) except that activations are rounded to f16
-// instead of q8_K.
+// Activation layout ("q16", produced by quant16_k8 below and by the decode attention kernels, q16.hpp) of a block of 16 tokens:
+//   planes  [K/8][16 tokens][16 B]: {hi[0..7], lo[0..7]} of elements 8q..8q+7 of the token
+//   dx      [K/32][16 tokens] f32: block scale;  sx [K/32][16 tokens] f32: block sum of x (= dx * sum of quants)
+// The 16 lanes of a lane group read 256 contiguous bytes of planes; columns beyond T hold whatever they held (an MFMA
+// row never mixes tokens, and those rows are not stored).
+//
+// Same math as ggml's mul_mat for K-quant weights (ggml_vec_dot_q4_K_q8_K / q6_K in third_party/llama.cpp
+// ggml-cpu/quants.c, reached from rpc_server::graph_compute, patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451)
+// -- an integer dot per sub-block, scales applied in f32 -- with 16-bit instead of 8-bit activations.
 
 #include "gemm.hpp"
 #include "gemv_device.hpp"
@@ -36,30 +40,13 @@ namespace mesh {
 constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
 constexpr int SK_DEPTH_Q4 = 4;            // weight tiles a wave keeps in flight (2304 B each)
-constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B and their fragments need more registers
-constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA N)
-constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
+constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B
+constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA M)
+constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
 
-// Phase timestamps for tuning builds (-DMESH_GEMV_TRACE); compiled out of the product.
-#ifdef MESH_GEMV_TRACE
-__device__ long long *g_skinny_trace = nullptr;
-extern "C" int mesh_debug_set_skinny_trace(long long *p) {
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_skinny_trace), &p, sizeof p) == hipSuccess ? 0 : -2;
-}
-#define SK_MARK(k)                                                                                 \
-    do {                                                                                           \
-        if (g_skinny_trace && (threadIdx.x & 63) == 0)                                             \
-            g_skinny_trace[((size_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (k)] = wall_clock64(); \
-    } while (0)
-#else
-#define SK_MARK(k) do { } while (0)
-#endif
-
-typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef int i4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 
 struct SkinnyKernelArgs {
     const uint8_t *wbase[3];      // matrix base minus its first tile-row, so a global tile-row index addresses it
@@ -68,166 +55,194 @@ struct SkinnyKernelArgs {
     const float *bias[3];
     int M[3];
     int ldy[3];
-    const _Float16 *x;            // k8-major block of 16 columns
     int K, T;
     const float *residual;
     int ldres;
     int epi;
-    _Float16 *y16;                // optional f16 copy of the output (matrix 0): k8-major block with M16 rows as its k
-    int M16;
     int ks;                       // waves along K
     GemvRope rope;                // rope.pos / rope.seq point at the launch's first column
     int kind[3];
 };
 
-// four bytes (values < 64) -> four f16 holding 1024 + value
-__device__ __forceinline__ void bytes_to_h1024(uint32_t v, h2_t &lo, h2_t &hi) {
-    lo = __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u));
-    hi = __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u));
-}
+__device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) { return (long)(((unsigned long long)hi << 32) | lo); }
 
-// Eight weights as an MFMA A fragment: bytes of v0, v1 hold the quants; w = (q - off) * s - mn.
-__device__ __forceinline__ h8_t dequant8(uint32_t v0, uint32_t v1, h2_t off, h2_t s, h2_t mn) {
-    h2_t p[4];
-    bytes_to_h1024(v0, p[0], p[1]);
-    bytes_to_h1024(v1, p[2], p[3]);
-    u4_t a;                                                          // built as four dwords: no half-register moves
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const h2_t q = p[i] - off;                                   // exact
-        a[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, s, mn));
+// A operands (activation planes) of one super-block for this lane, the same for both weight types: 32-element block s,
+// elements 32s + 8g .. + 7 of token m as {hi8 (x, y), lo8 (z, w)}.  The block scales take a detour through a wave-private
+// LDS table ([8 blocks][16 tokens] f32, two of them): a lane needs those of four tokens for every block -- 32 registers
+// per super-block if kept in registers -- but the table is only 128 floats, one 8-byte load per lane.
+struct XFrags {
+    uint4 p[8];
+    float2 dxpre;      // this lane's two entries of the super-block's scale table
+    float sxa, sxb;    // q4_K: block sums of token m, blocks g and g + 4 (operands of the minimum-term MFMAs)
+    __device__ __forceinline__ const uint4 *planes(const uint8_t *xq, int sb, int lane) const {
+        return reinterpret_cast<const uint4 *>(xq) + ((size_t)sb * 32 + (lane >> 4)) * 16 + (lane & 15);
     }
-    return __builtin_bit_cast(h8_t, a);
-}
-
-__device__ __forceinline__ h2_t h2_of(float v) {
-    const _Float16 h = (_Float16)v;
-    return h2_t{h, h};
-}
-
-// A fragments of one tile, MFMA by MFMA.  frag(t, ...) returns the fragment of MFMA t (0..7) and the element
-// offset within the super-block of this lane's 8 k-slots.
-template <int TYPE> struct TileFrags;
-
-template <> struct TileFrags<MESH_Q4_K> {
-    uint32_t w[8];
-    h2_t s_lo, s_hi, mn_lo, mn_hi;
-    int kbase;
-    __device__ __forceinline__ void prepare(const TileRegs<MESH_Q4_K> &R, int g) {
-        const float d = f16_bits_to_f32((uint16_t)(R.hdr.x & 0xFFFFu));
-        const float dmin = f16_bits_to_f32((uint16_t)(R.hdr.x >> 16));
-        // 6-bit (scale, min) of sub-blocks 2g and 2g+1 (get_scale_min_k4 of ggml-quants.c)
-        const uint32_t scw = g < 2 ? (R.hdr.y & 0x3F3F3F3Fu) : ((R.hdr.w & 0x0F0F0F0Fu) | ((R.hdr.y >> 2) & 0x30303030u));
-        const uint32_t mnw = g < 2 ? (R.hdr.z & 0x3F3F3F3Fu) : (((R.hdr.w >> 4) & 0x0F0F0F0Fu) | ((R.hdr.z >> 2) & 0x30303030u));
-        const int sh = (g & 1) * 16;
-        s_lo = h2_of(d * (float)((scw >> sh) & 0xFFu));
-        s_hi = h2_of(d * (float)((scw >> (sh + 8)) & 0xFFu));
-        mn_lo = h2_of(-dmin * (float)((mnw >> sh) & 0xFFu));
-        mn_hi = h2_of(-dmin * (float)((mnw >> (sh + 8)) & 0xFFu));
-        w[0] = R.qa.x; w[1] = R.qa.y; w[2] = R.qa.z; w[3] = R.qa.w;
-        w[4] = R.qb.x; w[5] = R.qb.y; w[6] = R.qb.z; w[7] = R.qb.w;
-        kbase = 64 * g;
-    }
-    // MFMA t: t < 4 low nibbles (sub-block 2g), bytes 8t..8t+7; t >= 4 high nibbles (sub-block 2g+1)
-    __device__ __forceinline__ h8_t frag(int t) const {
-        const int tt = t & 3;
-        const bool high = t >= 4;
-        const uint32_t v0 = (high ? w[2 * tt] >> 4 : w[2 * tt]) & 0x0F0F0F0Fu;
-        const uint32_t v1 = (high ? w[2 * tt + 1] >> 4 : w[2 * tt + 1]) & 0x0F0F0F0Fu;
-        const h2_t off = {(_Float16)1024.f, (_Float16)1024.f};
-        return dequant8(v0, v1, off, high ? s_hi : s_lo, high ? mn_hi : mn_lo);
-    }
-    __device__ __forceinline__ int koff(int t) const { return kbase + 32 * (t >> 2) + 8 * (t & 3); }
-};
-
-template <> struct TileFrags<MESH_Q6_K> {
-    uint32_t v[4][4];      // [t4][dword]: six-bit quants in bytes, elements 128n + 32 t4 + 16u + 4 dword + byte
-    h2_t s[4];
-    int kbase;
-    __device__ __forceinline__ void prepare(const TileRegs<MESH_Q6_K> &R, int g) {
-        const int n = g >> 1, u = g & 1;
-        const float d = f16_bits_to_f32((uint16_t)R.d);
-        const uint32_t la[4] = {R.qla.x, R.qla.y, R.qla.z, R.qla.w}, lb[4] = {R.qlb.x, R.qlb.y, R.qlb.z, R.qlb.w};
-        const uint32_t qh[4] = {R.qh.x, R.qh.y, R.qh.z, R.qh.w};
-        const uint32_t scw0 = n ? R.sc.z : R.sc.x, scw1 = n ? R.sc.w : R.sc.y;
-        s[0] = h2_of(d * (float)(int8_t)((scw0 >> (8 * u)) & 0xFFu));
-        s[1] = h2_of(d * (float)(int8_t)((scw0 >> (16 + 8 * u)) & 0xFFu));
-        s[2] = h2_of(d * (float)(int8_t)((scw1 >> (8 * u)) & 0xFFu));
-        s[3] = h2_of(d * (float)(int8_t)((scw1 >> (16 + 8 * u)) & 0xFFu));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v[0][j] = (la[j] & 0x0F0F0F0Fu) | ((qh[j] << 4) & 0x30303030u);
-            v[1][j] = (lb[j] & 0x0F0F0F0Fu) | ((qh[j] << 2) & 0x30303030u);
-            v[2][j] = ((la[j] >> 4) & 0x0F0F0F0Fu) | (qh[j] & 0x30303030u);
-            v[3][j] = ((lb[j] >> 4) & 0x0F0F0F0Fu) | ((qh[j] >> 2) & 0x30303030u);
-        }
-        kbase = 128 * n + 16 * u;
-    }
-    // MFMA t = 2 t4 + h: elements 8h..8h+7 of the 16-element scale group t4
-    __device__ __forceinline__ h8_t frag(int t) const {
-        const int t4 = t >> 1, h = t & 1;
-        const h2_t off = {(_Float16)1056.f, (_Float16)1056.f};       // 1024 + 32: quants are stored with a bias of 32
-        const h2_t zero = {(_Float16)0.f, (_Float16)0.f};
-        return dequant8(v[t4][2 * h], v[t4][2 * h + 1], off, s[t4], zero);
-    }
-    __device__ __forceinline__ int koff(int t) const { return kbase + 32 * (t >> 1) + 8 * (t & 1); }
-};
-
-// B fragments of one super-block for this lane: 8 MFMAs x 8 f16
-template <int TYPE>
-struct BFrags {
-    uint4 b[8];
-    // x: the k8-major block (uniform), lane_off: this lane's column and quarter offset in halfs
-    __device__ __forceinline__ void load(const _Float16 *x, int lane_off, int sb) {
-        const _Float16 *base = x + (size_t)sb * (QK_K * 16);      // uniform
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            int koff;                                      // compile-time part of the element offset
-            if (TYPE == MESH_Q4_K) koff = 32 * (t >> 2) + 8 * (t & 3);
-            else koff = 32 * (t >> 1) + 8 * (t & 1);
-            b[t] = ldg<uint4>(base + lane_off + koff * 16);
+    template <bool SUMS>
+    __device__ __forceinline__ void load_scales(const uint8_t *xq, int K, int sb, int lane) {
+        dxpre = ldg<float2>(reinterpret_cast<const float *>(xq + (size_t)K * 32) + (size_t)sb * 128 + 2 * lane);
+        if (SUMS) {
+            const float *sxp = reinterpret_cast<const float *>(xq + (size_t)K * 34) + (size_t)sb * 128 + (lane & 15);
+            sxa = ldg<float>(sxp + (lane >> 4) * 16);
+            sxb = ldg<float>(sxp + ((lane >> 4) + 4) * 16);
         }
     }
+    template <bool SUMS>
+    __device__ __forceinline__ void load(const uint8_t *xq, int K, int sb, int lane) {
+        const uint4 *pl = planes(xq, sb, lane);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) p[s] = ldg<uint4>(pl + s * 64);
+        load_scales<SUMS>(xq, K, sb, lane);
+    }
 };
 
-// Moves a tile loaded with the dense mapping (lane 4r + c holds row r, quarter c) to the MFMA mapping
-// (lane m + 16 g holds row m, quarter g).
-__device__ __forceinline__ uint32_t lane_gather(uint32_t v, int src_lane4) {
-    return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane4, (int)v);
+// The LDS unit executes a wave's accesses in order; the fences only keep the compiler from reordering them.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
-__device__ __forceinline__ uint4 lane_gather(const uint4 &v, int src_lane4) {
-    return make_uint4(lane_gather(v.x, src_lane4), lane_gather(v.y, src_lane4), lane_gather(v.z, src_lane4), lane_gather(v.w, src_lane4));
+
+// One tile: dense-mapped registers -> wave-private LDS slot (same arrangement as in memory) -> the view of lane (m, g):
+// row m's header and the quants of elements 32s + 8g .. + 7, s = 0..7, of that row.
+template <int TYPE> struct TileView;
+
+constexpr int Q4_ROW = 144;                       // LDS stride of a row's 128 quant bytes
+constexpr int Q6_ROW_L = 144, Q6_ROW_H = 80;      // of a row's 128 low-nibble bytes and 64 upper-bit bytes
+constexpr int Q6_LDS_QH = 16 * Q6_ROW_L, Q6_LDS_SC = Q6_LDS_QH + 16 * Q6_ROW_H, Q6_LDS_D = Q6_LDS_SC + 256;
+constexpr int LDS_TILE_Q4 = 256 + 16 * Q4_ROW, LDS_TILE_Q6 = Q6_LDS_D + 32;
+
+template <> struct TileView<MESH_Q4_K> {
+    uint4 hdr;
+    uint2 v[4];        // chunk c: bytes 8g .. 8g + 7 of qs[32c ..]: low nibbles block 2c, high nibbles block 2c + 1
+    __device__ __forceinline__ void stage(const TileRegs<MESH_Q4_K> &R, uint8_t *slot, int lane) {
+        const int m = lane & 15, g = lane >> 4;
+        wave_lds_sync();                                          // the previous tile's reads are issued before these writes
+        // (rows of quants are Q4_ROW bytes apart in LDS, not 128: the 16 rows a read instruction touches then fall into
+        // different banks instead of two)
+        if ((lane & 3) == 0) *reinterpret_cast<uint4 *>(slot + (lane >> 2) * 16) = R.hdr;
+        *reinterpret_cast<uint4 *>(slot + 256 + (lane >> 2) * Q4_ROW + (lane & 3) * 32) = R.qa;
+        *reinterpret_cast<uint4 *>(slot + 256 + (lane >> 2) * Q4_ROW + (lane & 3) * 32 + 16) = R.qb;
+        wave_lds_sync();
+        hdr = *reinterpret_cast<const uint4 *>(slot + m * 16);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = *reinterpret_cast<const uint2 *>(slot + 256 + m * Q4_ROW + 32 * c + 8 * g);
+    }
+};
+
+template <> struct TileView<MESH_Q6_K> {
+    uint2 la[2], lb[2], qh[2];     // half n: ql[64n + 8g ..], ql[64n + 32 + 8g ..], qh[32n + 8g ..], 8 bytes each
+    uint4 sc;
+    uint32_t d;
+    __device__ __forceinline__ void stage(const TileRegs<MESH_Q6_K> &R, uint8_t *slot, int lane) {
+        const int m = lane & 15, g = lane >> 4;
+        const int r = lane >> 2, c = lane & 3, n = c >> 1, u = c & 1;
+        wave_lds_sync();
+        *reinterpret_cast<uint4 *>(slot + r * Q6_ROW_L + 64 * n + 16 * u) = R.qla;
+        *reinterpret_cast<uint4 *>(slot + r * Q6_ROW_L + 64 * n + 32 + 16 * u) = R.qlb;
+        *reinterpret_cast<uint4 *>(slot + Q6_LDS_QH + r * Q6_ROW_H + 32 * n + 16 * u) = R.qh;
+        if (c == 0) {
+            *reinterpret_cast<uint4 *>(slot + Q6_LDS_SC + r * 16) = R.sc;
+            *reinterpret_cast<uint16_t *>(slot + Q6_LDS_D + r * 2) = (uint16_t)R.d;
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            la[h] = *reinterpret_cast<const uint2 *>(slot + m * Q6_ROW_L + 64 * h + 8 * g);
+            lb[h] = *reinterpret_cast<const uint2 *>(slot + m * Q6_ROW_L + 64 * h + 32 + 8 * g);
+            qh[h] = *reinterpret_cast<const uint2 *>(slot + Q6_LDS_QH + m * Q6_ROW_H + 32 * h + 8 * g);
+        }
+        sc = *reinterpret_cast<const uint4 *>(slot + Q6_LDS_SC + m * 16);
+        d = *reinterpret_cast<const uint16_t *>(slot + Q6_LDS_D + m * 2);
+    }
+};
+
+// acc[i] += sum over the tile's 256 elements of w[row m][k] * x[token 4g + i][k]
+__device__ __forceinline__ void tile_mac(const TileView<MESH_Q4_K> &V, const XFrags &X, const float *dxt, int lane, f4_t &acc) {
+    const int g = lane >> 4;
+    const float d = f16_bits_to_f32((uint16_t)(V.hdr.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(V.hdr.x >> 16));
+    // 6-bit scales / minima of the 8 sub-blocks as bytes (get_scale_min_k4 of ggml-quants.c)
+    const uint32_t sc_lo = V.hdr.y & 0x3F3F3F3Fu, sc_hi = (V.hdr.w & 0x0F0F0F0Fu) | ((V.hdr.y >> 2) & 0x30303030u);
+    const uint32_t mn_lo = V.hdr.z & 0x3F3F3F3Fu, mn_hi = ((V.hdr.w >> 4) & 0x0F0F0F0Fu) | ((V.hdr.z >> 2) & 0x30303030u);
+    const i4_t zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int c = s >> 1, h = s & 1;
+        const long w = pack64((V.v[c].x >> (4 * h)) & 0x0F0F0F0Fu, (V.v[c].y >> (4 * h)) & 0x0F0F0F0Fu);
+        const i4_t ih = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(X.p[s].x, X.p[s].y), w, zero, 0, 0, 0);
+        const i4_t il = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(X.p[s].z, X.p[s].w), w, zero, 0, 0, 0);
+        const float ds = d * (float)(((s < 4 ? sc_lo : sc_hi) >> (8 * (s & 3))) & 0xFFu);
+        const f4_t dx = *reinterpret_cast<const f4_t *>(dxt + s * 16 + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf((float)((ih[i] << 8) + il[i]) * dx[i], ds, acc[i]);
+    }
+    // - dmin * m_s * sum(x_s), s = 0..7: a [16 tokens x 8] . [8 x 16 rows] product in f32
+    const float nma = -dmin * (float)((mn_lo >> (8 * g)) & 0xFFu), nmb = -dmin * (float)((mn_hi >> (8 * g)) & 0xFFu);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X.sxa, nma, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X.sxb, nmb, acc, 0, 0, 0);
 }
-__device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q4_K> &R, int src_lane4) {
-    R.hdr = lane_gather(R.hdr, src_lane4);
-    R.qa = lane_gather(R.qa, src_lane4);
-    R.qb = lane_gather(R.qb, src_lane4);
+
+__device__ __forceinline__ uint32_t q6_to_i8(uint32_t v) {       // bytes 0..63 -> int8 bytes v - 32
+    return ((v | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
 }
-__device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_lane4) {
-    R.qla = lane_gather(R.qla, src_lane4);
-    R.qlb = lane_gather(R.qlb, src_lane4);
-    R.qh = lane_gather(R.qh, src_lane4);
-    R.sc = lane_gather(R.sc, src_lane4);
-    R.d = lane_gather(R.d, src_lane4);
+
+// q6_K scales cover 16 elements: of a 32-element block, lane groups 0-1 hold the first scale group and 2-3 the second, so
+// the block takes two MFMAs per plane, each with the other group's weights zeroed.
+__device__ __forceinline__ void tile_mac(const TileView<MESH_Q6_K> &V, const XFrags &X, const float *dxt, int lane, f4_t &acc) {
+    const int g = lane >> 4;
+    const float d = f16_bits_to_f32((uint16_t)V.d);
+    const uint32_t scs[4] = {V.sc.x, V.sc.y, V.sc.z, V.sc.w};
+    const uint32_t first = g < 2 ? 0xFFFFFFFFu : 0u;
+    const i4_t zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int n = s >> 2, t4 = s & 3;
+        const uint2 l = (t4 & 1) ? V.lb[n] : V.la[n], q = V.qh[n];
+        uint32_t w0, w1;
+        if (t4 == 0) { w0 = (l.x & 0x0F0F0F0Fu) | ((q.x << 4) & 0x30303030u); w1 = (l.y & 0x0F0F0F0Fu) | ((q.y << 4) & 0x30303030u); }
+        else if (t4 == 1) { w0 = (l.x & 0x0F0F0F0Fu) | ((q.x << 2) & 0x30303030u); w1 = (l.y & 0x0F0F0F0Fu) | ((q.y << 2) & 0x30303030u); }
+        else if (t4 == 2) { w0 = ((l.x >> 4) & 0x0F0F0F0Fu) | (q.x & 0x30303030u); w1 = ((l.y >> 4) & 0x0F0F0F0Fu) | (q.y & 0x30303030u); }
+        else { w0 = ((l.x >> 4) & 0x0F0F0F0Fu) | ((q.x >> 2) & 0x30303030u); w1 = ((l.y >> 4) & 0x0F0F0F0Fu) | ((q.y >> 2) & 0x30303030u); }
+        w0 = q6_to_i8(w0);
+        w1 = q6_to_i8(w1);
+        const uint32_t a0 = w0 & first, a1 = w1 & first;
+        const long wa = pack64(a0, a1), wb = pack64(w0 ^ a0, w1 ^ a1);
+        const long xh = pack64(X.p[s].x, X.p[s].y), xl = pack64(X.p[s].z, X.p[s].w);
+        const i4_t ah = __builtin_amdgcn_mfma_i32_16x16x32_i8(xh, wa, zero, 0, 0, 0);
+        const i4_t al = __builtin_amdgcn_mfma_i32_16x16x32_i8(xl, wa, zero, 0, 0, 0);
+        const i4_t bh = __builtin_amdgcn_mfma_i32_16x16x32_i8(xh, wb, zero, 0, 0, 0);
+        const i4_t bl = __builtin_amdgcn_mfma_i32_16x16x32_i8(xl, wb, zero, 0, 0, 0);
+        const uint32_t scw = scs[s >> 1] >> (16 * (s & 1));             // scale groups 2s and 2s + 1
+        const float dsa = d * (float)(int8_t)(scw & 0xFFu), dsb = d * (float)(int8_t)((scw >> 8) & 0xFFu);
+        const f4_t dx = *reinterpret_cast<const f4_t *>(dxt + s * 16 + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float t = fmaf((float)((bh[i] << 8) + bl[i]), dsb, (float)((ah[i] << 8) + al[i]) * dsa);
+            acc[i] = fmaf(t, dx[i], acc[i]);
+        }
+    }
 }
 
 template <int TYPE, int NU, int SEGS>
-__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
                                                                  int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
                                                                  const SkinnyKernelArgs a) {
-    // (p_begins = first tile-row of matrix 1 | of matrix 2 << 16; p_split = tile-rows per workgroup | workgroups with one
-    // more << 16, computed on the host: no division and no grid-size load stand before the first weight load)
+    // (leading scalar arguments: preloaded into SGPRs, see gemv.hip.  p_begins = first tile-row of matrix 1 | of matrix 2
+    // << 16; p_split = tile-rows per workgroup | workgroups with one more << 16, computed on the host: no division and
+    // no grid-size load stand before the first weight load)
     const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
-    // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
     extern __shared__ __align__(16) uint8_t smem[];
-    float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
     constexpr int TB = TileRegs<TYPE>::BYTES;
+    constexpr int SLOT = ((TYPE == MESH_Q4_K ? LDS_TILE_Q4 : LDS_TILE_Q6) + 255) / 256 * 256;
     constexpr int SK_DEPTH = TYPE == MESH_Q4_K ? SK_DEPTH_Q4 : SK_DEPTH_Q6;
+    constexpr bool SUMS = TYPE == MESH_Q4_K;
+    constexpr int WAVE_LDS = SLOT + 2 * 512;                               // tile slot + two scale tables
+    float *red = reinterpret_cast<float *>(smem + SK_WAVES * WAVE_LDS);   // [KS][rows_here][NU][16 rows][16 tokens]
     const int K = p_K, nsb = K / QK_K;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: tile addresses become SGPR base + lane offset
+    uint8_t *slot = smem + wave * WAVE_LDS;
+    float *dxt = reinterpret_cast<float *>(slot + SLOT);                   // [2][8][16]
     const int m = lane & 15, g = lane >> 4;
-    const int src_lane4 = 4 * (4 * m + g);                // byte address, for ds_bpermute, of the lane that loaded row m, quarter g
     const int KS = p_ks, LK = __builtin_ctz((unsigned)KS), RS = SK_WAVES >> LK;      // KS is a power of two
     const int ks = wave & (KS - 1), rs = wave >> LK;
     (void)p_rows;
@@ -236,8 +251,6 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     const int rows_here = sq + (bx < sr ? 1 : 0);
     const int n_i = rs < RS ? (nsb - ks + KS - 1) >> LK : 0;        // super-blocks of this wave (ks < KS <= nsb)
     const size_t row_stride = (size_t)nsb * TB;
-    // B fragments: lane (n = m, g) supplies column n, quarter g (columns beyond T hold zeros)
-    const int lane_off = (TYPE == MESH_Q4_K ? 64 * g : 128 * (g >> 1) + 16 * (g & 1)) * 16 + m * 8;
     // flat tile index f -> (ii, seg); seg -> (local tile-row j, matrix u)
     auto seg_valid = [&](int seg) { return rs + RS * (seg / NU) < rows_here; };
     auto tile_ptr = [&](int ii, int seg) -> const uint8_t * {
@@ -254,7 +267,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     const int total = seg_valid(0) ? n_i * SEGS : 0;
 
     TileRegs<TYPE> ring[SK_DEPTH];
-    BFrags<TYPE> B[2];
+    XFrags X[2];
     f4_t D[SEGS];
 #pragma unroll
     for (int s = 0; s < SEGS; ++s) D[s] = f4_t{0.f, 0.f, 0.f, 0.f};
@@ -267,72 +280,67 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         const bool ok = f < total && seg_valid(seg);
         dst.load(tile_ptr(ok ? f / SEGS : n_i - 1, ok ? seg : 0), lane);
     };
-    auto compute = [&](const TileRegs<TYPE> &loaded, const BFrags<TYPE> &bf, f4_t &acc) {
-        TileRegs<TYPE> tile = loaded;
-        to_mfma_lanes(tile, src_lane4);
-        TileFrags<TYPE> F;
-        F.prepare(tile, g);
-#pragma unroll
-        for (int t = 0; t < 8; ++t)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
+    // the scale table of super-block ii goes to LDS table ii & 1 before the super-block's first tile
+    auto publish = [&](const XFrags &x, int b) {
+        wave_lds_sync();
+        *reinterpret_cast<float2 *>(dxt + b * 128 + 2 * lane) = x.dxpre;
+        wave_lds_sync();
     };
-    SK_MARK(0);
+    auto sb_of = [&](int ii) { return ks + KS * (ii < n_i ? ii : n_i - 1); };
     if (total > 0) {
+        // Loads return in issue order, so waiting for a load also waits for everything issued before it.  Every wait
+        // in the loop below is therefore for something issued at least two super-blocks earlier: activations are
+        // fetched two super-blocks ahead, BEFORE the weight tile issued in the same iteration, and a weight tile is
+        // consumed SK_DEPTH - 1 iterations after its load was issued.
+        X[0].template load<SUMS>(p_xq, K, sb_of(0), lane);
+        X[1].template load<SUMS>(p_xq, K, sb_of(1), lane);
 #pragma unroll
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
-        B[0].load(p_x, lane_off, ks);
-        B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
-        SK_MARK(1);
-        if (n_i <= 2 && total <= SK_DEPTH) {
-            // short walk: everything it needs is already in flight
+        constexpr int RB0 = SEGS >= SK_DEPTH ? 1 : SK_DEPTH / SEGS;
+        constexpr int RB = RB0 < 2 ? 2 : RB0;              // super-blocks per unrolled block: even, so the activation buffer of a step is static
+        constexpr int UB = RB * SEGS;                        // tiles per unrolled block, a multiple of the ring depth
+        static_assert(UB % SK_DEPTH == 0 && RB % 2 == 0, "ring slots and activation buffers must be static inside a block");
+        // Software pipeline: the LDS round trip of tile f + 1 (its view) is started before tile f is multiplied.
+        TileView<TYPE> cur, nxt;
+        cur.stage(ring[0], slot, lane);
+        load_tile(ring[0], SK_DEPTH, SK_DEPTH % SEGS);
+        for (int blk = 0; blk * RB < n_i; ++blk) {
 #pragma unroll
-            for (int q = 0; q < SK_DEPTH; ++q)
-                if (q < total && seg_valid(q % SEGS)) compute(ring[q], B[(q / SEGS) % 2], D[q % SEGS]);
-        } else {
-            constexpr int RB = SEGS >= 2 ? 2 : 4;            // super-block rounds per unrolled block (even: B parity is static)
-            constexpr int UB = RB * SEGS;                    // tiles per block, a multiple of the ring depth
-            static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
-            for (int blk = 0; blk * RB < n_i; ++blk) {
-#pragma unroll
-                for (int q = 0; q < UB; ++q) {
-                    const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
-                    const int ii = blk * RB + r, f = ii * SEGS + seg;
-                    if (ii < n_i && seg_valid(seg)) compute(ring[slot], B[r % 2], D[seg]);
-                    // refill this slot with the tile DEPTH positions ahead
-                    load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
-                    // last segment of a super-block: its activation buffer is free for the one after next
-                    if (seg == SEGS - 1) B[r % 2].load(p_x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
-                    __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
-                }
+            for (int q = 0; q < UB; ++q) {
+                const int r = q / SEGS, seg = q % SEGS;
+                const int ii = blk * RB + r, f = ii * SEGS + seg;
+                nxt.stage(ring[(q + 1) % SK_DEPTH], slot, lane);
+                if (seg == 0) publish(X[r % 2], r % 2);
+                if (ii < n_i && seg_valid(seg)) tile_mac(cur, X[r % 2], dxt + (r % 2) * 128, lane, D[seg]);
+                // last segment of a super-block: its activation buffer is free for the one after next
+                if (seg == SEGS - 1) X[r % 2].template load<SUMS>(p_xq, K, sb_of(ii + 2), lane);
+                load_tile(ring[(q + 1) % SK_DEPTH], f + 1 + SK_DEPTH, (q + 1 + SK_DEPTH) % SEGS);
+                cur = nxt;
+                __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
             }
         }
     }
 
-    SK_MARK(2);
-    // partial sums of this wave: D[seg] holds rows 4g..4g+3, column m of segment seg
+    // partial sums of this wave: D[seg][i] belongs to weight row m, token 4g + i of segment seg
 #pragma unroll
     for (int seg = 0; seg < SEGS; ++seg) {
         if (total > 0 && seg_valid(seg)) {
             const int j = rs + RS * (seg / NU), u = seg % NU;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + 4 * g + i) * 16 + m] = D[seg][i];
+            for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + m) * 16 + 4 * g + i] = D[seg][i];
         }
     }
     __syncthreads();
 
-    SK_MARK(3);
     // outputs of this workgroup: rows_here x 16 rows x T columns
     for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
+        if (t >= a.T) continue;
         const int tr = tr0 + j;
         int mi = 0;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
         const int row = (tr - a.tile_begin[mi]) * TILE_ROWS + r;
         if (row >= a.M[mi]) continue;
-        if (t >= a.T) {                                    // unused columns of the f16 output block stay finite
-            if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
-            continue;
-        }
         float s0 = 0.f, s1 = 0.f;
         for (int k2 = 0; k2 < KS; ++k2) {
             s0 += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + r) * 16 + t];
@@ -370,32 +378,30 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         } else {
             out = s0;
         }
-        if (a.y[mi]) a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
-        if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)out;
+        a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
     }
-    SK_MARK(4);
 }
 
 template <int TYPE, int NU, int SEGS>
-static int launch_skinny(const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
+static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
         MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_kernel<TYPE, NU, SEGS>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(ka.x, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks,
-                                                                                                 ka.tile_begin[3], (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16),
-                                                                                                 (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
+    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(
+        xq, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks, ka.tile_begin[3],
+        (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
 template <int TYPE, int NU>
-static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
-    if (segs <= 1) return launch_skinny<TYPE, NU, NU>(ka, grid, smem, stream);       // NU == 2 needs two segments at least
-    if (segs <= 2) return launch_skinny<TYPE, NU, 2>(ka, grid, smem, stream);
-    return launch_skinny<TYPE, NU, 4>(ka, grid, smem, stream);
+static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, size_t smem, hipStream_t stream) {
+    if (segs <= 1) return launch_skinny<TYPE, NU, NU>(ka, xq, grid, smem, stream);       // NU == 2 needs two segments at least
+    if (segs <= 2) return launch_skinny<TYPE, NU, 2>(ka, xq, grid, smem, stream);
+    return launch_skinny<TYPE, NU, 4>(ka, xq, grid, smem, stream);
 }
 
 static int skinny_n_cu() {
@@ -409,11 +415,14 @@ static int skinny_n_cu() {
     return n;
 }
 
+size_t q16_block_bytes(int K) { return (size_t)K * 32 + 2 * (size_t)(K / 32) * 16 * sizeof(float); }
+
 // all matrices of `a` are tiled K-quants of one type
 static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     const int type = a.mat[0].type;
     const int nsb = a.K / QK_K, NU = a.epi == EPI_SWIGLU ? 2 : 1;
-    const size_t row_stride = (size_t)nsb * (type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES);
+    const int tile_bytes = type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
+    const size_t row_stride = (size_t)nsb * tile_bytes;
     SkinnyKernelArgs ka{};
     int total_rows = 0;
     for (int i = 0; i < a.n_mat; ++i) {
@@ -432,7 +441,6 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     ka.K = a.K;
     ka.ldres = a.ldres; ka.epi = a.epi;
     ka.rope = a.rope;
-    ka.M16 = a.mat[0].M;
     int KS = 1;
     while (KS * 2 <= nsb && KS * 2 <= SK_WAVES) KS *= 2;      // a power of two: the kernel splits its waves with shifts
     const int RS = SK_WAVES / KS;
@@ -447,26 +455,105 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
     if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d segments per wave", segs);
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d tile-rows in one launch", total_rows);
-    const size_t smem = sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
-    if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: reduction buffer of %zu bytes does not fit LDS", smem);
+    const int lds_tile = ((type == MESH_Q4_K ? LDS_TILE_Q4 : LDS_TILE_Q6) + 255) / 256 * 256;
+    const size_t smem = (size_t)SK_WAVES * (lds_tile + 2 * 512) + sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
+    if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %zu bytes of LDS needed", smem);
     for (int t = 0; t < a.T; t += SK_NT) {
         SkinnyKernelArgs kb = ka;
         kb.T = std::min(SK_NT, a.T - t);
         if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
-        kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
+        const uint8_t *xq = a.xq + (size_t)(t / SK_NT) * q16_block_bytes(a.K);
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
-        kb.y16 = a.y16 ? a.y16 + (size_t)t * a.mat[0].M : nullptr;
         for (int i = 0; i < a.n_mat; ++i)
             if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
         int rc;
-        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, grid, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, grid, smem, stream);
-        else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, grid, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, grid, smem, stream);
+        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, xq, grid, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, xq, grid, smem, stream);
+        else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, xq, grid, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, xq, grid, smem, stream);
         if (rc != MESH_OK) return rc;
     }
     return MESH_OK;
 }
 
-// ---- producers of the k8-major activation layout ------------------------------------------------------------------
+// ---- producer of the q16 activation layout -------------------------------------------------------------------------
+// y = quantise(x[t] * rsqrt(mean(x[t]^2) + eps) * w), or with w == null just quantise(x[t]).  Workgroup (chunk, t)
+// quantises elements [1024 chunk, 1024 chunk + 1024) of token t, eight per lane; four neighbouring lanes share a
+// 32-element block, as in the mat-vec kernel's prologue (gemv_device.hpp: x_quantise), with the same rounding.  With a
+// norm every workgroup of a token sums the whole row's squares itself (the row is a few KB in L2): no second launch.
+// Token slots beyond T are not written: an MFMA row never mixes tokens, and the GEMM does not store those rows.
+constexpr int Q16_THREADS = 128;
+__global__ __launch_bounds__(Q16_THREADS) void quant16_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int n,
+                                                              uint8_t *__restrict__ y) {
+    __shared__ float red[Q16_THREADS / 64];
+    const int tid = threadIdx.x, tok = blockIdx.y, t = tok & 15;
+    uint8_t *yb = y + (size_t)(tok >> 4) * ((size_t)n * 36);
+    uint4 *planes = reinterpret_cast<uint4 *>(yb);                                  // record (k / 8, t) at planes[(k / 8) * 16 + t]
+    float *dxp = reinterpret_cast<float *>(yb + (size_t)n * 32), *sxp = reinterpret_cast<float *>(yb + (size_t)n * 34);
+    const float *xt = x + (size_t)tok * n;
+    const int i = blockIdx.x * (Q16_THREADS * 8) + tid * 8;
+    const bool live = i < n;
+    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
+    if (live) {
+        a0 = *reinterpret_cast<const float4 *>(xt + i);
+        a1 = *reinterpret_cast<const float4 *>(xt + i + 4);
+        if (w) { g0 = *reinterpret_cast<const float4 *>(w + i); g1 = *reinterpret_cast<const float4 *>(w + i + 4); }
+    }
+    float scale = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int k = tid * 4; k < n; k += Q16_THREADS * 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(xt + k);
+            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int k = 0; k < Q16_THREADS / 64; ++k) tot += red[k];
+        scale = 1.0f / sqrtf(tot / (float)n + eps);
+    }
+    const float v[8] = {a0.x * scale * g0.x, a0.y * scale * g0.y, a0.z * scale * g0.z, a0.w * scale * g0.w,
+                        a1.x * scale * g1.x, a1.y * scale * g1.y, a1.z * scale * g1.z, a1.w * scale * g1.w};
+    float amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    const float inv = amax > 0.f ? XQ_LEVELS / amax : 0.f;
+    int hi[8], lo[8], isum = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int q = __float2int_rn(v[e] * inv);
+        lo[e] = ((q + 128) & 0xFF) - 128;
+        hi[e] = (q - lo[e]) >> 8;
+        isum += q;
+    }
+    isum += __shfl_xor(isum, 1);
+    isum += __shfl_xor(isum, 2);
+    if (live) {
+        planes[(size_t)(i >> 3) * 16 + t] = make_uint4(pack_bytes(hi[0], hi[1], hi[2], hi[3]), pack_bytes(hi[4], hi[5], hi[6], hi[7]),
+                                                       pack_bytes(lo[0], lo[1], lo[2], lo[3]), pack_bytes(lo[4], lo[5], lo[6], lo[7]));
+        if ((tid & 3) == 0) {
+            const float d = amax / XQ_LEVELS;
+            dxp[(i >> 5) * 16 + t] = d;
+            sxp[(i >> 5) * 16 + t] = d * (float)isum;
+        }
+    }
+}
+
+int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t *y, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (n % 32) return fail(MESH_ERR_INVALID, "quant16_k8: row length %d not a multiple of 32", n);
+    quant16_kernel<<<dim3((unsigned)((n + Q16_THREADS * 8 - 1) / (Q16_THREADS * 8)), (unsigned)T), dim3(Q16_THREADS), 0, stream>>>(x, w, eps, n, y);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// ---- producers of the k8-major f16 activation layout (read by the large-tile GEMM, gemm.hip) ------------------------
+// Tokens are grouped in blocks of 16 columns, and within a block the 8 consecutive k of every column sit together:
+// element (t, k) of block b = t / 16 is at ((b * K/8 + k/8) * 16 + t % 16) * 8 + k % 8.
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {
     const h2_t h = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, h);
@@ -589,17 +676,16 @@ int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream) {
 }
 
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
-    if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.T <= 0 || a.K <= 0) return fail(MESH_ERR_INVALID, "gemm_skinny: bad arguments");
-    if (a.K % QK_K || (reinterpret_cast<uintptr_t>(a.x) & 15))
+    if (a.n_mat < 1 || a.n_mat > 3 || !a.xq || a.T <= 0 || a.K <= 0) return fail(MESH_ERR_INVALID, "gemm_skinny: bad arguments");
+    if (a.K % QK_K || (reinterpret_cast<uintptr_t>(a.xq) & 15))
         return fail(MESH_ERR_INVALID, "gemm_skinny: K %d must be a multiple of 256 and the activations 16-byte aligned", a.K);
-    if (a.y16 && a.mat[0].M % 8) return fail(MESH_ERR_INVALID, "gemm_skinny: f16 output needs a row count that is a multiple of 8");
     if (a.epi == EPI_SWIGLU && (a.n_mat != 2 || a.mat[0].M != a.mat[1].M || a.mat[0].type != a.mat[1].type))
         return fail(MESH_ERR_INVALID, "gemm_skinny: SwiGLU needs a gate and an up matrix of equal shape and type");
     if (a.epi == EPI_RESIDUAL && !a.residual) return fail(MESH_ERR_INVALID, "gemm_skinny: residual epilogue without residual");
     if (a.rope.pos && (a.epi != EPI_STORE || a.rope.head_dim % 2 || a.rope.n_rot % 2)) return fail(MESH_ERR_INVALID, "gemm_skinny: rope epilogue needs a plain store");
     for (int i = 0; i < a.n_mat; ++i) {
         if (!a.mat[i].W || a.mat[i].M <= 0 || !type_is_tiled(a.mat[i].type)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d is not a tiled K-quant", i);
-        if (!a.mat[i].y && !(i == 1 && a.epi == EPI_SWIGLU) && !(i == 0 && a.y16)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d has no output", i);
+        if (!a.mat[i].y && !(i == 1 && a.epi == EPI_SWIGLU)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d has no output", i);
     }
     bool same = true;
     for (int i = 1; i < a.n_mat; ++i) same = same && a.mat[i].type == a.mat[0].type;
@@ -612,7 +698,6 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
         SkinnyArgs sub = a;
         sub.n_mat = j - i;
         for (int k2 = 0; k2 < sub.n_mat; ++k2) { sub.mat[k2] = a.mat[i + k2]; sub.kind[k2] = a.kind[i + k2]; }
-        sub.y16 = i == 0 ? a.y16 : nullptr;
         int rc = skinny_one_type(sub, stream);
         if (rc != MESH_OK) return rc;
         i = j;

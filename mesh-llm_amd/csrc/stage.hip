@@ -506,7 +506,7 @@ static int skinny_min_tokens() {
     static int v = 0;
     if (!v) {
         const char *e = getenv("MESH_SKINNY_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 4;
+        v = e && atoi(e) > 0 ? atoi(e) : 5;
     }
     return v;
 }
@@ -554,6 +554,14 @@ int session_new(mesh_stage *st, mesh_session **out) {
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
         MESH_HIP_TRY(hipMemsetAsync(p, 0, B16 * std::max<size_t>(hp.n_embd, QD) * 2, s->stream));     // unused token columns stay finite
+        {
+            // q16 activations of the skinny GEMM (calls below the large-tile GEMM's token count), widest projection input
+            const size_t tok = std::min<size_t>(B, (size_t)std::max(16, PREFILL_MIN_TOKENS - 1));
+            const size_t kmax = std::max<size_t>(std::max<size_t>(hp.n_embd, QD), hp.n_ff);
+            const size_t bytes = (tok + 15) / 16 * q16_block_bytes((int)((kmax + 255) / 256 * 256));
+            if ((rc = sess_alloc(s.get(), &p, bytes)) != MESH_OK) return rc;
+            s->xq = static_cast<uint8_t *>(p);
+        }
         if (hp.n_ff > 0) {
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
@@ -698,7 +706,8 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     bool rope_fused = false, attn_is_k8 = false;
     const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
     auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; return g; };
-    if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
+    if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+    else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
@@ -707,7 +716,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
-        qa.x = xn; qa.K = E; qa.T = T;
+        qa.xq = s->xq; qa.K = E; qa.T = T;
         if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
             !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
             qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;
@@ -786,12 +795,15 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
             rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
         }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
-            if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }         // straight into the output projection's input layout
+            // straight into the output projection's input layout
+            if (skinny) { aa.out_q16 = s->xq; attn_is_k8 = true; }
+            else if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }
             rc = attention_mma(aa, T, stream);
         } else rc = attention(aa, T, stream);
     }
     if (rc != MESH_OK) return rc;
     if (attn_is_k8) rc = MESH_OK;
+    else if (skinny) rc = quant16_k8(s->attn, nullptr, 0.f, T, QD, s->xq, stream);
     else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
     else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
     if (rc != MESH_OK) return rc;
@@ -799,7 +811,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         SkinnyArgs oa;
         oa.n_mat = 1;
         oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
-        oa.x = xn; oa.K = QD; oa.T = T;
+        oa.xq = s->xq; oa.K = QD; oa.T = T;
         oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny(oa, stream)) != MESH_OK) return rc;
@@ -810,24 +822,26 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
     if (attn_only) return MESH_OK;
-    if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
+    if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+    else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
     else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     if (rc != MESH_OK) return rc;
     if (skinny) {
-        // gate and up in one pass with the SwiGLU epilogue, written as f16 straight into the down projection's input
+        // gate and up in one pass with the SwiGLU epilogue; its f32 output is quantised for the down projection
         SkinnyArgs ga;
         ga.n_mat = 2;
-        ga.mat[0] = mat_of(L.w_gate, nullptr, FF, nullptr);
+        ga.mat[0] = mat_of(L.w_gate, s->ffn, FF, nullptr);
         ga.mat[1] = mat_of(L.w_up, nullptr, FF, nullptr);
-        ga.x = xn; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
-        ga.y16 = f16ffn;
+        ga.xq = s->xq; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
         SkinnyArgs da;
         da.n_mat = 1;
         da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
-        da.x = f16ffn; da.K = FF; da.T = T;
+        da.xq = s->xq; da.K = FF; da.T = T;
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_skinny(ga, stream); }
+        if (rc != MESH_OK) return rc;
+        if ((rc = quant16_k8(s->ffn, nullptr, 0.f, T, FF, s->xq, stream)) != MESH_OK) return rc;
         ProfScope ps(s, MESH_PROF_GEMV);
-        if ((rc = gemm_skinny(ga, stream)) != MESH_OK) return rc;
         return gemm_skinny(da, stream);
     }
     if (L.gate_up_gemm && k8 && s->gemm_fused) {
