@@ -200,16 +200,19 @@ int64_t mesh_session_persistent_steps(const mesh_session *session);
  * session creation turns graphs on: they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
 int64_t mesh_session_graph_replays(const mesh_session *session);
 
-/* Per-kernel-class timing of a session, measured with HIP events recorded on the session's stream around each
- * launch.  Off by default (it adds two event records per launch).  Kinds index the arrays below. */
+/* Per-kernel-class timing of a session: every kernel launched for the session while profiling is on carries its own
+ * start / stop event pair (stamped by the dispatch, nothing extra is queued between launches), so ms[] sums pure
+ * kernel durations -- the same spans a kernel trace shows -- and launches[] counts kernels.  Off by default.  Kinds
+ * index the arrays below. */
 #define MESH_PROF_GEMV 0      /* dequant-fused mat-vec launches (q/k/v, o, gate/up, down, output) */
 #define MESH_PROF_ROPE 1      /* rope + KV append */
 #define MESH_PROF_ATTN 2      /* attention (split + combine) */
 #define MESH_PROF_CODEC 3     /* boundary pack / unpack */
-#define MESH_PROF_KINDS 4
+#define MESH_PROF_PREP 4      /* activation preparation of the batched paths: RMS norm + quantise / f16 conversion, SwiGLU */
+#define MESH_PROF_KINDS 5
 typedef struct mesh_profile {
-    double ms[MESH_PROF_KINDS];           /* summed event time per kind since the last reset */
-    uint64_t launches[MESH_PROF_KINDS];   /* bracketed launch groups per kind */
+    double ms[MESH_PROF_KINDS];           /* summed kernel time per kind since the last reset */
+    uint64_t launches[MESH_PROF_KINDS];   /* kernels per kind */
 } mesh_profile;
 int mesh_session_profile(mesh_session *session, int enable);          /* also resets the counters */
 int mesh_session_profile_read(mesh_session *session, mesh_profile *out);   /* waits for the stream */

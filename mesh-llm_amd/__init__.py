@@ -74,10 +74,10 @@ class Batch(ctypes.Structure):
 
 class Profile(ctypes.Structure):
     """mesh_profile"""
-    _fields_ = [("ms", ctypes.c_double * 4), ("launches", ctypes.c_uint64 * 4)]
+    _fields_ = [("ms", ctypes.c_double * 5), ("launches", ctypes.c_uint64 * 5)]
 
 
-PROF_GEMV, PROF_ROPE, PROF_ATTN, PROF_CODEC = 0, 1, 2, 3
+PROF_GEMV, PROF_ROPE, PROF_ATTN, PROF_CODEC, PROF_PREP = 0, 1, 2, 3, 4
 TOKENS, LOGITS = 100, 101
 _pp = ctypes.POINTER(ctypes.c_void_p)
 _psz = ctypes.POINTER(ctypes.c_size_t)
@@ -347,7 +347,7 @@ class Session:
     def profile_read(self):
         p = Profile()
         check(lib().mesh_session_profile_read(self._h, ctypes.byref(p)))
-        names = ("gemv", "rope", "attn", "codec")
+        names = ("gemv", "rope", "attn", "codec", "prep")
         return {n: {"ms": p.ms[i], "launches": int(p.launches[i])} for i, n in enumerate(names)}
 
     def set_expert_mask(self, allowed):

@@ -79,7 +79,7 @@ int rope_kv(const RopeKvArgs &a, int T, hipStream_t stream) {
         return fail(MESH_ERR_INVALID, "rope: bad head_dim/n_rot %d/%d", a.head_dim, a.n_rot);
     if (!kv_type_supported(a.k_type) || !kv_type_supported(a.v_type) || ((a.k_type != MESH_F16 || a.v_type != MESH_F16) && a.head_dim % 32))
         return fail(MESH_ERR_UNSUPPORTED, "rope: KV cache types %d/%d with head_dim %d", a.k_type, a.v_type, a.head_dim);
-    rope_kv_kernel<<<dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream>>>(a.pos, a.seq, a.q, a.k, a.v, a.n_head, a.n_kv, a.head_dim, a);
+    MESH_LAUNCH(rope_kv_kernel, dim3((unsigned)(a.n_head + 2 * a.n_kv), (unsigned)T), dim3(64), 0, stream, a.pos, a.seq, a.q, a.k, a.v, a.n_head, a.n_kv, a.head_dim, a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -300,7 +300,7 @@ static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     const dim3 block(ATTN_THREADS);
 #define MESH_ATTN_CASE(GG)                                                                          \
     if (a.group == GG) {                                                                            \
-        attn_kernel<HD, GG, KT, VT><<<dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream>>>(a); \
+        MESH_LAUNCH((attn_kernel<HD, GG, KT, VT>), dim3((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block, 0, stream, a); \
         MESH_LAUNCH_CHECK();                                                                        \
         return MESH_OK;                                                                             \
     }
@@ -311,7 +311,7 @@ static int launch_attn(const AttnArgs &a, int T, hipStream_t stream) {
     if (HD == 64) { MESH_ATTN_CASE(7) }
 #undef MESH_ATTN_CASE
     // any other group size: one query head per workgroup (K/V re-read per head)
-    attn_kernel<HD, 1, KT, VT><<<dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream>>>(a);
+    MESH_LAUNCH((attn_kernel<HD, 1, KT, VT>), dim3((unsigned)a.n_splits, (unsigned)(a.n_kv * a.group), (unsigned)T), block, 0, stream, a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -342,7 +342,7 @@ int attention(const AttnArgs &a, int T, hipStream_t stream) {
 }
 
 int attention_combine(const AttnArgs &a, int T, hipStream_t stream) {
-    attn_combine_kernel<<<dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream>>>(a.part, a.ml, a.out, a.out16_k8, a.out_q16, a.n_splits, a.n_head, a.head_dim);
+    MESH_LAUNCH(attn_combine_kernel, dim3((unsigned)a.n_head, (unsigned)T), dim3((unsigned)a.head_dim), 0, stream, a.part, a.ml, a.out, a.out16_k8, a.out_q16, a.n_splits, a.n_head, a.head_dim);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -366,13 +366,13 @@ __global__ __launch_bounds__(64) void kv_export_kernel(int type, const uint8_t *
 
 int kv_import(int type, uint8_t *cache, const uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream) {
     if (!kv_type_supported(type) || head_dim > ROPE_HD_MAX || (type != MESH_F16 && head_dim % 32)) return fail(MESH_ERR_UNSUPPORTED, "kv_import: type %d, head_dim %d", type, head_dim);
-    kv_import_kernel<<<dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream>>>(type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
+    MESH_LAUNCH(kv_import_kernel, dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream, type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 int kv_export(int type, const uint8_t *cache, uint16_t *half, int n_kv, int n_ctx, int head_dim, int seq, int pos0, int n_pos, hipStream_t stream) {
     if (!kv_type_supported(type)) return fail(MESH_ERR_UNSUPPORTED, "kv_export: type %d", type);
-    kv_export_kernel<<<dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream>>>(type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
+    MESH_LAUNCH(kv_export_kernel, dim3((unsigned)n_kv, (unsigned)n_pos), dim3(64), 0, stream, type, cache, half, n_kv, n_ctx, head_dim, seq, pos0);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -264,9 +264,9 @@ __global__ __launch_bounds__(MMA_THREADS) void attn_mma_kernel(const float *p_q,
 template <int HD>
 static int launch_mma(const AttnArgs &a, int T, hipStream_t stream) {
     const dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)T), block(MMA_THREADS);
-    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) attn_mma_kernel<HD, MESH_F16, MESH_F16><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
-    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q8_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
-    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) attn_mma_kernel<HD, MESH_Q4_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_LAUNCH((attn_mma_kernel<HD, MESH_F16, MESH_F16>), grid, block, 0, stream, a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
+    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_mma_kernel<HD, MESH_Q8_0, MESH_Q4_0>), grid, block, 0, stream, a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
+    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_mma_kernel<HD, MESH_Q4_0, MESH_Q4_0>), grid, block, 0, stream, a.q, a.pos, a.seq, a.kcache, a.vcache, a.n_splits, a.n_ctx, a.n_kv, a.group, a.n_head, a.scale, a);
     else return fail(MESH_ERR_UNSUPPORTED, "attention_mma: KV cache types %d/%d", a.k_type, a.v_type);
     MESH_LAUNCH_CHECK();
     return MESH_OK;

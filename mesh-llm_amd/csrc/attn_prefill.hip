@@ -200,9 +200,9 @@ int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t str
     while (hpw > 8 || a.group % hpw) --hpw;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * hpw));
-    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) attn_chunk_kernel<MESH_F16, MESH_F16><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
-    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) attn_chunk_kernel<MESH_Q8_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
-    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) attn_chunk_kernel<MESH_Q4_0, MESH_Q4_0><<<grid, block, 0, stream>>>(a, T, pos0, seq, hpw);
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_LAUNCH((attn_chunk_kernel<MESH_F16, MESH_F16>), grid, block, 0, stream, a, T, pos0, seq, hpw);
+    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_chunk_kernel<MESH_Q8_0, MESH_Q4_0>), grid, block, 0, stream, a, T, pos0, seq, hpw);
+    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_chunk_kernel<MESH_Q4_0, MESH_Q4_0>), grid, block, 0, stream, a, T, pos0, seq, hpw);
     else return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: KV cache types %d/%d", a.k_type, a.v_type);
     MESH_LAUNCH_CHECK();
     return MESH_OK;

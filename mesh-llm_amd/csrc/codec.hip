@@ -224,8 +224,8 @@ int act_pack_dev(int fmt, const float *src, void *dst, int64_t n, hipStream_t st
             return MESH_OK;
         case MESH_F16: {
             const int64_t grid = (n + CODEC_THREADS * 8 - 1) / (CODEC_THREADS * 8);
-            if (al) pack_f16_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint16_t *)dst, n);
-            else pack_f16_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint16_t *)dst, n);
+            if (al) MESH_LAUNCH(pack_f16_kernel<true>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, src, (uint16_t *)dst, n);
+            else MESH_LAUNCH(pack_f16_kernel<false>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, src, (uint16_t *)dst, n);
             MESH_LAUNCH_CHECK();
             return MESH_OK;
         }
@@ -233,8 +233,8 @@ int act_pack_dev(int fmt, const float *src, void *dst, int64_t n, hipStream_t st
             if (n % QK8_0) return fail(MESH_ERR_INVALID, "mesh_act_pack: q8_0 needs a multiple of 32 elements, got %lld", (long long)n);
             const int64_t nblk = n / QK8_0;
             const int64_t grid = (nblk + Q8_PACK_WG_BLOCKS - 1) / Q8_PACK_WG_BLOCKS;
-            if (al) pack_q8_0_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint8_t *)dst, nblk);
-            else pack_q8_0_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>(src, (uint8_t *)dst, nblk);
+            if (al) MESH_LAUNCH(pack_q8_0_kernel<true>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, src, (uint8_t *)dst, nblk);
+            else MESH_LAUNCH(pack_q8_0_kernel<false>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, src, (uint8_t *)dst, nblk);
             MESH_LAUNCH_CHECK();
             return MESH_OK;
         }
@@ -253,8 +253,8 @@ int act_unpack_dev(int fmt, const void *src, float *dst, int64_t n, hipStream_t 
             return MESH_OK;
         case MESH_F16: {
             const int64_t grid = (n + CODEC_THREADS * 4 - 1) / (CODEC_THREADS * 4);
-            if (al) unpack_f16_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint16_t *)src, dst, n);
-            else unpack_f16_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint16_t *)src, dst, n);
+            if (al) MESH_LAUNCH(unpack_f16_kernel<true>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, (const uint16_t *)src, dst, n);
+            else MESH_LAUNCH(unpack_f16_kernel<false>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, (const uint16_t *)src, dst, n);
             MESH_LAUNCH_CHECK();
             return MESH_OK;
         }
@@ -262,8 +262,8 @@ int act_unpack_dev(int fmt, const void *src, float *dst, int64_t n, hipStream_t 
             if (n % QK8_0) return fail(MESH_ERR_INVALID, "mesh_act_unpack: q8_0 needs a multiple of 32 elements, got %lld", (long long)n);
             const int64_t nblk = n / QK8_0;
             const int64_t grid = (nblk + Q8_WG_BLOCKS - 1) / Q8_WG_BLOCKS;
-            if (al) unpack_q8_0_kernel<true><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint8_t *)src, dst, nblk);
-            else unpack_q8_0_kernel<false><<<dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream>>>((const uint8_t *)src, dst, nblk);
+            if (al) MESH_LAUNCH(unpack_q8_0_kernel<true>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, (const uint8_t *)src, dst, nblk);
+            else MESH_LAUNCH(unpack_q8_0_kernel<false>, dim3((unsigned)grid), dim3(CODEC_THREADS), 0, stream, (const uint8_t *)src, dst, nblk);
             MESH_LAUNCH_CHECK();
             return MESH_OK;
         }

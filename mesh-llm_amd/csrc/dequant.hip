@@ -95,16 +95,16 @@ int dequantize_dev(int type, const void *src, float *dst, int64_t n, hipStream_t
         case MESH_F16:
             return act_unpack_dev(type, src, dst, n, stream);
         case MESH_Q8_0:
-            dequant_q8_0_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(x, dst, n);
+            MESH_LAUNCH(dequant_q8_0_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, dst, n);
             break;
         case MESH_Q5_0:
-            dequant_q5_0_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(x, dst, n);
+            MESH_LAUNCH(dequant_q5_0_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, dst, n);
             break;
         case MESH_Q4_K:
-            dequant_q4_K_kernel<<<dim3((unsigned)(n / QK_K)), dim3(256), 0, stream>>>(x, dst, n / QK_K);
+            MESH_LAUNCH(dequant_q4_K_kernel, dim3((unsigned)(n / QK_K)), dim3(256), 0, stream, x, dst, n / QK_K);
             break;
         case MESH_Q6_K:
-            dequant_q6_K_kernel<<<dim3((unsigned)(n / QK_K)), dim3(256), 0, stream>>>(x, dst, n / QK_K);
+            MESH_LAUNCH(dequant_q6_K_kernel, dim3((unsigned)(n / QK_K)), dim3(256), 0, stream, x, dst, n / QK_K);
             break;
         default:
             return fail(MESH_ERR_UNSUPPORTED, "mesh_dequantize: no kernel for ggml type %d", type);

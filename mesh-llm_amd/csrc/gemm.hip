@@ -28,7 +28,11 @@ constexpr int GM = 128, GN = 128, GK = 64;     // workgroup tile: weight rows x 
 constexpr int LDS_LD = GK + 8;                 // f16 elements per LDS row (16-byte pad against bank conflicts)
 constexpr int GEMM_THREADS = 512;              // 4 matrix-core waves + 4 staging waves
 
+// f32 pair -> packed f16, saturating: a magnitude beyond the f16 range becomes +-65504 instead of an infinity that the
+// next layer's norm would turn into NaN for the whole token.
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+    a = __builtin_amdgcn_fmed3f(a, -65504.f, 65504.f);
+    b = __builtin_amdgcn_fmed3f(b, -65504.f, 65504.f);
     return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
 }
 
@@ -573,13 +577,13 @@ static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) 
         MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW><<<grid, dim3(GEMM_THREADS), smem, stream>>>(k);
+    MESH_LAUNCH((gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW>), grid, dim3(GEMM_THREADS), smem, stream, k);
     MESH_LAUNCH_CHECK();
     if (SPLIT) {
         const int t_pad = k.y16_k8 ? (k.T + 15) & ~15 : k.T;
         const size_t n = (size_t)t_pad * grid.x * (k.y16_k8 ? GM / 8 : GM / 4);
         const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
-        gemm_splitk_epilogue_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(k, (int)grid.x);
+        MESH_LAUNCH(gemm_splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, stream, k, (int)grid.x);
         MESH_LAUNCH_CHECK();
     }
     return MESH_OK;
@@ -708,8 +712,8 @@ int gemm_pack(int type, const void *tiled, void *packed, int64_t M, int64_t K, h
     const dim3 grid((unsigned)(K / GK), (unsigned)((M + GM - 1) / GM));
     const int M_pad = (int)((M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS), nsb = (int)(K / QK_K);
     if (grid.y > 65535u) return fail(MESH_ERR_UNSUPPORTED, "gemm_pack: %lld rows are too many", (long long)M);
-    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
-    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
+    if (type == MESH_Q4_K) MESH_LAUNCH(gemm_pack_kernel<MESH_Q4_K>, grid, dim3(256), 0, stream, static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
+    else MESH_LAUNCH(gemm_pack_kernel<MESH_Q6_K>, grid, dim3(256), 0, stream, static_cast<const uint8_t *>(tiled), nullptr, static_cast<uint8_t *>(packed), M_pad, nsb);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -727,8 +731,8 @@ int gemm_pack_pair(int type, const void *gate_tiled, const void *up_tiled, void 
     const int M_pad = (int)((M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS), nsb = (int)(K / QK_K);
     if (grid.y > 65535u) return fail(MESH_ERR_UNSUPPORTED, "gemm_pack_pair: %lld rows are too many", (long long)M);
     const uint8_t *g = static_cast<const uint8_t *>(gate_tiled), *u = static_cast<const uint8_t *>(up_tiled);
-    if (type == MESH_Q4_K) gemm_pack_kernel<MESH_Q4_K><<<grid, dim3(256), 0, stream>>>(g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
-    else gemm_pack_kernel<MESH_Q6_K><<<grid, dim3(256), 0, stream>>>(g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
+    if (type == MESH_Q4_K) MESH_LAUNCH(gemm_pack_kernel<MESH_Q4_K>, grid, dim3(256), 0, stream, g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
+    else MESH_LAUNCH(gemm_pack_kernel<MESH_Q6_K>, grid, dim3(256), 0, stream, g, u, static_cast<uint8_t *>(packed), M_pad, nsb);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -761,7 +765,7 @@ __global__ __launch_bounds__(256) void rmsnorm_f16_kernel(const float *__restric
 int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 4 || ldy % 4) return fail(MESH_ERR_INVALID, "rmsnorm: row length %d not a multiple of 4", n);
-    rmsnorm_f16_kernel<<<dim3((unsigned)T), dim3(256), 0, stream>>>(x, w, eps, n, y, ldy);
+    MESH_LAUNCH(rmsnorm_f16_kernel, dim3((unsigned)T), dim3(256), 0, stream, x, w, eps, n, y, ldy);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -780,7 +784,7 @@ __global__ __launch_bounds__(256) void swiglu_f16_kernel(const float *__restrict
 int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream) {
     if (n <= 0) return MESH_OK;
     if (n % 4) return fail(MESH_ERR_INVALID, "swiglu: count not a multiple of 4");
-    swiglu_f16_kernel<<<dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream>>>(gate, up, out, n / 4);
+    MESH_LAUNCH(swiglu_f16_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream, gate, up, out, n / 4);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

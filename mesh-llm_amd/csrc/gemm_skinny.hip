@@ -390,7 +390,7 @@ static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    gemm_skinny_kernel<TYPE, NU, SEGS><<<dim3((unsigned)grid), dim3(SK_THREADS), smem, stream>>>(
+    MESH_LAUNCH((gemm_skinny_kernel<TYPE, NU, SEGS>), dim3((unsigned)grid), dim3(SK_THREADS), smem, stream, 
         xq, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks, ka.tile_begin[3],
         (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
     MESH_LAUNCH_CHECK();
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(Q16_THREADS) void quant16_kernel(const float *__res
 int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 32) return fail(MESH_ERR_INVALID, "quant16_k8: row length %d not a multiple of 32", n);
-    quant16_kernel<<<dim3((unsigned)((n + Q16_THREADS * 8 - 1) / (Q16_THREADS * 8)), (unsigned)T), dim3(Q16_THREADS), 0, stream>>>(x, w, eps, n, y);
+    MESH_LAUNCH(quant16_kernel, dim3((unsigned)((n + Q16_THREADS * 8 - 1) / (Q16_THREADS * 8)), (unsigned)T), dim3(Q16_THREADS), 0, stream, x, w, eps, n, y);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -554,8 +554,8 @@ int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t 
 // Tokens are grouped in blocks of 16 columns, and within a block the 8 consecutive k of every column sit together:
 // element (t, k) of block b = t / 16 is at ((b * K/8 + k/8) * 16 + t % 16) * 8 + k % 8.
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {
-    const h2_t h = {(_Float16)a, (_Float16)b};
+__device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {       // saturating, like gemm.hip's pack_h2
+    const h2_t h = {(_Float16)__builtin_amdgcn_fmed3f(a, -65504.f, 65504.f), (_Float16)__builtin_amdgcn_fmed3f(b, -65504.f, 65504.f)};
     return __builtin_bit_cast(uint32_t, h);
 }
 
@@ -635,7 +635,7 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
-    to_k8_kernel<<<dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream>>>(x, w, eps, T, n, y);
+    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -666,7 +666,7 @@ __global__ __launch_bounds__(256) void swiglu_k8_kernel(const float *__restrict_
 int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "swiglu_f16_k8: row length %d not a multiple of 8", n);
-    swiglu_k8_kernel<<<dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream>>>(gate, up, T, n, y);
+    MESH_LAUNCH(swiglu_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, gate, up, T, n, y);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -221,7 +221,7 @@ static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStrea
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dot_kernel<TYPE, NB, NU, EXPERT><<<grid, dim3(GEMV_THREADS), smem, stream>>>(
+    MESH_LAUNCH((gemv_dot_kernel<TYPE, NB, NU, EXPERT>), grid, dim3(GEMV_THREADS), smem, stream, 
         ka.x, ka.norm_w, ka.wbase[0], ka.wbase[1], ka.wbase[2], (unsigned)ka.ldx | (grid.x << 16), rows | (q << 16),
         (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), r | ((unsigned)(ka.K / QK_K) << 16) | ((unsigned)ka.ks << 24), ka);
     MESH_LAUNCH_CHECK();
@@ -240,7 +240,7 @@ static int launch_grouped(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipS
     if (ka.K / QK_K > 0xFF || ka.tile_begin[3] > 0xFFFF || ka.ldx > 0xFFFF || ka.x_div > 0xFFFF || ka.expert_stride > 0xFFFFFFFFull || (w1d & 255) ||
         w1d / 256 > INT32_MAX || w1d / 256 < INT32_MIN)
         return fail(MESH_ERR_UNSUPPORTED, "gemv: grouped expert launch outside its packed argument ranges");
-    gemv_grouped_kernel<TYPE, NU><<<grid, dim3(GROUPED_THREADS), smem, stream>>>(
+    MESH_LAUNCH((gemv_grouped_kernel<TYPE, NU>), grid, dim3(GROUPED_THREADS), smem, stream, 
         ka.items, ka.n_items, ka.x, ka.norm_w, ka.wbase[0], (unsigned)(ka.K / QK_K) | ((unsigned)ka.ks << 8) | ((unsigned)ka.tile_begin[3] << 16),
         (unsigned)ka.ldx | ((unsigned)ka.x_div << 16), (unsigned)ka.expert_stride, (int)(w1d / 256), ka);
     MESH_LAUNCH_CHECK();
@@ -386,7 +386,7 @@ static int launch_dual2(const GemvKernelArgs &k4, const GemvKernelArgs &k6, int 
         MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dual_kernel<NB, SIMPLE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    gemv_dual_kernel<NB, SIMPLE><<<dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream>>>(
+    MESH_LAUNCH((gemv_dual_kernel<NB, SIMPLE>), dim3((unsigned)(n4 + n6)), dim3(GEMV_THREADS), smem, stream, 
         k4.x, k4.norm_w, k4.wbase[0], k4.wbase[1], k6.wbase[0], (unsigned)k4.ldx | ((unsigned)n4 << 16),
         (unsigned)k4.tile_begin[3] | ((unsigned)k6.tile_begin[3] << 16), (unsigned)k4.tile_begin[1] | ((unsigned)(n4 + n6) << 16),
         (unsigned)(k4.K / QK_K) | ((unsigned)k4.ks << 8), k4, k6);

@@ -172,7 +172,7 @@ static int launch_generic(const GenArgs &ka, int grid, hipStream_t stream) {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         attr_set = true;
     }
-    gemv_generic_kernel<NB><<<dim3((unsigned)grid), dim3(GEN_THREADS), smem, stream>>>(ka);
+    MESH_LAUNCH(gemv_generic_kernel<NB>, dim3((unsigned)grid), dim3(GEN_THREADS), smem, stream, ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

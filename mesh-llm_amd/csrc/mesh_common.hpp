@@ -4,10 +4,14 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <hip/hip_ext.h>
+
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <tuple>
+#include <utility>
 
 #include "../../include/mesh_stage.h"
 
@@ -33,6 +37,32 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
             return ::mesh::fail(MESH_ERR_DEVICE, "kernel launch failed: %s (%s:%d)",         \
                                 hipGetErrorString(_e), __FILE__, __LINE__);                  \
     } while (0)
+
+// ---- kernel launches --------------------------------------------------------------------------------------------
+// Every kernel goes out through MESH_LAUNCH.  While the calling thread is inside a profiled scope of a session
+// (mesh_session_profile), the launch carries a start / stop event pair of its own: the runtime stamps them from the
+// dispatch itself, so the measured span is the kernel's and nothing is added to the stream between launches (an event
+// recorded around a launch adds a marker packet on either side, which at a few microseconds per kernel is a
+// perturbation of the same order as the thing measured).  Otherwise both events are null and this is a plain launch.
+struct LaunchTimer {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+LaunchTimer launch_timer();
+
+template <typename... KArgs, size_t... I>
+inline void launch_kernel_impl(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t stream, std::tuple<KArgs...> &formal,
+                               std::index_sequence<I...>) {
+    void *ptrs[sizeof...(KArgs) ? sizeof...(KArgs) : 1] = {static_cast<void *>(&std::get<I>(formal))...};
+    const LaunchTimer t = launch_timer();
+    (void)hipExtLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, smem, stream, t.start, t.stop, 0);
+}
+template <typename... KArgs, typename... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t stream, Args &&...args) {
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count differs from the kernel's parameter list");
+    std::tuple<KArgs...> formal(static_cast<KArgs>(args)...);       // the arguments in the kernel's own parameter types
+    launch_kernel_impl(kernel, grid, block, smem, stream, formal, std::index_sequence_for<KArgs...>{});
+}
+#define MESH_LAUNCH(kernel, grid, block, smem, stream, ...) ::mesh::launch_kernel(kernel, grid, block, smem, stream, ##__VA_ARGS__)
 
 // block geometry of the GGUF types on the stage path
 constexpr int QK8_0 = 32, Q8_0_BYTES = 34;

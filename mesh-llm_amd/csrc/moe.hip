@@ -158,10 +158,10 @@ int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float
     if (!moe_router_fused_supported(E, a.n_expert, a.top_k)) return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d / %d experts", E, a.n_expert);
     const dim3 grid((unsigned)T), block(ROUTER_THREADS);
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 2: MESH_LAUNCH(moe_router_fused_kernel<2>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 4: MESH_LAUNCH(moe_router_fused_kernel<4>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 8: MESH_LAUNCH(moe_router_fused_kernel<8>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+        case 16: MESH_LAUNCH(moe_router_fused_kernel<16>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
@@ -175,7 +175,7 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (a.n_expert < 1 || a.n_expert > 64 * ROUTE_MAX_PER_LANE || a.top_k < 1 || a.top_k > 64 || a.top_k > a.n_expert)
         return fail(MESH_ERR_UNSUPPORTED, "moe: %d experts / top-%d outside what the router kernel handles", a.n_expert, a.top_k);
-    moe_route_kernel<<<dim3((unsigned)T), dim3(64), 0, stream>>>(a);
+    MESH_LAUNCH(moe_route_kernel, dim3((unsigned)T), dim3(64), 0, stream, a);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -271,16 +271,16 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
     const dim3 grid((unsigned)T, (unsigned)split), block(ROUTER_THREADS);
     MoeRouteArgs la = a;
     switch (E / 256) {
-        case 2: moe_router_fused_kernel<2><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
-        case 4: moe_router_fused_kernel<4><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
-        case 8: moe_router_fused_kernel<8><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
-        case 16: moe_router_fused_kernel<16><<<grid, block, 0, stream>>>(x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 2: MESH_LAUNCH(moe_router_fused_kernel<2>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 4: MESH_LAUNCH(moe_router_fused_kernel<4>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 8: MESH_LAUNCH(moe_router_fused_kernel<8>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
+        case 16: MESH_LAUNCH(moe_router_fused_kernel<16>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
         default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
     }
     MESH_LAUNCH_CHECK();
     la.logits = logits;
     const size_t smem = ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
-    moe_route_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(la.logits, la.mask, la.ids, la.weights, T, la.n_expert, la.top_k, la.norm_w,
+    MESH_LAUNCH(moe_route_group_kernel, dim3(1), dim3(GROUP_THREADS), smem, stream, la.logits, la.mask, la.ids, la.weights, T, la.n_expert, la.top_k, la.norm_w,
                                                                            items, n_items);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
@@ -302,7 +302,7 @@ int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int
         attr_set = true;
     }
     const size_t smem = ((size_t)n_pairs + 2 * (size_t)n_expert) * sizeof(int32_t);
-    moe_group_kernel<<<dim3(1), dim3(GROUP_THREADS), smem, stream>>>(ids, n_pairs, n_expert, items, n_items);
+    MESH_LAUNCH(moe_group_kernel, dim3(1), dim3(GROUP_THREADS), smem, stream, ids, n_pairs, n_expert, items, n_items);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float *__restrict__ x,
 
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
-    moe_combine_kernel<<<dim3((unsigned)((n_embd + 255) / 256), (unsigned)T), dim3(256), 0, stream>>>(x, y, w, n_embd, top_k);
+    MESH_LAUNCH(moe_combine_kernel, dim3((unsigned)((n_embd + 255) / 256), (unsigned)T), dim3(256), 0, stream, x, y, w, n_embd, top_k);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -69,11 +69,11 @@ static int repack_common(bool to_tiled, int type, const void *src, void *dst, in
     const uint8_t *s = static_cast<const uint8_t *>(src);
     uint8_t *d = static_cast<uint8_t *>(dst);
     if (type == MESH_Q4_K) {
-        if (to_tiled) repack_q4k_kernel<true><<<grid, dim3(64), 0, stream>>>(s, d, (int)M, nsb);
-        else repack_q4k_kernel<false><<<grid, dim3(64), 0, stream>>>(s, d, (int)M, nsb);
+        if (to_tiled) MESH_LAUNCH(repack_q4k_kernel<true>, grid, dim3(64), 0, stream, s, d, (int)M, nsb);
+        else MESH_LAUNCH(repack_q4k_kernel<false>, grid, dim3(64), 0, stream, s, d, (int)M, nsb);
     } else {
-        if (to_tiled) repack_q6k_kernel<true><<<grid, dim3(64), 0, stream>>>(s, d, (int)M, nsb);
-        else repack_q6k_kernel<false><<<grid, dim3(64), 0, stream>>>(s, d, (int)M, nsb);
+        if (to_tiled) MESH_LAUNCH(repack_q6k_kernel<true>, grid, dim3(64), 0, stream, s, d, (int)M, nsb);
+        else MESH_LAUNCH(repack_q6k_kernel<false>, grid, dim3(64), 0, stream, s, d, (int)M, nsb);
     }
     MESH_LAUNCH_CHECK();
     return MESH_OK;

@@ -635,35 +635,49 @@ static int attn_splits_for(int T, int n_kv, int max_keys) {
 }
 
 // ---- optional timing -----------------------------------------------------------------------------
-struct ProfScope {
-    mesh_session *s;
-    bool on;
-    ProfScope(mesh_session *ses, int kind) : s(ses), on(ses->profile) {
-        if (!on) return;
-        if (s->prof_used + 2 > s->prof_events.size()) {
-            for (int i = 0; i < 2; ++i) {
-                hipEvent_t e;
-                if (hipEventCreate(&e) != hipSuccess) { on = false; return; }
-                s->prof_events.push_back(e);
-            }
+// A ProfScope names the kernel class of the launches made while it lives; launch_timer() (mesh_common.hpp) hands each of
+// them an event pair of the session, which profile_collect reads back.
+namespace {
+thread_local mesh_session *t_prof_session = nullptr;
+thread_local int t_prof_kind = 0;
+}  // namespace
+
+LaunchTimer launch_timer() {
+    LaunchTimer t;
+    mesh_session *s = t_prof_session;
+    if (!s) return t;
+    if (s->prof_used + 2 > s->prof_events.size()) {
+        for (int i = 0; i < 2; ++i) {
+            hipEvent_t e;
+            if (hipEventCreate(&e) != hipSuccess) { (void)hipGetLastError(); return t; }
+            s->prof_events.push_back(e);
         }
-        s->prof_kinds.push_back(kind);
-        (void)hipEventRecord(s->prof_events[s->prof_used], s->stream);
     }
-    ~ProfScope() {
-        if (!on) return;
-        (void)hipEventRecord(s->prof_events[s->prof_used + 1], s->stream);
-        s->prof_used += 2;
+    s->prof_kinds.push_back(t_prof_kind);
+    t.start = s->prof_events[s->prof_used];
+    t.stop = s->prof_events[s->prof_used + 1];
+    s->prof_used += 2;
+    return t;
+}
+
+struct ProfScope {
+    mesh_session *prev_s;
+    int prev_kind;
+    ProfScope(mesh_session *ses, int kind) : prev_s(t_prof_session), prev_kind(t_prof_kind) {
+        if (ses->profile) { t_prof_session = ses; t_prof_kind = kind; }
     }
+    ~ProfScope() { t_prof_session = prev_s; t_prof_kind = prev_kind; }
 };
 
 int profile_collect(mesh_session *s) {
     MESH_HIP_TRY(hipStreamSynchronize(s->stream));
-    for (size_t i = 0; i + 1 < s->prof_used + 1 && i / 2 < s->prof_kinds.size(); i += 2) {
+    for (size_t i = 0; i + 1 < s->prof_used && i / 2 < s->prof_kinds.size(); i += 2) {
         float ms = 0.f;
         if (hipEventElapsedTime(&ms, s->prof_events[i], s->prof_events[i + 1]) == hipSuccess) {
             s->prof_ms[s->prof_kinds[i / 2]] += ms;
             s->prof_launches[s->prof_kinds[i / 2]] += 1;
+        } else {
+            (void)hipGetLastError();
         }
     }
     s->prof_used = 0;
@@ -706,9 +720,12 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     bool rope_fused = false, attn_is_k8 = false;
     const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
     auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; return g; };
-    if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
-    else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
-    else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    {
+        ProfScope ps(s, MESH_PROF_PREP);
+        if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
+        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    }
     if (rc != MESH_OK) return rc;
     if (skinny) {
         SkinnyArgs qa;
@@ -802,10 +819,13 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         } else rc = attention(aa, T, stream);
     }
     if (rc != MESH_OK) return rc;
-    if (attn_is_k8) rc = MESH_OK;
-    else if (skinny) rc = quant16_k8(s->attn, nullptr, 0.f, T, QD, s->xq, stream);
-    else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
-    else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
+    {
+        ProfScope ps(s, MESH_PROF_PREP);
+        if (attn_is_k8) rc = MESH_OK;
+        else if (skinny) rc = quant16_k8(s->attn, nullptr, 0.f, T, QD, s->xq, stream);
+        else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
+        else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
+    }
     if (rc != MESH_OK) return rc;
     if (skinny) {
         SkinnyArgs oa;
@@ -822,9 +842,12 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_kquant(go, stream)) != MESH_OK) return rc;
     }
     if (attn_only) return MESH_OK;
-    if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
-    else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
-    else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    {
+        ProfScope ps(s, MESH_PROF_PREP);
+        if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
+        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+    }
     if (rc != MESH_OK) return rc;
     if (skinny) {
         // gate and up in one pass with the SwiGLU epilogue; its f32 output is quantised for the down projection
@@ -840,7 +863,8 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
         { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_skinny(ga, stream); }
         if (rc != MESH_OK) return rc;
-        if ((rc = quant16_k8(s->ffn, nullptr, 0.f, T, FF, s->xq, stream)) != MESH_OK) return rc;
+        { ProfScope ps(s, MESH_PROF_PREP); rc = quant16_k8(s->ffn, nullptr, 0.f, T, FF, s->xq, stream); }
+        if (rc != MESH_OK) return rc;
         ProfScope ps(s, MESH_PROF_GEMV);
         return gemm_skinny(da, stream);
     }
@@ -858,8 +882,11 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
             if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, s->ffn, FF, nullptr)), stream)) != MESH_OK) return rc;
             if ((rc = gemm_kquant(gemm_k8(gemm_of(L.w_up, s->xn16, E, T, s->ffn_up, FF, nullptr)), stream)) != MESH_OK) return rc;
         }
-        if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
-        else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
+        {
+            ProfScope ps(s, MESH_PROF_PREP);
+            if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
+            else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
+        }
         if (rc != MESH_OK) return rc;
     }
     {

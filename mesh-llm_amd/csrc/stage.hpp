@@ -140,7 +140,7 @@ struct mesh_session {
     std::vector<hipEvent_t> prof_events;      // pairs (begin, end)
     std::vector<int> prof_kinds;
     size_t prof_used = 0;
-    double prof_ms[MESH_PROF_KINDS] = {0, 0, 0, 0};
-    uint64_t prof_launches[MESH_PROF_KINDS] = {0, 0, 0, 0};
+    double prof_ms[MESH_PROF_KINDS] = {};
+    uint64_t prof_launches[MESH_PROF_KINDS] = {};
     ~mesh_session();
 };
