@@ -98,6 +98,22 @@ def run_codec(torch, m, steps, warmup, T=4096, h=4096):
         ms, _ = time_on_stream(torch, stream, fn, steps, warmup)
         gbs = n * bpe / ms / 1e6
         res[name] = {"ms": round(ms, 5), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+    # yardstick: a plain streaming kernel of the same traffic shape over the same buffers, timed the same way (f32 side
+    # n * 4 bytes; the other side a quarter of that for q8_0, whose packed side is really 0.266 of it, half for f16)
+    big = n * 4
+    plain = {
+        "pack_q8_0": lambda i: m.hbm_mix_probe_dev(xs[i % nbuf].data_ptr(), packed[i % nbuf].data_ptr(), big, 4, True, s),
+        "unpack_q8_0": lambda i: m.hbm_mix_probe_dev(packed[i % nbuf].data_ptr(), backs[i % nbuf].data_ptr(), big, 4, False, s),
+        "pack_f16": lambda i: m.hbm_mix_probe_dev(xs[i % nbuf].data_ptr(), halves[i % nbuf].data_ptr(), big, 2, True, s),
+        "unpack_f16": lambda i: m.hbm_mix_probe_dev(halves[i % nbuf].data_ptr(), backs[i % nbuf].data_ptr(), big, 2, False, s),
+    }
+    for name, fn in plain.items():
+        ms, _ = time_on_stream(torch, stream, fn, steps, warmup)
+        ratio = 4 if "q8_0" in name else 2
+        gbs = (big + big // ratio) / ms / 1e6
+        res[name]["plain_stream_ms"] = round(ms, 5)
+        res[name]["plain_stream_GBps"] = round(gbs, 1)
+        res[name]["frac_of_plain_stream"] = round(res[name]["GBps"] / gbs, 4)
     return res
 
 

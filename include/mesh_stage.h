@@ -66,6 +66,13 @@ int mesh_device_select(const char *device);
  * taken by the caller; its output feeds mesh-llm/src/system/benchmark.rs:11-29). */
 int mesh_hbm_read_probe(size_t bytes, int warmup_runs, int timed_runs, double *gbps);
 
+/* Plain streaming kernel of a given traffic shape, the yardstick for the codec kernels: moves `big_bytes` on the
+ * larger side (read if big_is_read, else written) and big_bytes / ratio on the other (ratio 1, 2 or 4), non-temporal
+ * 16-byte vectors, queued on `stream` and not waited for; the caller times it like any other launch.  big_bytes must be
+ * a multiple of 4096 * ratio.  Same purpose as mesh_hbm_read_probe (mesh-llm/benchmarks/membench-fingerprint.hip:24-39),
+ * for kernels that write as well as read. */
+int mesh_hbm_mix_probe_dev(const void *d_src, void *d_dst, size_t big_bytes, int ratio, int big_is_read, void *stream);
+
 /* ---- boundary activation codec -------------------------------------------------------------------
  * The inter-stage hidden state [n_tokens, n_embd] f32, packed for transport.  Replaces the raw-f32
  * ggml_backend_tensor_get -> TCP -> ggml_backend_tensor_set hop of push_tensor_to_peer

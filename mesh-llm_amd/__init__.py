@@ -34,6 +34,7 @@ SIGNATURES = {
     "mesh_device_count": (_i32, []),
     "mesh_device_select": (_i32, [_cp]),
     "mesh_hbm_read_probe": (_i32, [_sz, _i32, _i32, _vp]),
+    "mesh_hbm_mix_probe_dev": (_i32, [_vp, _vp, _sz, _i32, _i32, _vp]),
     "mesh_act_packed_size": (_sz, [_i32, _i64, _i64]),
     "mesh_act_pack": (_i32, [_i32, _vp, _vp, _i64]),
     "mesh_act_unpack": (_i32, [_i32, _vp, _vp, _i64]),
@@ -151,6 +152,12 @@ def hbm_read_probe(nbytes=512 << 20, warmup=3, runs=20):
     out = (ctypes.c_double * runs)()
     check(lib().mesh_hbm_read_probe(nbytes, warmup, runs, out))
     return sorted(out)
+
+
+def hbm_mix_probe_dev(src_ptr, dst_ptr, big_bytes, ratio, big_is_read, stream=0):
+    """Queue one plain streaming kernel that moves big_bytes on its larger side and big_bytes / ratio on the other
+    (mesh_hbm_mix_probe_dev); device pointers, not waited for."""
+    check(lib().mesh_hbm_mix_probe_dev(src_ptr, dst_ptr, big_bytes, ratio, int(bool(big_is_read)), stream))
 
 
 def act_packed_size(fmt, n_tokens, n_embd):

@@ -28,6 +28,30 @@ __global__ __launch_bounds__(MB_THREADS) void memread_kernel(const uint4 *__rest
     if (acc == 0x9E3779B9u) atomicAdd(sink, acc);     // never true for a zero-filled buffer; keeps the loads alive
 }
 
+// Plain streaming mix: every workgroup pass reads RD and writes WR 16-byte vectors per thread, each instruction of a
+// wave covering one contiguous kilobyte, non-temporal both ways, one pass per workgroup.  No arithmetic to speak of:
+// what this reaches for a given read : write ratio and size is what the memory system gives a kernel of that traffic
+// shape, the yardstick for the codec kernels (q8_0 pack reads 3.8 bytes per byte written, f16 pack 2, the unpacks the
+// reverse).
+typedef unsigned int mb_u32x4 __attribute__((ext_vector_type(4)));
+template <int RD, int WR>
+__global__ __launch_bounds__(MB_THREADS) void memmix_kernel(const mb_u32x4 *__restrict__ src, mb_u32x4 *__restrict__ dst) {
+    const mb_u32x4 *s = src + (size_t)blockIdx.x * MB_THREADS * RD + threadIdx.x;
+    mb_u32x4 *d = dst + (size_t)blockIdx.x * MB_THREADS * WR + threadIdx.x;
+    mb_u32x4 v[RD];
+#pragma unroll
+    for (int r = 0; r < RD; ++r) v[r] = __builtin_nontemporal_load(s + r * MB_THREADS);
+    mb_u32x4 a = v[0];
+#pragma unroll
+    for (int r = 1; r < RD; ++r) a ^= v[r];
+#pragma unroll
+    for (int w = 0; w < WR; ++w) {
+        mb_u32x4 o = a;
+        o.x += w;
+        __builtin_nontemporal_store(o, d + w * MB_THREADS);
+    }
+}
+
 }  // namespace mesh
 
 using namespace mesh;
@@ -72,4 +96,22 @@ extern "C" int mesh_hbm_read_probe(size_t bytes, int warmup_runs, int timed_runs
     }
 #undef MB_TRY
     return done(rc);
+}
+
+extern "C" int mesh_hbm_mix_probe_dev(const void *d_src, void *d_dst, size_t big_bytes, int ratio, int big_is_read, void *stream) {
+    if (!d_src || !d_dst || (ratio != 1 && ratio != 2 && ratio != 4)) return fail(MESH_ERR_INVALID, "mesh_hbm_mix_probe_dev: bad arguments");
+    const size_t per_wg = (size_t)MB_THREADS * 16 * ratio;        // bytes of the larger side one workgroup moves
+    if (big_bytes < per_wg || big_bytes % per_wg) return fail(MESH_ERR_INVALID, "mesh_hbm_mix_probe_dev: %zu bytes is not a multiple of %zu", big_bytes, per_wg);
+    if ((reinterpret_cast<uintptr_t>(d_src) | reinterpret_cast<uintptr_t>(d_dst)) & 15u) return fail(MESH_ERR_INVALID, "mesh_hbm_mix_probe_dev: pointers must be 16-byte aligned");
+    const dim3 grid((unsigned)(big_bytes / per_wg)), block(MB_THREADS);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const mb_u32x4 *s = static_cast<const mb_u32x4 *>(d_src);
+    mb_u32x4 *d = static_cast<mb_u32x4 *>(d_dst);
+    if (ratio == 1) MESH_LAUNCH((memmix_kernel<1, 1>), grid, block, 0, st, s, d);
+    else if (ratio == 2 && big_is_read) MESH_LAUNCH((memmix_kernel<2, 1>), grid, block, 0, st, s, d);
+    else if (ratio == 2) MESH_LAUNCH((memmix_kernel<1, 2>), grid, block, 0, st, s, d);
+    else if (big_is_read) MESH_LAUNCH((memmix_kernel<4, 1>), grid, block, 0, st, s, d);
+    else MESH_LAUNCH((memmix_kernel<1, 4>), grid, block, 0, st, s, d);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
 }
