@@ -45,6 +45,19 @@ def codec_input(T, h=4096):
     return x
 
 
+def profiled_ratio(fname, key):
+    """The number on the line `<key> = <number>` of profiles/<fname> (HBM traffic measured with rocprofv3 counters, as
+    a multiple of the algorithmic bytes); None when the file or the line is not there."""
+    try:
+        with open(os.path.join(ROOT, "profiles", fname)) as f:
+            for line in f:
+                if line.startswith(key + " ="):
+                    return float(line.split("=", 1)[1].split()[0])
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def time_on_stream(torch, stream, fn, steps, warmup):
     """Average ms per call of fn(i) over `steps` calls: events recorded on `stream`, host clock beside it."""
     for i in range(warmup):
@@ -138,13 +151,18 @@ def bench_codec(args):
     m.lib()
     res = run_codec(torch, m, args.steps, args.warmup)
     gbs, ms = res["pack_q8_0"]["GBps"], res["pack_q8_0"]["ms"]
+    codec_ratio = profiled_ratio(CODEC_TRAFFIC_PROFILE, "pack_q8_0_traffic_over_algorithmic")
     out = {
         "metric": "activation pack GB/s (q8_0, [4096,4096] f32)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32->i8+f16", "data": "synthetic",
         "config": {"workload": "codec: pack_q8_0 of hidden state [4096,4096] f32, N(0,1) with 0.1% channels x50"},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "measured_stream_read_GBps": hbm_probe(m)},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": int(round(codec_ratio * 4096 * 4096 * Q8_BPE)) if codec_ratio else None,
+                     "traffic_source": "profiles/" + CODEC_TRAFFIC_PROFILE if codec_ratio else None,
+                     "plain_stream_GBps": res["pack_q8_0"]["plain_stream_GBps"], "frac_of_plain_stream": res["pack_q8_0"]["frac_of_plain_stream"],
+                     "measured_stream_read_GBps": hbm_probe(m)},
         "codec": res,
     }
     if not args.no_cpu:
@@ -158,6 +176,8 @@ STAGE_LAYERS = 16
 # bytes of one head_dim-128 cache row: f16, q8_0 (32 x 34-byte blocks' worth: 128 quants + 4 scales), q4_0 (64 + 8)
 HD_BYTES_F16, HD_BYTES_Q8_0, HD_BYTES_Q4_0 = 256, 136, 72
 PREFILL_T = 2048
+TRAFFIC_PROFILE = "stage_decode_llama3_8b_l0_15_hbm_traffic.txt"
+CODEC_TRAFFIC_PROFILE = "codec_4096x4096_hbm_traffic.txt"
 BURN_IN_SECONDS = 2.0
 
 
@@ -249,7 +269,7 @@ def bench_stage(args):
             ses.decode_dev(x.data_ptr(), pos, out.data_ptr(), out.numel(), seq=seq, in_fmt=m.F32, out_fmt=m.Q8_0)
 
         ms, wall = time_on_stream(torch, stream, step, args.steps, args.warmup)
-        # per-kernel-class durations, from a few extra steps with event brackets around every launch
+        # per-kernel-class durations over a few extra steps: every launch carries its own start / stop stamps
         ses.profile(True)
         for i in range(5):
             step(i)
@@ -280,11 +300,15 @@ def bench_stage(args):
         mm_flop = 2.0 * PREFILL_T * STAGE_LAYERS * (E * H * HD * 2 + E * HK * HD * 2 + 3 * E * FF)
         at_flop = 4.0 * STAGE_LAYERS * H * HD * PREFILL_T * (PREFILL_T + 1) / 2
         gemm_ms = pprof["gemv"]["ms"]
+        # what the matrix pipes sustain from registers alone on this GPU (20 launches of ~15 ms each, median)
+        mp = m.mfma_f16_probe(20000, 2, 20)
+        mfma_probe = mp[len(mp) // 2]
         prefill = {"tokens": PREFILL_T, "ms": round(pms, 2), "tok_s": round(PREFILL_T * 1e3 / pms, 1),
                    "matmul_TFLOP": round(mm_flop / 1e12, 3), "attention_TFLOP": round(at_flop / 1e12, 3),
                    "stage_TFLOPs": round((mm_flop + at_flop) / pms / 1e9, 1),
                    "gemm_ms": round(gemm_ms, 2), "gemm_TFLOPs": round(mm_flop / gemm_ms / 1e9, 1),
                    "gemm_frac_mfma_f16_peak": round(mm_flop / gemm_ms / 1e9 / 2500.0, 4),
+                   "mfma_f16_probe_TFLOPs": round(mfma_probe, 1), "gemm_frac_of_mfma_probe": round(mm_flop / gemm_ms / 1e9 / mfma_probe, 4),
                    "kernel_ms": {k: round(v["ms"], 2) for k, v in pprof.items()}}
     b1 = results[batches[0]]
     # roofline of the dominant kernel (the dequant-fused GEMV): all of a step's weight bytes pass through its
@@ -292,6 +316,7 @@ def bench_stage(args):
     g_ms = b1["kernel_ms_per_step"]["gemv"]
     g_n = b1["kernel_launches_per_step"]["gemv"]
     gemv_gbs = weight_bytes / g_ms / 1e6
+    traffic_ratio = profiled_ratio(TRAFFIC_PROFILE, "gemv_batch1_traffic_over_algorithmic")
     codec = run_codec(torch, m, max(10, args.steps // 2), args.warmup)
     probe = hbm_probe(m)
     out = {
@@ -303,9 +328,10 @@ def bench_stage(args):
                    "weight_bytes": weight_bytes, "kv_bytes_per_seq": kv_bytes_per_seq},
         "roofline": {"bound": "hbm", "kernel": "gemv_dot_kernel<type,1,NU> (q4_K/q6_K dequant-fused mat-vec, all instantiations)",
                      "achieved": round(gemv_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gemv_gbs / HBM_PEAK_GBS, 4),
-                     # HBM bytes per average launch: rocprofv3 FETCH_SIZE (x2.0 calibration) + WRITE_SIZE of the gemv
-                     # launches, profiles/stage_decode_llama3_8b_l0_15_hbm_traffic.txt: 1.006 x algorithmic
-                     "traffic": int(round(1.006 * weight_bytes / g_n)), "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
+                     # HBM bytes per average launch: the ratio of counted (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated
+                     # on a copy of known size) to algorithmic bytes recorded in the committed profile summary
+                     "traffic": int(round(traffic_ratio * weight_bytes / g_n)) if traffic_ratio else None,
+                     "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic_ratio else None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
                      "algorithmic_bytes_per_launch": weight_bytes // g_n,
                      "measured_stream_read_GBps": probe, "frac_of_measured_p90": round(gemv_gbs / probe["p90"], 4)},
         "stage_frac_hbm": b1["frac_hbm"],
@@ -325,7 +351,7 @@ def bench_stage(args):
 SHAPES = {
     "c4": dict(model="qwen2.5-32b", layers=32, n_ctx=8192, batches=[1, 8, 32], prefill=4096, n_expert_local=None, kv="q8_0/q4_0",
                metric="stage decode tok/s @32B Q4_K_M, layers 0-31 of 64"),
-    "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=1024, n_expert_local=64, kv="q8_0/q4_0",
+    "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=1024, n_expert_local=64, kv="q8_0/q4_0", router="zipf",
                metric="expert-shard decode tok/s @Qwen3-30B-A3B Q4_K_M, 64 of 128 experts, batch 16"),
 }
 
@@ -344,7 +370,9 @@ def bench_shape(args):
     kv_row = {m.F16: HD_BYTES_F16, m.Q8_0: HD_BYTES_Q8_0, m.Q4_0: HD_BYTES_Q4_0}
     path = os.path.join(models.tmp_dir(), "mesh_bench_%s.gguf" % args.workload)
     t0 = time.perf_counter()
-    tensors = models.write_model(path, cfg, range(sp["layers"]), seed=42, fast=True, n_expert_local=sp["n_expert_local"])
+    zipf = sp.get("router") == "zipf"
+    tensors = models.write_model(path, cfg, range(sp["layers"]), seed=42, fast=True, n_expert_local=sp["n_expert_local"],
+                                 router=sp.get("router"))
     t_gen = time.perf_counter() - t0
     expert_bytes = sum(d.nbytes for n, (_, _, d) in tensors.items() if "_exps." in n)
     del tensors
@@ -382,7 +410,8 @@ def bench_shape(args):
     results = {}
     for B in batches:
         print("[bench] decode batch %d" % B, file=sys.stderr, flush=True)
-        x = torch.from_numpy(rng.standard_normal((B, E)).astype(np.float32)).cuda()
+        # router="zipf": the expert bias rides on a constant channel of the hidden state (tests/models.py)
+        x = torch.from_numpy(models.zipf_hidden_state(rng, B, E) if zipf else rng.standard_normal((B, E)).astype(np.float32)).cuda()
         out = torch.empty(m.act_packed_size(m.Q8_0, B, E), dtype=torch.uint8, device="cuda")
         pos = np.full(B, n_ctx - 1, np.int32)
         seq = np.arange(B, dtype=np.int32)
@@ -403,6 +432,14 @@ def bench_shape(args):
             ids = ses.moe_last_ids(B)
             distinct = int(np.unique(ids).size)
             r["distinct_experts_last_layer"] = distinct
+            if zipf:
+                # how much of the carrier channel's level survives 48 layers of residual updates
+                back = torch.empty(B * E, dtype=torch.float32, device="cuda")
+                m.act_unpack_dev(m.Q8_0, out.data_ptr(), back.data_ptr(), B * E, stream.cuda_stream)
+                stream.synchronize()
+                h = back.cpu().numpy().reshape(B, E)
+                r["carrier_channel_over_rms_in_out"] = [round(float(models.ZIPF_LEVEL / np.sqrt(((E - 1) + models.ZIPF_LEVEL ** 2) / E)), 3),
+                                                        round(float(np.mean(h[:, models.ZIPF_CHANNEL] / np.sqrt(np.mean(h * h, axis=1)))), 3)]
             step_bytes = (st.weight_bytes - expert_bytes) + expert_bytes * distinct / sp["n_expert_local"] + kv_bytes_per_seq * B
         else:
             step_bytes = st.weight_bytes + kv_bytes_per_seq * B

@@ -73,6 +73,13 @@ int mesh_hbm_read_probe(size_t bytes, int warmup_runs, int timed_runs, double *g
  * for kernels that write as well as read. */
 int mesh_hbm_mix_probe_dev(const void *d_src, void *d_dst, size_t big_bytes, int ratio, int big_is_read, void *stream);
 
+/* Sustained f16 matrix-core rate of the current GPU: `timed_runs` event-timed launches (after `warmup_runs` untimed
+ * ones) of a kernel in which every wave issues `iters` x 4 independent v_mfma_f32_32x32x16_f16 from registers, four
+ * waves per SIMD; TFLOP/s of each launch into tflops[timed_runs].  The yardstick for the prefill GEMM beside the
+ * nominal 2.5 PFLOP/s: it shows the clock the chip holds with the matrix pipes saturated.  No counterpart in the
+ * reference (its fingerprint benchmark, mesh-llm/benchmarks/membench-fingerprint.hip, measures memory only). */
+int mesh_mfma_f16_probe(int iters, int warmup_runs, int timed_runs, double *tflops);
+
 /* ---- boundary activation codec -------------------------------------------------------------------
  * The inter-stage hidden state [n_tokens, n_embd] f32, packed for transport.  Replaces the raw-f32
  * ggml_backend_tensor_get -> TCP -> ggml_backend_tensor_set hop of push_tensor_to_peer

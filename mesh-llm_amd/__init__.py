@@ -35,6 +35,7 @@ SIGNATURES = {
     "mesh_device_select": (_i32, [_cp]),
     "mesh_hbm_read_probe": (_i32, [_sz, _i32, _i32, _vp]),
     "mesh_hbm_mix_probe_dev": (_i32, [_vp, _vp, _sz, _i32, _i32, _vp]),
+    "mesh_mfma_f16_probe": (_i32, [_i32, _i32, _i32, _vp]),
     "mesh_act_packed_size": (_sz, [_i32, _i64, _i64]),
     "mesh_act_pack": (_i32, [_i32, _vp, _vp, _i64]),
     "mesh_act_unpack": (_i32, [_i32, _vp, _vp, _i64]),
@@ -151,6 +152,13 @@ def hbm_read_probe(nbytes=512 << 20, warmup=3, runs=20):
     """GB/s of `runs` streaming-read passes over a buffer of nbytes (mesh_hbm_read_probe), ascending."""
     out = (ctypes.c_double * runs)()
     check(lib().mesh_hbm_read_probe(nbytes, warmup, runs, out))
+    return sorted(out)
+
+
+def mfma_f16_probe(iters=4000, warmup=3, runs=20):
+    """TFLOP/s of `runs` launches of the register-only f16 matrix-core kernel (mesh_mfma_f16_probe), ascending."""
+    out = (ctypes.c_double * runs)()
+    check(lib().mesh_mfma_f16_probe(iters, warmup, runs, out))
     return sorted(out)
 
 

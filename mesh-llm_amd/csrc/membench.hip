@@ -52,6 +52,40 @@ __global__ __launch_bounds__(MB_THREADS) void memmix_kernel(const mb_u32x4 *__re
     }
 }
 
+// Matrix-core issue probe: every wave keeps four independent v_mfma_f32_32x32x16_f16 accumulation chains going from
+// registers alone (no memory traffic at all), four waves per SIMD.  What this sustains is what the matrix pipes deliver
+// at the clock the chip holds under that load, the yardstick beside the nominal 2.5 PFLOP/s for the prefill GEMM.
+typedef _Float16 mb_half8 __attribute__((ext_vector_type(8)));
+typedef float mb_float16 __attribute__((ext_vector_type(16)));
+constexpr int MFMA_PROBE_CHAINS = 4;
+__global__ __launch_bounds__(MB_THREADS) void mfma_probe_kernel(float *sink, int iters) {
+    // operands of mixed sign and magnitude below one, different in every lane, so the accumulators wander instead of running away
+    uint32_t h = (uint32_t)(blockIdx.x * MB_THREADS + threadIdx.x) * 2654435761u + 12345u;
+    mb_half8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        h = h * 1664525u + 1013904223u;
+        a[i] = (_Float16)(((int)(h >> 20) - 2048) * (1.0f / 2048.0f));
+        h = h * 1664525u + 1013904223u;
+        b[i] = (_Float16)(((int)(h >> 20) - 2048) * (1.0f / 2048.0f));
+    }
+    mb_float16 c[MFMA_PROBE_CHAINS];
+#pragma unroll
+    for (int k = 0; k < MFMA_PROBE_CHAINS; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) c[k][i] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int k = 0; k < MFMA_PROBE_CHAINS; ++k) c[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c[k], 0, 0, 0);
+    }
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < MFMA_PROBE_CHAINS; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t += c[k][i];
+    if (t == 123456.789f) sink[0] = t;       // keeps the chains alive; practically never true
+}
+
 }  // namespace mesh
 
 using namespace mesh;
@@ -114,4 +148,38 @@ extern "C" int mesh_hbm_mix_probe_dev(const void *d_src, void *d_dst, size_t big
     else MESH_LAUNCH((memmix_kernel<1, 4>), grid, block, 0, st, s, d);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
+}
+
+extern "C" int mesh_mfma_f16_probe(int iters, int warmup_runs, int timed_runs, double *tflops) {
+    if (iters < 1 || timed_runs < 1 || warmup_runs < 0 || !tflops) return fail(MESH_ERR_INVALID, "mesh_mfma_f16_probe: bad arguments");
+    float *sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto done = [&](int r) {
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+        if (sink) (void)hipFree(sink);
+        return r;
+    };
+#define MB_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return done(fail(MESH_ERR_DEVICE, "mesh_mfma_f16_probe: %s", hipGetErrorString(e_))); } while (0)
+    MB_TRY(hipMalloc(reinterpret_cast<void **>(&sink), sizeof(float)));
+    MB_TRY(hipEventCreate(&e0));
+    MB_TRY(hipEventCreate(&e1));
+    int dev = 0;
+    hipDeviceProp_t prop;
+    MB_TRY(hipGetDevice(&dev));
+    MB_TRY(hipGetDeviceProperties(&prop, dev));
+    const unsigned grid = (unsigned)prop.multiProcessorCount * 4;          // four 4-wave workgroups per CU: four waves per SIMD
+    const double flop = (double)grid * (MB_THREADS / 64) * (double)iters * MFMA_PROBE_CHAINS * (2.0 * 32 * 32 * 16);
+    for (int i = 0; i < warmup_runs + timed_runs; ++i) {
+        MB_TRY(hipEventRecord(e0, nullptr));
+        mfma_probe_kernel<<<dim3(grid), dim3(MB_THREADS), 0, nullptr>>>(sink, iters);
+        MB_TRY(hipGetLastError());
+        MB_TRY(hipEventRecord(e1, nullptr));
+        MB_TRY(hipEventSynchronize(e1));
+        float ms = 0.f;
+        MB_TRY(hipEventElapsedTime(&ms, e0, e1));
+        if (i >= warmup_runs) tflops[i - warmup_runs] = flop / ((double)ms * 1e-3) / 1e12;
+    }
+#undef MB_TRY
+    return done(MESH_OK);
 }
