@@ -204,11 +204,6 @@ int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const 
 /* The session's hipStream_t (for events), and a wait for everything queued on it. */
 void *mesh_session_stream(mesh_session *session);
 int mesh_session_synchronize(mesh_session *session);
-/* Number of decode steps of this session that ran through the persistent single-launch decode kernel (batches of up
- * to 4 single-token sequences on a dense K-quant stage with head_dim 128; environment MESH_STAGE_PERSISTENT=1 at
- * session creation turns that kernel on).  -1 for a null session.  No counterpart in the reference; it lets tests and
- * benchmarks tell which path produced a result. */
-int64_t mesh_session_persistent_steps(const mesh_session *session);
 /* Number of decode steps of this session whose layer launches were replayed from a captured HIP graph (batches of up to
  * 32 tokens, from the third call with the same token count and KV split count on; environment MESH_STAGE_GRAPHS=1 at
  * session creation turns graphs on: they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
@@ -247,6 +242,30 @@ int mesh_session_kv_write(mesh_session *session, int layer, int seq_id, int pos0
                           const uint16_t *k, const uint16_t *v);
 int mesh_session_kv_read(mesh_session *session, int layer, int seq_id, int pos0, int n_pos,
                          uint16_t *k, uint16_t *v);
+
+/* ---- single graph nodes ---------------------------------------------------------------------------
+ * The layer's activation producers and its decode attention on their own: the nodes rpc_server::graph_compute
+ * (patches/0002:443-451) runs between the mat-muls -- rms_norm + mul, swiglu, flash_attn_ext -- in the forms the
+ * batched paths of this library use.  Device pointers; queued on `stream` (the session's stream for attention). */
+
+/* y = quantise(rms_norm(x, eps) * w) for n_tokens rows of n floats (n a multiple of 32; w NULL: quantise(x)) in the
+ * "q16" activation layout of the batched decode GEMM: per block of 16 tokens 36 * n bytes = for every 8-element group g
+ * and token t a 16-byte record at (g * 16 + t) * 16 holding the high bytes of eight 16-bit fixed-point values, then their
+ * low bytes (value = (hi * 256 + lo) * d, lo and hi signed); at 32 * n the f32 scales d[(k / 32) * 16 + t] of the
+ * 32-element blocks (d = max|v| / 32512), at 34 * n the f32 block sums.  mesh_op_q16_bytes: bytes of that buffer. */
+size_t mesh_op_q16_bytes(int64_t n_tokens, int64_t n);
+int mesh_op_rms_norm_q16_dev(const float *d_x, const float *d_w, float eps, int64_t n_tokens, int64_t n, void *d_q16, void *stream);
+/* y = f16(rms_norm(x, eps) * w), saturating, in the "k8-major" layout of the prefill GEMM: blocks of 16 tokens, element
+ * (t, k) of block t / 16 at ((k / 8) * 16 + t % 16) * 8 + k % 8 within the block's 16 * n halfs; rows beyond n_tokens
+ * are zero.  d_y16 holds ceil(n_tokens / 16) * 16 * n halfs. */
+int mesh_op_rms_norm_f16k8_dev(const float *d_x, const float *d_w, float eps, int64_t n_tokens, int64_t n, void *d_y16, void *stream);
+/* y = f16(silu(gate) * up), saturating, same layout. */
+int mesh_op_swiglu_f16k8_dev(const float *d_gate, const float *d_up, int64_t n_tokens, int64_t n, void *d_y16, void *stream);
+/* Decode attention of one (absolute) layer over the session's KV cache: token i of the batch attends to positions
+ * [0, pos[i]] of its sequence; d_q holds already rotated queries [n_tokens][n_head][head_dim] f32, d_out receives
+ * [n_tokens][n_head][head_dim] f32.  matrix_cores != 0 picks the kernel the stage uses (queries and probabilities
+ * rounded to f16), 0 the all-f32 one.  Waits for the session's stream before it queues its own work. */
+int mesh_session_attn_dev(mesh_session *session, int layer, const float *d_q, const mesh_batch *batch, float *d_out, int matrix_cores);
 
 #ifdef __cplusplus
 }

@@ -102,7 +102,6 @@ SIGNATURES.update({
     "mesh_stage_decode_dev": (_i32, [_vp, ctypes.POINTER(Batch), _vp, _i32, _vp, _i32, _sz, _psz]),
     "mesh_session_stream": (_vp, [_vp]),
     "mesh_session_synchronize": (_i32, [_vp]),
-    "mesh_session_persistent_steps": (_i64, [_vp]),
     "mesh_session_graph_replays": (_i64, [_vp]),
     "mesh_session_profile": (_i32, [_vp, _i32]),
     "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
@@ -110,6 +109,11 @@ SIGNATURES.update({
     "mesh_session_moe_last_ids": (_i32, [_vp, _vp, _i32]),
     "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
+    "mesh_op_q16_bytes": (_sz, [_i64, _i64]),
+    "mesh_op_rms_norm_q16_dev": (_i32, [_vp, _vp, ctypes.c_float, _i64, _i64, _vp, _vp]),
+    "mesh_op_rms_norm_f16k8_dev": (_i32, [_vp, _vp, ctypes.c_float, _i64, _i64, _vp, _vp]),
+    "mesh_op_swiglu_f16k8_dev": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
+    "mesh_session_attn_dev": (_i32, [_vp, _i32, _vp, ctypes.POINTER(Batch), _vp, _i32]),
 })
 
 _lib = None
@@ -166,6 +170,22 @@ def hbm_mix_probe_dev(src_ptr, dst_ptr, big_bytes, ratio, big_is_read, stream=0)
     """Queue one plain streaming kernel that moves big_bytes on its larger side and big_bytes / ratio on the other
     (mesh_hbm_mix_probe_dev); device pointers, not waited for."""
     check(lib().mesh_hbm_mix_probe_dev(src_ptr, dst_ptr, big_bytes, ratio, int(bool(big_is_read)), stream))
+
+
+def op_q16_bytes(n_tokens, n):
+    return int(lib().mesh_op_q16_bytes(n_tokens, n))
+
+
+def op_rms_norm_q16_dev(x_ptr, w_ptr, eps, n_tokens, n, out_ptr, stream=0):
+    check(lib().mesh_op_rms_norm_q16_dev(x_ptr, w_ptr, eps, n_tokens, n, out_ptr, stream))
+
+
+def op_rms_norm_f16k8_dev(x_ptr, w_ptr, eps, n_tokens, n, out_ptr, stream=0):
+    check(lib().mesh_op_rms_norm_f16k8_dev(x_ptr, w_ptr, eps, n_tokens, n, out_ptr, stream))
+
+
+def op_swiglu_f16k8_dev(gate_ptr, up_ptr, n_tokens, n, out_ptr, stream=0):
+    check(lib().mesh_op_swiglu_f16k8_dev(gate_ptr, up_ptr, n_tokens, n, out_ptr, stream))
 
 
 def act_packed_size(fmt, n_tokens, n_embd):
@@ -346,10 +366,10 @@ class Session:
     def synchronize(self):
         check(lib().mesh_session_synchronize(self._h))
 
-    @property
-    def persistent_steps(self):
-        """Decode steps so far that ran through the persistent single-launch kernel."""
-        return int(lib().mesh_session_persistent_steps(self._h))
+    def attn_dev(self, layer, d_q, pos, d_out, seq=None, matrix_cores=True):
+        """Decode attention of one layer over this session's KV cache (mesh_session_attn_dev); device pointers."""
+        b, keep = self._batch(pos, seq)
+        check(lib().mesh_session_attn_dev(self._h, layer, d_q, ctypes.byref(b), d_out, 1 if matrix_cores else 0))
 
     @property
     def graph_replays(self):

@@ -160,11 +160,7 @@ void *mesh_session_stream(mesh_session *session) { return session ? static_cast<
 int mesh_session_synchronize(mesh_session *session) {
     if (!session) return fail(MESH_ERR_INVALID, "mesh_session_synchronize: null session");
     MESH_HIP_TRY(hipStreamSynchronize(session->stream));
-    return mega_check(session);
-}
-
-int64_t mesh_session_persistent_steps(const mesh_session *session) {
-    return session ? session->mega.steps : -1;
+    return MESH_OK;
 }
 
 int64_t mesh_session_graph_replays(const mesh_session *session) {

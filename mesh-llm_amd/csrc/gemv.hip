@@ -57,23 +57,6 @@ struct GemvKernelArgs {
     int kind[3];
 };
 
-// Phase timestamps for tuning builds (-DMESH_GEMV_TRACE); compiled out of the product.
-#ifdef MESH_GEMV_TRACE
-__device__ long long *g_gemv_trace = nullptr;
-__device__ int g_gemv_trace_sel = -1;      // -1: every launch; else only kernels with (GROUPED ? 1 : 0) | (NU == 2 ? 2 : 0) | (expert_ids ? 4 : 0) == sel
-extern "C" int mesh_debug_set_gemv_trace(long long *p, int sel) {
-    if (hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace_sel), &sel, sizeof sel) != hipSuccess) return -2;
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace), &p, sizeof p) == hipSuccess ? 0 : -2;
-}
-#define GEMV_MARK(k)                                                                              \
-    do {                                                                                          \
-        if (g_gemv_trace && (threadIdx.x & 63) == 0 &&                                            \
-            (g_gemv_trace_sel < 0 || g_gemv_trace_sel == ((GROUPED ? 1 : 0) | (NU == 2 ? 2 : 0) | (a.expert_ids ? 4 : 0))))    \
-            g_gemv_trace[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * WAVES + (threadIdx.x >> 6)) * 8 + (k)] = wall_clock64(); \
-    } while (0)
-#else
-#define GEMV_MARK(k) do { } while (0)
-#endif
 
 
 // rows per workgroup by division (kernels that do not get them from the host)

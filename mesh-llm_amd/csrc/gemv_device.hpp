@@ -1,6 +1,5 @@
-// Device-side building blocks of the dequant-fused GEMV, shared by the per-projection kernel (gemv.hip) and the
-// persistent decode kernel (decode_mega.hip): the 16-bit fixed-point activation staging in LDS, and the per-tile
-// integer dot products for q4_K / q6_K tiles.  See gemv.hip for the design notes.
+// Device-side building blocks of the dequant-fused GEMV (gemv.hip): the 16-bit fixed-point activation staging in LDS,
+// and the per-tile integer dot products for q4_K / q6_K tiles.  See gemv.hip for the design notes.
 #pragma once
 
 #include "gemv.hpp"

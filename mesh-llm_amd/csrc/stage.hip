@@ -17,7 +17,6 @@
 #include <mutex>
 
 #include "attn.hpp"
-#include "decode_mega.hpp"
 #include "gemm.hpp"
 #include "gemv.hpp"
 #include "moe.hpp"
@@ -306,179 +305,6 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
 static int sess_alloc(mesh_session *s, void **p, size_t bytes);
 static bool layer_is_kquant_dense(const LayerWeights &L);
 
-// ------------------------------------------------------------------------------------------------ persistent decode
-// Uncached device blocks are recycled through a process-wide list and never freed: memory allocated uncached must
-// not be released before the process ends once a kernel has read it.
-namespace {
-struct UncachedBlock { void *p; size_t bytes; int device; };
-std::mutex g_uncached_mu;
-std::vector<UncachedBlock> g_uncached_free;
-
-void *uncached_acquire(size_t bytes, int device) {
-    {
-        std::lock_guard<std::mutex> lk(g_uncached_mu);
-        for (size_t i = 0; i < g_uncached_free.size(); ++i)
-            if (g_uncached_free[i].device == device && g_uncached_free[i].bytes >= bytes) {
-                void *p = g_uncached_free[i].p;
-                g_uncached_free.erase(g_uncached_free.begin() + (long)i);
-                return p;
-            }
-    }
-    void *p = nullptr;
-    if (hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    return p;
-}
-void uncached_release(void *p, size_t bytes, int device) {
-    std::lock_guard<std::mutex> lk(g_uncached_mu);
-    g_uncached_free.push_back({p, bytes, device});
-}
-}  // namespace
-
-void mega_pool_release(void *p, size_t bytes, int device) { uncached_release(p, bytes, device); }
-
-// Reads the abort flag of the persistent kernel (after the stream has drained).  A set flag means a grid barrier
-// timed out: the step's output is invalid, and the session falls back to the per-projection kernels from then on.
-int mega_check(mesh_session *s) {
-    if (!s->mega.ready || s->mega.failed) return MESH_OK;
-    int flag = 0;
-    MESH_HIP_TRY(hipMemcpy(&flag, s->mega.abort_flag, sizeof flag, hipMemcpyDeviceToHost));
-    if (flag) {
-        s->mega.failed = true;
-        return fail(MESH_ERR_DEVICE, "persistent decode kernel: grid barrier timed out; the last step's output is invalid");
-    }
-    return MESH_OK;
-}
-
-static bool mega_eligible(const mesh_stage *st) {
-    const HParams &hp = st->hp;
-    const char *env = getenv("MESH_STAGE_PERSISTENT");       // opt-in while it is slower than the per-projection kernels
-    if (!env || env[0] != '1') return false;
-    if (hp.head_dim != 128 || hp.n_ff == 0 || hp.n_head_kv == 0 || hp.n_head % hp.n_head_kv) return false;
-    if (st->k_type != MESH_F16 || st->v_type != MESH_F16) return false;
-    if (!mega_group_supported((int)(hp.n_head / hp.n_head_kv))) return false;
-    const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, FF = hp.n_ff;
-    if (E % 256 || QD % 256 || FF % 256) return false;
-    for (const LayerWeights &L : st->layers) {
-        if (!layer_is_kquant_dense(L) || L.q_norm.present() || L.k_norm.present()) return false;
-        if (L.w_gate.type != L.w_up.type) return false;
-    }
-    return !st->layers.empty();
-}
-
-static int mega_setup(mesh_session *s) {
-    mesh_stage *st = s->stage;
-    if (!mega_eligible(st)) return MESH_OK;
-    const HParams &hp = st->hp;
-    hipDeviceProp_t prop;
-    MESH_HIP_TRY(hipGetDeviceProperties(&prop, st->device));
-    if (!prop.cooperativeLaunch) return MESH_OK;
-    const int grid = prop.multiProcessorCount;
-    const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
-    auto &m = s->mega;
-    const size_t nB = MEGA_BATCH_MAX;
-    size_t off = 0;
-    auto carve = [&](size_t floats) { const size_t o = off; off += (floats * 4 + 255) / 256 * 256; return o; };
-    // replica strides are not multiples of a large power of two, so the copies fall on different memory channels
-    const size_t xs = nB * E + 1088, as = nB * QD + 1088, fs = nB * FF + 1088;
-    const size_t o_x = carve(MEGA_REPLICAS * xs), o_q = carve(nB * QD), o_k = carve(nB * KD), o_v = carve(nB * KD), o_attn = carve(MEGA_REPLICAS * as),
-                 o_ffn = carve(MEGA_REPLICAS * fs), o_part = carve(nB * QD * MEGA_SPLITS_MAX), o_ml = carve(nB * hp.n_head * MEGA_SPLITS_MAX * 2),
-                 o_bar = carve(64);
-    m.pool_bytes = off;
-    m.pool = uncached_acquire(m.pool_bytes, st->device);
-    if (!m.pool) return MESH_OK;         // no uncached memory: stay on the per-projection kernels
-    uint8_t *base = static_cast<uint8_t *>(m.pool);
-    m.x = reinterpret_cast<float *>(base + o_x); m.q = reinterpret_cast<float *>(base + o_q);
-    m.k = reinterpret_cast<float *>(base + o_k); m.v = reinterpret_cast<float *>(base + o_v);
-    m.attn = reinterpret_cast<float *>(base + o_attn); m.ffn = reinterpret_cast<float *>(base + o_ffn);
-    m.part = reinterpret_cast<float *>(base + o_part); m.ml = reinterpret_cast<float *>(base + o_ml);
-    m.bar = reinterpret_cast<unsigned *>(base + o_bar);
-    m.abort_flag = reinterpret_cast<int *>(base + o_bar + 64);
-    MESH_HIP_TRY(hipMemsetAsync(m.pool, 0, m.pool_bytes, s->stream));
-    m.bar_value = 0;
-    std::vector<MegaLayer> tbl(st->layers.size());
-    for (size_t il = 0; il < st->layers.size(); ++il) {
-        const LayerWeights &L = st->layers[il];
-        MegaLayer &d = tbl[il];
-        memset(&d, 0, sizeof d);
-        auto w = [](const DevTensor &t) { return static_cast<const uint8_t *>(t.data); };
-        auto f = [](const DevTensor &t) { return t.present() ? static_cast<const float *>(t.data) : nullptr; };
-        MegaPhase &qkv = d.ph[0], &o = d.ph[1], &gu = d.ph[2], &dn = d.ph[3];
-        qkv.n_part = 3;
-        qkv.part[0] = MegaPart{w(L.wq), nullptr, L.wq.type, QD, 0, QD, m.q, f(L.bq), 1, 0};
-        qkv.part[1] = MegaPart{w(L.wk), nullptr, L.wk.type, KD, QD / TILE_ROWS, KD, m.k, f(L.bk), 1, 0};
-        qkv.part[2] = MegaPart{w(L.wv), nullptr, L.wv.type, KD, (QD + KD) / TILE_ROWS, KD, m.v, f(L.bv), 1, 0};
-        qkv.total_rows = (QD + 2 * KD) / TILE_ROWS;
-        qkv.x = m.x; qkv.x_rep_stride = xs; qkv.ldx = E; qkv.K = E; qkv.norm_w = f(L.attn_norm); qkv.epi = EPI_STORE;
-        o.n_part = 1;
-        o.part[0] = MegaPart{w(L.wo), nullptr, L.wo.type, E, 0, E, m.x, nullptr, MEGA_REPLICAS, xs};
-        o.total_rows = E / TILE_ROWS;
-        o.x = m.attn; o.x_rep_stride = as; o.ldx = QD; o.K = QD; o.norm_w = nullptr; o.epi = EPI_RESIDUAL;
-        gu.n_part = 1;
-        gu.part[0] = MegaPart{w(L.w_gate), w(L.w_up), L.w_gate.type, FF, 0, FF, m.ffn, nullptr, MEGA_REPLICAS, fs};
-        gu.total_rows = FF / TILE_ROWS;
-        gu.x = m.x; gu.x_rep_stride = xs; gu.ldx = E; gu.K = E; gu.norm_w = f(L.ffn_norm); gu.epi = EPI_SWIGLU;
-        dn.n_part = 1;
-        dn.part[0] = MegaPart{w(L.w_down), nullptr, L.w_down.type, E, 0, E, m.x, nullptr, MEGA_REPLICAS, xs};
-        dn.total_rows = E / TILE_ROWS;
-        dn.x = m.ffn; dn.x_rep_stride = fs; dn.ldx = FF; dn.K = FF; dn.norm_w = nullptr; dn.epi = EPI_RESIDUAL;
-        d.kc = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
-        d.vc = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
-    }
-    // widest batch whose LDS need fits one workgroup
-    const int group = (int)(hp.n_head / hp.n_head_kv);
-    m.max_batch = 0;
-    for (int nb = 1; nb <= MEGA_BATCH_MAX; nb *= 2) {
-        const size_t need = mega_smem_bytes(tbl[0], nb, group, grid);
-        if (need > 160 * 1024) break;          // LDS of one gfx950 CU
-        m.max_batch = nb;
-        m.smem[nb] = need;
-    }
-    if (m.max_batch == 0) return MESH_OK;
-    int rc = sess_alloc(s, &m.layers, tbl.size() * sizeof(MegaLayer));
-    if (rc != MESH_OK) return rc;
-    void *rope_tab = nullptr;
-    if ((rc = sess_alloc(s, &rope_tab, 2 * nB * 64 * sizeof(float))) != MESH_OK) return rc;
-    m.rope_cs = static_cast<float *>(rope_tab);
-    m.rope_sn = m.rope_cs + nB * 64;
-    m.x_rep_stride = xs;
-    m.attn_rep_stride = as;
-    MESH_HIP_TRY(hipMemcpy(m.layers, tbl.data(), tbl.size() * sizeof(MegaLayer), hipMemcpyHostToDevice));
-    m.grid = grid;
-    m.ready = true;
-    return MESH_OK;
-}
-
-// One decode step of T <= 4 single-token sequences through the persistent kernel.  The input is already unpacked
-// into mega.x; the result is left there.
-static int mega_step(mesh_session *s, int T, int max_keys) {
-    mesh_stage *st = s->stage;
-    const HParams &hp = st->hp;
-    auto &m = s->mega;
-    MegaArgs ma{};
-    ma.layers = static_cast<const MegaLayer *>(m.layers);
-    ma.n_layers = (int)st->layers.size();
-    ma.B = T;
-    ma.E = (int)hp.n_embd;
-    ma.n_head = (int)hp.n_head; ma.n_kv = (int)hp.n_head_kv; ma.group = (int)(hp.n_head / hp.n_head_kv);
-    ma.n_rot = (int)hp.n_rot; ma.rope_mode = (int)hp.rope_mode; ma.n_ctx = st->n_ctx;
-    int ns = 1;
-    while (ns * 2 <= MEGA_SPLITS_MAX && T * ma.n_kv * ns * 2 <= m.grid && ns * 2 * 32 <= max_keys) ns *= 2;
-    ma.n_splits = ns;
-    ma.eps = hp.rms_eps; ma.attn_scale = 1.0f / sqrtf((float)hp.head_dim);
-    ma.x = m.x; ma.x_rep_stride = m.x_rep_stride; ma.attn_rep_stride = m.attn_rep_stride;
-    ma.q = m.q; ma.k = m.k; ma.v = m.v; ma.attn = m.attn; ma.part = m.part; ma.ml = m.ml;
-    ma.rope_cs = m.rope_cs; ma.rope_sn = m.rope_sn;
-    ma.pos = s->d_pos; ma.seq = s->d_seq; ma.inv_freq = st->rope_inv_freq;
-    ma.bar = m.bar; ma.bar_base = m.bar_value; ma.abort_flag = m.abort_flag;
-    ma.spin_limit = 400000;
-    const int nb = T <= 1 ? 1 : T <= 2 ? 2 : 4;
-    int rc = decode_mega(ma, m.grid, m.smem[nb], s->stream);
-    if (rc != MESH_OK) return rc;
-    m.bar_value += (unsigned)mega_barriers_per_launch(ma.n_layers) * (unsigned)m.grid;
-    ++m.steps;
-    return MESH_OK;
-}
-
 // ------------------------------------------------------------------------------------------------ session
 static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
     hipError_t e = hipMalloc(p, bytes ? bytes : 16);
@@ -600,7 +426,6 @@ int session_new(mesh_stage *st, mesh_session **out) {
     s->io_out_bytes = std::max(s->io_stage_bytes, st->output.present() ? std::min<size_t>(B, LOGITS_TOKENS_MAX) * (size_t)st->output.M * sizeof(float) : 0);
     if ((rc = sess_alloc(s.get(), &s->io_stage, s->io_stage_bytes + s->io_out_bytes)) != MESH_OK) return rc;
     MESH_HIP_TRY(hipHostMalloc(&s->h_io, s->io_stage_bytes + s->io_out_bytes, hipHostMallocDefault));
-    if ((rc = mega_setup(s.get())) != MESH_OK) return rc;
     MESH_HIP_TRY(hipStreamSynchronize(s->stream));
     *out = s.release();
     return MESH_OK;
@@ -1164,16 +989,6 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
         // embedding rows: one dequantize per token (ids are read on the host side by the caller's contract)
         return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_decode_dev: token input is only available through the host-pointer entry point");
     }
-    // a batch of single-token sequences goes through the persistent kernel when the stage qualifies
-    bool use_mega = s->mega.ready && !s->mega.failed && !s->profile && T <= s->mega.max_batch && !logits_out;
-    for (int i = 0; use_mega && i < T; ++i)
-        for (int j = 0; j < i; ++j)
-            if ((b->seq_id ? b->seq_id[i] : 0) == (b->seq_id ? b->seq_id[j] : 0)) use_mega = false;
-    if (use_mega) {
-        if ((rc = act_unpack_dev(in_fmt, d_in, s->mega.x, (int64_t)T * hp.n_embd, stream)) != MESH_OK) return rc;
-        if (mega_step(s, T, max_keys) == MESH_OK) return act_pack_dev(out_fmt, s->mega.x, d_out, (int64_t)T * hp.n_embd, stream);
-        s->mega.failed = true;       // the launch was refused (nothing ran): use the per-projection kernels from now on
-    }
     { ProfScope ps(s, MESH_PROF_CODEC); rc = act_unpack_dev(in_fmt, d_in, s->x, (int64_t)T * hp.n_embd, stream); }
     if (rc != MESH_OK) return rc;
     if ((rc = run_layers_graphed(s, T, max_keys)) != MESH_OK) return rc;
@@ -1232,9 +1047,45 @@ int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fm
     uint8_t *h_out = static_cast<uint8_t *>(s->h_io) + s->io_stage_bytes;
     MESH_HIP_TRY(hipMemcpyAsync(h_out, d_out, len, hipMemcpyDeviceToHost, stream));
     MESH_HIP_TRY(hipStreamSynchronize(stream));
-    if ((rc = mega_check(s)) != MESH_OK) return rc;
     memcpy(out, h_out, len);
     return MESH_OK;
+}
+
+// ---- single graph nodes -------------------------------------------------------------------------
+// Decode attention of one layer over the session's KV cache, for callers that bring their own (already rotated) queries.
+int session_attention(mesh_session *s, int layer, const float *d_q, const mesh_batch *b, float *d_out, int matrix_cores) {
+    const mesh_stage *st = s->stage;
+    const HParams &hp = st->hp;
+    const int il = layer - st->layer_begin;
+    if (il < 0 || il >= (int)st->layers.size()) return fail(MESH_ERR_INVALID, "mesh_session_attn_dev: layer %d is not in this stage", layer);
+    const int T = b->n_tokens;
+    if (T < 1 || T > st->n_batch_max || !b->pos) return fail(MESH_ERR_INVALID, "mesh_session_attn_dev: bad batch");
+    int max_keys = 0;
+    std::vector<int32_t> seq((size_t)T, 0);
+    for (int i = 0; i < T; ++i) {
+        if (b->seq_id) seq[i] = b->seq_id[i];
+        if (b->pos[i] < 0 || b->pos[i] >= st->n_ctx || seq[i] < 0 || seq[i] >= st->n_seq_max)
+            return fail(MESH_ERR_INVALID, "mesh_session_attn_dev: token %d has position %d / sequence %d outside the cache", i, b->pos[i], seq[i]);
+        max_keys = std::max(max_keys, b->pos[i] + 1);
+    }
+    MESH_HIP_TRY(hipStreamSynchronize(s->stream));
+    MESH_HIP_TRY(hipMemcpy(s->d_pos, b->pos, (size_t)T * sizeof(int32_t), hipMemcpyHostToDevice));
+    MESH_HIP_TRY(hipMemcpy(s->d_seq, seq.data(), (size_t)T * sizeof(int32_t), hipMemcpyHostToDevice));
+    AttnArgs aa;
+    aa.q = d_q;
+    aa.kcache = s->kcache + il * s->k_layer_bytes;
+    aa.vcache = s->vcache + il * s->v_layer_bytes;
+    aa.k_type = st->k_type; aa.v_type = st->v_type; aa.pos = s->d_pos; aa.seq = s->d_seq;
+    aa.part = s->attn_part; aa.ml = s->attn_ml; aa.out = d_out;
+    aa.scale = 1.0f / sqrtf((float)hp.head_dim);
+    aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
+    aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
+    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;
+    if (matrix_cores) {
+        if (!attention_mma_supported(aa)) return fail(MESH_ERR_UNSUPPORTED, "mesh_session_attn_dev: the matrix-core kernel does not cover this shape");
+        return attention_mma(aa, T, s->stream);
+    }
+    return attention(aa, T, s->stream);
 }
 
 }  // namespace mesh
@@ -1247,7 +1098,6 @@ mesh_session::~mesh_session() {
     if (stream) (void)hipStreamSynchronize(stream);
     for (hipEvent_t e : prof_events) (void)hipEventDestroy(e);
     for (void *p : allocations) (void)hipFree(p);
-    if (mega.pool && stage) mesh::mega_pool_release(mega.pool, mega.pool_bytes, stage->device);
     for (auto &kv : graphs)
         if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
     if (h_meta) (void)hipHostFree(h_meta);

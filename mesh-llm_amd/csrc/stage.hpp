@@ -56,8 +56,7 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
 int session_new(mesh_stage *st, mesh_session **out);
 int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fmt, void *out, int out_fmt, size_t out_cap, size_t *out_len);
 int profile_collect(mesh_session *s);
-int mega_check(mesh_session *s);
-void mega_pool_release(void *p, size_t bytes, int device);
+int session_attention(mesh_session *s, int layer, const float *d_q, const mesh_batch *b, float *d_out, int matrix_cores);
 int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int in_fmt, void *d_out, int out_fmt, size_t out_cap, size_t *out_len);
 }  // namespace mesh
 
@@ -109,24 +108,6 @@ struct mesh_session {
     int attn_splits_max = 0;
     // set per call: the batch is one run of consecutive positions of one sequence (first position, sequence), else -1
     int chunk_pos0 = -1, chunk_seq = -1;
-    // persistent decode kernel (decode_mega.hip): exchange buffers in uncached device memory, per-layer table
-    struct Mega {
-        bool ready = false;
-        void *pool = nullptr;             // one uncached block, returned to a process-wide free list, never hipFree'd
-        size_t pool_bytes = 0;
-        float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr, *part = nullptr, *ml = nullptr;
-        float *rope_cs = nullptr, *rope_sn = nullptr;   // ordinary device memory
-        size_t x_rep_stride = 0, attn_rep_stride = 0;
-        unsigned *bar = nullptr;
-        int *abort_flag = nullptr;
-        void *layers = nullptr;           // device array of MegaLayer
-        unsigned bar_value = 0;           // counter value once every queued launch has finished
-        int grid = 0;
-        int max_batch = 0;                // widest batch (1, 2 or 4 columns) whose LDS need fits
-        size_t smem[5] = {0, 0, 0, 0, 0}; // LDS bytes per column count
-        bool failed = false;
-        int64_t steps = 0;                // decode steps that went through the persistent kernel
-    } mega;
     std::vector<void *> allocations;
     // optional per-kernel-class timing (HIP events on `stream` around every launch group)
     bool profile = false;

@@ -94,7 +94,7 @@ CONFIGS = {
     "tiny-qwen2": dict(arch="qwen2", n_layer=3, n_embd=512, n_head=4, n_head_kv=1, head_dim=128, n_ff=768, n_vocab=768, eps=1e-6, rope=1e6, bias=True, tied=True),
     "tiny-qwen3": dict(arch="qwen3", n_layer=2, n_embd=256, n_head=8, n_head_kv=4, head_dim=64, n_ff=768, n_vocab=256, eps=1e-6, rope=1e6, qk_norm=True),
     "tiny-moe": dict(arch="qwen3moe", n_layer=2, n_embd=512, n_head=4, n_head_kv=2, head_dim=128, n_ff=0, n_vocab=256, eps=1e-6, rope=1e6, n_expert=8, n_expert_used=2, n_ff_exp=256, qk_norm=True),
-    # head_dim 128 shapes for the persistent decode kernel: query heads per KV head 5, 8, 2 and 7
+    # head_dim 128 shapes with 5, 8, 2 and 7 query heads per KV head
     "tiny-g5": dict(arch="qwen2", n_layer=2, n_embd=1280, n_head=10, n_head_kv=2, head_dim=128, n_ff=1536, n_vocab=256, eps=1e-6, rope=1e6, bias=True),
     "tiny-g8": dict(arch="llama", n_layer=2, n_embd=1024, n_head=8, n_head_kv=1, head_dim=128, n_ff=1024, n_vocab=256, eps=1e-5, rope=5e5),
     "tiny-g2": dict(arch="llama", n_layer=2, n_embd=512, n_head=4, n_head_kv=2, head_dim=128, n_ff=512, n_vocab=256, eps=1e-5, rope=1e4),
