@@ -5,6 +5,8 @@
 
 namespace mesh {
 
+constexpr int SKINNY_ITEM_PAIRS = 16;      // pairs per work item of an expert launch of the skinny GEMM: one MFMA's columns
+
 struct GemmArgs {
     const void *W = nullptr;         // tiled q4_K / q6_K matrix [M][K]
     const void *Wp = nullptr;        // optional: the same matrix in the GEMM layout (gemm_pack); used instead of W when set
@@ -80,6 +82,13 @@ struct SkinnyArgs {
     // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+    // Expert launch (mixture of experts): mat[] describe expert 0 of stacked, equally shaped tiled matrices; work
+    // item i (blockIdx.y) = {expert, n, pair[0..n)} in the grouping kernel's format with SKINNY_ITEM_PAIRS pairs per item
+    // (moe.hpp); slot j of an item reads activation column pair[j] / x_div of xq (any block of 16) and writes output row
+    // pair[j].  One matrix or a gate / up pair (EPI_SWIGLU); T is not used.
+    const int32_t *items = nullptr, *n_items = nullptr;
+    int max_items = 0;
+    int x_div = 1;
 };
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
 // Bytes of one 16-token block of the q16 layout for rows of K elements.

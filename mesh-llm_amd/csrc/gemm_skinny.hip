@@ -44,6 +44,7 @@ constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B
 constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA M)
 constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
+constexpr int SK_ITEM_INTS = (2 + SKINNY_ITEM_PAIRS + 3) / 4 * 4;   // expert, n, pairs, padded to a multiple of 4 (moe_item_ints)
 
 typedef int i4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -62,36 +63,68 @@ struct SkinnyKernelArgs {
     int ks;                       // waves along K
     GemvRope rope;                // rope.pos / rope.seq point at the launch's first column
     int kind[3];
+    // expert launches: blockIdx.y = work item {expert, n, pair[0..n)} of SK_ITEM_INTS int32 (n <= 16 pairs of one expert);
+    // the matrices are that expert's (expert_stride bytes apart), slot j's activation column is pair[j] / x_div and its
+    // output row pair[j]
+    const int32_t *items, *n_items;
+    size_t expert_stride;
+    int x_div;
 };
 
 __device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) { return (long)(((unsigned long long)hi << 32) | lo); }
 
+// Where a lane finds its activations.  Plain launches: token column m = lane % 16 of the launch's block of 16.  Expert
+// launches (mixture of experts): the column is whatever (token or pair) the work item lists for slot m, in whichever block
+// of 16 it lives, so every lane carries its own base pointers.
+struct XSrc {
+    const uint4 *pl;        // record (k-group g, own column), super-block 0
+    const float *dxa, *dxb; // block-scale entries this lane fetches for the wave's table: block lane / 8, slots 2 (lane % 8) and + 1
+    const float *sx;        // block sum (block 0, own column)
+    __device__ __forceinline__ static XSrc plain(const uint8_t *xq, int K, int lane) {
+        XSrc x;
+        x.pl = reinterpret_cast<const uint4 *>(xq) + (lane >> 4) * 16 + (lane & 15);
+        x.dxa = reinterpret_cast<const float *>(xq + (size_t)K * 32) + 2 * lane;
+        x.dxb = x.dxa + 1;
+        x.sx = reinterpret_cast<const float *>(xq + (size_t)K * 34) + (lane & 15);
+        return x;
+    }
+    // col: this lane's column (slot lane % 16 of the item); cola / colb: the columns of slots 2 (lane % 8) and + 1
+    __device__ __forceinline__ static XSrc gathered(const uint8_t *xq, int K, int lane, int col, int cola, int colb) {
+        const size_t bb = (size_t)K * 36;
+        XSrc x;
+        const uint8_t *blk = xq + (size_t)(col >> 4) * bb;
+        x.pl = reinterpret_cast<const uint4 *>(blk) + (lane >> 4) * 16 + (col & 15);
+        x.sx = reinterpret_cast<const float *>(blk + (size_t)K * 34) + (col & 15);
+        x.dxa = reinterpret_cast<const float *>(xq + (size_t)(cola >> 4) * bb + (size_t)K * 32) + (lane >> 3) * 16 + (cola & 15);
+        x.dxb = reinterpret_cast<const float *>(xq + (size_t)(colb >> 4) * bb + (size_t)K * 32) + (lane >> 3) * 16 + (colb & 15);
+        return x;
+    }
+};
+
 // A operands (activation planes) of one super-block for this lane, the same for both weight types: 32-element block s,
-// elements 32s + 8g .. + 7 of token m as {hi8 (x, y), lo8 (z, w)}.  The block scales take a detour through a wave-private
-// LDS table ([8 blocks][16 tokens] f32, two of them): a lane needs those of four tokens for every block -- 32 registers
-// per super-block if kept in registers -- but the table is only 128 floats, one 8-byte load per lane.
+// elements 32s + 8g .. + 7 of the lane's column as {hi8 (x, y), lo8 (z, w)}.  The block scales take a detour through a
+// wave-private LDS table ([8 blocks][16 slots] f32, two of them): a lane needs those of four columns for every block -- 32
+// registers per super-block if kept in registers -- but the table is only 128 floats, two entries per lane.
 struct XFrags {
     uint4 p[8];
     float2 dxpre;      // this lane's two entries of the super-block's scale table
-    float sxa, sxb;    // q4_K: block sums of token m, blocks g and g + 4 (operands of the minimum-term MFMAs)
-    __device__ __forceinline__ const uint4 *planes(const uint8_t *xq, int sb, int lane) const {
-        return reinterpret_cast<const uint4 *>(xq) + ((size_t)sb * 32 + (lane >> 4)) * 16 + (lane & 15);
-    }
-    template <bool SUMS>
-    __device__ __forceinline__ void load_scales(const uint8_t *xq, int K, int sb, int lane) {
-        dxpre = ldg<float2>(reinterpret_cast<const float *>(xq + (size_t)K * 32) + (size_t)sb * 128 + 2 * lane);
+    float sxa, sxb;    // q4_K: block sums of the lane's column, blocks g and g + 4 (operands of the minimum-term MFMAs)
+    template <bool SUMS, bool GATHER>
+    __device__ __forceinline__ void load(const XSrc &x, int sb, int lane) {
+        const uint4 *pl = x.pl + (size_t)sb * 512;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) p[s] = ldg<uint4>(pl + s * 64);
+        if (GATHER) {
+            dxpre.x = ldg<float>(x.dxa + (size_t)sb * 128);
+            dxpre.y = ldg<float>(x.dxb + (size_t)sb * 128);
+        } else {
+            dxpre = ldg<float2>(x.dxa + (size_t)sb * 128);
+        }
         if (SUMS) {
-            const float *sxp = reinterpret_cast<const float *>(xq + (size_t)K * 34) + (size_t)sb * 128 + (lane & 15);
+            const float *sxp = x.sx + (size_t)sb * 128;
             sxa = ldg<float>(sxp + (lane >> 4) * 16);
             sxb = ldg<float>(sxp + ((lane >> 4) + 4) * 16);
         }
-    }
-    template <bool SUMS>
-    __device__ __forceinline__ void load(const uint8_t *xq, int K, int sb, int lane) {
-        const uint4 *pl = planes(xq, sb, lane);
-#pragma unroll
-        for (int s = 0; s < 8; ++s) p[s] = ldg<uint4>(pl + s * 64);
-        load_scales<SUMS>(xq, K, sb, lane);
     }
 };
 
@@ -222,7 +255,7 @@ __device__ __forceinline__ void tile_mac(const TileView<MESH_Q6_K> &V, const XFr
     }
 }
 
-template <int TYPE, int NU, int SEGS>
+template <int TYPE, int NU, int SEGS, bool GROUPED>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
                                                                  int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
                                                                  const SkinnyKernelArgs a) {
@@ -230,6 +263,22 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
     // << 16; p_split = tile-rows per workgroup | workgroups with one more << 16, computed on the host: no division and
     // no grid-size load stand before the first weight load)
     const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
+    // expert launches: this workgroup's item; workgroups past the item count have nothing to do
+    int it_n = SK_NT, it_pair = 0;
+    if (GROUPED) {
+        // item count and item are fetched together (the item buffer holds max_items entries, so the read is in bounds even
+        // for a workgroup past the count): one memory round trip before the first weight load instead of two
+        const int32_t *it = a.items + (size_t)blockIdx.y * SK_ITEM_INTS;
+        const int n_live = ldg<int>(a.n_items);
+        const int2 head = ldg<int2>(reinterpret_cast<const int2 *>(it));
+        const int slot_l = (int)(threadIdx.x & 15);
+        const int p_mine = ldg<int>(it + 2 + slot_l), p_first = ldg<int>(it + 2);
+        if ((int)blockIdx.y >= n_live) return;
+        const size_t eoff = (size_t)head.x * a.expert_stride;
+        p_w0 += eoff; p_w1 += eoff; p_w2 += eoff;
+        it_n = head.y;
+        it_pair = slot_l < it_n ? p_mine : p_first;              // unused slots repeat slot 0: computed, never stored
+    }
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int TB = TileRegs<TYPE>::BYTES;
     constexpr int SLOT = ((TYPE == MESH_Q4_K ? LDS_TILE_Q4 : LDS_TILE_Q6) + 255) / 256 * 256;
@@ -266,6 +315,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
     // segment has nothing at all
     const int total = seg_valid(0) ? n_i * SEGS : 0;
 
+    XSrc xs;
+    if (GROUPED) {
+        const int col = it_pair / a.x_div;
+        xs = XSrc::gathered(p_xq, K, lane, col, __shfl(col, 2 * (lane & 7)), __shfl(col, 2 * (lane & 7) + 1));
+    } else {
+        xs = XSrc::plain(p_xq, K, lane);
+    }
     TileRegs<TYPE> ring[SK_DEPTH];
     XFrags X[2];
     f4_t D[SEGS];
@@ -292,8 +348,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
         // in the loop below is therefore for something issued at least two super-blocks earlier: activations are
         // fetched two super-blocks ahead, BEFORE the weight tile issued in the same iteration, and a weight tile is
         // consumed SK_DEPTH - 1 iterations after its load was issued.
-        X[0].template load<SUMS>(p_xq, K, sb_of(0), lane);
-        X[1].template load<SUMS>(p_xq, K, sb_of(1), lane);
+        X[0].template load<SUMS, GROUPED>(xs, sb_of(0), lane);
+        X[1].template load<SUMS, GROUPED>(xs, sb_of(1), lane);
 #pragma unroll
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
         constexpr int RB0 = SEGS >= SK_DEPTH ? 1 : SK_DEPTH / SEGS;
@@ -313,7 +369,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
                 if (seg == 0) publish(X[r % 2], r % 2);
                 if (ii < n_i && seg_valid(seg)) tile_mac(cur, X[r % 2], dxt + (r % 2) * 128, lane, D[seg]);
                 // last segment of a super-block: its activation buffer is free for the one after next
-                if (seg == SEGS - 1) X[r % 2].template load<SUMS>(p_xq, K, sb_of(ii + 2), lane);
+                if (seg == SEGS - 1) X[r % 2].template load<SUMS, GROUPED>(xs, sb_of(ii + 2), lane);
                 load_tile(ring[(q + 1) % SK_DEPTH], f + 1 + SK_DEPTH, (q + 1 + SK_DEPTH) % SEGS);
                 cur = nxt;
                 __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
@@ -335,7 +391,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
     // outputs of this workgroup: rows_here x 16 rows x T columns
     for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
-        if (t >= a.T) continue;
+        if (t >= (GROUPED ? it_n : a.T)) continue;
+        // output row of column t: the token itself, or the pair the item lists for this slot
+        const size_t orow = GROUPED ? (size_t)a.items[(size_t)blockIdx.y * SK_ITEM_INTS + 2 + t] : (size_t)t;
         const int tr = tr0 + j;
         int mi = 0;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
@@ -347,7 +405,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
             if (NU == 2) s1 += red[((((size_t)k2 * rows_here + j) * NU + 1) * 16 + r) * 16 + t];
         }
         if (a.bias[mi]) s0 += a.bias[mi][row];
-        if (NU == 1 && a.rope.pos && a.kind[mi] != GEMV_KIND_PLAIN) {
+        if (!GROUPED && NU == 1 && a.rope.pos && a.kind[mi] != GEMV_KIND_PLAIN) {
             // q / k / v row of a token (see gemv.hpp): rotate q and k with the neighbouring row, k and v go to the cache
             const int kind = a.kind[mi], hd = a.rope.head_dim;
             const int head = row / hd, dd = row - head * hd;
@@ -374,23 +432,23 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
             if (a.bias[1]) s1 += a.bias[1][row];
             out = (s0 / (1.0f + expf(-s0))) * s1;
         } else if (a.epi == EPI_RESIDUAL) {
-            out = a.residual[(size_t)t * a.ldres + row] + s0;
+            out = a.residual[orow * a.ldres + row] + s0;
         } else {
             out = s0;
         }
-        a.y[mi][(size_t)t * a.ldy[mi] + row] = out;
+        a.y[mi][orow * a.ldy[mi] + row] = out;
     }
 }
 
-template <int TYPE, int NU, int SEGS>
-static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, size_t smem, hipStream_t stream) {
+template <int TYPE, int NU, int SEGS, bool GROUPED>
+static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, int grid_y, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_kernel<TYPE, NU, SEGS>),
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_kernel<TYPE, NU, SEGS, GROUPED>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    MESH_LAUNCH((gemm_skinny_kernel<TYPE, NU, SEGS>), dim3((unsigned)grid), dim3(SK_THREADS), smem, stream, 
+    MESH_LAUNCH((gemm_skinny_kernel<TYPE, NU, SEGS, GROUPED>), dim3((unsigned)grid, (unsigned)grid_y), dim3(SK_THREADS), smem, stream, 
         xq, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks, ka.tile_begin[3],
         (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
     MESH_LAUNCH_CHECK();
@@ -398,10 +456,14 @@ static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid
 }
 
 template <int TYPE, int NU>
-static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, size_t smem, hipStream_t stream) {
-    if (segs <= 1) return launch_skinny<TYPE, NU, NU>(ka, xq, grid, smem, stream);       // NU == 2 needs two segments at least
-    if (segs <= 2) return launch_skinny<TYPE, NU, 2>(ka, xq, grid, smem, stream);
-    return launch_skinny<TYPE, NU, 4>(ka, xq, grid, smem, stream);
+static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, int grid_y, size_t smem, hipStream_t stream) {
+    if (ka.items) {
+        if (segs <= 2) return launch_skinny<TYPE, NU, 2, true>(ka, xq, grid, grid_y, smem, stream);
+        return launch_skinny<TYPE, NU, 4, true>(ka, xq, grid, grid_y, smem, stream);
+    }
+    if (segs <= 1) return launch_skinny<TYPE, NU, NU, false>(ka, xq, grid, 1, smem, stream);       // NU == 2 needs two segments at least
+    if (segs <= 2) return launch_skinny<TYPE, NU, 2, false>(ka, xq, grid, 1, smem, stream);
+    return launch_skinny<TYPE, NU, 4, false>(ka, xq, grid, 1, smem, stream);
 }
 
 static int skinny_n_cu() {
@@ -441,14 +503,18 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     ka.K = a.K;
     ka.ldres = a.ldres; ka.epi = a.epi;
     ka.rope = a.rope;
+    const bool grouped = a.items != nullptr;
+    ka.items = a.items; ka.n_items = a.n_items; ka.expert_stride = (size_t)tiled_bytes(type, a.mat[0].M, a.K); ka.x_div = a.x_div > 0 ? a.x_div : 1;
     int KS = 1;
-    while (KS * 2 <= nsb && KS * 2 <= SK_WAVES) KS *= 2;      // a power of two: the kernel splits its waves with shifts
+    // a power of two: the kernel splits its waves with shifts.  Expert matrices are short in K (a few super-blocks), so
+    // their waves go along the rows instead and each still walks several super-blocks
+    while (KS * 2 <= nsb && KS * 2 <= (grouped ? 2 : SK_WAVES)) KS *= 2;
     const int RS = SK_WAVES / KS;
     ka.ks = KS;
     // tile-rows per workgroup: spread over the CUs, bounded by the segments a wave can hold
     const int rows_cap = std::max(1, SK_SEGS_MAX / NU) * RS;
     const int ncu = skinny_n_cu();
-    int rows_per_wg = std::min((total_rows + ncu - 1) / ncu, rows_cap);
+    int rows_per_wg = grouped ? rows_cap : std::min((total_rows + ncu - 1) / ncu, rows_cap);     // expert launches have many items: few, long workgroups each
     rows_per_wg = std::max(1, rows_per_wg);
     const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
     const int rows_max = (total_rows + grid - 1) / grid;
@@ -458,6 +524,11 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     const int lds_tile = ((type == MESH_Q4_K ? LDS_TILE_Q4 : LDS_TILE_Q6) + 255) / 256 * 256;
     const size_t smem = (size_t)SK_WAVES * (lds_tile + 2 * 512) + sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
     if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %zu bytes of LDS needed", smem);
+    if (grouped) {
+        ka.T = SK_NT;
+        if (type == MESH_Q4_K) return NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, ka, a.xq, grid, a.max_items, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, ka, a.xq, grid, a.max_items, smem, stream);
+        return NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, ka, a.xq, grid, a.max_items, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, ka, a.xq, grid, a.max_items, smem, stream);
+    }
     for (int t = 0; t < a.T; t += SK_NT) {
         SkinnyKernelArgs kb = ka;
         kb.T = std::min(SK_NT, a.T - t);
@@ -467,8 +538,8 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
         for (int i = 0; i < a.n_mat; ++i)
             if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
         int rc;
-        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, xq, grid, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, xq, grid, smem, stream);
-        else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, xq, grid, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, xq, grid, smem, stream);
+        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, xq, grid, 1, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, xq, grid, 1, smem, stream);
+        else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, xq, grid, 1, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, xq, grid, 1, smem, stream);
         if (rc != MESH_OK) return rc;
     }
     return MESH_OK;
@@ -683,6 +754,11 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
         return fail(MESH_ERR_INVALID, "gemm_skinny: SwiGLU needs a gate and an up matrix of equal shape and type");
     if (a.epi == EPI_RESIDUAL && !a.residual) return fail(MESH_ERR_INVALID, "gemm_skinny: residual epilogue without residual");
     if (a.rope.pos && (a.epi != EPI_STORE || a.rope.head_dim % 2 || a.rope.n_rot % 2)) return fail(MESH_ERR_INVALID, "gemm_skinny: rope epilogue needs a plain store");
+    if (a.items) {
+        bool ok = a.n_items && a.max_items >= 1 && a.max_items <= 65535 && !a.rope.pos && a.epi != EPI_RESIDUAL && a.n_mat <= 2;
+        for (int i = 1; i < a.n_mat; ++i) ok = ok && a.mat[i].type == a.mat[0].type && a.mat[i].M == a.mat[0].M;
+        if (!ok) return fail(MESH_ERR_INVALID, "gemm_skinny: an expert launch takes one matrix or a gate / up pair of one type, no rope, no residual");
+    }
     for (int i = 0; i < a.n_mat; ++i) {
         if (!a.mat[i].W || a.mat[i].M <= 0 || !type_is_tiled(a.mat[i].type)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d is not a tiled K-quant", i);
         if (!a.mat[i].y && !(i == 1 && a.epi == EPI_SWIGLU)) return fail(MESH_ERR_INVALID, "gemm_skinny: matrix %d has no output", i);

@@ -51,10 +51,12 @@ struct GemvMat {
 // at the token's position, v rows go to the V cache.  Same arithmetic, hence the same bits, as rope_kv_kernel.
 // A work item of a grouped expert launch: MOE_ITEM_INTS int32 = {expert, n, pair[0..n), unused...}, 1 <= n <= MOE_ITEM_PAIRS.
 constexpr int MOE_ITEM_PAIRS = 4, MOE_ITEM_INTS = 8;
-// upper bound on the items n_pairs pairs over n_expert experts can form (sum over experts of ceil(count / 4))
-inline int moe_max_items(int n_pairs, int n_expert) {
+// int32 per item when an item holds up to item_pairs pairs: expert, n, the pairs, padded to a multiple of 4
+__host__ __device__ inline int moe_item_ints(int item_pairs) { return (2 + item_pairs + 3) / 4 * 4; }
+// upper bound on the items n_pairs pairs over n_expert experts can form (sum over experts of ceil(count / item_pairs))
+inline int moe_max_items(int n_pairs, int n_expert, int item_pairs = MOE_ITEM_PAIRS) {
     const int used = n_pairs < n_expert ? n_pairs : n_expert;
-    const int bound = used + n_pairs / MOE_ITEM_PAIRS;
+    const int bound = used + n_pairs / item_pairs;
     return bound < n_pairs ? bound : n_pairs;
 }
 

@@ -185,8 +185,10 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream) {
 // experts' item counts -- to write each pair into its item.
 constexpr int GROUP_THREADS = 1024, GROUP_WAVES = GROUP_THREADS / 64;
 // (whole workgroup; lds: n_pairs + 2 * n_expert ints)
+// ipairs: most pairs per item; an item takes iints = moe_item_ints(ipairs) int32
 __device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int n_pairs, int n_expert, int32_t *__restrict__ items,
-                                            int32_t *__restrict__ n_items, int32_t *lds) {
+                                            int32_t *__restrict__ n_items, int32_t *lds, int ipairs) {
+    const int iints = moe_item_ints(ipairs);
     int32_t *s_ids = lds, *s_cnt = lds + n_pairs, *s_base = s_cnt + n_expert;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (int p = tid; p < n_pairs; p += GROUP_THREADS) s_ids[p] = ids[p];
@@ -204,7 +206,7 @@ __device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int
         // exclusive prefix of items per expert: each lane sums a run of experts, the runs are scanned across the wave
         const int per = (n_expert + 63) / 64, e0 = lane * per;
         int mine = 0;
-        for (int e = e0; e < e0 + per && e < n_expert; ++e) mine += (s_cnt[e] + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+        for (int e = e0; e < e0 + per && e < n_expert; ++e) mine += (s_cnt[e] + ipairs - 1) / ipairs;
         int incl = mine;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
@@ -214,7 +216,7 @@ __device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int
         int run = incl - mine;
         for (int e = e0; e < e0 + per && e < n_expert; ++e) {
             s_base[e] = run;
-            run += (s_cnt[e] + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+            run += (s_cnt[e] + ipairs - 1) / ipairs;
         }
         if (lane == 63) n_items[0] = incl;
     }
@@ -228,22 +230,22 @@ __device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int
             const unsigned long long m = __ballot(hit);
             if (hit) {
                 const int r = seen + __popcll(m & ((1ull << lane) - 1ull));
-                items[(size_t)(base + r / MOE_ITEM_PAIRS) * MOE_ITEM_INTS + 2 + r % MOE_ITEM_PAIRS] = p;
+                items[(size_t)(base + r / ipairs) * iints + 2 + r % ipairs] = p;
             }
             seen += __popcll(m);
         }
-        const int n_it = (cnt + MOE_ITEM_PAIRS - 1) / MOE_ITEM_PAIRS;
+        const int n_it = (cnt + ipairs - 1) / ipairs;
         for (int i = lane; i < n_it; i += 64) {
-            items[(size_t)(base + i) * MOE_ITEM_INTS + 0] = e;
-            items[(size_t)(base + i) * MOE_ITEM_INTS + 1] = i + 1 < n_it ? MOE_ITEM_PAIRS : cnt - i * MOE_ITEM_PAIRS;
+            items[(size_t)(base + i) * iints + 0] = e;
+            items[(size_t)(base + i) * iints + 1] = i + 1 < n_it ? ipairs : cnt - i * ipairs;
         }
     }
 }
 
 __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs, int n_expert,
-                                                                  int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
+                                                                  int32_t *__restrict__ items, int32_t *__restrict__ n_items, int ipairs) {
     extern __shared__ int32_t g_lds[];
-    group_pairs(ids, n_pairs, n_expert, items, n_items, g_lds);
+    group_pairs(ids, n_pairs, n_expert, items, n_items, g_lds, ipairs);
 }
 
 // Routing of a small batch and the grouping of its pairs in one single-workgroup launch: wave w routes tokens w,
@@ -252,18 +254,18 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int32_t 
 // (the routing arguments as leading scalars: preloaded into SGPRs, see gemv.hip)
 __global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(const float *p_logits, const float *p_mask, int32_t *p_ids, float *p_weights,
                                                                         int T, int p_n_expert, int p_top_k, int p_norm_w,
-                                                                        int32_t *__restrict__ items, int32_t *__restrict__ n_items) {
+                                                                        int32_t *__restrict__ items, int32_t *__restrict__ n_items, int ipairs) {
     extern __shared__ int32_t g_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     MoeRouteArgs a;
     a.logits = p_logits; a.mask = p_mask; a.ids = p_ids; a.weights = p_weights; a.n_expert = p_n_expert; a.top_k = p_top_k; a.norm_w = p_norm_w;
     for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(p_logits + (size_t)t * p_n_expert, a, t, lane);
     __syncthreads();
-    group_pairs(p_ids, T * p_top_k, p_n_expert, items, n_items, g_lds);
+    group_pairs(p_ids, T * p_top_k, p_n_expert, items, n_items, g_lds, ipairs);
 }
 
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
-                     float *logits, int T, int32_t *items, int32_t *n_items, hipStream_t stream) {
+                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (!moe_router_group_supported(E, a.n_expert, a.top_k, T) || !logits)
         return fail(MESH_ERR_UNSUPPORTED, "moe: split router for hidden size %d / %d experts / %d tokens", E, a.n_expert, T);
@@ -281,7 +283,7 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
     la.logits = logits;
     const size_t smem = ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
     MESH_LAUNCH(moe_route_group_kernel, dim3(1), dim3(GROUP_THREADS), smem, stream, la.logits, la.mask, la.ids, la.weights, T, la.n_expert, la.top_k, la.norm_w,
-                                                                           items, n_items);
+                                                                           items, n_items, item_pairs);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -294,7 +296,7 @@ bool moe_group_supported(int n_pairs, int n_expert) {
     return n_pairs >= 1 && n_expert >= 1 && ((size_t)n_pairs + 2 * (size_t)n_expert) * sizeof(int32_t) <= 128 * 1024;
 }
 
-int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, hipStream_t stream) {
+int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream) {
     if (!moe_group_supported(n_pairs, n_expert)) return fail(MESH_ERR_UNSUPPORTED, "moe: %d pairs over %d experts do not fit the grouping kernel", n_pairs, n_expert);
     static bool attr_set = false;
     if (!attr_set) {
@@ -302,7 +304,7 @@ int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int
         attr_set = true;
     }
     const size_t smem = ((size_t)n_pairs + 2 * (size_t)n_expert) * sizeof(int32_t);
-    MESH_LAUNCH(moe_group_kernel, dim3(1), dim3(GROUP_THREADS), smem, stream, ids, n_pairs, n_expert, items, n_items);
+    MESH_LAUNCH(moe_group_kernel, dim3(1), dim3(GROUP_THREADS), smem, stream, ids, n_pairs, n_expert, items, n_items, item_pairs);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -21,17 +21,18 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream);
 bool moe_router_fused_supported(int E, int n_expert, int top_k);
 int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
                      float *logits_out, int T, hipStream_t stream);
-// Groups the n_pairs (token, slot) pairs of ids by expert into work items for the expert mat-vec launches (gemv.hpp:
-// MOE_ITEM_INTS int32 per item = {expert, n, pair[0..n)}, n <= MOE_ITEM_PAIRS pairs of that expert, in ascending pair
-// order; experts in ascending order).  *n_items receives the count.  The order is a function of ids alone.
+// Groups the n_pairs (token, slot) pairs of ids by expert into work items for the expert launches: moe_item_ints(item_pairs)
+// int32 per item = {expert, n, pair[0..n)}, n <= item_pairs pairs of that expert, in ascending pair order; experts in
+// ascending order (gemv.hpp; item_pairs = MOE_ITEM_PAIRS for the mat-vec kernel, SKINNY_ITEM_PAIRS for the matrix-core
+// one).  *n_items receives the count.  The order is a function of ids alone.
 bool moe_group_supported(int n_pairs, int n_expert);
-int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, hipStream_t stream);
+int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream);
 // Small batches (T <= 64): router logits with the experts split over several workgroups per token, then routing and
 // grouping in one single-workgroup launch.  Same results as moe_router_fused followed by moe_group; `logits`
 // ([T][n_expert]) is required.
 bool moe_router_group_supported(int E, int n_expert, int top_k, int T);
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
-                     float *logits, int T, int32_t *items, int32_t *n_items, hipStream_t stream);
+                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream);
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 

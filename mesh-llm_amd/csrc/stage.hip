@@ -382,9 +382,13 @@ int session_new(mesh_stage *st, mesh_session **out) {
         MESH_HIP_TRY(hipMemsetAsync(p, 0, B16 * std::max<size_t>(hp.n_embd, QD) * 2, s->stream));     // unused token columns stay finite
         {
             // q16 activations of the skinny GEMM (calls below the large-tile GEMM's token count), widest projection input
-            const size_t tok = std::min<size_t>(B, (size_t)std::max(16, PREFILL_MIN_TOKENS - 1));
+            // (mixture-of-experts stages also run their prefill expert products from this layout: every token)
+            const size_t tok = hp.n_expert ? B : std::min<size_t>(B, (size_t)std::max(16, PREFILL_MIN_TOKENS - 1));
+            s->xq_tokens = tok;
             const size_t kmax = std::max<size_t>(std::max<size_t>(hp.n_embd, QD), hp.n_ff);
-            const size_t bytes = (tok + 15) / 16 * q16_block_bytes((int)((kmax + 255) / 256 * 256));
+            size_t bytes = (tok + 15) / 16 * q16_block_bytes((int)((kmax + 255) / 256 * 256));
+            // mixture of experts: the down projections read one row of n_ff_exp per (token, slot) pair
+            if (hp.n_expert) bytes = std::max(bytes, (tok * hp.n_expert_used + 15) / 16 * q16_block_bytes((int)((hp.n_ff_exp + 255) / 256 * 256)));
             if ((rc = sess_alloc(s.get(), &p, bytes)) != MESH_OK) return rc;
             s->xq = static_cast<uint8_t *>(p);
         }
@@ -408,7 +412,9 @@ int session_new(mesh_stage *st, mesh_session **out) {
             return rc;
         if ((rc = sess_alloc(s.get(), &p, B * k * sizeof(int32_t))) != MESH_OK) return rc;
         s->moe_ids = static_cast<int32_t *>(p);
-        const size_t items = (size_t)moe_max_items((int)(B * k), (int)ne);
+        // work items: 4 pairs each for the mat-vec kernel, 16 for the matrix-core one; the buffer fits either
+        const size_t items = (size_t)std::max(moe_max_items((int)(B * k), (int)ne) * MOE_ITEM_INTS,
+                                              moe_max_items((int)(B * k), (int)ne, SKINNY_ITEM_PAIRS) * moe_item_ints(SKINNY_ITEM_PAIRS)) / MOE_ITEM_INTS + 1;
         if ((rc = sess_alloc(s.get(), &p, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t))) != MESH_OK) return rc;
         s->moe_items = static_cast<int32_t *>(p);
         s->moe_n_items = s->moe_items + items * MOE_ITEM_INTS;
@@ -817,13 +823,20 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             mr.logits = s->moe_logits; mr.mask = s->expert_mask_on ? s->expert_mask : nullptr;
             mr.ids = s->moe_ids; mr.weights = s->moe_w; mr.n_expert = ne; mr.top_k = k; mr.norm_w = 1;
             const bool want_groups = s->moe_grouped && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
+            // a batch of decode steps over K-quant experts: the expert products on the matrix cores, 16 pairs of an expert per pass
+            // (worth it from about four pairs per expert: below that the mat-vec kernel, which only computes the columns an
+            // item has, is as fast)
+            const bool mfma = want_groups && s->xq && (size_t)T <= s->xq_tokens && T * k >= 4 * ne && E % 256 == 0 && ffe % 256 == 0 &&
+                              type_is_tiled(L.gate_exps.type) && L.up_exps.type == L.gate_exps.type && type_is_tiled(L.down_exps.type) &&
+                              moe_max_items(T * k, ne, SKINNY_ITEM_PAIRS) <= 65535;
+            const int item_pairs = mfma ? SKINNY_ITEM_PAIRS : MOE_ITEM_PAIRS;
             bool grouped_done = false;
             if (want_groups && L.gate_inp.type == MESH_F32 && moe_router_group_supported(E, ne, k, T)) {
                 // a batch of decode steps: logits over many workgroups, then routing and grouping in one launch
                 ProfScope ps(s, MESH_PROF_GEMV);
                 if ((rc = moe_router_group(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
                                            static_cast<const float *>(L.gate_inp.data), E, s->moe_logits, T, s->moe_items, s->moe_n_items,
-                                           stream)) != MESH_OK) return rc;
+                                           item_pairs, stream)) != MESH_OK) return rc;
                 grouped_done = true;
             } else if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
                 // the router matrix is small and f32: logits and routing in one launch
@@ -842,7 +855,33 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             }
             // pairs of one expert share a pass over its weights
             const bool grouped = want_groups;
-            if (grouped && !grouped_done && (rc = moe_group(s->moe_ids, T * k, ne, s->moe_items, s->moe_n_items, stream)) != MESH_OK) return rc;
+            if (grouped && !grouped_done && (rc = moe_group(s->moe_ids, T * k, ne, s->moe_items, s->moe_n_items, item_pairs, stream)) != MESH_OK) return rc;
+            if (mfma) {
+                const int max_items = moe_max_items(T * k, ne, SKINNY_ITEM_PAIRS);
+                { ProfScope ps(s, MESH_PROF_PREP); rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream); }
+                if (rc != MESH_OK) return rc;
+                SkinnyArgs ga;
+                ga.n_mat = 2;
+                ga.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);
+                ga.mat[1] = mat_of(L.up_exps, nullptr, ffe, nullptr);
+                ga.xq = s->xq; ga.K = E; ga.T = 1; ga.epi = EPI_SWIGLU;
+                ga.items = s->moe_items; ga.n_items = s->moe_n_items; ga.max_items = max_items;
+                ga.x_div = k;
+                { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_skinny(ga, stream); }
+                if (rc != MESH_OK) return rc;
+                { ProfScope ps(s, MESH_PROF_PREP); rc = quant16_k8(s->ffn, nullptr, 0.f, T * k, ffe, s->xq, stream); }
+                if (rc != MESH_OK) return rc;
+                SkinnyArgs da;
+                da.n_mat = 1;
+                da.mat[0] = mat_of(L.down_exps, s->moe_out, E, nullptr);
+                da.xq = s->xq; da.K = ffe; da.T = 1;
+                da.items = s->moe_items; da.n_items = s->moe_n_items; da.max_items = max_items;
+                da.x_div = 1;
+                { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_skinny(da, stream); }
+                if (rc != MESH_OK) return rc;
+                if ((rc = moe_combine(s->x, s->moe_out, s->moe_w, T, E, k, stream)) != MESH_OK) return rc;
+                continue;
+            }
             GemvArgs ea;
             ea.n_mat = 2;
             ea.mat[0] = mat_of(L.gate_exps, s->ffn, ffe, nullptr);

@@ -247,9 +247,10 @@ def test_moe_stage_matches_oracle_with_and_without_mask(tmp_path):
 
 def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path, monkeypatch):
     """The expert launches walk (token, slot) pairs grouped by expert, up to four pairs of an expert per pass over its
-    weights; MESH_MOE_GROUP=0 runs every pair as its own product.  A column's arithmetic does not depend on its
-    neighbours, so both must give the same bits, whatever the group sizes (8 experts, top-2: 1 to 40 tokens make
-    groups of every size 1..4 and experts with more than one group)."""
+    weights (mat-vec kernel, fewer than 5 tokens) or up to sixteen (matrix-core kernel); MESH_MOE_GROUP=0 runs every pair
+    as its own product.  A column's arithmetic does not depend on its neighbours, so the mat-vec groups give the same
+    bits as pair-by-pair, whatever the group sizes (8 experts, top-2: 1 to 30 tokens make groups of every size and
+    experts with more than one group)."""
     m, cfg, tensors, st = _open(tmp_path, "tiny-moe", range(0, 2), 0, 2, n_ctx=64, n_batch=64)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(77))
@@ -259,12 +260,17 @@ def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path, monkeypatch):
     monkeypatch.delenv("MESH_MOE_GROUP")
     orc = StageOracle(cfg, tensors, 0, 2, 64)
     pos0 = 0
-    for T in (1, 2, 5, 23, 3, 30):
+    for T in (1, 2, 4, 3, 5, 23, 26):           # the bit-exact cases first: afterwards the two caches differ in the last bits
         x = rng.standard_normal((T, E)).astype(np.float32)
         pos = np.arange(pos0, pos0 + T)
         a = ses.decode(x, pos).view(np.float32).reshape(T, E)
         b = ses0.decode(x, pos).view(np.float32).reshape(T, E)
-        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), T
+        if T < 5:
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), T
+        else:
+            # from 5 tokens on the grouped launches run on the matrix cores (16 pairs of an expert per pass): 16-bit
+            # fixed-point activations and exact integer dot products like the mat-vec kernel, f32 sums in another order
+            assert rel_l2(a, b) <= 5e-5, T
         assert np.array_equal(ses.moe_last_ids(T), ses0.moe_last_ids(T))
         assert rel_l2(a, orc.forward(x, pos)) <= 1e-3
         pos0 += T
