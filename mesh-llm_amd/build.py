@@ -76,6 +76,22 @@ def build_rpc_server_hostmem(out_path):
     return out_path
 
 
+PLUGIN = os.path.join(HERE, "mesh-stage-plugin")
+
+
+def build_plugin(out_path=PLUGIN):
+    """Links mesh-llm_amd/mesh-stage-plugin: the stage as a mesh-llm plugin process with an inference endpoint (host code
+    over the C ABI of libmeshstage.so)."""
+    src = os.path.join(CSRC, "plugin", "plugin_main.cpp")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-pthread", src, "-L" + HERE, "-lmeshstage", "-L/opt/rocm/lib",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + HERE, "-Wl,-rpath,/opt/rocm/lib", "-o", out_path]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("mesh-stage-plugin build failed:\n%s\n%s" % (" ".join(cmd), r.stderr))
+    return out_path
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
     print(build_rpc_server())
+    print(build_plugin())
