@@ -217,3 +217,42 @@ def test_c5_expert_shard_layer_zipf_router_on_filled_cache(tmp_path):
     print("[fullsize] C5 distinct experts touched by 16 tokens x top-8: %s" % distinct, file=sys.stderr, flush=True)
     assert max(distinct) <= 44
     ses.close(); st.close()
+
+
+def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path):
+    """The same shard with enough tokens per expert for the matrix-core expert kernel (from four pairs per expert on
+    average: 32 tokens x top-8 over 64 experts): a 96-token prompt chunk of one sequence, then a decode batch of 40
+    sequences, Zipf router, against the oracle; routing decisions identical."""
+    m = mesh()
+    cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
+    path = os.path.join(str(tmp_path), "shard.gguf")
+    tensors = models.write_model(path, cfg, [5, 6], seed=9, n_expert_local=64, fast=True, router="zipf")
+    n_ctx, E = 128, 2048
+    st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=40, n_batch_max=96)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 5, 7, n_ctx, n_seq_max=40)
+    rng = np.random.Generator(np.random.PCG64(56))
+    # prompt chunk
+    T = 96
+    x = models.zipf_hidden_state(rng, T, E)
+    pos = np.arange(T, dtype=np.int32)
+    got = ses.decode(x, pos).view(np.float32).reshape(T, E)
+    ref = orc.forward(x, pos)
+    r = rel_l2(got - x, ref - x)
+    report("C5 shard layers 5-6, 96-token prefill (matrix-core expert products; of the layers' contribution)", r)
+    assert r <= NORTH_STAR
+    assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+    # wide decode batch: sequence 0 continues its prompt, the others start
+    T = 40
+    x = models.zipf_hidden_state(rng, T, E)
+    pos = np.zeros(T, np.int32)
+    pos[0] = 96
+    seq = np.arange(T, dtype=np.int32)
+    got = ses.decode(x, pos, seq=seq).view(np.float32).reshape(T, E)
+    ref = orc.forward(x, pos, seq=seq)
+    r = rel_l2(got - x, ref - x)
+    report("C5 shard layers 5-6, decode batch 40 (matrix-core expert products)", r)
+    assert r <= NORTH_STAR
+    assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+    ses.close(); st.close()
