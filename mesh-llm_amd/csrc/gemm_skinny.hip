@@ -505,17 +505,29 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     ka.rope = a.rope;
     const bool grouped = a.items != nullptr;
     ka.items = a.items; ka.n_items = a.n_items; ka.expert_stride = (size_t)tiled_bytes(type, a.mat[0].M, a.K); ka.x_div = a.x_div > 0 ? a.x_div : 1;
-    int KS = 1;
-    // a power of two: the kernel splits its waves with shifts.  Expert matrices are short in K (a few super-blocks), so
-    // their waves go along the rows instead and each still walks several super-blocks
-    while (KS * 2 <= nsb && KS * 2 <= (grouped ? 2 : SK_WAVES)) KS *= 2;
+    // How the 8 waves of a workgroup are arranged (KS along K, a power of two: the kernel splits its waves with shifts; the
+    // other 8 / KS along tile-rows) decides how many workgroups the launch has and how long each wave's chain of tiles is.
+    // A workgroup costs a fixed start-up / reduction time plus its waves' tiles one after the other, and workgroups beyond one
+    // per CU wait for a second round: take the arrangement for which that estimate is smallest (ties: more waves along K).
+    // Expert matrices are short in K (a few super-blocks) and their launches have many items, so they get few, long
+    // workgroups: at most 2 waves along K and as many tile-rows as a workgroup can hold.
+    const int ncu = skinny_n_cu();
+    int KS = 1, rows_per_wg = 1;
+    {
+        double best = 1e30;
+        for (int ks = 1; ks <= (grouped ? 2 : SK_WAVES) && ks <= nsb; ks *= 2) {
+            const int rs = SK_WAVES / ks;
+            const int cap = std::max(1, SK_SEGS_MAX / NU) * rs;
+            const int rpw = grouped ? cap : std::max(1, std::min((total_rows + ncu - 1) / ncu, cap));
+            const int wgs = (total_rows + rpw - 1) / rpw;
+            const int rounds = grouped ? 1 : (wgs + ncu - 1) / ncu;
+            const int tiles = ((rpw + rs - 1) / rs) * NU * ((nsb + ks - 1) / ks);
+            const double cost = rounds * (5.0 + 0.9 * tiles);
+            if (cost <= best) { best = cost; KS = ks; rows_per_wg = rpw; }
+        }
+    }
     const int RS = SK_WAVES / KS;
     ka.ks = KS;
-    // tile-rows per workgroup: spread over the CUs, bounded by the segments a wave can hold
-    const int rows_cap = std::max(1, SK_SEGS_MAX / NU) * RS;
-    const int ncu = skinny_n_cu();
-    int rows_per_wg = grouped ? rows_cap : std::min((total_rows + ncu - 1) / ncu, rows_cap);     // expert launches have many items: few, long workgroups each
-    rows_per_wg = std::max(1, rows_per_wg);
     const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
     const int rows_max = (total_rows + grid - 1) / grid;
     const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
