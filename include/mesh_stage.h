@@ -208,10 +208,6 @@ int mesh_session_synchronize(mesh_session *session);
  * 32 tokens, from the third call with the same token count and KV split count on; environment MESH_STAGE_GRAPHS=1 at
  * session creation turns graphs on: they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
 int64_t mesh_session_graph_replays(const mesh_session *session);
-/* Number of one-token decode steps of this session that ran as a single launch sharded over the GPU's compute dies
- * (stages of the Llama-3-8B shape with an f16 KV cache on a 256-CU device, when the environment has MESH_DECODE_DIE=1 at
- * session creation; otherwise every step takes the launch-per-projection path).  -1 for a null session.  No counterpart in the reference. */
-int64_t mesh_session_single_launch_steps(const mesh_session *session);
 
 /* Per-kernel-class timing of a session: every kernel launched for the session while profiling is on carries its own
  * start / stop event pair (stamped by the dispatch, nothing extra is queued between launches), so ms[] sums pure

@@ -103,7 +103,6 @@ SIGNATURES.update({
     "mesh_session_stream": (_vp, [_vp]),
     "mesh_session_synchronize": (_i32, [_vp]),
     "mesh_session_graph_replays": (_i64, [_vp]),
-    "mesh_session_single_launch_steps": (_i64, [_vp]),
     "mesh_session_profile": (_i32, [_vp, _i32]),
     "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
     "mesh_session_set_expert_mask": (_i32, [_vp, _vp, _i32]),
@@ -376,11 +375,6 @@ class Session:
     def graph_replays(self):
         """Decode steps so far whose layer launches were replayed from a captured graph."""
         return int(lib().mesh_session_graph_replays(self._h))
-
-    @property
-    def single_launch_steps(self):
-        """One-token decode steps so far that ran as one launch sharded over the compute dies."""
-        return int(lib().mesh_session_single_launch_steps(self._h))
 
     def profile(self, enable):
         check(lib().mesh_session_profile(self._h, 1 if enable else 0))

@@ -167,10 +167,6 @@ int64_t mesh_session_graph_replays(const mesh_session *session) {
     return session ? session->graph_replays : -1;
 }
 
-int64_t mesh_session_single_launch_steps(const mesh_session *session) {
-    return session ? session->die_steps : -1;
-}
-
 int mesh_session_profile(mesh_session *session, int enable) {
     if (!session) return fail(MESH_ERR_INVALID, "mesh_session_profile: null session");
     int rc = profile_collect(session);

@@ -17,7 +17,6 @@
 #include <mutex>
 
 #include "attn.hpp"
-#include "decode_die.hpp"
 #include "gemm.hpp"
 #include "gemv.hpp"
 #include "moe.hpp"
@@ -434,8 +433,6 @@ int session_new(mesh_stage *st, mesh_session **out) {
     if ((rc = sess_alloc(s.get(), &s->io_stage, s->io_stage_bytes + s->io_out_bytes)) != MESH_OK) return rc;
     MESH_HIP_TRY(hipHostMalloc(&s->h_io, s->io_stage_bytes + s->io_out_bytes, hipHostMallocDefault));
     MESH_HIP_TRY(hipStreamSynchronize(s->stream));
-    // one-token steps of stages of the shape it is built for run as a single launch sharded over the compute dies
-    if (!s->graphs_on && (rc = die_decode_create(s.get(), &s->die)) != MESH_OK) return rc;
     *out = s.release();
     return MESH_OK;
 }
@@ -952,11 +949,6 @@ static int validate_batch(const mesh_session *s, const mesh_batch *b, int *max_k
 constexpr int GRAPH_MAX_TOKENS = 32;
 constexpr size_t GRAPH_MAX_ENTRIES = 96;
 static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
-    if (T == 1 && s->die) {
-        ProfScope ps(s, MESH_PROF_GEMV);
-        ++s->die_steps;
-        return die_decode_step(s, s->die);
-    }
     if (!s->graphs_on || s->profile || T > GRAPH_MAX_TOKENS) return run_layers(s, T, max_keys);
     // A prefill chunk (consecutive positions of one sequence, enough tokens for the large-tile GEMM) runs the chunk
     // attention kernel, whose first position and sequence are launch arguments: a replay would carry the captured
@@ -1094,7 +1086,6 @@ int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fm
     uint8_t *h_out = static_cast<uint8_t *>(s->h_io) + s->io_stage_bytes;
     MESH_HIP_TRY(hipMemcpyAsync(h_out, d_out, len, hipMemcpyDeviceToHost, stream));
     MESH_HIP_TRY(hipStreamSynchronize(stream));
-    if ((rc = die_decode_check(s, s->die)) != MESH_OK) return rc;
     memcpy(out, h_out, len);
     return MESH_OK;
 }
@@ -1144,7 +1135,6 @@ mesh_stage::~mesh_stage() {
 
 mesh_session::~mesh_session() {
     if (stream) (void)hipStreamSynchronize(stream);
-    mesh::die_decode_destroy(die);
     for (hipEvent_t e : prof_events) (void)hipEventDestroy(e);
     for (void *p : allocations) (void)hipFree(p);
     for (auto &kv : graphs)

@@ -52,7 +52,6 @@ struct LayerWeights {
 }  // namespace mesh
 
 namespace mesh {
-struct DieDecode;
 int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stage_opts *opts, mesh_stage **out);
 int session_new(mesh_stage *st, mesh_session **out);
 int stage_decode(mesh_session *s, const mesh_batch *b, const void *in, int in_fmt, void *out, int out_fmt, size_t out_cap, size_t *out_len);
@@ -119,8 +118,6 @@ struct mesh_session {
     struct LayerGraph { hipGraphExec_t exec = nullptr; int uses = 0; };
     std::unordered_map<uint64_t, LayerGraph> graphs;
     int64_t graph_replays = 0;
-    int64_t die_steps = 0;
-    mesh::DieDecode *die = nullptr;  // single-launch one-token step (decode_die.hpp), null when the stage or device does not fit it
     bool graphs_on = false;          // MESH_STAGE_GRAPHS=1 at session creation turns them on; a failed capture turns them off
     std::vector<hipEvent_t> prof_events;      // pairs (begin, end)
     std::vector<int> prof_kinds;
