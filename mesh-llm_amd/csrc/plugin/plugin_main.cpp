@@ -13,6 +13,7 @@
 // packed boundary activations in, packed boundary activations (or logits) out.  Chat / completion routes answer 501: a
 // pipeline stage has no tokenizer and no sampler, those stay with the process that owns both ends of the pipeline.
 
+#include <algorithm>
 #include <arpa/inet.h>
 #include <netinet/in.h>
 #include <netinet/tcp.h>
@@ -231,7 +232,7 @@ static void handle_decode(int fd, State &st, const std::string &head, const std:
     const int pos0 = atoi(header_value(head, "X-Mesh-Pos0").c_str());
     const int seq = atoi(header_value(head, "X-Mesh-Seq").c_str());
     const int in_fmt = format_id(header_value(head, "X-Mesh-In-Format"), MESH_Q8_0), out_fmt = format_id(header_value(head, "X-Mesh-Out-Format"), MESH_Q8_0);
-    if (T < 1 || T > st.cfg.n_batch_max || pos0 < 0 || in_fmt < 0 || out_fmt < 0 || in_fmt == MESH_LOGITS || out_fmt == MESH_TOKENS)
+    if (T < 1 || T > st.cfg.n_batch_max || pos0 < 0 || pos0 > (1 << 30) || seq < 0 || in_fmt < 0 || out_fmt < 0 || in_fmt == MESH_LOGITS || out_fmt == MESH_TOKENS)
         return http_error(fd, "400 Bad Request", "X-Mesh-Tokens / X-Mesh-Pos0 / formats out of range", "invalid_request_error");
     const size_t want = in_fmt == MESH_TOKENS ? (size_t)T * 4 : mesh_act_packed_size(in_fmt, T, st.info.n_embd);
     if (body.size() != want) return http_error(fd, "400 Bad Request", "body has " + std::to_string(body.size()) + " bytes, " + std::to_string(want) + " expected", "invalid_request_error");
@@ -265,7 +266,9 @@ static void http_client(int fd, State *st) {
     const std::string head = req.substr(0, head_end + 2);
     const size_t clen = (size_t)strtoull(header_value(head, "Content-Length").c_str(), nullptr, 10);
     std::string body = req.substr(head_end + 4);
-    if (clen > (1u << 30)) { http_error(fd, "413 Payload Too Large", "body too large", "invalid_request_error"); ::close(fd); return; }
+    // (the largest body a stage takes is a batch of f32 rows)
+    const size_t body_max = std::max<size_t>(1u << 20, st->session ? (size_t)st->cfg.n_batch_max * st->info.n_embd * 4 : 0);
+    if (clen > body_max) { http_error(fd, "413 Payload Too Large", "body too large", "invalid_request_error"); ::close(fd); return; }
     while (body.size() < clen) {
         const ssize_t n = ::recv(fd, buf, sizeof buf, 0);
         if (n <= 0) break;

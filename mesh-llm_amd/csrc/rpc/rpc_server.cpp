@@ -6,6 +6,7 @@
 
 #include "rpc_server.hpp"
 
+#include <algorithm>
 #include <arpa/inet.h>
 #include <netdb.h>
 #include <netinet/in.h>
@@ -354,7 +355,13 @@ bool Server::push_tensor_to_peer(const PushTensorToPeerReq &req) {
 }
 
 void Server::serve_client(Conn &conn) {
-    constexpr uint64_t MSG_LIMIT = (uint64_t)64 << 30;
+    // a tensor payload cannot be larger than the largest live buffer it could land in
+    auto payload_limit = [this]() {
+        std::lock_guard<std::mutex> lk(mu_);
+        uint64_t largest = 0;
+        for (const auto &kv : buffers_) largest = std::max(largest, kv.second->size);
+        return largest + sizeof(Tensor) + sizeof(uint64_t);
+    };
     uint8_t cmd;
     if (!conn.recv_all(&cmd, 1)) return;
     if (cmd != CMD_HELLO) {
@@ -480,7 +487,7 @@ void Server::serve_client(Conn &conn) {
             }
             case CMD_SET_TENSOR: {
                 std::vector<uint8_t> input;
-                if (!conn.recv_msg(input, MSG_LIMIT) || !set_tensor(input)) return;
+                if (!conn.recv_msg(input, payload_limit()) || !set_tensor(input)) return;
                 break;                  // no reply
             }
             case CMD_SET_TENSOR_HASH: {
@@ -545,7 +552,7 @@ void Server::serve_client(Conn &conn) {
             }
             case CMD_PEER_TENSOR_DATA: {
                 std::vector<uint8_t> input;
-                if (!conn.recv_msg(input, MSG_LIMIT)) return;
+                if (!conn.recv_msg(input, payload_limit())) return;
                 const uint8_t result = set_tensor(input) ? 1 : 0;
                 if (!conn.send_msg(&result, 1)) return;
                 break;
