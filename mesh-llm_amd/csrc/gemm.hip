@@ -476,6 +476,214 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         }
 }
 
+// ---- the same product on a 256 x 128 workgroup tile ----------------------------------------------------------
+// What bounds the 128 x 128 kernel above is operand traffic, not the matrix cores: a wave that owns 64 x 64 of the tile
+// needs 1 KB of fragments per v_mfma_f32_32x32x16_f16 (2 x 2 register blocking: two weight fragments from LDS and two
+// activation fragments from memory per four MFMAs), and four SIMDs at one MFMA per 32 cycles then ask the vector memory
+// path for its whole 64 B per cycle and LDS for three quarters of its 128.  Here a matrix-core wave owns 128 weight rows x
+// 64 tokens (4 x 2 blocking, 128 accumulator registers): 0.5 KB of weight fragments and 0.25 KB of activation fragments
+// per MFMA, half of either path.  The price is one workgroup per CU and one matrix-core wave per SIMD, which therefore
+// fetches the weight fragments of the next k16 step before it multiplies the current one; a staging wave shares the
+// SIMD and dequantises while the MFMAs execute.
+// Production layout only (GEMM-layout weights, k8-major activations), K not split, an even number of 128-row blocks:
+// a workgroup takes row blocks 2 * blockIdx.x and + 1, one per pair of matrix-core waves, so everything that depends on
+// the row block (matrix of a multi-matrix launch, SwiGLU pairing) is per wave.
+constexpr int BGM = 256;
+// Workgroup barrier that orders LDS only.  __syncthreads() also waits for every outstanding global load, i.e. at the end
+// of each k-step for the activation fragments requested a moment ago for the NEXT step -- with one matrix-core wave per
+// SIMD nothing else would run during that wait.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+template <int TYPE>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_big_kernel(GemmArgs a) {
+    extern __shared__ __align__(16) _Float16 gemm_smem[];
+    _Float16 *Ws = gemm_smem;                                  // [2][BGM][LDS_LD]
+    using Sub = PackedSub<TYPE>;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t0 = blockIdx.y * GN;
+    const int n_steps = a.K / GK;
+
+    if (wave >= 4) {
+        // ---- staging waves: thread s: (row s / 2, sub-block half s % 2) of both row blocks
+        const int st = tid - 256;
+        const uint8_t *chunk0 = static_cast<const uint8_t *>(a.Wp) + (size_t)(2 * blockIdx.x) * n_steps * Sub::CHUNK;
+        const uint8_t *chunk1 = chunk0 + (size_t)n_steps * Sub::CHUNK;
+        _Float16 *dst = Ws + (st >> 1) * LDS_LD + 32 * (st & 1);
+        Sub rw[2][2];
+        auto fetch = [&](int kc, Sub (&w)[2]) {
+            w[0].load(chunk0 + (size_t)kc * Sub::CHUNK, st);
+            w[1].load(chunk1 + (size_t)kc * Sub::CHUNK, st);
+        };
+        auto stage = [&](int buf, const Sub (&w)[2]) {
+            w[0].store(dst + buf * BGM * LDS_LD);
+            w[1].store(dst + (buf * BGM + GM) * LDS_LD);
+        };
+        fetch(0, rw[0]);
+        fetch(n_steps > 1 ? 1 : 0, rw[1]);
+        stage(0, rw[0]);
+        lds_barrier();
+        for (int kc0 = 0; kc0 < n_steps; kc0 += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int kc = kc0 + u;
+                if (kc >= n_steps) break;
+                fetch(kc + 2 < n_steps ? kc + 2 : n_steps - 1, rw[u]);
+                if (kc + 1 < n_steps) stage(u ^ 1, rw[u ^ 1]);
+                lds_barrier();
+            }
+        }
+        return;
+    }
+
+    // ---- multiplying waves: row block (wave & 1), token half (wave >> 1)
+    const int vb = 2 * (int)blockIdx.x + (wave & 1);           // this wave's 128-row block of the launch
+    const int wm = (wave & 1) * GM, wn = (wave >> 1) * 64;
+    float16v acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    const int n_blk = (a.T + 15) >> 4, n_g = n_steps * (GK / 16);
+    const _Float16 *bp[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int tok = t0 + wn + 32 * i + (lane & 31);
+        const int blk = (tok >> 4) < n_blk ? (tok >> 4) : n_blk - 1;
+        bp[i] = a.X + (size_t)blk * 16 * a.K + ((lane >> 5) * 16 + (tok & 15)) * 8;
+    }
+    half8 ring[GK / 16][2];
+#pragma unroll
+    for (int ks = 0; ks < GK / 16; ++ks)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)(ks < n_g ? ks : n_g - 1) * 256);
+    const int a_off = (wm + (lane & 31)) * LDS_LD + 8 * (lane >> 5);
+    lds_barrier();
+    for (int kc = 0; kc < n_steps; ++kc) {
+        const _Float16 *Wb = Ws + (kc & 1) * BGM * LDS_LD + a_off;
+        half8 af[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[0][i] = *reinterpret_cast<const half8 *>(Wb + 32 * i * LDS_LD);
+#pragma unroll
+        for (int ks = 0; ks < GK / 16; ++ks) {
+            if (ks + 1 < GK / 16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) af[(ks + 1) & 1][i] = *reinterpret_cast<const half8 *>(Wb + 32 * i * LDS_LD + 16 * (ks + 1));
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1][i], ring[ks][j], acc[i][j], 0, 0, 0);
+            int gn = (kc + 1) * (GK / 16) + ks;
+            gn = gn < n_g ? gn : n_g - 1;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) ring[ks][i] = *reinterpret_cast<const half8 *>(bp[i] + (size_t)gn * 256);
+            // Issue order inside the step: the next step's four fragment reads go out between the first MFMAs (an MFMA
+            // holds the matrix pipe for 32 cycles, the wave is free to issue meanwhile), the two activation refills after
+            // the last.  Left to itself the scheduler puts the reads behind all eight MFMAs, and the next step then
+            // starts by waiting out the LDS latency.
+            if (ks + 1 < GK / 16) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // one LDS read
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);              // the two global loads
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        lds_barrier();
+    }
+
+    // D[m][t]: lane holds column t = lane % 32 and rows 8 * (e / 4) + 4 * (lane / 32) + e % 4 of each 32 x 32 block
+    if (a.y16_k8) {
+        // SwiGLU pair: the row block's rows 0..63 are gate rows, 64..127 the up rows of the same outputs: blocks
+        // acc[0..1] and acc[2..3] of this very lane
+        const int t_pad = (a.T + 15) & ~15;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int t = t0 + wn + 32 * j + (lane & 31);
+                if (t >= t_pad) continue;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const int m = vb * (GM / 2) + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                    if (m >= a.M) continue;
+                    float o[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float g = acc[i][j][4 * e4 + c], u = acc[i + 2][j][4 * e4 + c];
+                        o[c] = t < a.T ? g / (1.0f + expf(-g)) * u : 0.f;
+                    }
+                    *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
+                        make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
+                }
+            }
+        return;
+    }
+    float *Y = a.Y;
+    const float *bias = a.bias;
+    int M = a.M, ldy = a.ldy, mb0 = vb * GM;
+    if (a.n_seg > 1) {
+        const int sg = (vb >= a.seg_begin[1] ? 1 : 0) + (a.n_seg > 2 && vb >= a.seg_begin[2] ? 1 : 0);
+        Y = sg == 0 ? a.seg_Y[0] : sg == 1 ? a.seg_Y[1] : a.seg_Y[2];
+        bias = sg == 0 ? a.seg_bias[0] : sg == 1 ? a.seg_bias[1] : a.seg_bias[2];
+        M = sg == 0 ? a.seg_M[0] : sg == 1 ? a.seg_M[1] : a.seg_M[2];
+        ldy = sg == 0 ? a.seg_ldy[0] : sg == 1 ? a.seg_ldy[1] : a.seg_ldy[2];
+        mb0 = (vb - (sg == 0 ? 0 : sg == 1 ? a.seg_begin[1] : a.seg_begin[2])) * GM;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int t = t0 + wn + 32 * j + (lane & 31);
+            if (t >= a.T) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int m = mb0 + 32 * i + 8 * e4 + 4 * (lane >> 5);
+                if (m >= M) continue;
+                float4 o = make_float4(acc[i][j][4 * e4], acc[i][j][4 * e4 + 1], acc[i][j][4 * e4 + 2], acc[i][j][4 * e4 + 3]);
+                if (bias) {
+                    const float4 b = *reinterpret_cast<const float4 *>(bias + m);
+                    o.x += b.x; o.y += b.y; o.z += b.z; o.w += b.w;
+                }
+                if (a.residual) {
+                    const float4 r = *reinterpret_cast<const float4 *>(a.residual + (size_t)t * a.ldres + m);
+                    o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
+                }
+                *reinterpret_cast<float4 *>(Y + (size_t)t * ldy + m) = o;
+            }
+        }
+}
+
+template <int TYPE>
+static int launch_gemm_big(const GemmArgs &k, int row_blocks, int t_blocks, hipStream_t stream) {
+    constexpr size_t smem = sizeof(_Float16) * 2 * BGM * LDS_LD;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_big_kernel<TYPE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    MESH_LAUNCH((gemm_big_kernel<TYPE>), dim3((unsigned)(row_blocks / 2), (unsigned)t_blocks), dim3(GEMM_THREADS), smem, stream, k);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// MESH_GEMM_BIG=0: every call keeps the 128 x 128 tile (for comparison)
+static bool gemm_big_on() {
+    const char *e = getenv("MESH_GEMM_BIG");
+    return !(e && e[0] == '0');
+}
+
 // Second kernel of a split launch: adds the slices of part[slice][token][row] in slice order and applies the epilogue
 // of the unsplit kernel.  One thread per (token, four consecutive rows); rows run fastest, so partial reads and output
 // writes are contiguous.
@@ -665,6 +873,10 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
         return fail(MESH_ERR_INVALID, "gemm: RoPE / KV append on a launch it does not fit");
     if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
+    // enough workgroups of the 256 x 128 tile to give every CU one: the big tile (gemm_big_kernel)
+    if (a.x_k8 && packed && k.ksplit <= 1 && !a.rope.pos && row_blocks % 2 == 0 && gemm_big_on() &&
+        (row_blocks / 2) * (int)grid.y >= gemm_n_cu())
+        return q4 ? launch_gemm_big<MESH_Q4_K>(k, row_blocks, (int)grid.y, stream) : launch_gemm_big<MESH_Q6_K>(k, row_blocks, (int)grid.y, stream);
     if (a.x_k8) {
         if (packed) return q4 ? launch_gemm<MESH_Q4_K, true, true>(k, grid, stream) : launch_gemm<MESH_Q6_K, true, true>(k, grid, stream);
         return q4 ? launch_gemm<MESH_Q4_K, false, true>(k, grid, stream) : launch_gemm<MESH_Q6_K, false, true>(k, grid, stream);

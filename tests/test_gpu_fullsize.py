@@ -85,7 +85,7 @@ def test_c3_sixteen_layer_stage_decode_at_kv_depth_4095(c3_model):
     ses.close(); st.close()
 
 
-def test_c3_prefill_2048_tokens_two_layers(c3_model):
+def test_c3_prefill_2048_tokens_two_layers(c3_model, monkeypatch):
     m = mesh()
     cfg, tensors, path = c3_model
     T = 2048
@@ -100,6 +100,12 @@ def test_c3_prefill_2048_tokens_two_layers(c3_model):
     report("C3 layers 3-4, prefill 2048 tokens", r)
     assert r <= NORTH_STAR
     assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR
+    # launches that fill the chip with 256 x 128 tiles take the big-tile kernel; with MESH_GEMM_BIG=0 all keep the
+    # 128 x 128 one.  Same fragments, same order along K: the same bits.
+    monkeypatch.setenv("MESH_GEMM_BIG", "0")
+    small = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, 4096)
+    monkeypatch.delenv("MESH_GEMM_BIG")
+    assert np.array_equal(got, small)
     # one decode token on top of the 2048 cached positions
     x1 = rng.standard_normal((1, 4096)).astype(np.float32)
     r1 = rel_l2(ses.decode(x1, [T]).view(np.float32), orc.forward(x1, [T]))
