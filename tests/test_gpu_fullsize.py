@@ -136,6 +136,33 @@ def test_c3_prefill_256_tokens_sixteen_layers(c3_model):
     ses.close(); st.close()
 
 
+def test_c4_long_prefill_takes_the_big_tile_with_biases(tmp_path, monkeypatch):
+    """1664 tokens through one Qwen2.5-32B-shaped layer: every projection launch has enough 256-row tiles to fill the chip,
+    so the fused q / k / v launch (three matrices, biases, 40 + 8 + 8 row blocks) and the q6_K down projection run on the
+    256 x 128 tile; against the oracle, and bit for bit against the 128 x 128 kernel."""
+    m = mesh()
+    cfg = models.CONFIGS["qwen2.5-32b"]
+    path = os.path.join(str(tmp_path), "c4l.gguf")
+    tensors = models.write_model(path, cfg, [7], seed=42, fast=True)
+    T, E = 1664, 5120
+    st = m.Stage(path, 7, 8, n_ctx=T, n_seq_max=1, n_batch_max=T)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 7, 8, T, blas=True)
+    rng = np.random.Generator(np.random.PCG64(1664))
+    x = rng.standard_normal((T, E)).astype(np.float32)
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
+    ref = orc.forward(x, np.arange(T))
+    r = rel_l2(got, ref)
+    report("C4 layer 7, prefill 1664 tokens (big tile)", r)
+    assert r <= NORTH_STAR
+    monkeypatch.setenv("MESH_GEMM_BIG", "0")
+    small = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
+    monkeypatch.delenv("MESH_GEMM_BIG")
+    assert np.array_equal(got, small)
+    ses.close(); st.close()
+
+
 @pytest.mark.parametrize("kv", ["f16", "q8_0/q4_0"])
 def test_c4_qwen25_32b_layers_wide_batches_and_prefill(tmp_path, kv):
     """Layers 7 (q6_K attn_v / ffn_down) and 8 (all q4_K) of the 64-layer model."""
