@@ -26,7 +26,12 @@ namespace mesh {
 constexpr int PF_HD = 128;
 constexpr int PF_TILE = 32;                 // queries per workgroup and keys per step
 constexpr int PF_KPITCH = PF_HD + 8;        // halfs per key row of the K tile in LDS (bank-conflict padding)
-constexpr int PF_VPITCH = PF_TILE + 4;      // halfs per dim row of the transposed V tile
+constexpr int PF_VPITCH = PF_TILE / 2 + 2;  // dwords (key pairs) per dim row of the transposed V tile
+
+// Column (dword) of key pair kp in dim row `dim` of the transposed V tile.  Rows 32 apart start on the same LDS bank
+// (32 * 18 dwords is a multiple of the 64 banks), and the staging writes of a wave touch four such rows at once; the
+// XOR moves them onto different banks.  It keeps dwords 2j, 2j + 1 neighbours, which the 8-byte fragment reads need.
+__device__ __forceinline__ int pf_vcol(int dim, int kp) { return kp ^ ((dim >> 5) << 2); }
 constexpr float PF_RESCALE_STEP = 8.f;      // the softmax reference moves only when the running maximum exceeds it by this (log2)
 
 typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
@@ -54,11 +59,12 @@ __device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
     }
 }
 
-template <int KT, int VT>
+// NP: (key, 8-dim piece) pairs of a tile one thread carries, at least 512 / (threads of the workgroup).
+template <int KT, int VT, int NP>
 __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw) {
     constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
     __shared__ __align__(16) _Float16 sK[PF_TILE * PF_KPITCH];
-    __shared__ __align__(16) _Float16 sVt[PF_HD * PF_VPITCH];
+    __shared__ __align__(16) uint32_t sVt[PF_HD * PF_VPITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
     const int qcol = lane & 31, half = lane >> 5;
     const int qt = blockIdx.x, kvh = blockIdx.y;
@@ -90,21 +96,59 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
     const int q_end = qt * PF_TILE + PF_TILE < T ? qt * PF_TILE + PF_TILE : T;      // queries of this tile: [qt*32, q_end)
     const int n_keys = pos0 + q_end;                                                // keys any of them may see
-    for (int k0 = 0; k0 < n_keys; k0 += PF_TILE) {
-        // stage the K tile as it is and the V tile transposed; rows past the context end are clamped (masked below)
-        for (int p = tid; p < PF_TILE * 16; p += nthreads) {
-            const int key = p >> 4, piece = p & 15;
-            int kr = k0 + key;
-            kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
-            const uint4 kv = pf_row_piece<KT>(a.kcache + (base + kr) * KRB, piece);
-            const uint4 vv = pf_row_piece<VT>(a.vcache + (base + kr) * VRB, piece);
-            *reinterpret_cast<uint4 *>(sK + key * PF_KPITCH + piece * 8) = kv;
-            const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
+    // The rows of a tile travel through registers: a thread fetches its share of tile k0 + 32 right after it has written
+    // that of tile k0 to LDS, so the loads are in flight while the tile is multiplied.  K: (key, 8-dim piece) pairs, 16
+    // bytes each.  V: the same 8 dims of two neighbouring keys, so that the transposed tile is written as dwords.
+    // Rows past the context end are clamped (masked below).
+    constexpr int NPV = (NP + 1) / 2;
+    uint4 rk[NP], rv[NPV][2];
+    auto fetch_tile = [&](int k0) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                reinterpret_cast<uint16_t *>(sVt)[(piece * 8 + e) * PF_VPITCH + key] = (uint16_t)(vw[e >> 1] >> (16 * (e & 1)));
+        for (int i = 0; i < NP; ++i) {
+            const int p = tid + i * nthreads;
+            if (p < PF_TILE * 16) {
+                int kr = k0 + (p >> 4);
+                kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
+                rk[i] = pf_row_piece<KT>(a.kcache + (base + kr) * KRB, p & 15);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            const int p = tid + i * nthreads;
+            if (p < PF_TILE * 8) {
+                int kr0 = k0 + 2 * (p >> 4), kr1 = kr0 + 1;
+                kr0 = kr0 < a.n_ctx ? kr0 : a.n_ctx - 1;
+                kr1 = kr1 < a.n_ctx ? kr1 : a.n_ctx - 1;
+                rv[i][0] = pf_row_piece<VT>(a.vcache + (base + kr0) * VRB, p & 15);
+                rv[i][1] = pf_row_piece<VT>(a.vcache + (base + kr1) * VRB, p & 15);
+            }
+        }
+    };
+    fetch_tile(0);
+    for (int k0 = 0; k0 < n_keys; k0 += PF_TILE) {
+        // the K tile as it is
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int p = tid + i * nthreads;
+            if (p < PF_TILE * 16) *reinterpret_cast<uint4 *>(sK + (p >> 4) * PF_KPITCH + (p & 15) * 8) = rk[i];
+        }
+        // the V tile transposed: 8 dwords, one per dim, each holding the pair of keys
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            const int p = tid + i * nthreads;
+            if (p < PF_TILE * 8) {
+                const int kp = p >> 4, piece = p & 15;
+                const uint32_t w0[4] = {rv[i][0].x, rv[i][0].y, rv[i][0].z, rv[i][0].w}, w1[4] = {rv[i][1].x, rv[i][1].y, rv[i][1].z, rv[i][1].w};
+                uint32_t *dst = sVt + piece * 8 * PF_VPITCH + pf_vcol(piece * 8, kp);
+#pragma unroll
+                for (int e2 = 0; e2 < 4; ++e2) {
+                    dst[(2 * e2) * PF_VPITCH] = (w0[e2] & 0xffffu) | (w1[e2] << 16);
+                    dst[(2 * e2 + 1) * PF_VPITCH] = (w0[e2] >> 16) | (w1[e2] & 0xffff0000u);
+                }
+            }
         }
         __syncthreads();
+        if (k0 + PF_TILE < n_keys) fetch_tile(k0 + PF_TILE);
 
         // S^T = K . Q^T : lane (key row = lane % 32 of the A operand, query column = lane % 32 of the result)
         pf_f16v s;
@@ -144,7 +188,7 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         }
         float p[16], ps = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { p[i] = exp2f(s[i] - m); ps += p[i]; }
+        for (int i = 0; i < 16; ++i) { p[i] = __builtin_amdgcn_exp2f(s[i] - m); ps += p[i]; }     // s - m <= PF_RESCALE_STEP; far below, 0
         ps += __shfl_xor(ps, 32);
         l += ps;
         // P^T as the B operand: the lane's own registers, 8 per MFMA
@@ -153,9 +197,10 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         const pf_h8 p1 = __builtin_bit_cast(pf_h8, pu1), p2 = __builtin_bit_cast(pf_h8, pu2);
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-            const _Float16 *vrow = sVt + (db * 32 + qcol) * PF_VPITCH + 4 * half;     // dim row, this half's keys
-            const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow), a1 = *reinterpret_cast<const uint2 *>(vrow + 8);
-            const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 16), a3 = *reinterpret_cast<const uint2 *>(vrow + 24);
+            // dim row db * 32 + qcol, this half's keys: key pairs 2 * half + 4 * j (+ 1), j = 0 .. 3
+            const uint32_t *vrow = sVt + (db * 32 + qcol) * PF_VPITCH + 2 * half;
+            const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow + 4 * (0 ^ db)), a1 = *reinterpret_cast<const uint2 *>(vrow + 4 * (1 ^ db));
+            const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 4 * (2 ^ db)), a3 = *reinterpret_cast<const uint2 *>(vrow + 4 * (3 ^ db));
             const pf_u4 v1 = {a0.x, a0.y, a1.x, a1.y}, v2 = {a2.x, a2.y, a3.x, a3.y};
             o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v1), p1, o[db], 0, 0, 0);
             o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v2), p2, o[db], 0, 0, 0);
@@ -200,10 +245,17 @@ int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t str
     while (hpw > 8 || a.group % hpw) --hpw;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * hpw));
-    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_LAUNCH((attn_chunk_kernel<MESH_F16, MESH_F16>), grid, block, 0, stream, a, T, pos0, seq, hpw);
-    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_chunk_kernel<MESH_Q8_0, MESH_Q4_0>), grid, block, 0, stream, a, T, pos0, seq, hpw);
-    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) MESH_LAUNCH((attn_chunk_kernel<MESH_Q4_0, MESH_Q4_0>), grid, block, 0, stream, a, T, pos0, seq, hpw);
+#define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
+    do {                                                                                                                  \
+        if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw);        \
+        else if (hpw >= 2) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4>), grid, block, 0, stream, a, T, pos0, seq, hpw);   \
+        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 8>), grid, block, 0, stream, a, T, pos0, seq, hpw);                  \
+    } while (0)
+    if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_CHUNK_LAUNCH(MESH_F16, MESH_F16);
+    else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q8_0, MESH_Q4_0);
+    else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q4_0, MESH_Q4_0);
     else return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: KV cache types %d/%d", a.k_type, a.v_type);
+#undef MESH_CHUNK_LAUNCH
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
