@@ -461,8 +461,13 @@ def bench_shape(args):
         H = cfg["n_head"]
         FF = cfg["n_ff_exp"] * cfg["n_expert_used"] if cfg.get("n_expert") else cfg["n_ff"]      # FFN rows a token passes through
         mm_flop = 2.0 * T * L * (E * H * HD * 2 + E * HK * HD * 2 + 3 * E * FF)
+        ses.profile(True)
+        pstep(0)
+        pprof = ses.profile_read()
+        ses.profile(False)
         prefill = {"tokens": T, "ms": round(pms, 2), "tok_s": round(T * 1e3 / pms, 1), "matmul_TFLOP": round(mm_flop / 1e12, 2),
-                   "matmul_TFLOPs_over_whole_step": round(mm_flop / pms / 1e9, 1)}
+                   "matmul_TFLOPs_over_whole_step": round(mm_flop / pms / 1e9, 1),
+                   "kernel_ms": {k: round(v["ms"], 2) for k, v in pprof.items()}}
     head = results[batches[0]]
     out = {"metric": sp["metric"], "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -39,6 +39,9 @@ struct AttnArgs {
     _Float16 *out16_k8 = nullptr;
     // or, when set, quantised into the q16 activation layout of the skinny GEMM (gemm.hpp), also instead of `out`
     uint8_t *out_q16 = nullptr;
+    // attention_chunk only, optional: scratch of 2 * n_kv * n_ctx * head_dim f16 values; with it a long chunk over a
+    // quantised cache decodes the rows it needs once, into the scratch, instead of once per query tile
+    _Float16 *chunk_kv16 = nullptr;
     float scale = 1.f;
     int n_head = 0, n_kv = 0, group = 1, head_dim = 0, n_ctx = 0, n_splits = 1;
 };

@@ -24,14 +24,16 @@
 namespace mesh {
 
 constexpr int PF_HD = 128;
-constexpr int PF_TILE = 32;                 // queries per workgroup and keys per step
+constexpr int PF_TILE = 32;                 // queries per workgroup
+constexpr int PF_KEYS = 64;                 // keys per step (two MFMA tiles)
 constexpr int PF_KPITCH = PF_HD + 8;        // halfs per key row of the K tile in LDS (bank-conflict padding)
-constexpr int PF_VPITCH = PF_TILE / 2 + 2;  // dwords (key pairs) per dim row of the transposed V tile
+constexpr int PF_VPITCH = PF_KEYS / 2 + 2;  // dwords (key pairs) per dim row of the transposed V tile
 
 // Column (dword) of key pair kp in dim row `dim` of the transposed V tile.  Rows 32 apart start on the same LDS bank
-// (32 * 18 dwords is a multiple of the 64 banks), and the staging writes of a wave touch four such rows at once; the
+// (32 * 34 dwords is a multiple of the 64 banks), and the staging writes of a wave touch four such rows at once; the
 // XOR moves them onto different banks.  It keeps dwords 2j, 2j + 1 neighbours, which the 8-byte fragment reads need.
 __device__ __forceinline__ int pf_vcol(int dim, int kp) { return kp ^ ((dim >> 5) << 2); }
+constexpr int PF_EXPAND_MIN_T = 128;         // chunks from this many tokens decode a quantised cache to f16 once, ahead of the walk
 constexpr float PF_RESCALE_STEP = 8.f;      // the softmax reference moves only when the running maximum exceeds it by this (log2)
 
 typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
@@ -59,15 +61,18 @@ __device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
     }
 }
 
-// NP: (key, 8-dim piece) pairs of a tile one thread carries, at least 512 / (threads of the workgroup).
+// NP: (key, 8-dim piece) pairs of a step one thread carries in registers, at least 1024 / (threads of the workgroup);
+// 0 for small workgroups, which load each step's rows where they write them.
 template <int KT, int VT, int NP>
 __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw) {
     constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
-    __shared__ __align__(16) _Float16 sK[PF_TILE * PF_KPITCH];
+    __shared__ __align__(16) _Float16 sK[PF_KEYS * PF_KPITCH];
     __shared__ __align__(16) uint32_t sVt[PF_HD * PF_VPITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
     const int qcol = lane & 31, half = lane >> 5;
-    const int qt = blockIdx.x, kvh = blockIdx.y;
+    // the last query tile of a chunk walks the most keys: the launch hands the tiles out from the last one backwards, so
+    // that the longest walks start first when the workgroups do not all fit on the chip at once
+    const int qt = (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
     const int h = kvh * a.group + blockIdx.z * hpw + wave;
     const int tq = qt * PF_TILE + qcol;
     const bool q_live = tq < T;
@@ -96,86 +101,112 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
     const int q_end = qt * PF_TILE + PF_TILE < T ? qt * PF_TILE + PF_TILE : T;      // queries of this tile: [qt*32, q_end)
     const int n_keys = pos0 + q_end;                                                // keys any of them may see
-    // The rows of a tile travel through registers: a thread fetches its share of tile k0 + 32 right after it has written
-    // that of tile k0 to LDS, so the loads are in flight while the tile is multiplied.  K: (key, 8-dim piece) pairs, 16
-    // bytes each.  V: the same 8 dims of two neighbouring keys, so that the transposed tile is written as dwords.
-    // Rows past the context end are clamped (masked below).
-    constexpr int NPV = (NP + 1) / 2;
-    uint4 rk[NP], rv[NPV][2];
-    auto fetch_tile = [&](int k0) {
+    // K is staged as it is: (key, 8-dim piece) pairs, 16 bytes each.  V is staged transposed: an item is the same 8 dims
+    // of two neighbouring keys, written as 8 dwords, one per dim, each holding the pair of keys.  Rows past the context
+    // end are clamped (masked below).
+    auto k_row = [&](int k0, int p) {
+        int kr = k0 + (p >> 4);
+        kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
+        return pf_row_piece<KT>(a.kcache + (base + kr) * KRB, p & 15);
+    };
+    auto v_row = [&](int k0, int p, int second) {
+        int kr = k0 + 2 * (p >> 4) + second;
+        kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
+        return pf_row_piece<VT>(a.vcache + (base + kr) * VRB, p & 15);
+    };
+    auto k_put = [&](int p, const uint4 &r) { *reinterpret_cast<uint4 *>(sK + (p >> 4) * PF_KPITCH + (p & 15) * 8) = r; };
+    auto v_put = [&](int p, const uint4 &r0, const uint4 &r1) {
+        const int kp = p >> 4, piece = p & 15;
+        const uint32_t w0[4] = {r0.x, r0.y, r0.z, r0.w}, w1[4] = {r1.x, r1.y, r1.z, r1.w};
+        uint32_t *dst = sVt + piece * 8 * PF_VPITCH + pf_vcol(piece * 8, kp);
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int p = tid + i * nthreads;
-            if (p < PF_TILE * 16) {
-                int kr = k0 + (p >> 4);
-                kr = kr < a.n_ctx ? kr : a.n_ctx - 1;
-                rk[i] = pf_row_piece<KT>(a.kcache + (base + kr) * KRB, p & 15);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < NPV; ++i) {
-            const int p = tid + i * nthreads;
-            if (p < PF_TILE * 8) {
-                int kr0 = k0 + 2 * (p >> 4), kr1 = kr0 + 1;
-                kr0 = kr0 < a.n_ctx ? kr0 : a.n_ctx - 1;
-                kr1 = kr1 < a.n_ctx ? kr1 : a.n_ctx - 1;
-                rv[i][0] = pf_row_piece<VT>(a.vcache + (base + kr0) * VRB, p & 15);
-                rv[i][1] = pf_row_piece<VT>(a.vcache + (base + kr1) * VRB, p & 15);
-            }
+        for (int e2 = 0; e2 < 4; ++e2) {
+            dst[(2 * e2) * PF_VPITCH] = (w0[e2] & 0xffffu) | (w1[e2] << 16);
+            dst[(2 * e2 + 1) * PF_VPITCH] = (w0[e2] >> 16) | (w1[e2] & 0xffff0000u);
         }
     };
-    fetch_tile(0);
-    for (int k0 = 0; k0 < n_keys; k0 += PF_TILE) {
-        // the K tile as it is
+    // With NP > 0 the rows of a step travel through registers: a thread fetches its share of step k0 + 64 right after it
+    // has written that of step k0 to LDS, so the loads are in flight while the step is multiplied.
+    constexpr int NPK = NP > 0 ? NP : 1, NPV = NP > 0 ? (NP + 1) / 2 : 1;
+    uint4 rk[NPK], rv[NPV][2];
+    auto fetch_step = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
+        for (int i = 0; i < NPK; ++i) {
             const int p = tid + i * nthreads;
-            if (p < PF_TILE * 16) *reinterpret_cast<uint4 *>(sK + (p >> 4) * PF_KPITCH + (p & 15) * 8) = rk[i];
+            if (p < PF_KEYS * 16) rk[i] = k_row(k0, p);
         }
-        // the V tile transposed: 8 dwords, one per dim, each holding the pair of keys
 #pragma unroll
         for (int i = 0; i < NPV; ++i) {
             const int p = tid + i * nthreads;
-            if (p < PF_TILE * 8) {
-                const int kp = p >> 4, piece = p & 15;
-                const uint32_t w0[4] = {rv[i][0].x, rv[i][0].y, rv[i][0].z, rv[i][0].w}, w1[4] = {rv[i][1].x, rv[i][1].y, rv[i][1].z, rv[i][1].w};
-                uint32_t *dst = sVt + piece * 8 * PF_VPITCH + pf_vcol(piece * 8, kp);
+            if (p < PF_KEYS * 8) { rv[i][0] = v_row(k0, p, 0); rv[i][1] = v_row(k0, p, 1); }
+        }
+    };
+    if constexpr (NP > 0) fetch_step(0);
+    for (int k0 = 0; k0 < n_keys; k0 += PF_KEYS) {
+        if constexpr (NP > 0) {
 #pragma unroll
-                for (int e2 = 0; e2 < 4; ++e2) {
-                    dst[(2 * e2) * PF_VPITCH] = (w0[e2] & 0xffffu) | (w1[e2] << 16);
-                    dst[(2 * e2 + 1) * PF_VPITCH] = (w0[e2] >> 16) | (w1[e2] & 0xffff0000u);
-                }
+            for (int i = 0; i < NPK; ++i) {
+                const int p = tid + i * nthreads;
+                if (p < PF_KEYS * 16) k_put(p, rk[i]);
             }
+#pragma unroll
+            for (int i = 0; i < NPV; ++i) {
+                const int p = tid + i * nthreads;
+                if (p < PF_KEYS * 8) v_put(p, rv[i][0], rv[i][1]);
+            }
+        } else {
+            for (int p = tid; p < PF_KEYS * 16; p += nthreads) k_put(p, k_row(k0, p));
+            for (int p = tid; p < PF_KEYS * 8; p += nthreads) v_put(p, v_row(k0, p, 0), v_row(k0, p, 1));
         }
         __syncthreads();
-        if (k0 + PF_TILE < n_keys) fetch_tile(k0 + PF_TILE);
-
-        // S^T = K . Q^T : lane (key row = lane % 32 of the A operand, query column = lane % 32 of the result)
-        pf_f16v s;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#pragma unroll
-        for (int kc = 0; kc < 8; ++kc) {
-            const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + qcol * PF_KPITCH + kc * 16 + 8 * half);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s, 0, 0, 0);
+        if constexpr (NP > 0) {
+            if (k0 + PF_KEYS < n_keys) fetch_step(k0 + PF_KEYS);
         }
-        // register i of the result is key k0 + 8 * (i / 4) + 4 * half + i % 4 for query qcol.  Only a tile that reaches
-        // past the first query's position has anything to mask (a dead query column has q = 0 and is never stored).
-        if (k0 + PF_TILE - 1 > pos0 + qt * PF_TILE) {
+        // the second 32 keys of the step lie past every query of the tile at the end of the walk
+        const bool two = k0 + 32 < n_keys;
+
+        // S^T = K . Q^T, two tiles of 32 keys x 32 queries: lane (key row = lane % 32 of the A operand, query column =
+        // lane % 32 of the result); two independent accumulation chains
+        pf_f16v s[2];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = k0 + 8 * (i >> 2) + 4 * half + (i & 3);
-                s[i] = key <= pos_q ? s[i] : -INFINITY;
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[t][i] = t == 0 ? 0.f : (two ? 0.f : -INFINITY);
+        if (two) {
+#pragma unroll
+            for (int kc = 0; kc < 8; ++kc)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + (32 * t + qcol) * PF_KPITCH + kc * 16 + 8 * half);
+                    s[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s[t], 0, 0, 0);
+                }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < 8; ++kc) {
+                const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + qcol * PF_KPITCH + kc * 16 + 8 * half);
+                s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s[0], 0, 0, 0);
             }
         }
-        float mx = s[0];
+        // register i of tile t is key k0 + 32 * t + 8 * (i / 4) + 4 * half + i % 4 for query qcol.  Only a step that
+        // reaches past the first query's position has anything to mask (a dead query column has q = 0 and is never stored).
+        if (k0 + PF_KEYS - 1 > pos0 + qt * PF_TILE) {
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
+                    s[t][i] = key <= pos_q ? s[t][i] : -INFINITY;
+                }
+        }
+        float mx0 = s[0][0], mx1 = s[1][0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) { mx0 = fmaxf(mx0, s[0][i]); mx1 = fmaxf(mx1, s[1][i]); }
+        float mx = fmaxf(mx0, mx1);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         // m is the reference the exponentials are taken against.  It follows the running maximum only when that has
         // moved by more than PF_RESCALE_STEP (log2 units), so that most steps skip the rescale of the 64 accumulator
         // registers; in between p <= 2^PF_RESCALE_STEP, which f16 holds comfortably.  (Key 0 is visible to every
-        // query, so after the first tile m is finite for every live column.)
+        // query, so after the first step m is finite for every live column.)
         if (__builtin_amdgcn_ballot_w64(mx > m + PF_RESCALE_STEP) != 0ull) {
             const float m_new = mx > m + PF_RESCALE_STEP ? mx : m;
             const float corr = exp2f(m - m_new);                    // exp2(-inf) = 0 while nothing is accumulated; 1 for lanes that stay
@@ -186,24 +217,37 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o[db][i] *= corr;
         }
-        float p[16], ps = 0.f;
+        // P^T as the B operand: the lane's own registers, 8 per MFMA
+        pf_h8 pf[2][2];
+        float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { p[i] = __builtin_amdgcn_exp2f(s[i] - m); ps += p[i]; }     // s - m <= PF_RESCALE_STEP; far below, 0
+        for (int t = 0; t < 2; ++t) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(s[t][i] - m);     // s - m <= PF_RESCALE_STEP; far below, 0
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) { ps0 += p[i]; ps1 += p[i + 1]; }
+            const pf_u4 pu1 = {pf_pack(p[0], p[1]), pf_pack(p[2], p[3]), pf_pack(p[4], p[5]), pf_pack(p[6], p[7])};
+            const pf_u4 pu2 = {pf_pack(p[8], p[9]), pf_pack(p[10], p[11]), pf_pack(p[12], p[13]), pf_pack(p[14], p[15])};
+            pf[t][0] = __builtin_bit_cast(pf_h8, pu1);
+            pf[t][1] = __builtin_bit_cast(pf_h8, pu2);
+        }
+        float ps = ps0 + ps1;
         ps += __shfl_xor(ps, 32);
         l += ps;
-        // P^T as the B operand: the lane's own registers, 8 per MFMA
-        const pf_u4 pu1 = {pf_pack(p[0], p[1]), pf_pack(p[2], p[3]), pf_pack(p[4], p[5]), pf_pack(p[6], p[7])};
-        const pf_u4 pu2 = {pf_pack(p[8], p[9]), pf_pack(p[10], p[11]), pf_pack(p[12], p[13]), pf_pack(p[14], p[15])};
-        const pf_h8 p1 = __builtin_bit_cast(pf_h8, pu1), p2 = __builtin_bit_cast(pf_h8, pu2);
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-            // dim row db * 32 + qcol, this half's keys: key pairs 2 * half + 4 * j (+ 1), j = 0 .. 3
+            // dim row db * 32 + qcol, this half's keys of tile t: key pairs 16 * t + 2 * half + 4 * j (+ 1), j = 0 .. 3
             const uint32_t *vrow = sVt + (db * 32 + qcol) * PF_VPITCH + 2 * half;
-            const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow + 4 * (0 ^ db)), a1 = *reinterpret_cast<const uint2 *>(vrow + 4 * (1 ^ db));
-            const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 4 * (2 ^ db)), a3 = *reinterpret_cast<const uint2 *>(vrow + 4 * (3 ^ db));
-            const pf_u4 v1 = {a0.x, a0.y, a1.x, a1.y}, v2 = {a2.x, a2.y, a3.x, a3.y};
-            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v1), p1, o[db], 0, 0, 0);
-            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v2), p2, o[db], 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (t == 1 && !two) break;
+                const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (0 ^ db)), a1 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (1 ^ db));
+                const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (2 ^ db)), a3 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (3 ^ db));
+                const pf_u4 v1 = {a0.x, a0.y, a1.x, a1.y}, v2 = {a2.x, a2.y, a3.x, a3.y};
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v1), pf[t][0], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v2), pf[t][1], o[db], 0, 0, 0);
+            }
         }
         __syncthreads();        // the tiles are overwritten by the next step
     }
@@ -236,20 +280,54 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
     }
 }
 
-int attention_chunk(const AttnArgs &a, int T, int pos0, int seq, hipStream_t stream) {
+// Rows [0, n_keys) of one sequence's K and V, every KV head, as f16 rows [n_kv][n_ctx][128] (the values the staging
+// of attn_chunk_kernel would decode): one thread per (row, 8-dim piece).
+template <int KT, int VT>
+__global__ __launch_bounds__(256) void kv_expand_kernel(const uint8_t *kcache, const uint8_t *vcache, uint4 *k16, uint4 *v16, int n_keys, int n_ctx,
+                                                        int n_kv, int seq) {
+    constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int piece = (int)(idx & 15);
+    const size_t row = idx >> 4;
+    if (row >= (size_t)n_kv * n_keys) return;
+    const int kvh = (int)(row / n_keys), key = (int)(row % n_keys);
+    const size_t src = ((size_t)seq * n_kv + kvh) * n_ctx + key, dst = (size_t)kvh * n_ctx + key;
+    k16[dst * 16 + piece] = pf_row_piece<KT>(kcache + src * KRB, piece);
+    v16[dst * 16 + piece] = pf_row_piece<VT>(vcache + src * VRB, piece);
+}
+
+int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
+    AttnArgs a = a_in;
     if (a.head_dim != PF_HD) return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: head_dim %d (128 only)", a.head_dim);
     if (a.group < 1 || a.n_head != a.group * a.n_kv || pos0 < 0 || pos0 + T > a.n_ctx || seq < 0)
         return fail(MESH_ERR_INVALID, "attention_chunk: bad head layout or chunk [%d, %d) outside the context of %d", pos0, pos0 + T, a.n_ctx);
+    if (a.k_type != MESH_F16 && a.chunk_kv16 && T >= PF_EXPAND_MIN_T) {
+        // Every query tile's workgroup would decode the quantised rows it walks.  Decode them once instead, into the
+        // caller's f16 scratch, and run the f16 kernel on that: the same values reach the matrix cores.
+        const int n_keys = pos0 + T;
+        uint4 *k16 = reinterpret_cast<uint4 *>(a.chunk_kv16), *v16 = k16 + (size_t)a.n_kv * a.n_ctx * 16;
+        const unsigned blocks = (unsigned)(((size_t)a.n_kv * n_keys * 16 + 255) / 256);
+        if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0)
+            MESH_LAUNCH((kv_expand_kernel<MESH_Q8_0, MESH_Q4_0>), dim3(blocks), dim3(256), 0, stream, a.kcache, a.vcache, k16, v16, n_keys, a.n_ctx, a.n_kv, seq);
+        else if (a.k_type == MESH_Q4_0 && a.v_type == MESH_Q4_0)
+            MESH_LAUNCH((kv_expand_kernel<MESH_Q4_0, MESH_Q4_0>), dim3(blocks), dim3(256), 0, stream, a.kcache, a.vcache, k16, v16, n_keys, a.n_ctx, a.n_kv, seq);
+        else return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: KV cache types %d/%d", a.k_type, a.v_type);
+        MESH_LAUNCH_CHECK();
+        a.kcache = reinterpret_cast<const uint8_t *>(k16);
+        a.vcache = reinterpret_cast<const uint8_t *>(v16);
+        a.k_type = a.v_type = MESH_F16;
+        seq = 0;
+    }
     int hpw = a.group;                       // heads (waves) per workgroup: the largest divisor of the group up to 8
     while (hpw > 8 || a.group % hpw) --hpw;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * hpw));
 #define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
     do {                                                                                                                  \
-        if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw);        \
-        else if (hpw >= 2) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4>), grid, block, 0, stream, a, T, pos0, seq, hpw);   \
-        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 8>), grid, block, 0, stream, a, T, pos0, seq, hpw);                  \
+        if (hpw == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw);        \
+        else if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4>), grid, block, 0, stream, a, T, pos0, seq, hpw);   \
+        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 0>), grid, block, 0, stream, a, T, pos0, seq, hpw);                  \
     } while (0)
     if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_CHUNK_LAUNCH(MESH_F16, MESH_F16);
     else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q8_0, MESH_Q4_0);

@@ -392,6 +392,15 @@ int session_new(mesh_stage *st, mesh_session **out) {
             if ((rc = sess_alloc(s.get(), &p, bytes)) != MESH_OK) return rc;
             s->xq = static_cast<uint8_t *>(p);
         }
+        const char *ckv = getenv("MESH_CHUNK_KV16");      // =0 at session creation: every query tile decodes the quantised rows itself
+        if (st->k_type != MESH_F16 && hp.head_dim == 128 && B >= 128 && !(ckv && atoi(ckv) == 0)) {
+            // f16 copy of one sequence's K and V rows of one layer: a long prefill chunk decodes the quantised cache once
+            // per layer into it (attn.hpp: chunk_kv16).  Zeroed, so that rows past a chunk's last key are finite.
+            const size_t bytes = 2 * (size_t)hp.n_head_kv * st->n_ctx * hp.head_dim * 2;
+            if ((rc = sess_alloc(s.get(), &p, bytes)) != MESH_OK) return rc;
+            s->chunk_kv16 = static_cast<uint16_t *>(p);
+            MESH_HIP_TRY(hipMemsetAsync(p, 0, bytes, s->stream));
+        }
         if (hp.n_ff > 0) {
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
@@ -640,6 +649,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         ProfScope ps(s, MESH_PROF_ATTN);
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) {
             if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }          // straight into the output projection's input layout
+            aa.chunk_kv16 = reinterpret_cast<_Float16 *>(s->chunk_kv16);
             rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
         }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {

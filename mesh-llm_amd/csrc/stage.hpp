@@ -87,6 +87,7 @@ struct mesh_session {
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
     uint16_t *xn16 = nullptr, *ffn16 = nullptr;
+    uint16_t *chunk_kv16 = nullptr;      // quantised KV caches: f16 rows of one sequence and layer for long prefill chunks (attn.hpp)
     size_t xq_tokens = 0;               // tokens the q16 buffer below is sized for
     uint8_t *xq = nullptr;               // 16-bit fixed-point activations of the skinny GEMM (gemm.hpp: q16 layout)
     float *gemm_part = nullptr;          // partial tiles of large-tile GEMM launches that split K (gemm.hpp)

@@ -108,7 +108,7 @@ def test_stage_with_quantised_kv_matches_oracle(tmp_path, name, kv_types):
 
 
 @pytest.mark.parametrize("kv_types", PAIRS)
-def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types):
+def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types, monkeypatch):
     """Two real-shape layers over a 300-deep quantised cache: split-KV decode at batch 1 and 4, the batched (skinny
     GEMM) path at batch 9, and a 200-token prefill chunk through the matrix-core attention kernel."""
     name = "llama3-8b"
@@ -148,6 +148,23 @@ def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types):
     ref = orc.forward(xp, np.arange(T), seq=np.full(T, 9, np.int32))
     assert rel_l2(got, ref) <= 3e-2
     assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 8e-2
+    # a second chunk on top of the first (136 tokens at positions 200 .. 335): chunks this long decode the cache rows
+    # they attend to once, into an f16 scratch, before the walk; that has to cover the first chunk's rows too
+    T2 = 136
+    xp2 = rng.standard_normal((T2, 4096)).astype(np.float32)
+    got2 = ses.decode(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32)).view(np.float32).reshape(T2, 4096)
+    ref2 = orc.forward(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32))
+    assert rel_l2(got2, ref2) <= 3e-2
+    ses.close()
+    # the same two chunks with the scratch switched off (every query tile decodes the rows itself): the same values
+    # reach the matrix cores in the same order, so the hidden states are bit-identical
+    monkeypatch.setenv("MESH_CHUNK_KV16", "0")
+    ses = st.session()
+    monkeypatch.delenv("MESH_CHUNK_KV16")
+    got_b = ses.decode(xp, np.arange(T), seq=np.full(T, 9, np.int32)).view(np.float32).reshape(T, 4096)
+    got2_b = ses.decode(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32)).view(np.float32).reshape(T2, 4096)
+    assert np.array_equal(got_b.view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(got2_b.view(np.uint32), got2.view(np.uint32))
     ses.close()
     st.close()
 
