@@ -230,15 +230,27 @@ template <> struct PackedSub<MESH_Q6_K> {
 // 16 k is four contiguous 256-byte pieces of that layout, so each lane fetches its 16 bytes straight from memory (L2),
 // four k16 steps ahead, into a ring of registers.  That halves the LDS reads per MFMA and leaves the staging waves only
 // the weights.
-template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW>
+// GROUPED: an expert launch (gemm.hpp): the workgroup's token tile and matrix come from a.tiles[blockIdx.y].
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW, bool GROUPED = false>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
+    static_assert(!GROUPED || (PACKED && XDIRECT && !SPLIT && !NARROW), "expert launches: GEMM layout, k8-major activations, one k range");
     extern __shared__ __align__(16) _Float16 gemm_smem[];
     _Float16 *Ws = gemm_smem;                                  // [2][GM][LDS_LD]
     _Float16 *Xs = gemm_smem + 2 * GM * LDS_LD;                // [2][GN][LDS_LD]
     constexpr int TB = TYPE == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int m0 = blockIdx.x * GM, t0 = blockIdx.y * GN;
+    // token tile [t0, t_end) of this workgroup and its matrix
+    int t0 = blockIdx.y * GN, t_end = a.T;
+    const uint8_t *Wp = static_cast<const uint8_t *>(a.Wp);
+    if constexpr (GROUPED) {
+        if ((int)blockIdx.y >= *a.n_tiles) return;
+        const int4 tl = reinterpret_cast<const int4 *>(a.tiles)[blockIdx.y];
+        Wp += (size_t)tl.x * a.expert_stride;
+        t0 = tl.y;
+        t_end = tl.y + tl.z;
+    }
+    const int m0 = blockIdx.x * GM;
     const int nsb = a.K / QK_K, n_all = a.K / GK;
     // k-steps [k0, k0 + n_steps) of this workgroup: all of them, or slice blockIdx.z of a split launch
     // (a template parameter: the unsplit kernel must not carry the offsets, they cost it 6%)
@@ -251,7 +263,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         const int srow = st >> 1, sh = st & 1;
         const int wrow = m0 + srow;                                  // rows beyond M are zero tiles (M padded to 16)
         const bool wlive = PACKED || wrow < a.M_pad;                 // (the GEMM layout holds its zero rows)
-        const uint8_t *wtile_row = PACKED ? static_cast<const uint8_t *>(a.Wp) + ((size_t)blockIdx.x * n_all + k0) * PackedSub<TYPE>::CHUNK
+        const uint8_t *wtile_row = PACKED ? Wp + ((size_t)blockIdx.x * n_all + k0) * PackedSub<TYPE>::CHUNK
                                           : static_cast<const uint8_t *>(a.W) + (size_t)((wlive ? wrow : 0) >> 4) * nsb * TB;
         using Sub = typename std::conditional<PACKED, PackedSub<TYPE>, RawSub<TYPE>>::type;
         const int tok = t0 + srow;
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
         }
         __syncthreads();
         if (is_up) return;
-        const int t_pad = (a.T + 15) & ~15;
+        const int t_pad = (t_end + 15) & ~15;
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -431,7 +443,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         const float g = acc[i][j][4 * e4 + c], u = xch[((pair + i * 2 + j) * 16 + 4 * e4 + c) * 64 + lane];
-                        o[c] = t < a.T ? g / (1.0f + expf(-g)) * u : 0.f;       // padding columns of the last token block hold zeros
+                        o[c] = t < t_end ? g / (1.0f + expf(-g)) * u : 0.f;       // padding columns of the last token block hold zeros
                     }
                     *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
                         make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
@@ -457,7 +469,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int t = t0 + wn + 32 * j + (lane & 31);
-            if (t >= a.T) continue;
+            if (t >= t_end) continue;
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
                 const int m = mb0 + wm + 32 * i + 8 * e4 + 4 * (lane >> 5);
@@ -776,16 +788,16 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
     }
 }
 
-template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW>
+template <int TYPE, bool PACKED, bool XDIRECT, bool SPLIT, bool NARROW, bool GROUPED = false>
 static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) {
     // two stages of the weight slab, and of the activation slab unless the activations bypass LDS: 73 728 / 36 864 B
     constexpr size_t smem = sizeof(_Float16) * 2 * (GM + (XDIRECT ? 0 : GN)) * LDS_LD;
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW, GROUPED>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    MESH_LAUNCH((gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW>), grid, dim3(GEMM_THREADS), smem, stream, k);
+    MESH_LAUNCH((gemm_kq_kernel<TYPE, PACKED, XDIRECT, SPLIT, NARROW, GROUPED>), grid, dim3(GEMM_THREADS), smem, stream, k);
     MESH_LAUNCH_CHECK();
     if (SPLIT) {
         const int t_pad = k.y16_k8 ? (k.T + 15) & ~15 : k.T;
@@ -861,6 +873,17 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     GemmArgs k = a;
     k.M_pad = (a.M + TILE_ROWS - 1) / TILE_ROWS * TILE_ROWS;
     const int row_blocks = a.y16_k8 ? (a.M + GM / 2 - 1) / (GM / 2) : (a.M + GM - 1) / GM;
+    if (a.tiles) {
+        // expert launch: one workgroup row per tile of the list (those past *n_tiles leave at once)
+        if (!a.Wp || !a.x_k8 || !a.n_tiles || a.max_tiles <= 0 || a.n_seg > 1 || a.bias || a.residual || a.rope.pos || a.expert_stride % 16)
+            return fail(MESH_ERR_INVALID, "gemm: an expert launch needs the GEMM layout, k8-major activations and a plain or SwiGLU epilogue");
+        if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
+        const dim3 g((unsigned)row_blocks, (unsigned)a.max_tiles);
+        k.ksplit = 1;
+        k.k_per_split = a.K / GK;
+        return a.type == MESH_Q4_K ? launch_gemm_kernel<MESH_Q4_K, true, true, false, false, true>(k, g, stream)
+                                   : launch_gemm_kernel<MESH_Q6_K, true, true, false, false, true>(k, g, stream);
+    }
     dim3 grid((unsigned)row_blocks, (unsigned)((a.T + GN - 1) / GN));
     // A launch of fewer workgroups than CUs walks all of K in each of them while the rest of the chip idles: split K
     // over blockIdx.z (slices of at least 8 k-steps, at most one workgroup per CU in total, partial tiles within the

@@ -43,6 +43,14 @@ struct GemmArgs {
     // the f16 KV cache instead of storing them to their outputs, like the projection epilogues of the decode kernels.
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+    // Expert launch (mixture of experts; GEMM layout and k8-major activations only, plain store or SwiGLU): X holds the
+    // (token, slot) pairs sorted by expert (moe.hpp: moe_sort), T is its capacity in pair slots, and tile i of `tiles` =
+    // {expert, first slot, slots, 0} multiplies slots [first, first + slots) (at most 128; first a multiple of 16) by the
+    // matrix at Wp + expert * expert_stride.  *n_tiles (device) tiles are live, max_tiles bounds them for the grid.
+    // Outputs are indexed by slot.
+    const int32_t *tiles = nullptr, *n_tiles = nullptr;
+    size_t expert_stride = 0;
+    int max_tiles = 0;
 };
 int gemm_kquant(const GemmArgs &a, hipStream_t stream);
 // Number of K slices gemm_kquant will use for this launch (1: not split).
@@ -100,6 +108,8 @@ int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t 
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream);
 int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream);
+// the same as rmsnorm_f16_k8 for n_slots (a multiple of 16) gathered rows: slot i holds row row_of_slot[i] / row_div of x, zeros when negative
+int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream);
 int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream);
 
 int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream);

@@ -644,16 +644,24 @@ __device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {       // satu
 
 // y = f16(x[t] * rsqrt(mean(x[t]^2) + eps) * w), or with w == null just f16(x[t]); one workgroup per token slot of the
 // padded batch (slots >= T write zeros).
+// row_of_slot set: slot t takes row row_of_slot[t] / row_div of x, or zeros when that is negative (gathered expert inputs).
 __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int T, int n,
-                                                    _Float16 *__restrict__ y) {
+                                                    _Float16 *__restrict__ y, const int32_t *__restrict__ row_of_slot, int row_div) {
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     _Float16 *yb = y + (size_t)(t / 16) * 16 * n + (size_t)(t % 16) * 8;        // element (t, k) at yb + (k / 8) * 128 + k % 8
-    if (t >= T) {
+    int src = t;
+    bool dead = t >= T;
+    if (row_of_slot && !dead) {
+        const int r = row_of_slot[t];
+        dead = r < 0;
+        src = r / row_div;
+    }
+    if (dead) {
         for (int i = tid * 8; i < n; i += 2048) *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = make_uint4(0u, 0u, 0u, 0u);
         return;
     }
-    const float *xt = x + (size_t)t * n;
+    const float *xt = x + (size_t)src * n;
     constexpr int RC = 4;                                   // rows of up to 2048 * RC elements stay in registers: one read
     if (w && n <= 2048 * RC) {
         float4 v[RC][2], g[RC][2];
@@ -718,7 +726,15 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
-    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y);
+    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y, (const int32_t *)nullptr, 1);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream) {
+    if (n_slots <= 0) return MESH_OK;
+    if (n % 8 || n_slots % 16 || !row_of_slot || row_div < 1) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8_gather: bad arguments (row length %d, %d slots)", n, n_slots);
+    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)n_slots), dim3(256), 0, stream, x, w, eps, n_slots, n, y, row_of_slot, row_div);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

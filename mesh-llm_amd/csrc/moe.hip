@@ -4,6 +4,8 @@
 // softmax of the router logits over every expert in the file; a 0 / -inf mask is ADDED to the probabilities used
 // for selection only; the weights are the unmasked probabilities of the selected experts, renormalised to sum 1.
 
+#include <algorithm>
+
 #include "moe.hpp"
 #include "gemv.hpp"
 
@@ -323,6 +325,92 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float *__restrict__ x,
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     MESH_LAUNCH(moe_combine_kernel, dim3((unsigned)((n_embd + 255) / 256), (unsigned)T), dim3(256), 0, stream, x, y, w, n_embd, top_k);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// the same with the rows of y at the slots of moe_sort: x[t][i] += sum_s w[t][s] * y[slot_of_pair[t*top_k + s]][i], four columns a thread
+__global__ __launch_bounds__(256) void moe_combine_slots_kernel(float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ w,
+                                                                const int32_t *__restrict__ slot_of_pair, int n_embd, int top_k) {
+    const int t = blockIdx.y;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n_embd) return;
+    float4 acc = *reinterpret_cast<const float4 *>(x + (size_t)t * n_embd + i);
+    for (int s = 0; s < top_k; ++s) {
+        const float ws = w[(size_t)t * top_k + s];
+        const float4 v = *reinterpret_cast<const float4 *>(y + (size_t)slot_of_pair[(size_t)t * top_k + s] * n_embd + i);
+        acc.x = fmaf(ws, v.x, acc.x); acc.y = fmaf(ws, v.y, acc.y); acc.z = fmaf(ws, v.z, acc.z); acc.w = fmaf(ws, v.w, acc.w);
+    }
+    *reinterpret_cast<float4 *>(x + (size_t)t * n_embd + i) = acc;
+}
+
+int moe_combine_slots(float *x, const float *y, const float *w, const int32_t *slot_of_pair, int T, int n_embd, int top_k, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (n_embd % 4) return fail(MESH_ERR_INVALID, "moe_combine_slots: row length %d not a multiple of 4", n_embd);
+    MESH_LAUNCH(moe_combine_slots_kernel, dim3((unsigned)((n_embd / 4 + 255) / 256), (unsigned)T), dim3(256), 0, stream, x, y, w, slot_of_pair, n_embd, top_k);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// ---- pairs sorted by expert for the large-tile GEMM ------------------------------------------------------------
+// One workgroup: counts per expert (LDS atomics), a scan over the experts for the first slot (a multiple of 16) and the
+// first tile of each, then every pair takes the next free slot of its expert.  Which slot of its expert a pair gets
+// depends on the order the atomics land in; nothing computed from the slots does (a column of a matrix product depends
+// on that column alone, and the combine step finds its rows through slot_of_pair).
+constexpr int SORT_THREADS = 1024;
+__global__ __launch_bounds__(SORT_THREADS) void moe_sort_kernel(const int32_t *__restrict__ ids, int n_pairs, int n_expert, int cap_slots,
+                                                                int32_t *__restrict__ slot_of_pair, int32_t *__restrict__ pair_of_slot,
+                                                                int32_t *__restrict__ tiles, int32_t *__restrict__ counts) {
+    extern __shared__ int32_t s_lds[];
+    int32_t *s_cnt = s_lds, *s_off = s_cnt + n_expert, *s_tile = s_off + n_expert, *s_cur = s_tile + n_expert;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < n_expert; e += SORT_THREADS) { s_cnt[e] = 0; s_cur[e] = 0; }
+    for (int sl = tid; sl < cap_slots; sl += SORT_THREADS) pair_of_slot[sl] = -1;
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += SORT_THREADS) atomicAdd(&s_cnt[ids[p]], 1);
+    __syncthreads();
+    if (wave == 0) {
+        // exclusive prefixes of padded slots and of tiles per expert: each lane sums a run of experts, the runs are scanned across the wave
+        const int per = (n_expert + 63) / 64, e0 = lane * per;
+        int my_s = 0, my_t = 0;
+        for (int e = e0; e < e0 + per && e < n_expert; ++e) { my_s += (s_cnt[e] + 15) & ~15; my_t += (s_cnt[e] + 127) >> 7; }
+        int in_s = my_s, in_t = my_t;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int vs = __shfl_up(in_s, o), vt = __shfl_up(in_t, o);
+            if (lane >= o) { in_s += vs; in_t += vt; }
+        }
+        int run_s = in_s - my_s, run_t = in_t - my_t;
+        for (int e = e0; e < e0 + per && e < n_expert; ++e) {
+            s_off[e] = run_s; s_tile[e] = run_t;
+            run_s += (s_cnt[e] + 15) & ~15; run_t += (s_cnt[e] + 127) >> 7;
+        }
+        if (lane == 63) { counts[0] = in_t; counts[1] = in_s; }
+    }
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += SORT_THREADS) {
+        const int cnt = s_cnt[e];
+        for (int j = 0; j * 128 < cnt; ++j) {
+            int32_t *tl = tiles + (size_t)(s_tile[e] + j) * 4;
+            tl[0] = e; tl[1] = s_off[e] + 128 * j; tl[2] = cnt - 128 * j < 128 ? cnt - 128 * j : 128; tl[3] = 0;
+        }
+    }
+    for (int p = tid; p < n_pairs; p += SORT_THREADS) {
+        const int e = ids[p];
+        const int sl = s_off[e] + atomicAdd(&s_cur[e], 1);
+        slot_of_pair[p] = sl;
+        pair_of_slot[sl] = p;
+    }
+}
+
+int moe_sort_slots(int n_pairs, int n_expert) { return (n_pairs + 15 * std::min(n_pairs, n_expert) + 15) / 16 * 16; }
+int moe_sort_max_tiles(int n_pairs, int n_expert) { return n_pairs / 128 + std::min(n_pairs, n_expert); }
+
+int moe_sort(const int32_t *ids, int n_pairs, int n_expert, const MoeSorted &out, hipStream_t stream) {
+    if (n_pairs < 1 || n_expert < 1 || n_expert > 4096 || !ids || !out.slot_of_pair || !out.pair_of_slot || !out.tiles || !out.counts)
+        return fail(MESH_ERR_INVALID, "moe_sort: bad arguments (%d pairs, %d experts)", n_pairs, n_expert);
+    MESH_LAUNCH(moe_sort_kernel, dim3(1), dim3(SORT_THREADS), 4 * (size_t)n_expert * sizeof(int32_t), stream, ids, n_pairs, n_expert,
+                moe_sort_slots(n_pairs, n_expert), out.slot_of_pair, out.pair_of_slot, out.tiles, out.counts);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -36,4 +36,19 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 
+// The pairs sorted by expert, for the expert launches of the large-tile GEMM (gemm.hpp): the pairs of an expert take
+// consecutive slots from a multiple of 16 on (padding slots in between hold no pair), experts in ascending order, and
+// every run of up to 128 slots of one expert is a tile {expert, first slot, pairs, 0}.
+struct MoeSorted {
+    int32_t *slot_of_pair = nullptr;   // [n_pairs]
+    int32_t *pair_of_slot = nullptr;   // [moe_sort_slots()], -1 for a padding slot
+    int32_t *tiles = nullptr;          // [moe_sort_max_tiles()][4]
+    int32_t *counts = nullptr;         // [2]: tiles, slots in use
+};
+int moe_sort_slots(int n_pairs, int n_expert);         // slot capacity for any routing
+int moe_sort_max_tiles(int n_pairs, int n_expert);
+int moe_sort(const int32_t *ids, int n_pairs, int n_expert, const MoeSorted &out, hipStream_t stream);
+// x[t] += sum_s weights[t][s] * y[slot_of_pair[t*top_k + s]]
+int moe_combine_slots(float *x, const float *y, const float *w, const int32_t *slot_of_pair, int T, int n_embd, int top_k, hipStream_t stream);
+
 }  // namespace mesh

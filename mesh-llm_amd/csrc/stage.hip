@@ -188,6 +188,29 @@ struct Loader {
         }
         return MESH_OK;
     }
+    // the expert matrices of a mixture-of-experts layer, for prefill chunks (expert launches of the large-tile GEMM): every
+    // expert's gate / up pair and down projection in the GEMM layout, experts back to back
+    int pack_experts(LayerWeights &L) {
+        if (!gemm_layout) return MESH_OK;
+        const DevTensor &g = L.gate_exps, &u = L.up_exps, &d = L.down_exps;
+        if (!g.present() || !g.tiled || !u.tiled || !d.tiled || g.type != u.type || g.M != u.M || g.K != u.K || g.M % 64 || g.E != u.E || g.E != d.E) return MESH_OK;
+        const size_t pair_b = gemm_packed_pair_bytes(g.type, g.M, g.K), down_b = gemm_packed_bytes(d.type, d.M, d.K);
+        if (!pair_b || !down_b) return MESH_OK;
+        int rc;
+        if ((rc = dev_alloc(&L.exps_gate_up_gemm, pair_b * (size_t)g.E)) != MESH_OK || (rc = dev_alloc(&L.exps_down_gemm, down_b * (size_t)g.E)) != MESH_OK) return rc;
+        const size_t g_e = tiled_bytes(g.type, g.M, g.K), d_e = tiled_bytes(d.type, d.M, d.K);
+        for (int64_t e = 0; e < g.E; ++e) {
+            if ((rc = gemm_pack_pair(g.type, static_cast<const uint8_t *>(g.data) + e * g_e, static_cast<const uint8_t *>(u.data) + e * g_e,
+                                     static_cast<uint8_t *>(L.exps_gate_up_gemm) + e * pair_b, g.M, g.K, nullptr)) != MESH_OK ||
+                (rc = gemm_pack(d.type, static_cast<const uint8_t *>(d.data) + e * d_e, static_cast<uint8_t *>(L.exps_down_gemm) + e * down_b, d.M, d.K, nullptr)) != MESH_OK)
+                return rc;
+        }
+        L.exps_gate_up_stride = pair_b;
+        L.exps_down_stride = down_b;
+        st.gemm_layout_bytes += (pair_b + down_b) * (size_t)g.E;
+        MESH_HIP_TRY(hipDeviceSynchronize());
+        return MESH_OK;
+    }
 };
 
 }  // namespace
@@ -272,6 +295,7 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
                 (rc = ld.load(p + "ffn_up_exps.weight", L.up_exps, E, ffe, ne, true, true, false)) ||
                 (rc = ld.load(p + "ffn_down_exps.weight", L.down_exps, ffe, E, ne, true, true, false)))
                 return rc;
+            if ((rc = ld.pack_experts(L)) != MESH_OK) return rc;
         }
     }
     if (layer_begin == 0) {
@@ -327,6 +351,14 @@ static int gemm_min_tokens() {
     return v;
 }
 #define PREFILL_MIN_TOKENS gemm_min_tokens()
+// mixture of experts: calls with at least this many (token, slot) pairs per expert on average run the expert products as
+// tiles of the large-tile GEMM (below that, 16 pairs at a time on the integer matrix cores)
+constexpr size_t MOE_GEMM_MIN_PAIRS_PER_EXPERT = 16;
+// MESH_MOE_GEMM=0: never (for comparison)
+static bool moe_gemm_on() {
+    const char *e = getenv("MESH_MOE_GEMM");
+    return !(e && e[0] == '0');
+}
 // calls with at least this many tokens (and fewer than the above) take the skinny MFMA GEMM (MESH_SKINNY_MIN_TOKENS)
 static int skinny_min_tokens() {
     static int v = 0;
@@ -429,6 +461,24 @@ int session_new(mesh_stage *st, mesh_session **out) {
         s->moe_n_items = s->moe_items + items * MOE_ITEM_INTS;
         MESH_HIP_TRY(hipMemsetAsync(s->moe_items, 0, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t), s->stream));
         MESH_HIP_TRY(hipMemsetAsync(s->expert_mask, 0, ne * sizeof(float), s->stream));
+        if (st->layers[0].exps_gate_up_gemm && s->xn16 && B * k >= MOE_GEMM_MIN_PAIRS_PER_EXPERT * ne) {
+            // prefill chunks: the pairs sorted by expert, their inputs / SwiGLU outputs in the k8-major f16 layout and their
+            // down-projection rows, all indexed by slot (moe.hpp: moe_sort)
+            const size_t slots = (size_t)moe_sort_slots((int)(B * k), (int)ne), tiles = (size_t)moe_sort_max_tiles((int)(B * k), (int)ne);
+            const size_t pairs4 = (B * k + 3) / 4 * 4;
+            if ((rc = sess_alloc(s.get(), &p, (pairs4 + slots + 4 * tiles + 4) * sizeof(int32_t))) != MESH_OK) return rc;
+            s->moe_sorted.slot_of_pair = static_cast<int32_t *>(p);
+            s->moe_sorted.pair_of_slot = s->moe_sorted.slot_of_pair + pairs4;
+            s->moe_sorted.tiles = s->moe_sorted.pair_of_slot + slots;           // (a multiple of 16 ints in: 16-byte aligned)
+            s->moe_sorted.counts = s->moe_sorted.tiles + 4 * tiles;
+            if ((rc = sess_alloc(s.get(), &p, slots * hp.n_embd * 2)) != MESH_OK) return rc;
+            s->moe_x16 = static_cast<uint16_t *>(p);
+            if ((rc = sess_alloc(s.get(), &p, slots * (size_t)hp.n_ff_exp * 2)) != MESH_OK) return rc;
+            s->moe_ffn16 = static_cast<uint16_t *>(p);
+            if ((rc = fbuf(&s->moe_out_slots, slots * hp.n_embd)) != MESH_OK) return rc;
+            MESH_HIP_TRY(hipMemsetAsync(s->moe_x16, 0, slots * hp.n_embd * 2, s->stream));          // unused slots stay finite
+            MESH_HIP_TRY(hipMemsetAsync(s->moe_ffn16, 0, slots * (size_t)hp.n_ff_exp * 2, s->stream));
+        }
     }
     if ((rc = sess_alloc(s.get(), &p, 3 * B * sizeof(int32_t))) != MESH_OK) return rc;
     s->d_pos = static_cast<int32_t *>(p);
@@ -839,6 +889,51 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             const bool mfma = want_groups && s->xq && (size_t)T <= s->xq_tokens && T * k >= 4 * ne && E % 256 == 0 && ffe % 256 == 0 &&
                               type_is_tiled(L.gate_exps.type) && L.up_exps.type == L.gate_exps.type && type_is_tiled(L.down_exps.type) &&
                               moe_max_items(T * k, ne, SKINNY_ITEM_PAIRS) <= 65535;
+            // a prefill chunk (from MOE_GEMM_MIN_PAIRS_PER_EXPERT pairs per expert on average): the pairs sorted by expert and
+            // the expert products as tiles of the large-tile GEMM, up to 128 pairs of an expert per pass over its weights
+            const bool big = s->moe_sorted.tiles && s->moe_grouped && (size_t)T * k >= (size_t)MOE_GEMM_MIN_PAIRS_PER_EXPERT * ne &&
+                             moe_gemm_on() && E % 256 == 0 && ffe % 256 == 0;
+            if (big) {
+                if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
+                    ProfScope ps(s, MESH_PROF_GEMV);
+                    if ((rc = moe_router_fused(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
+                                               static_cast<const float *>(L.gate_inp.data), E, s->moe_logits, T, stream)) != MESH_OK) return rc;
+                } else {
+                    GemvArgs ra2;
+                    ra2.n_mat = 1;
+                    ra2.mat[0] = mat_of(L.gate_inp, s->moe_logits, ne, nullptr);
+                    ra2.x = s->x; ra2.ldx = E; ra2.K = E; ra2.T = T;
+                    ra2.norm_w = static_cast<const float *>(L.ffn_norm.data); ra2.eps = hp.rms_eps;
+                    { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ra2, stream); }
+                    if (rc != MESH_OK) return rc;
+                    if ((rc = moe_route(mr, T, stream)) != MESH_OK) return rc;
+                }
+                const int slots = moe_sort_slots(T * k, ne), max_tiles = moe_sort_max_tiles(T * k, ne);
+                {
+                    ProfScope ps(s, MESH_PROF_PREP);
+                    if ((rc = moe_sort(s->moe_ids, T * k, ne, s->moe_sorted, stream)) != MESH_OK) return rc;
+                    if ((rc = rmsnorm_f16_k8_gather(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, s->moe_sorted.pair_of_slot, k, slots, E,
+                                                    reinterpret_cast<_Float16 *>(s->moe_x16), stream)) != MESH_OK) return rc;
+                }
+                GemmArgs g;
+                g.W = L.gate_exps.data; g.Wp = L.exps_gate_up_gemm; g.type = L.gate_exps.type;
+                g.M = ffe; g.K = E; g.T = slots;
+                g.X = reinterpret_cast<const _Float16 *>(s->moe_x16); g.ldx = E; g.x_k8 = true;
+                g.y16_k8 = reinterpret_cast<_Float16 *>(s->moe_ffn16);
+                g.tiles = s->moe_sorted.tiles; g.n_tiles = s->moe_sorted.counts; g.max_tiles = max_tiles; g.expert_stride = L.exps_gate_up_stride;
+                { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_kquant(g, stream); }
+                if (rc != MESH_OK) return rc;
+                GemmArgs d;
+                d.W = L.down_exps.data; d.Wp = L.exps_down_gemm; d.type = L.down_exps.type;
+                d.M = E; d.K = ffe; d.T = slots;
+                d.X = reinterpret_cast<const _Float16 *>(s->moe_ffn16); d.ldx = ffe; d.x_k8 = true;
+                d.Y = s->moe_out_slots; d.ldy = E;
+                d.tiles = s->moe_sorted.tiles; d.n_tiles = s->moe_sorted.counts; d.max_tiles = max_tiles; d.expert_stride = L.exps_down_stride;
+                { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_kquant(d, stream); }
+                if (rc != MESH_OK) return rc;
+                if ((rc = moe_combine_slots(s->x, s->moe_out_slots, s->moe_w, s->moe_sorted.slot_of_pair, T, E, k, stream)) != MESH_OK) return rc;
+                continue;
+            }
             const int item_pairs = mfma ? SKINNY_ITEM_PAIRS : MOE_ITEM_PAIRS;
             bool grouped_done = false;
             if (want_groups && L.gate_inp.type == MESH_F32 && moe_router_group_supported(E, ne, k, T)) {

@@ -8,6 +8,7 @@
 
 #include "gguf.hpp"
 #include "mesh_common.hpp"
+#include "moe.hpp"
 
 namespace mesh {
 
@@ -47,6 +48,9 @@ struct LayerWeights {
     // packed as a SwiGLU pair.
     int qkv_fused = 0;
     void *gate_up_gemm = nullptr;
+    // mixture of experts: every expert's gate / up pair and down projection in the GEMM layout, experts back to back
+    void *exps_gate_up_gemm = nullptr, *exps_down_gemm = nullptr;
+    size_t exps_gate_up_stride = 0, exps_down_stride = 0;
 };
 
 }  // namespace mesh
@@ -97,6 +101,10 @@ struct mesh_session {
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
     int32_t *moe_items = nullptr, *moe_n_items = nullptr;      // (token, slot) pairs grouped by expert, see moe_group
+    // prefill chunks: the pairs sorted by expert (moe_sort) and their buffers, rows indexed by slot
+    mesh::MoeSorted moe_sorted;
+    uint16_t *moe_x16 = nullptr, *moe_ffn16 = nullptr;          // k8-major f16: normalised inputs, SwiGLU outputs
+    float *moe_out_slots = nullptr;                            // down-projection rows
     bool gemm_fused = true;          // MESH_GEMM_FUSED=0 at session creation: q / k / v and gate / up as separate prefill GEMM launches
     bool gemm_x_k8 = true;           // MESH_GEMM_XDIRECT=0 at session creation: the prefill GEMM stages row-major activations through LDS
     bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product

@@ -289,3 +289,48 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path):
     assert r <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     ses.close(); st.close()
+
+
+def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch):
+    """The same shard with a 272-token prompt chunk (34 pairs per expert on average; ragged: 272 = 2 * 128 + 16): the
+    pairs are sorted by expert and the expert products run as tiles of the large-tile f16 GEMM.  Against the oracle, the
+    routing decisions identical; then a second chunk on top; then the first chunk again through the 16-pair
+    integer matrix-core kernel (MESH_MOE_GEMM=0), which has to agree to within both paths' distance from the oracle."""
+    m = mesh()
+    cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
+    path = os.path.join(str(tmp_path), "shard.gguf")
+    tensors = models.write_model(path, cfg, [5, 6], seed=9, n_expert_local=64, fast=True, router="zipf")
+    n_ctx, E = 512, 2048
+    st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=2, n_batch_max=272)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 5, 7, n_ctx, n_seq_max=2)
+    rng = np.random.Generator(np.random.PCG64(57))
+    T = 272
+    x = models.zipf_hidden_state(rng, T, E)
+    pos = np.arange(T, dtype=np.int32)
+    got = ses.decode(x, pos).view(np.float32).reshape(T, E)
+    ref = orc.forward(x, pos)
+    r = rel_l2(got - x, ref - x)
+    report("C5 shard layers 5-6, 272-token prefill (expert products as large-tile GEMM tiles; of the layers' contribution)", r)
+    assert r <= NORTH_STAR
+    assert max(rel_l2(got[i] - x[i], ref[i] - x[i]) for i in range(T)) <= 3 * NORTH_STAR
+    assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
+    T2 = 150
+    x2 = models.zipf_hidden_state(rng, T2, E)
+    pos2 = np.arange(T, T + T2, dtype=np.int32)
+    got2 = ses.decode(x2, pos2).view(np.float32).reshape(T2, E)
+    ref2 = orc.forward(x2, pos2)
+    r2 = rel_l2(got2 - x2, ref2 - x2)
+    report("C5 shard layers 5-6, second chunk of 150 tokens on top (same path)", r2)
+    assert r2 <= NORTH_STAR
+    ses.close()
+    monkeypatch.setenv("MESH_MOE_GEMM", "0")
+    ses = st.session()
+    alt = ses.decode(x, pos).view(np.float32).reshape(T, E)
+    monkeypatch.delenv("MESH_MOE_GEMM")
+    ra = rel_l2(alt - x, ref - x)
+    report("C5 shard layers 5-6, the same 272 tokens through the 16-pair integer kernel", ra)
+    assert ra <= NORTH_STAR
+    assert rel_l2(got - x, alt - x) <= r + ra
+    ses.close(); st.close()
