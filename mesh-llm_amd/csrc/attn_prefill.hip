@@ -25,12 +25,10 @@ namespace mesh {
 
 constexpr int PF_HD = 128;
 constexpr int PF_TILE = 32;                 // queries per workgroup
-constexpr int PF_KEYS = 64;                 // keys per step (two MFMA tiles)
 constexpr int PF_KPITCH = PF_HD + 8;        // halfs per key row of the K tile in LDS (bank-conflict padding)
-constexpr int PF_VPITCH = PF_KEYS / 2 + 2;  // dwords (key pairs) per dim row of the transposed V tile
 
 // Column (dword) of key pair kp in dim row `dim` of the transposed V tile.  Rows 32 apart start on the same LDS bank
-// (32 * 34 dwords is a multiple of the 64 banks), and the staging writes of a wave touch four such rows at once; the
+// (32 rows of 18 or 34 dwords are a multiple of the 64 banks), and the staging writes of a wave touch four such rows at once; the
 // XOR moves them onto different banks.  It keeps dwords 2j, 2j + 1 neighbours, which the 8-byte fragment reads need.
 __device__ __forceinline__ int pf_vcol(int dim, int kp) { return kp ^ ((dim >> 5) << 2); }
 constexpr int PF_EXPAND_MIN_T = 128;         // chunks from this many tokens decode a quantised cache to f16 once, ahead of the walk
@@ -61,18 +59,23 @@ __device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
     }
 }
 
-// NP: (key, 8-dim piece) pairs of a step one thread carries in registers, at least 1024 / (threads of the workgroup);
-// 0 for small workgroups, which load each step's rows where they write them.
-template <int KT, int VT, int NP>
-__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw) {
+// NT: tiles of 32 keys per step (1 or 2; two give the wave two independent score chains and half the barriers per key, at
+// ~50 more registers).  NP: (key, 8-dim piece) pairs of a step one thread carries in registers, at least 512 NT /
+// (threads of the workgroup); 0 for small workgroups, which load each step's rows where they write them.
+template <int KT, int VT, int NP, int NT>
+__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw, int fwd_from) {
     constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
+    constexpr int PF_KEYS = 32 * NT;                // keys per step
+    constexpr int PF_VPITCH = PF_KEYS / 2 + 2;      // dwords (key pairs) per dim row of the transposed V tile
     __shared__ __align__(16) _Float16 sK[PF_KEYS * PF_KPITCH];
     __shared__ __align__(16) uint32_t sVt[PF_HD * PF_VPITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
     const int qcol = lane & 31, half = lane >> 5;
     // the last query tile of a chunk walks the most keys: the launch hands the tiles out from the last one backwards, so
     // that the longest walks start first when the workgroups do not all fit on the chip at once
-    const int qt = (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
+    // (a launch whose workgroups all fit at once, two per CU, runs its second half forwards: see attention_chunk)
+    const int lin = (int)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
+    const int qt = lin >= fwd_from ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
     const int h = kvh * a.group + blockIdx.z * hpw + wave;
     const int tq = qt * PF_TILE + qcol;
     const bool q_live = tq < T;
@@ -163,20 +166,20 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
             if (k0 + PF_KEYS < n_keys) fetch_step(k0 + PF_KEYS);
         }
         // the second 32 keys of the step lie past every query of the tile at the end of the walk
-        const bool two = k0 + 32 < n_keys;
+        const bool two = NT == 2 && k0 + 32 < n_keys;
 
         // S^T = K . Q^T, two tiles of 32 keys x 32 queries: lane (key row = lane % 32 of the A operand, query column =
         // lane % 32 of the result); two independent accumulation chains
-        pf_f16v s[2];
+        pf_f16v s[NT];
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) s[t][i] = t == 0 ? 0.f : (two ? 0.f : -INFINITY);
         if (two) {
 #pragma unroll
             for (int kc = 0; kc < 8; ++kc)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int t = 0; t < NT; ++t) {
                     const pf_h8 kf = *reinterpret_cast<const pf_h8 *>(sK + (32 * t + qcol) * PF_KPITCH + kc * 16 + 8 * half);
                     s[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kc], s[t], 0, 0, 0);
                 }
@@ -191,17 +194,21 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         // reaches past the first query's position has anything to mask (a dead query column has q = 0 and is never stored).
         if (k0 + PF_KEYS - 1 > pos0 + qt * PF_TILE) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
                     s[t][i] = key <= pos_q ? s[t][i] : -INFINITY;
                 }
         }
-        float mx0 = s[0][0], mx1 = s[1][0];
+        float mxt[NT];
 #pragma unroll
-        for (int i = 1; i < 16; ++i) { mx0 = fmaxf(mx0, s[0][i]); mx1 = fmaxf(mx1, s[1][i]); }
-        float mx = fmaxf(mx0, mx1);
+        for (int t = 0; t < NT; ++t) mxt[t] = s[t][0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) mxt[t] = fmaxf(mxt[t], s[t][i]);
+        float mx = NT == 2 ? fmaxf(mxt[0], mxt[NT - 1]) : mxt[0];
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         // m is the reference the exponentials are taken against.  It follows the running maximum only when that has
         // moved by more than PF_RESCALE_STEP (log2 units), so that most steps skip the rescale of the 64 accumulator
@@ -218,10 +225,10 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
                 for (int i = 0; i < 16; ++i) o[db][i] *= corr;
         }
         // P^T as the B operand: the lane's own registers, 8 per MFMA
-        pf_h8 pf[2][2];
+        pf_h8 pf[NT][2];
         float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < NT; ++t) {
             float p[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(s[t][i] - m);     // s - m <= PF_RESCALE_STEP; far below, 0
@@ -240,7 +247,7 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
             // dim row db * 32 + qcol, this half's keys of tile t: key pairs 16 * t + 2 * half + 4 * j (+ 1), j = 0 .. 3
             const uint32_t *vrow = sVt + (db * 32 + qcol) * PF_VPITCH + 2 * half;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < NT; ++t) {
                 if (t == 1 && !two) break;
                 const uint2 a0 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (0 ^ db)), a1 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (1 ^ db));
                 const uint2 a2 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (2 ^ db)), a3 = *reinterpret_cast<const uint2 *>(vrow + 16 * t + 4 * (3 ^ db));
@@ -296,6 +303,17 @@ __global__ __launch_bounds__(256) void kv_expand_kernel(const uint8_t *kcache, c
     v16[dst * 16 + piece] = pf_row_piece<VT>(vcache + src * VRB, piece);
 }
 
+static int pf_n_cu() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
 int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     AttnArgs a = a_in;
@@ -323,11 +341,18 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     while (hpw > 8 || a.group % hpw) --hpw;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * hpw));
+    // When the whole launch is resident at once with two workgroups per CU, the hardware has been seen to give a CU
+    // workgroups i and i + (half the launch): handing the second half its query tiles in forward order pairs a long
+    // walk with a short one on every CU.  (A guess about placement costs nothing when wrong: the tiles are the same.)
+    const int total = (int)(grid.x * grid.y * grid.z);
+    const int fwd_from = (hpw <= 4 && total % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
+    // (Two tiles per step everywhere.  With 5 heads per KV head one tile per step keeps the kernel under 170 registers, so
+    // that two 5-wave workgroups share a CU instead of one: measured slower, 16.5 against 14.8 ms over 32 layers of 4096 tokens.)
 #define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
     do {                                                                                                                  \
-        if (hpw == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw);        \
-        else if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4>), grid, block, 0, stream, a, T, pos0, seq, hpw);   \
-        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 0>), grid, block, 0, stream, a, T, pos0, seq, hpw);                  \
+        if (hpw == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);       \
+        else if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);  \
+        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 0, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);                 \
     } while (0)
     if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_CHUNK_LAUNCH(MESH_F16, MESH_F16);
     else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q8_0, MESH_Q4_0);
