@@ -644,24 +644,16 @@ __device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {       // satu
 
 // y = f16(x[t] * rsqrt(mean(x[t]^2) + eps) * w), or with w == null just f16(x[t]); one workgroup per token slot of the
 // padded batch (slots >= T write zeros).
-// row_of_slot set: slot t takes row row_of_slot[t] / row_div of x, or zeros when that is negative (gathered expert inputs).
 __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int T, int n,
-                                                    _Float16 *__restrict__ y, const int32_t *__restrict__ row_of_slot, int row_div) {
+                                                    _Float16 *__restrict__ y) {
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     _Float16 *yb = y + (size_t)(t / 16) * 16 * n + (size_t)(t % 16) * 8;        // element (t, k) at yb + (k / 8) * 128 + k % 8
-    int src = t;
-    bool dead = t >= T;
-    if (row_of_slot && !dead) {
-        const int r = row_of_slot[t];
-        dead = r < 0;
-        src = r / row_div;
-    }
-    if (dead) {
+    if (t >= T) {
         for (int i = tid * 8; i < n; i += 2048) *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = make_uint4(0u, 0u, 0u, 0u);
         return;
     }
-    const float *xt = x + (size_t)src * n;
+    const float *xt = x + (size_t)t * n;
     constexpr int RC = 4;                                   // rows of up to 2048 * RC elements stay in registers: one read
     if (w && n <= 2048 * RC) {
         float4 v[RC][2], g[RC][2];
@@ -726,15 +718,61 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
-    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y, (const int32_t *)nullptr, 1);
+    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
+// The gathered form with one workgroup per block of 16 slots: each wave first sums the squares of four of the block's rows,
+// then thread (k8 group, slot) converts 8 values at a time, so that 16 neighbouring threads write one contiguous 256-byte
+// run of the block.  The sum of squares is taken in another order than in to_k8_kernel (one wave per row instead of four),
+// so the scale can differ from that kernel's in its last bit.
+__global__ __launch_bounds__(256) void gather_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int n,
+                                                        _Float16 *__restrict__ y, const int32_t *__restrict__ row_of_slot, int row_div) {
+    __shared__ float s_scale[16];
+    __shared__ int s_row[16];
+    const int blk = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < 16) {
+        const int r = row_of_slot[blk * 16 + tid];
+        s_row[tid] = r < 0 ? -1 : r / row_div;
+    }
+    __syncthreads();
+    for (int i = 0; i < 4; ++i) {
+        const int sl = wave * 4 + i, row = s_row[sl];
+        float ss = 0.f;
+        if (row >= 0) {
+            const float *xt = x + (size_t)row * n;
+            for (int k = lane * 8; k < n; k += 512) {
+                const float4 a = *reinterpret_cast<const float4 *>(xt + k), b = *reinterpret_cast<const float4 *>(xt + k + 4);
+                ss += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
+                ss += (b.x * b.x + b.y * b.y) + (b.z * b.z + b.w * b.w);
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if (lane == 0) s_scale[sl] = 1.0f / sqrtf(ss / (float)n + eps);
+    }
+    __syncthreads();
+    const int sl = tid & 15, row = s_row[sl];
+    const float sc = s_scale[sl];
+    _Float16 *yb = y + (size_t)blk * 16 * n + (size_t)sl * 8;
+    for (int k8 = tid >> 4; k8 < n / 8; k8 += 16) {
+        uint4 o = make_uint4(0u, 0u, 0u, 0u);
+        if (row >= 0) {
+            const float *xt = x + (size_t)row * n + k8 * 8;
+            const float4 v0 = *reinterpret_cast<const float4 *>(xt), v1 = *reinterpret_cast<const float4 *>(xt + 4);
+            const float4 g0 = *reinterpret_cast<const float4 *>(w + k8 * 8), g1 = *reinterpret_cast<const float4 *>(w + k8 * 8 + 4);
+            o = make_uint4(sk_pack_h2(v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(v0.z * sc * g0.z, v0.w * sc * g0.w),
+                           sk_pack_h2(v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(v1.z * sc * g1.z, v1.w * sc * g1.w));
+        }
+        *reinterpret_cast<uint4 *>(yb + (size_t)k8 * 128) = o;
+    }
+}
+
 int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream) {
     if (n_slots <= 0) return MESH_OK;
-    if (n % 8 || n_slots % 16 || !row_of_slot || row_div < 1) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8_gather: bad arguments (row length %d, %d slots)", n, n_slots);
-    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)n_slots), dim3(256), 0, stream, x, w, eps, n_slots, n, y, row_of_slot, row_div);
+    if (n % 8 || n_slots % 16 || !row_of_slot || row_div < 1 || !w) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8_gather: bad arguments (row length %d, %d slots)", n, n_slots);
+    MESH_LAUNCH(gather_k8_kernel, dim3((unsigned)(n_slots / 16)), dim3(256), 0, stream, x, w, eps, n, y, row_of_slot, row_div);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
