@@ -103,6 +103,10 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream);
 size_t q16_block_bytes(int K);
 // y (q16 layout) = quantise(rms_norm(x) * w) for T rows of n floats (w == null: quantise(x)); n a multiple of 32
 int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t *y, hipStream_t stream);
+// Mixture of experts: x[t] += sum_s w[t][s] * y[t * top_k + s] (moe.hpp: moe_combine) and, from the new x, the q16 activations
+// quant16_k8(x, norm_w, eps) would produce, in one launch: the same bits as the two launches.  Rows of n <= 8192.
+bool moe_combine_quant16_supported(int n);
+int moe_combine_quant16(float *x, const float *y, const float *w, int T, int n, int top_k, const float *norm_w, float eps, uint8_t *yq, hipStream_t stream);
 // The "k8-major" f16 layout the large-tile GEMM reads: blocks of 16 tokens, element (t, k) of block t / 16 at
 // ((k / 8) * 16 + t % 16) * 8 + k % 8 within the block of 16 * K halfs; columns beyond T hold zeros.
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion

@@ -564,40 +564,11 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
 // norm every workgroup of a token sums the whole row's squares itself (the row is a few KB in L2): no second launch.
 // Token slots beyond T are not written: an MFMA row never mixes tokens, and the GEMM does not store those rows.
 constexpr int Q16_THREADS = 128;
-__global__ __launch_bounds__(Q16_THREADS) void quant16_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int n,
-                                                              uint8_t *__restrict__ y) {
-    __shared__ float red[Q16_THREADS / 64];
-    const int tid = threadIdx.x, tok = blockIdx.y, t = tok & 15;
-    uint8_t *yb = y + (size_t)(tok >> 4) * ((size_t)n * 36);
+// 8 consecutive values v of token slot t (elements i .. i + 7 of a row of n) into the q16 block at yb; the four lanes of a
+// 32-element block (tid % 4) share its scale.  Every lane of the wave calls it (`live` guards the stores).
+__device__ __forceinline__ void q16_store8(const float (&v)[8], int i, int t, int n, uint8_t *yb, bool live, int tid) {
     uint4 *planes = reinterpret_cast<uint4 *>(yb);                                  // record (k / 8, t) at planes[(k / 8) * 16 + t]
     float *dxp = reinterpret_cast<float *>(yb + (size_t)n * 32), *sxp = reinterpret_cast<float *>(yb + (size_t)n * 34);
-    const float *xt = x + (size_t)tok * n;
-    const int i = blockIdx.x * (Q16_THREADS * 8) + tid * 8;
-    const bool live = i < n;
-    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
-    if (live) {
-        a0 = *reinterpret_cast<const float4 *>(xt + i);
-        a1 = *reinterpret_cast<const float4 *>(xt + i + 4);
-        if (w) { g0 = *reinterpret_cast<const float4 *>(w + i); g1 = *reinterpret_cast<const float4 *>(w + i + 4); }
-    }
-    float scale = 1.f;
-    if (w) {
-        float ss = 0.f;
-        for (int k = tid * 4; k < n; k += Q16_THREADS * 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(xt + k);
-            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-        if ((tid & 63) == 0) red[tid >> 6] = ss;
-        __syncthreads();
-        float tot = 0.f;
-#pragma unroll
-        for (int k = 0; k < Q16_THREADS / 64; ++k) tot += red[k];
-        scale = 1.0f / sqrtf(tot / (float)n + eps);
-    }
-    const float v[8] = {a0.x * scale * g0.x, a0.y * scale * g0.y, a0.z * scale * g0.z, a0.w * scale * g0.w,
-                        a1.x * scale * g1.x, a1.y * scale * g1.y, a1.z * scale * g1.z, a1.w * scale * g1.w};
     float amax = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
@@ -625,10 +596,112 @@ __global__ __launch_bounds__(Q16_THREADS) void quant16_kernel(const float *__res
     }
 }
 
+__global__ __launch_bounds__(Q16_THREADS) void quant16_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int n,
+                                                              uint8_t *__restrict__ y) {
+    __shared__ float red[Q16_THREADS / 64];
+    const int tid = threadIdx.x, tok = blockIdx.y, t = tok & 15;
+    uint8_t *yb = y + (size_t)(tok >> 4) * ((size_t)n * 36);
+    const float *xt = x + (size_t)tok * n;
+    const int i = blockIdx.x * (Q16_THREADS * 8) + tid * 8;
+    const bool live = i < n;
+    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
+    if (live) {
+        a0 = *reinterpret_cast<const float4 *>(xt + i);
+        a1 = *reinterpret_cast<const float4 *>(xt + i + 4);
+        if (w) { g0 = *reinterpret_cast<const float4 *>(w + i); g1 = *reinterpret_cast<const float4 *>(w + i + 4); }
+    }
+    float scale = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int k = tid * 4; k < n; k += Q16_THREADS * 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(xt + k);
+            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int k = 0; k < Q16_THREADS / 64; ++k) tot += red[k];
+        scale = 1.0f / sqrtf(tot / (float)n + eps);
+    }
+    const float v[8] = {a0.x * scale * g0.x, a0.y * scale * g0.y, a0.z * scale * g0.z, a0.w * scale * g0.w,
+                        a1.x * scale * g1.x, a1.y * scale * g1.y, a1.z * scale * g1.z, a1.w * scale * g1.w};
+    q16_store8(v, i, t, n, yb, live, tid);
+}
+
 int quant16_k8(const float *x, const float *w, float eps, int T, int n, uint8_t *y, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (n % 32) return fail(MESH_ERR_INVALID, "quant16_k8: row length %d not a multiple of 32", n);
     MESH_LAUNCH(quant16_kernel, dim3((unsigned)((n + Q16_THREADS * 8 - 1) / (Q16_THREADS * 8)), (unsigned)T), dim3(Q16_THREADS), 0, stream, x, w, eps, n, y);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// The combine step of a mixture-of-experts layer and the q16 activations of the next layer's first projections in one
+// launch, one workgroup per token: x[t] += sum_s w[t][s] * y[t * top_k + s] (the sums of moe_combine_kernel, in its order),
+// then y16 = quantise(rms_norm(x[t]) * norm_w) exactly as quant16_kernel forms it: the same partition of the row for the sum
+// of squares (its thread j of 128 adds the float4 groups j, j + 128, ... in turn) and the same 8 values per lane for the blocks;
+// the row and the groups' squares pass through LDS.  Rows of up to Q16F_MAX_N elements.
+constexpr int Q16F_MAX_N = 8192, Q16F_THREADS = 512;
+__global__ __launch_bounds__(Q16F_THREADS) void moe_combine_quant16_kernel(float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ wts,
+                                                                           int top_k, const float *__restrict__ norm_w, float eps, int n,
+                                                                           uint8_t *__restrict__ yq) {
+    __shared__ float red[Q16_THREADS / 64];
+    __shared__ __align__(16) float row[Q16F_MAX_N];
+    __shared__ float psq[Q16F_MAX_N / 4];
+    const int tid = threadIdx.x, tok = blockIdx.x, t = tok & 15;
+    uint8_t *yb = yq + (size_t)(tok >> 4) * ((size_t)n * 36);
+    float *xt = x + (size_t)tok * n;
+    // one float4 group per thread and pass: the new hidden state and the group's sum of squares
+    for (int g = tid; g < n / 4; g += Q16F_THREADS) {
+        float4 acc = *reinterpret_cast<const float4 *>(xt + 4 * g);
+        for (int s = 0; s < top_k; ++s) {
+            const float ws = wts[(size_t)tok * top_k + s];
+            const float4 v = *reinterpret_cast<const float4 *>(y + ((size_t)tok * top_k + s) * n + 4 * g);
+            acc.x = fmaf(ws, v.x, acc.x); acc.y = fmaf(ws, v.y, acc.y); acc.z = fmaf(ws, v.z, acc.z); acc.w = fmaf(ws, v.w, acc.w);
+        }
+        *reinterpret_cast<float4 *>(xt + 4 * g) = acc;
+        *reinterpret_cast<float4 *>(row + 4 * g) = acc;
+        psq[g] = (acc.x * acc.x + acc.y * acc.y) + (acc.z * acc.z + acc.w * acc.w);
+    }
+    __syncthreads();
+    // the row's sum of squares in quant16_kernel's order: thread j of 128 adds its groups j, j + 128, ... one after the other
+    if (tid < Q16_THREADS) {
+        float ss = 0.f;
+        for (int g = tid; g < n / 4; g += Q16_THREADS) ss += psq[g];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+    }
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int k = 0; k < Q16_THREADS / 64; ++k) tot += red[k];
+    const float scale = 1.0f / sqrtf(tot / (float)n + eps);
+    for (int i0 = 0; i0 < n; i0 += Q16F_THREADS * 8) {
+        const int i = i0 + tid * 8;
+        const bool live = i < n;
+        float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
+        if (live) {
+            a0 = *reinterpret_cast<const float4 *>(row + i);
+            a1 = *reinterpret_cast<const float4 *>(row + i + 4);
+            g0 = *reinterpret_cast<const float4 *>(norm_w + i);
+            g1 = *reinterpret_cast<const float4 *>(norm_w + i + 4);
+        }
+        const float v[8] = {a0.x * scale * g0.x, a0.y * scale * g0.y, a0.z * scale * g0.z, a0.w * scale * g0.w,
+                            a1.x * scale * g1.x, a1.y * scale * g1.y, a1.z * scale * g1.z, a1.w * scale * g1.w};
+        q16_store8(v, i, t, n, yb, live, tid);
+    }
+}
+
+bool moe_combine_quant16_supported(int n) { return n % 32 == 0 && n <= Q16F_MAX_N; }
+
+int moe_combine_quant16(float *x, const float *y, const float *w, int T, int n, int top_k, const float *norm_w, float eps, uint8_t *yq, hipStream_t stream) {
+    if (T <= 0) return MESH_OK;
+    if (!moe_combine_quant16_supported(n) || !norm_w || !yq) return fail(MESH_ERR_INVALID, "moe_combine_quant16: row length %d", n);
+    MESH_LAUNCH(moe_combine_quant16_kernel, dim3((unsigned)T), dim3(Q16F_THREADS), 0, stream, x, y, w, top_k, norm_w, eps, n, yq);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

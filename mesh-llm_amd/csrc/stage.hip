@@ -380,6 +380,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
+    if (const char *e = getenv("MESH_MOE_FUSE_QUANT")) s->moe_fuse_quant = e[0] != '0';
     if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
     if (const char *e = getenv("MESH_GEMM_FUSED")) s->gemm_fused = e[0] != '0';
     if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
@@ -612,7 +613,8 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; return g; };
     {
         ProfScope ps(s, MESH_PROF_PREP);
-        if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        if (skinny && s->xq_layer == (int)il) rc = MESH_OK;     // the previous layer's combine step has left them in s->xq
+        else if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
         else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
         else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
     }
@@ -796,6 +798,23 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     hipStream_t stream = s->stream;
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim);
     int rc;
+    s->xq_layer = -1;
+    // a mixture-of-experts layer whose attention block runs on the batched-decode (integer matrix-core) path
+    auto moe_attn_skinny = [&](const LayerWeights &Ln) {
+        return !Ln.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && T < PREFILL_MIN_TOKENS && s->xn16 && layer_attn_is_kquant(Ln) &&
+               hp.n_embd % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0;
+    };
+    // the combine step at the end of a mixture-of-experts layer; when the next layer starts by quantising the new hidden
+    // state for its projections, the same launch does that too (the same bits) and the layer finds them in s->xq
+    auto combine = [&](size_t il, int top_k) {
+        if (s->moe_fuse_quant && il + 1 < st->layers.size() && moe_attn_skinny(st->layers[il + 1]) && moe_combine_quant16_supported(E)) {
+            const int r = moe_combine_quant16(s->x, s->moe_out, s->moe_w, T, E, top_k, static_cast<const float *>(st->layers[il + 1].attn_norm.data), hp.rms_eps,
+                                              s->xq, stream);
+            if (r == MESH_OK) s->xq_layer = (int)il + 1;
+            return r;
+        }
+        return moe_combine(s->x, s->moe_out, s->moe_w, T, E, top_k, stream);
+    };
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
         if (T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
@@ -984,7 +1003,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                 da.x_div = 1;
                 { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_skinny(da, stream); }
                 if (rc != MESH_OK) return rc;
-                if ((rc = moe_combine(s->x, s->moe_out, s->moe_w, T, E, k, stream)) != MESH_OK) return rc;
+                if ((rc = combine(il, k)) != MESH_OK) return rc;
                 continue;
             }
             GemvArgs ea;
@@ -1006,7 +1025,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             if (grouped) { xa.items = s->moe_items; xa.n_items = s->moe_n_items; xa.max_items = ea.max_items; }
             { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(xa, stream); }
             if (rc != MESH_OK) return rc;
-            if ((rc = moe_combine(s->x, s->moe_out, s->moe_w, T, E, k, stream)) != MESH_OK) return rc;
+            if ((rc = combine(il, k)) != MESH_OK) return rc;
             continue;
         }
         // ffn = silu(Wgate . n) * (Wup . n),  n = rms_norm(x)

@@ -108,6 +108,8 @@ struct mesh_session {
     bool gemm_fused = true;          // MESH_GEMM_FUSED=0 at session creation: q / k / v and gate / up as separate prefill GEMM launches
     bool gemm_x_k8 = true;           // MESH_GEMM_XDIRECT=0 at session creation: the prefill GEMM stages row-major activations through LDS
     bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product
+    bool moe_fuse_quant = true;      // MESH_MOE_FUSE_QUANT=0 at session creation: the combine step never quantises for the next layer
+    int xq_layer = -1;               // layer whose attention-norm activations the previous layer's combine step has left in xq (-1: none)
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)
     unsigned meta_counter = 0;

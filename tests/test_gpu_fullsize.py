@@ -334,3 +334,31 @@ def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch
     assert ra <= NORTH_STAR
     assert rel_l2(got - x, alt - x) <= r + ra
     ses.close(); st.close()
+
+
+def test_c5_combine_step_quantises_for_the_next_layer_bit_identically(tmp_path, monkeypatch):
+    """Decode batch 16 over three shard layers: the combine step at the end of a mixture-of-experts layer also writes the
+    quantised activations the next layer's q / k / v launch reads.  The same bits as with the two separate launches
+    (MESH_MOE_FUSE_QUANT=0), step after step."""
+    m = mesh()
+    cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
+    path = os.path.join(str(tmp_path), "shard.gguf")
+    models.write_model(path, cfg, [5, 6, 7], seed=9, n_expert_local=64, fast=True, router="zipf")
+    E = 2048
+    st = m.Stage(path, 5, 8, n_ctx=64, n_seq_max=16, n_batch_max=16)
+    os.unlink(path)
+    rng = np.random.Generator(np.random.PCG64(58))
+    xs = [models.zipf_hidden_state(rng, 16, E) for _ in range(3)]
+    outs = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("MESH_MOE_FUSE_QUANT", fuse)
+        ses = st.session()
+        got = []
+        for step, x in enumerate(xs):
+            got.append(ses.decode(x, np.full(16, step, np.int32), seq=np.arange(16, dtype=np.int32)).view(np.uint32).copy())
+        outs.append(got)
+        ses.close()
+    monkeypatch.delenv("MESH_MOE_FUSE_QUANT")
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+    st.close()
