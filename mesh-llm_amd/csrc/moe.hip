@@ -43,6 +43,42 @@ __device__ __forceinline__ void route_wave(const float *lg, const float *mask, i
     }
     float wsum = 0.f, my_w = 0.f;
     int my_id = 0;
+    if constexpr (NPL <= 2) {
+        // Up to 128 experts: every candidate counts the experts that come before it in the order (value descending, id
+        // ascending) -- one broadcast per expert, no dependent cross-lane chain -- and the candidate counting k is the
+        // k-th pick.  The same picks in the same order as the loop below (each round of which takes the first expert
+        // left in that order).
+        int rank[NPL];
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) rank[i] = lane + 64 * i < n_expert ? 0 : 0x7FFFFFFF;
+#pragma unroll
+        for (int ii = 0; ii < NPL; ++ii) {
+            for (int j = 0; j < 64 && j + 64 * ii < n_expert; ++j) {
+                const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sel[ii]), j));
+                const int oe = j + 64 * ii;
+#pragma unroll
+                for (int i = 0; i < NPL; ++i) {
+                    const int e = lane + 64 * i;
+                    rank[i] += (ov > sel[i] || (ov == sel[i] && oe < e)) ? 1 : 0;
+                }
+            }
+        }
+        for (int k = 0; k < top_k; ++k) {
+            int bi = 0;
+            float bp = 0.f;
+#pragma unroll
+            for (int i = 0; i < NPL; ++i) {
+                const unsigned long long m = __builtin_amdgcn_ballot_w64(rank[i] == k);
+                if (m != 0ull) {
+                    const int src = __builtin_ctzll(m);
+                    bi = src + 64 * i;
+                    bp = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p[i]), src));
+                }
+            }
+            if (lane == k) { my_id = bi; my_w = bp; }
+            wsum += bp;
+        }
+    } else {
     unsigned taken = 0;        // bit i: expert lane + 64*i has been selected
     for (int k = 0; k < top_k; ++k) {
         // best remaining (value, id) of this lane, then of the wave; ties go to the lower id
@@ -66,6 +102,7 @@ __device__ __forceinline__ void route_wave(const float *lg, const float *mask, i
             if (lane + 64 * i == bi) taken |= 1u << i;
         if (lane == k) { my_id = bi; my_w = bp; }
         wsum += bp;
+    }
     }
     if (lane < top_k) {
         ids[lane] = my_id;
