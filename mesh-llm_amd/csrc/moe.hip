@@ -130,12 +130,15 @@ __global__ __launch_bounds__(64) void moe_route_kernel(MoeRouteArgs a) {
 // With gridDim.y > 1 the experts are split over blockIdx.y and the kernel only writes logits_out (routing follows in
 // moe_route_group_kernel): small batches then have enough workgroups to pull the router matrix through quickly.
 constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64;
-template <int NV>      // float4 groups per lane = E / 256
+// (RT: threads of the workgroup.  A decode batch has few tokens and wants every wave it can get on a token's expert rows;
+// a prefill chunk has a workgroup per token anyway, and small workgroups, eight to a CU, hide each other's row loads.)
+constexpr int ROUTER_THREADS_WIDE = 256, ROUTER_WIDE_MIN_TOKENS = 512;
+template <int NV, int RT = ROUTER_THREADS>      // float4 groups per lane = E / 256
 // (scalar arguments first: preloaded into SGPRs, see gemv.hip)
-__global__ __launch_bounds__(ROUTER_THREADS) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+__global__ __launch_bounds__(RT) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
                                                                           const float *__restrict__ W, float *__restrict__ logits_out,
                                                                           int ldx, float eps, int p_n_expert, const MoeRouteArgs a) {
-    constexpr int E = NV * 256;
+    constexpr int E = NV * 256, ROUTER_WAVES = RT / 64;
     __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // element index of a lane's values: 4 * (lane + 64 * i) + c
@@ -195,7 +198,20 @@ int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float
                      float *logits_out, int T, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (!moe_router_fused_supported(E, a.n_expert, a.top_k)) return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d / %d experts", E, a.n_expert);
-    const dim3 grid((unsigned)T), block(ROUTER_THREADS);
+    const dim3 grid((unsigned)T);
+    if (T >= ROUTER_WIDE_MIN_TOKENS) {
+        const dim3 block(ROUTER_THREADS_WIDE);
+        switch (E / 256) {
+            case 2: MESH_LAUNCH((moe_router_fused_kernel<2, ROUTER_THREADS_WIDE>), grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+            case 4: MESH_LAUNCH((moe_router_fused_kernel<4, ROUTER_THREADS_WIDE>), grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+            case 8: MESH_LAUNCH((moe_router_fused_kernel<8, ROUTER_THREADS_WIDE>), grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+            case 16: MESH_LAUNCH((moe_router_fused_kernel<16, ROUTER_THREADS_WIDE>), grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
+            default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
+        }
+        MESH_LAUNCH_CHECK();
+        return MESH_OK;
+    }
+    const dim3 block(ROUTER_THREADS);
     switch (E / 256) {
         case 2: MESH_LAUNCH(moe_router_fused_kernel<2>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;
         case 4: MESH_LAUNCH(moe_router_fused_kernel<4>, grid, block, 0, stream, x, norm_w, W, logits_out, ldx, eps, a.n_expert, a); break;

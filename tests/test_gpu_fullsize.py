@@ -300,8 +300,8 @@ def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch
     cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
     path = os.path.join(str(tmp_path), "shard.gguf")
     tensors = models.write_model(path, cfg, [5, 6], seed=9, n_expert_local=64, fast=True, router="zipf")
-    n_ctx, E = 512, 2048
-    st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=2, n_batch_max=272)
+    n_ctx, E = 640, 2048
+    st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=2, n_batch_max=520)
     os.unlink(path)
     ses = st.session()
     orc = StageOracle(cfg, tensors, 5, 7, n_ctx, n_seq_max=2)
@@ -324,6 +324,16 @@ def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch
     r2 = rel_l2(got2 - x2, ref2 - x2)
     report("C5 shard layers 5-6, second chunk of 150 tokens on top (same path)", r2)
     assert r2 <= NORTH_STAR
+    # a 520-token chunk of the other sequence (from 512 tokens the router runs as small workgroups, one per token)
+    T3 = 520
+    x3 = models.zipf_hidden_state(rng, T3, E)
+    pos3 = np.arange(T3, dtype=np.int32)
+    got3 = ses.decode(x3, pos3, seq=np.ones(T3, np.int32)).view(np.float32).reshape(T3, E)
+    ref3 = orc.forward(x3, pos3, seq=np.ones(T3, np.int32))
+    r3 = rel_l2(got3 - x3, ref3 - x3)
+    report("C5 shard layers 5-6, 520-token prefill of a second sequence (same path)", r3)
+    assert r3 <= NORTH_STAR
+    assert np.array_equal(np.sort(ses.moe_last_ids(T3), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     ses.close()
     monkeypatch.setenv("MESH_MOE_GEMM", "0")
     ses = st.session()
