@@ -194,11 +194,85 @@ __global__ __launch_bounds__(RT) void moe_router_fused_kernel(const float *__res
     if (wave == 0) route_wave_any(s_logits, a, t, lane);
 }
 
+// The same for a prefill chunk, four tokens per workgroup of eight waves: every wave keeps the four normalised hidden
+// states in registers and walks every eighth expert row, so a row fetched from L2 serves four tokens (a workgroup per
+// token re-reads the whole router matrix per token: 512 MB per launch at 1024 tokens x 64 experts x 2048).  Every
+// (token, expert) logit is the sum the kernel above forms, in its order; waves 0 to 3 then route one token each.
+constexpr int CHUNK_TOKENS = 4, CHUNK_WAVES = 8, CHUNK_THREADS = 64 * CHUNK_WAVES;
+template <int NV>
+__global__ __launch_bounds__(CHUNK_THREADS) void moe_router_chunk_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+                                                                         const float *__restrict__ W, float *__restrict__ logits_out,
+                                                                         int ldx, float eps, int T, const MoeRouteArgs a) {
+    constexpr int E = NV * 256;
+    __shared__ float s_logits[CHUNK_TOKENS][64 * ROUTE_MAX_PER_LANE];
+    const int t0 = blockIdx.x * CHUNK_TOKENS, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float4 xr[CHUNK_TOKENS][NV];
+#pragma unroll
+    for (int k = 0; k < CHUNK_TOKENS; ++k) {
+        const int t = t0 + k < T ? t0 + k : T - 1;
+        const float *xt = x + (size_t)t * ldx;
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            xr[k][i] = *reinterpret_cast<const float4 *>(xt + 4 * (lane + 64 * i));
+            ss += xr[k][i].x * xr[k][i].x + xr[k][i].y * xr[k][i].y + xr[k][i].z * xr[k][i].z + xr[k][i].w * xr[k][i].w;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        const float scale = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const float4 w = *reinterpret_cast<const float4 *>(norm_w + 4 * (lane + 64 * i));
+            xr[k][i].x = xr[k][i].x * scale * w.x; xr[k][i].y = xr[k][i].y * scale * w.y;
+            xr[k][i].z = xr[k][i].z * scale * w.z; xr[k][i].w = xr[k][i].w * scale * w.w;
+        }
+    }
+    for (int e = wave; e < a.n_expert; e += CHUNK_WAVES) {
+        const float *wr = W + (size_t)e * E;
+        float4 r[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) r[i] = *reinterpret_cast<const float4 *>(wr + 4 * (lane + 64 * i));
+        float acc[CHUNK_TOKENS];
+#pragma unroll
+        for (int k = 0; k < CHUNK_TOKENS; ++k) {
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                v = fmaf(xr[k][i].x, r[i].x, v); v = fmaf(xr[k][i].y, r[i].y, v); v = fmaf(xr[k][i].z, r[i].z, v); v = fmaf(xr[k][i].w, r[i].w, v);
+            }
+            acc[k] = v;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+#pragma unroll
+            for (int k = 0; k < CHUNK_TOKENS; ++k) acc[k] += __shfl_xor(acc[k], o);
+        if (lane == 0) {
+#pragma unroll
+            for (int k = 0; k < CHUNK_TOKENS; ++k) {
+                s_logits[k][e] = acc[k];
+                if (logits_out && t0 + k < T) logits_out[(size_t)(t0 + k) * a.n_expert + e] = acc[k];
+            }
+        }
+    }
+    __syncthreads();
+    if (wave < CHUNK_TOKENS && t0 + wave < T) route_wave_any(s_logits[wave], a, t0 + wave, lane);
+}
+
 int moe_router_fused(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
                      float *logits_out, int T, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     if (!moe_router_fused_supported(E, a.n_expert, a.top_k)) return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d / %d experts", E, a.n_expert);
     const dim3 grid((unsigned)T);
+    if (T >= ROUTER_WIDE_MIN_TOKENS && E <= 2048) {
+        const dim3 cgrid((unsigned)((T + CHUNK_TOKENS - 1) / CHUNK_TOKENS)), cblock(CHUNK_THREADS);
+        switch (E / 256) {
+            case 2: MESH_LAUNCH(moe_router_chunk_kernel<2>, cgrid, cblock, 0, stream, x, norm_w, W, logits_out, ldx, eps, T, a); break;
+            case 4: MESH_LAUNCH(moe_router_chunk_kernel<4>, cgrid, cblock, 0, stream, x, norm_w, W, logits_out, ldx, eps, T, a); break;
+            default: MESH_LAUNCH(moe_router_chunk_kernel<8>, cgrid, cblock, 0, stream, x, norm_w, W, logits_out, ldx, eps, T, a); break;
+        }
+        MESH_LAUNCH_CHECK();
+        return MESH_OK;
+    }
     if (T >= ROUTER_WIDE_MIN_TOKENS) {
         const dim3 block(ROUTER_THREADS_WIDE);
         switch (E / 256) {
