@@ -339,6 +339,8 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     }
     int hpw = a.group;                       // heads (waves) per workgroup: the largest divisor of the group up to 8
     while (hpw > 8 || a.group % hpw) --hpw;
+    // eight heads per KV head: two workgroups of four waves when one of eight per (query tile, KV head) would leave CUs idle
+    if (hpw == 8 && ((T + PF_TILE - 1) / PF_TILE) * a.n_kv < pf_n_cu()) hpw = 4;
     const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * hpw));
     // When the whole launch is resident at once with two workgroups per CU, the hardware has been seen to give a CU
