@@ -303,11 +303,27 @@ def bench_stage(args):
         # what the matrix pipes sustain from registers alone on this GPU (20 launches of ~15 ms each, median)
         mp = m.mfma_f16_probe(20000, 2, 20)
         mfma_probe = mp[len(mp) // 2]
+        # and what the vendor library's plain f16 GEMM reaches on the largest projection's shape (gate + up: tokens x
+        # 2 n_ff x n_embd) with weights that are already f16: no dequantisation, no epilogue, 2 bytes per weight
+        va = torch.randn(PREFILL_T, E, device="cuda", dtype=torch.float16)
+        vb = torch.randn(2 * FF, E, device="cuda", dtype=torch.float16)
+        for _ in range(3):
+            vc = va @ vb.t()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(10):
+            vc = va @ vb.t()
+        ev1.record()
+        torch.cuda.synchronize()
+        vendor_tflops = 2.0 * PREFILL_T * 2 * FF * E * 10 / ev0.elapsed_time(ev1) / 1e9
+        del va, vb, vc
         prefill = {"tokens": PREFILL_T, "ms": round(pms, 2), "tok_s": round(PREFILL_T * 1e3 / pms, 1),
                    "matmul_TFLOP": round(mm_flop / 1e12, 3), "attention_TFLOP": round(at_flop / 1e12, 3),
                    "stage_TFLOPs": round((mm_flop + at_flop) / pms / 1e9, 1),
                    "gemm_ms": round(gemm_ms, 2), "gemm_TFLOPs": round(mm_flop / gemm_ms / 1e9, 1),
                    "gemm_frac_mfma_f16_peak": round(mm_flop / gemm_ms / 1e9 / 2500.0, 4),
+                   "vendor_plain_f16_gemm_TFLOPs_gate_up_shape": round(vendor_tflops, 1),
                    "mfma_f16_probe_TFLOPs": round(mfma_probe, 1), "gemm_frac_of_mfma_probe": round(mm_flop / gemm_ms / 1e9 / mfma_probe, 4),
                    "kernel_ms": {k: round(v["ms"], 2) for k, v in pprof.items()}}
     b1 = results[batches[0]]
