@@ -212,6 +212,31 @@ def cpu_stage_baseline(cfg, tensors, n_layers=2):
                       "CPU restatement of ggml's reference routines (f32 activations), not llama.cpp" % (n_layers - 1, reps, STAGE_LAYERS // n_layers)}
 
 
+def vendor_f16_matvec(torch, cfg):
+    """The vendor library's mat-vec (torch.matmul of an f16 matrix and a vector) on the four projection shapes of a
+    layer, launched back to back with no dependence between launches: what a plain f16 kernel of that size costs on
+    this GPU, next to the average launch of the dequant-fused mat-vec in `roofline`."""
+    E, FF = cfg["n_embd"], cfg["n_ff"]
+    QKV = (cfg["n_head"] + 2 * cfg["n_head_kv"]) * cfg["head_dim"]
+    out = {}
+    for name, (M, K) in (("qkv", (QKV, E)), ("o", (E, cfg["n_head"] * cfg["head_dim"])), ("gate_up", (2 * FF, E)), ("down", (E, FF))):
+        w = torch.randn(M, K, device="cuda", dtype=torch.float16)
+        x = torch.randn(K, 1, device="cuda", dtype=torch.float16)
+        for _ in range(5):
+            y = w @ x
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(50):
+            y = w @ x
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / 50 * 1e3
+        out[name] = {"rows": M, "k": K, "MB": round(M * K * 2 / 1e6, 1), "us": round(us, 2), "GBps": round(M * K * 2 / us / 1e3, 1)}
+        del w, x, y
+    return out
+
+
 def bench_stage(args):
     import torch
     import __graft_entry__ as graft
@@ -335,6 +360,7 @@ def bench_stage(args):
     traffic_ratio = profiled_ratio(TRAFFIC_PROFILE, "gemv_batch1_traffic_over_algorithmic")
     codec = run_codec(torch, m, max(10, args.steps // 2), args.warmup)
     probe = hbm_probe(m)
+    vendor_matvec = vendor_f16_matvec(torch, cfg)
     out = {
         "metric": "stage decode tok/s @8B Q4_K_M", "value": b1["tok_s"], "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": b1["ms_per_step"], "higher_is_better": True,
@@ -349,7 +375,8 @@ def bench_stage(args):
                      "traffic": int(round(traffic_ratio * weight_bytes / g_n)) if traffic_ratio else None,
                      "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic_ratio else None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
                      "algorithmic_bytes_per_launch": weight_bytes // g_n,
-                     "measured_stream_read_GBps": probe, "frac_of_measured_p90": round(gemv_gbs / probe["p90"], 4)},
+                     "measured_stream_read_GBps": probe, "frac_of_measured_p90": round(gemv_gbs / probe["p90"], 4),
+                     "vendor_f16_matvec_same_shapes": vendor_matvec},
         "stage_frac_hbm": b1["frac_hbm"],
         "decode": {str(k): v for k, v in results.items()},
         "prefill": prefill,
