@@ -347,7 +347,8 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     // workgroups i and i + (half the launch): handing the second half its query tiles in forward order pairs a long
     // walk with a short one on every CU.  (A guess about placement costs nothing when wrong: the tiles are the same.)
     const int total = (int)(grid.x * grid.y * grid.z);
-    const int fwd_from = (hpw <= 4 && total % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
+    // (half the launch has to be whole rows of query tiles: an even number of (KV head, head group) rows)
+    const int fwd_from = (hpw <= 4 && (grid.y * grid.z) % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
     // (Two tiles per step everywhere.  With 5 heads per KV head one tile per step keeps the kernel under 170 registers, so
     // that two 5-wave workgroups share a CU instead of one: measured slower, 16.5 against 14.8 ms over 32 layers of 4096 tokens.)
 #define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
