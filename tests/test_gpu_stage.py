@@ -412,6 +412,25 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
     ses.close(); st.close()
 
 
+def test_long_chunk_with_an_odd_number_of_head_rows(tmp_path):
+    """2816 tokens of a model with three KV heads, one query head each: the chunk attention launch has 88 query tiles x 3
+    head rows = 264 workgroups, between one and two per CU, an even count with an odd number of rows -- the shape for which a launch
+    must not hand the second half of its workgroups their tiles in forward order (half the launch would not be whole
+    rows, and tiles would be computed twice or not at all).  Also the single-wave-per-workgroup kernel at length."""
+    T = 2816
+    m, cfg, tensors, st = _open(tmp_path, "tiny-mha3", [0], 0, 1, n_ctx=T, n_seq=1, n_batch=T)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(44))
+    orc = StageOracle(cfg, tensors, 0, 1, T, n_seq_max=1)
+    ses = st.session()
+    x = rng.standard_normal((T, E)).astype(np.float32)
+    got = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
+    ref = orc.forward(x, np.arange(T))
+    assert rel_l2(got, ref) <= 3e-3
+    assert max(rel_l2(got[i], ref[i]) for i in range(0, T, 29)) <= 1e-2
+    ses.close(); st.close()
+
+
 def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
     """Decode batches of 4..16 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
     (one with q6_K attn_v / ffn_down, so q/k/v split into two launches), 16 sequences at KV depth 300, full and ragged
