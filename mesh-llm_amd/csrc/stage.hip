@@ -517,9 +517,16 @@ static int attn_mma_min_tokens() {
     return v;
 }
 
-static int attn_splits_for(int T, int n_kv, int max_keys) {
-    // one workgroup per compute unit (256 on gfx950) measured best from batch 1 to 16 with the matrix-core kernel
-    constexpr int target = 256;
+// quantised: the cache rows are q8_0 / q4_0
+static int attn_splits_for(int T, int n_kv, int max_keys, bool quantised) {
+    // One workgroup per compute unit (256 on gfx950) measured best from batch 1 to 16 with f16 rows, which that many
+    // workgroups stream at the memory's rate.  Quantised rows are bound by the instructions that decode them, and two
+    // workgroups per CU hide each other's waits: 3-7% of the step at batch 8-32 (Qwen2.5-32B shape, q8_0 / q4_0 cache:
+    // 9.86 -> 9.18 ms at batch 32, which otherwise runs unsplit); four per CU lose again, and so do 64 splits of a single
+    // token's walk (from 64 (token, KV head) pairs on).
+    // (MESH_ATTN_SPLIT_TARGET: the workgroup count aimed at, for experiments)
+    static const int forced = getenv("MESH_ATTN_SPLIT_TARGET") ? std::max(1, atoi(getenv("MESH_ATTN_SPLIT_TARGET"))) : 0;
+    const int target = forced ? forced : (quantised && T * n_kv >= 64) ? 512 : 256;
     int s = target / std::max(1, T * n_kv);
     s = std::min(s, (max_keys + 63) / 64);
     return std::max(1, std::min(s, ATTN_SPLITS_MAX));
@@ -696,7 +703,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;     // a batch of decode steps still splits the long KV
+    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;     // a batch of decode steps still splits the long KV
     {
         ProfScope ps(s, MESH_PROF_ATTN);
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) {
@@ -878,7 +885,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         aa.scale = 1.0f / sqrtf((float)hp.head_dim);
         aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
         aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-        aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys);
+        aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16);
         {
             ProfScope ps(s, MESH_PROF_ATTN);
             rc = T >= attn_mma_min_tokens() && attention_mma_supported(aa) ? attention_mma(aa, T, stream) : attention(aa, T, stream);
@@ -1079,7 +1086,7 @@ static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
     // chunk's.  Such calls are always launched eagerly.
     if (s->chunk_pos0 >= 0 && T >= PREFILL_MIN_TOKENS) return run_layers(s, T, max_keys);
     const mesh_stage *st = s->stage;
-    const int n_splits = attn_splits_for(T, (int)st->hp.n_head_kv, max_keys);
+    const int n_splits = attn_splits_for(T, (int)st->hp.n_head_kv, max_keys, st->k_type != MESH_F16);
     const uint64_t key = (uint64_t)T | ((uint64_t)n_splits << 8) | ((uint64_t)(s->expert_mask_on ? 1 : 0) << 20);
     auto it = s->graphs.find(key);
     if (it == s->graphs.end()) {
@@ -1243,7 +1250,7 @@ int session_attention(mesh_session *s, int layer, const float *d_q, const mesh_b
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys) : 1;
+    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;
     if (matrix_cores) {
         if (!attention_mma_supported(aa)) return fail(MESH_ERR_UNSUPPORTED, "mesh_session_attn_dev: the matrix-core kernel does not cover this shape");
         return attention_mma(aa, T, s->stream);
