@@ -352,8 +352,14 @@ static int gemm_min_tokens() {
 }
 #define PREFILL_MIN_TOKENS gemm_min_tokens()
 // mixture of experts: calls with at least this many (token, slot) pairs per expert on average run the expert products as
-// tiles of the large-tile GEMM (below that, 16 pairs at a time on the integer matrix cores)
-constexpr size_t MOE_GEMM_MIN_PAIRS_PER_EXPERT = 16;
+// tiles of the large-tile GEMM (measured against the other kernels on a 64-expert shard with top-8 routing, four layers:
+// 0.607 against 0.659 ms at 4 pairs per expert, 0.536 against 0.485 at 2; MESH_MOE_GEMM_MIN_PAIRS moves it).  Below that the
+// mat-vec kernel; the 16-pair integer matrix-core kernel covers stages without GEMM-layout copies of the experts.
+static size_t moe_gemm_min_pairs() {
+    static const size_t v = getenv("MESH_MOE_GEMM_MIN_PAIRS") ? (size_t)std::max(1, atoi(getenv("MESH_MOE_GEMM_MIN_PAIRS"))) : 4;
+    return v;
+}
+#define MOE_GEMM_MIN_PAIRS_PER_EXPERT moe_gemm_min_pairs()
 // MESH_MOE_GEMM=0: never (for comparison)
 static bool moe_gemm_on() {
     const char *e = getenv("MESH_MOE_GEMM");

@@ -252,10 +252,13 @@ def test_c5_expert_shard_layer_zipf_router_on_filled_cache(tmp_path):
     ses.close(); st.close()
 
 
-def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path):
-    """The same shard with enough tokens per expert for the matrix-core expert kernel (from four pairs per expert on
-    average: 32 tokens x top-8 over 64 experts): a 96-token prompt chunk of one sequence, then a decode batch of 40
-    sequences, Zipf router, against the oracle; routing decisions identical."""
+@pytest.mark.parametrize("expert_gemm", ["1", "0"])
+def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, monkeypatch, expert_gemm):
+    """The same shard with enough tokens per expert for the matrix cores (from four pairs per expert on average: 32
+    tokens x top-8 over 64 experts): a 96-token prompt chunk of one sequence, then a decode batch of 40 sequences, Zipf
+    router, against the oracle; routing decisions identical.  Once with the expert products as tiles of the large-tile
+    f16 GEMM (the default), once through the 16-pair integer kernel (MESH_MOE_GEMM=0)."""
+    monkeypatch.setenv("MESH_MOE_GEMM", expert_gemm)
     m = mesh()
     cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
     path = os.path.join(str(tmp_path), "shard.gguf")
@@ -273,7 +276,7 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path):
     got = ses.decode(x, pos).view(np.float32).reshape(T, E)
     ref = orc.forward(x, pos)
     r = rel_l2(got - x, ref - x)
-    report("C5 shard layers 5-6, 96-token prefill (matrix-core expert products; of the layers' contribution)", r)
+    report("C5 shard layers 5-6, 96-token prefill (matrix-core expert products, MESH_MOE_GEMM=%s; of the layers' contribution)" % expert_gemm, r)
     assert r <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     # wide decode batch: sequence 0 continues its prompt, the others start
@@ -285,7 +288,7 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path):
     got = ses.decode(x, pos, seq=seq).view(np.float32).reshape(T, E)
     ref = orc.forward(x, pos, seq=seq)
     r = rel_l2(got - x, ref - x)
-    report("C5 shard layers 5-6, decode batch 40 (matrix-core expert products)", r)
+    report("C5 shard layers 5-6, decode batch 40 (matrix-core expert products, MESH_MOE_GEMM=%s)" % expert_gemm, r)
     assert r <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     ses.close(); st.close()
