@@ -63,19 +63,23 @@ __device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
 // ~50 more registers).  NP: (key, 8-dim piece) pairs of a step one thread carries in registers, at least 512 NT /
 // (threads of the workgroup); 0 for small workgroups, which load each step's rows where they write them.
 template <int KT, int VT, int NP, int NT>
-__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw, int fwd_from) {
+__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw, int fwd_from, int qtiles) {
     constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
     constexpr int PF_KEYS = 32 * NT;                // keys per step
     constexpr int PF_VPITCH = PF_KEYS / 2 + 2;      // dwords (key pairs) per dim row of the transposed V tile
     __shared__ __align__(16) _Float16 sK[PF_KEYS * PF_KPITCH];
     __shared__ __align__(16) uint32_t sVt[PF_HD * PF_VPITCH];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+    const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x;
+    // wave -> (head of the workgroup, one of its `qtiles` consecutive query tiles): groups of fewer than four heads fill the
+    // workgroup with several query tiles of the same heads, which share the K / V tiles like heads do
+    const int wave = (tid >> 6) % hpw, qtl = (tid >> 6) / hpw;
     const int qcol = lane & 31, half = lane >> 5;
     // the last query tile of a chunk walks the most keys: the launch hands the tiles out from the last one backwards, so
     // that the longest walks start first when the workgroups do not all fit on the chip at once
     // (a launch whose workgroups all fit at once, two per CU, runs its second half forwards: see attention_chunk)
     const int lin = (int)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
-    const int qt = lin >= fwd_from ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
+    const int qg = lin >= fwd_from ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
+    const int qt = qg * qtiles + qtl;           // (past the last tile of the chunk: a wave without queries, q_live false)
     const int h = kvh * a.group + blockIdx.z * hpw + wave;
     const int tq = qt * PF_TILE + qcol;
     const bool q_live = tq < T;
@@ -103,7 +107,9 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
 
     const size_t base = ((size_t)seq * a.n_kv + kvh) * a.n_ctx;
     const int q_end = qt * PF_TILE + PF_TILE < T ? qt * PF_TILE + PF_TILE : T;      // queries of this tile: [qt*32, q_end)
-    const int n_keys = pos0 + q_end;                                                // keys any of them may see
+    const int n_keys_own = qt * PF_TILE < T ? pos0 + q_end : 0;                     // keys any of them may see
+    const int wg_end = (qg + 1) * qtiles * PF_TILE < T ? (qg + 1) * qtiles * PF_TILE : T;
+    const int n_keys = pos0 + wg_end;                                               // keys the workgroup's last tile walks
     // K is staged as it is: (key, 8-dim piece) pairs, 16 bytes each.  V is staged transposed: an item is the same 8 dims
     // of two neighbouring keys, written as 8 dwords, one per dim, each holding the pair of keys.  Rows past the context
     // end are clamped (masked below).
@@ -165,8 +171,9 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         if constexpr (NP > 0) {
             if (k0 + PF_KEYS < n_keys) fetch_step(k0 + PF_KEYS);
         }
+        if (k0 < n_keys_own) {      // (an earlier query tile of the workgroup is done before the last one)
         // the second 32 keys of the step lie past every query of the tile at the end of the walk
-        const bool two = NT == 2 && k0 + 32 < n_keys;
+        const bool two = NT == 2 && k0 + 32 < n_keys_own;
 
         // S^T = K . Q^T, two tiles of 32 keys x 32 queries: lane (key row = lane % 32 of the A operand, query column =
         // lane % 32 of the result); two independent accumulation chains
@@ -256,6 +263,7 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_h8, v2), pf[t][1], o[db], 0, 0, 0);
             }
         }
+        }
         __syncthreads();        // the tiles are overwritten by the next step
     }
     if (a.out16_k8) {
@@ -341,21 +349,25 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     while (hpw > 8 || a.group % hpw) --hpw;
     // eight heads per KV head: two workgroups of four waves when one of eight per (query tile, KV head) would leave CUs idle
     if (hpw == 8 && ((T + PF_TILE - 1) / PF_TILE) * a.n_kv < pf_n_cu()) hpw = 4;
-    const dim3 grid((unsigned)((T + PF_TILE - 1) / PF_TILE), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
-    const dim3 block((unsigned)(64 * hpw));
+    // groups of fewer than four heads: several consecutive query tiles per workgroup (they share the K / V tiles like heads do)
+    const int qtiles = hpw >= 4 ? 1 : hpw == 1 ? 4 : 2;
+    const int waves = hpw * qtiles, n_tiles = (T + PF_TILE - 1) / PF_TILE;
+    const dim3 grid((unsigned)((n_tiles + qtiles - 1) / qtiles), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
+    const dim3 block((unsigned)(64 * waves));
     // When the whole launch is resident at once with two workgroups per CU, the hardware has been seen to give a CU
     // workgroups i and i + (half the launch): handing the second half its query tiles in forward order pairs a long
     // walk with a short one on every CU.  (A guess about placement costs nothing when wrong: the tiles are the same.)
     const int total = (int)(grid.x * grid.y * grid.z);
     // (half the launch has to be whole rows of query tiles: an even number of (KV head, head group) rows)
-    const int fwd_from = (hpw <= 4 && (grid.y * grid.z) % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
+    const int fwd_from = (waves <= 4 && (grid.y * grid.z) % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
     // (Two tiles per step everywhere.  With 5 heads per KV head one tile per step keeps the kernel under 170 registers, so
     // that two 5-wave workgroups share a CU instead of one: measured slower, 16.5 against 14.8 ms over 32 layers of 4096 tokens.)
+    // NP by the threads of the workgroup: 1024 / threads pairs each, rounded up
 #define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
     do {                                                                                                                  \
-        if (hpw == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);       \
-        else if (hpw >= 4) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);  \
-        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 0, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from);                 \
+        if (waves == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles);      \
+        else if (waves == 6) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 3, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles); \
+        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles);                  \
     } while (0)
     if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_CHUNK_LAUNCH(MESH_F16, MESH_F16);
     else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q8_0, MESH_Q4_0);

@@ -97,8 +97,10 @@ CONFIGS = {
     # head_dim 128 shapes with 5, 8, 2 and 7 query heads per KV head
     "tiny-g5": dict(arch="qwen2", n_layer=2, n_embd=1280, n_head=10, n_head_kv=2, head_dim=128, n_ff=1536, n_vocab=256, eps=1e-6, rope=1e6, bias=True),
     "tiny-g8": dict(arch="llama", n_layer=2, n_embd=1024, n_head=8, n_head_kv=1, head_dim=128, n_ff=1024, n_vocab=256, eps=1e-5, rope=5e5),
-    # three KV heads with one query head each: an odd number of head rows in the chunk attention launch
-    "tiny-mha3": dict(arch="llama", n_layer=1, n_embd=768, n_head=3, n_head_kv=3, head_dim=128, n_ff=768, n_vocab=256, eps=1e-5, rope=1e4),
+    # three KV heads of four query heads: an odd number of head rows in the chunk attention launch
+    "tiny-kv3": dict(arch="llama", n_layer=1, n_embd=1536, n_head=12, n_head_kv=3, head_dim=128, n_ff=768, n_vocab=256, eps=1e-5, rope=1e4),
+    # one query head per KV head (row lengths a multiple of 256, so that every projection is a K-quant)
+    "tiny-mha": dict(arch="llama", n_layer=1, n_embd=512, n_head=4, n_head_kv=4, head_dim=128, n_ff=512, n_vocab=256, eps=1e-5, rope=1e4),
     "tiny-g2": dict(arch="llama", n_layer=2, n_embd=512, n_head=4, n_head_kv=2, head_dim=128, n_ff=512, n_vocab=256, eps=1e-5, rope=1e4),
     "tiny-g7": dict(arch="qwen2", n_layer=2, n_embd=1792, n_head=14, n_head_kv=2, head_dim=128, n_ff=2048, n_vocab=256, eps=1e-6, rope=1e6, bias=True),
     "tiny-odd": dict(arch="qwen2", n_layer=2, n_embd=320, n_head=5, n_head_kv=1, head_dim=64, n_ff=640, n_vocab=96, eps=1e-6, rope=1e4, bias=True, tied=True),

@@ -413,12 +413,12 @@ def test_prefill_path_small_model_with_bias_and_neox(tmp_path):
 
 
 def test_long_chunk_with_an_odd_number_of_head_rows(tmp_path):
-    """2816 tokens of a model with three KV heads, one query head each: the chunk attention launch has 88 query tiles x 3
-    head rows = 264 workgroups, between one and two per CU, an even count with an odd number of rows -- the shape for which a launch
-    must not hand the second half of its workgroups their tiles in forward order (half the launch would not be whole
-    rows, and tiles would be computed twice or not at all).  Also the single-wave-per-workgroup kernel at length."""
+    """2816 tokens of a model with three KV heads of four query heads: the chunk attention launch has 88 query tiles x 3
+    head rows = 264 workgroups, between one and two per CU, an even count with an odd number of rows -- the shape for
+    which a launch must not hand the second half of its workgroups their tiles in forward order (half the launch would
+    not be whole rows, and tiles would be computed twice or not at all)."""
     T = 2816
-    m, cfg, tensors, st = _open(tmp_path, "tiny-mha3", [0], 0, 1, n_ctx=T, n_seq=1, n_batch=T)
+    m, cfg, tensors, st = _open(tmp_path, "tiny-kv3", [0], 0, 1, n_ctx=T, n_seq=1, n_batch=T)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(44))
     orc = StageOracle(cfg, tensors, 0, 1, T, n_seq_max=1)
@@ -428,6 +428,25 @@ def test_long_chunk_with_an_odd_number_of_head_rows(tmp_path):
     ref = orc.forward(x, np.arange(T))
     assert rel_l2(got, ref) <= 3e-3
     assert max(rel_l2(got[i], ref[i]) for i in range(0, T, 29)) <= 1e-2
+    ses.close(); st.close()
+
+
+def test_prefill_chunks_of_a_model_with_one_query_head_per_kv_head(tmp_path):
+    """Groups of fewer than four query heads fill a chunk attention workgroup with several consecutive query tiles (four for
+    one head per KV head): 300 tokens from position 0 (ragged: 9 full tiles + 12 tokens, so the last workgroup has a tile
+    without queries), a second chunk of 100 on top, against the oracle."""
+    m, cfg, tensors, st = _open(tmp_path, "tiny-mha", [0], 0, 1, n_ctx=512, n_seq=1, n_batch=300)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(45))
+    orc = StageOracle(cfg, tensors, 0, 1, 512, n_seq_max=1)
+    ses = st.session()
+    for T, pos0 in ((300, 0), (100, 300)):
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        pos = np.arange(pos0, pos0 + T)
+        got = ses.decode(x, pos).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos)
+        assert rel_l2(got, ref) <= 3e-3, (T, pos0)
+        assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 1e-2, (T, pos0)
     ses.close(); st.close()
 
 
