@@ -33,6 +33,7 @@ struct AttnArgs {
     const int32_t *pos = nullptr, *seq = nullptr;
     float *part = nullptr;         // [T][n_head][n_splits][head_dim]
     float *ml = nullptr;           // [T][n_head][n_splits][2]
+    size_t part_rows = 0;          // attention_chunk only: (token, split) rows part / ml have room for (0: it never splits the keys)
     float *out = nullptr;          // [T][n_head][head_dim]
     // attention_mma only: when set, the result is written as f16 in the k8-major activation layout of the batched GEMM
     // (gemm.hpp; row length n_head * head_dim) INSTEAD of `out`, so the output projection can read it as it is

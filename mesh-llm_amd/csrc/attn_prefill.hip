@@ -19,6 +19,8 @@
 // rpc_server::graph_compute, third_party/llama.cpp/patches/0002-rpc-add-direct-peer-tensor-transfers.patch:443-451)
 // except that Q and the probabilities are rounded to f16 for the matrix cores; sums are f32.
 
+#include <algorithm>
+
 #include "attn.hpp"
 
 namespace mesh {
@@ -63,7 +65,7 @@ __device__ __forceinline__ uint4 pf_row_piece(const uint8_t *row, int piece) {
 // ~50 more registers).  NP: (key, 8-dim piece) pairs of a step one thread carries in registers, at least 512 NT /
 // (threads of the workgroup); 0 for small workgroups, which load each step's rows where they write them.
 template <int KT, int VT, int NP, int NT>
-__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw, int fwd_from, int qtiles) {
+__global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T, int pos0, int seq, int hpw, int fwd_from, int qtiles, int n_ksplit) {
     constexpr int KRB = kv_row_bytes(KT, PF_HD), VRB = kv_row_bytes(VT, PF_HD);
     constexpr int PF_KEYS = 32 * NT;                // keys per step
     constexpr int PF_VPITCH = PF_KEYS / 2 + 2;      // dwords (key pairs) per dim row of the transposed V tile
@@ -80,7 +82,10 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
     const int lin = (int)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
     const int qg = lin >= fwd_from ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x), kvh = blockIdx.y;
     const int qt = qg * qtiles + qtl;           // (past the last tile of the chunk: a wave without queries, q_live false)
-    const int h = kvh * a.group + blockIdx.z * hpw + wave;
+    // blockIdx.z = (head group, key split): with n_ksplit > 1 the workgroup walks one n_ksplit-th of the keys and leaves
+    // an un-normalised partial for attn_combine_kernel (short chunks on a long history, which have few query tiles)
+    const int ks = (int)blockIdx.z % n_ksplit;
+    const int h = kvh * a.group + ((int)blockIdx.z / n_ksplit) * hpw + wave;
     const int tq = qt * PF_TILE + qcol;
     const bool q_live = tq < T;
     const int pos_q = pos0 + tq;
@@ -109,7 +114,11 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
     const int q_end = qt * PF_TILE + PF_TILE < T ? qt * PF_TILE + PF_TILE : T;      // queries of this tile: [qt*32, q_end)
     const int n_keys_own = qt * PF_TILE < T ? pos0 + q_end : 0;                     // keys any of them may see
     const int wg_end = (qg + 1) * qtiles * PF_TILE < T ? (qg + 1) * qtiles * PF_TILE : T;
-    const int n_keys = pos0 + wg_end;                                               // keys the workgroup's last tile walks
+    const int n_keys_wg = pos0 + wg_end;                                            // keys the workgroup's last tile walks
+    const int per_split = (((n_keys_wg + n_ksplit - 1) / n_ksplit) + 63) & ~63;
+    const int k_lo = ks * per_split;
+    const int n_keys = k_lo + per_split < n_keys_wg ? k_lo + per_split : n_keys_wg;   // end of this workgroup's walk
+    const int n_keys_mine = n_keys_own < n_keys ? n_keys_own : n_keys;              // and of this wave's
     // K is staged as it is: (key, 8-dim piece) pairs, 16 bytes each.  V is staged transposed: an item is the same 8 dims
     // of two neighbouring keys, written as 8 dwords, one per dim, each holding the pair of keys.  Rows past the context
     // end are clamped (masked below).
@@ -150,8 +159,8 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
             if (p < PF_KEYS * 8) { rv[i][0] = v_row(k0, p, 0); rv[i][1] = v_row(k0, p, 1); }
         }
     };
-    if constexpr (NP > 0) fetch_step(0);
-    for (int k0 = 0; k0 < n_keys; k0 += PF_KEYS) {
+    if constexpr (NP > 0) fetch_step(k_lo);
+    for (int k0 = k_lo; k0 < n_keys; k0 += PF_KEYS) {
         if constexpr (NP > 0) {
 #pragma unroll
             for (int i = 0; i < NPK; ++i) {
@@ -171,9 +180,9 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         if constexpr (NP > 0) {
             if (k0 + PF_KEYS < n_keys) fetch_step(k0 + PF_KEYS);
         }
-        if (k0 < n_keys_own) {      // (an earlier query tile of the workgroup is done before the last one)
+        if (k0 < n_keys_mine) {     // (an earlier query tile of the workgroup is done before the last one)
         // the second 32 keys of the step lie past every query of the tile at the end of the walk
-        const bool two = NT == 2 && k0 + 32 < n_keys_own;
+        const bool two = NT == 2 && k0 + 32 < n_keys_mine;
 
         // S^T = K . Q^T, two tiles of 32 keys x 32 queries: lane (key row = lane % 32 of the A operand, query column =
         // lane % 32 of the result); two independent accumulation chains
@@ -231,6 +240,9 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o[db][i] *= corr;
         }
+        // (Without key splits key 0 is visible to every query, so m is finite from the first step on.  In a later split a
+        // query may see no key at all: all its scores are -inf and so is m; the reference 0 then gives p = 0, not NaN.)
+        const float mref = m == -INFINITY ? 0.f : m;
         // P^T as the B operand: the lane's own registers, 8 per MFMA
         pf_h8 pf[NT][2];
         float ps0 = 0.f, ps1 = 0.f;
@@ -238,7 +250,7 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         for (int t = 0; t < NT; ++t) {
             float p[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(s[t][i] - m);     // s - m <= PF_RESCALE_STEP; far below, 0
+            for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(s[t][i] - mref);  // s - m <= PF_RESCALE_STEP; far below, 0
 #pragma unroll
             for (int i = 0; i < 16; i += 2) { ps0 += p[i]; ps1 += p[i + 1]; }
             const pf_u4 pu1 = {pf_pack(p[0], p[1]), pf_pack(p[2], p[3]), pf_pack(p[4], p[5]), pf_pack(p[6], p[7])};
@@ -265,6 +277,21 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         }
         }
         __syncthreads();        // the tiles are overwritten by the next step
+    }
+    if (n_ksplit > 1) {
+        // un-normalised partial and (maximum, sum) of this key split, in the layout of the split-KV decode kernels
+        if (q_live) {
+            const size_t prow = ((size_t)tq * a.n_head + h) * n_ksplit + ks;
+            float *pp = a.part + prow * PF_HD;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4)
+                    *reinterpret_cast<float4 *>(pp + db * 32 + 8 * i4 + 4 * half) =
+                        make_float4(o[db][4 * i4], o[db][4 * i4 + 1], o[db][4 * i4 + 2], o[db][4 * i4 + 3]);
+            if (half == 0) { a.ml[prow * 2] = m; a.ml[prow * 2 + 1] = l; }
+        }
+        return;
     }
     if (a.out16_k8) {
         // f16, in the k8-major layout the output projection's GEMM reads (gemm.hpp); the padding columns of the last
@@ -322,6 +349,12 @@ static int pf_n_cu() {
     return n;
 }
 
+// MESH_ATTN_CHUNK_KSPLIT=0: a chunk's walks are never split over workgroups (for comparison)
+static bool pf_ksplit_on() {
+    const char *e = getenv("MESH_ATTN_CHUNK_KSPLIT");
+    return !(e && e[0] == '0');
+}
+
 int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     AttnArgs a = a_in;
@@ -352,22 +385,33 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     // groups of fewer than four heads: several consecutive query tiles per workgroup (they share the K / V tiles like heads do)
     const int qtiles = hpw >= 4 ? 1 : hpw == 1 ? 4 : 2;
     const int waves = hpw * qtiles, n_tiles = (T + PF_TILE - 1) / PF_TILE;
-    const dim3 grid((unsigned)((n_tiles + qtiles - 1) / qtiles), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
+    dim3 grid((unsigned)((n_tiles + qtiles - 1) / qtiles), (unsigned)a.n_kv, (unsigned)(a.group / hpw));
     const dim3 block((unsigned)(64 * waves));
+    // A short chunk on a long history has few query tiles, each with a long walk: split the keys of every walk over
+    // several workgroups (partials in the caller's split buffers, merged by attn_combine_kernel) until the launch has a
+    // workgroup per CU, at most 8 ways, at least 256 keys each, within the buffers' rows of (token, split).
+    int n_ksplit = 1;
+    {
+        const int wgs = (int)(grid.x * grid.y * grid.z), n_keys = pos0 + T;
+        if (a.part && a.ml && pf_ksplit_on() && wgs < pf_n_cu())
+            n_ksplit = std::max(1, std::min(std::min(pf_n_cu() / wgs, 8), std::min(n_keys / 256, (int)(a.part_rows / (size_t)T))));
+        if (n_ksplit > ATTN_SPLITS_CAP) n_ksplit = ATTN_SPLITS_CAP;
+    }
+    grid.z *= (unsigned)n_ksplit;
     // When the whole launch is resident at once with two workgroups per CU, the hardware has been seen to give a CU
     // workgroups i and i + (half the launch): handing the second half its query tiles in forward order pairs a long
     // walk with a short one on every CU.  (A guess about placement costs nothing when wrong: the tiles are the same.)
     const int total = (int)(grid.x * grid.y * grid.z);
     // (half the launch has to be whole rows of query tiles: an even number of (KV head, head group) rows)
-    const int fwd_from = (waves <= 4 && (grid.y * grid.z) % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
+    const int fwd_from = (n_ksplit == 1 && waves <= 4 && (grid.y * grid.z) % 2 == 0 && total <= 2 * pf_n_cu() && total > pf_n_cu()) ? total / 2 : INT32_MAX;
     // (Two tiles per step everywhere.  With 5 heads per KV head one tile per step keeps the kernel under 170 registers, so
     // that two 5-wave workgroups share a CU instead of one: measured slower, 16.5 against 14.8 ms over 32 layers of 4096 tokens.)
     // NP by the threads of the workgroup: 1024 / threads pairs each, rounded up
 #define MESH_CHUNK_LAUNCH(KT, VT)                                                                                         \
     do {                                                                                                                  \
-        if (waves == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles);      \
-        else if (waves == 6) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 3, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles); \
-        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles);                  \
+        if (waves == 8) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 2, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles, n_ksplit);      \
+        else if (waves == 6) MESH_LAUNCH((attn_chunk_kernel<KT, VT, 3, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles, n_ksplit); \
+        else MESH_LAUNCH((attn_chunk_kernel<KT, VT, 4, 2>), grid, block, 0, stream, a, T, pos0, seq, hpw, fwd_from, qtiles, n_ksplit);                  \
     } while (0)
     if (a.k_type == MESH_F16 && a.v_type == MESH_F16) MESH_CHUNK_LAUNCH(MESH_F16, MESH_F16);
     else if (a.k_type == MESH_Q8_0 && a.v_type == MESH_Q4_0) MESH_CHUNK_LAUNCH(MESH_Q8_0, MESH_Q4_0);
@@ -375,6 +419,10 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     else return fail(MESH_ERR_UNSUPPORTED, "attention_chunk: KV cache types %d/%d", a.k_type, a.v_type);
 #undef MESH_CHUNK_LAUNCH
     MESH_LAUNCH_CHECK();
+    if (n_ksplit > 1) {
+        a.n_splits = n_ksplit;
+        return attention_combine(a, T, stream);
+    }
     return MESH_OK;
 }
 

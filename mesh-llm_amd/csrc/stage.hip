@@ -410,6 +410,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
         return r;
     };
     const size_t part_rows = std::max<size_t>(B, ATTN_PART_ROWS_MIN);
+    s->attn_part_rows = part_rows;
     if ((rc = fbuf(&s->x, B * hp.n_embd)) || (rc = fbuf(&s->q, B * QD)) || (rc = fbuf(&s->k, B * KD)) ||
         (rc = fbuf(&s->v, B * KD)) || (rc = fbuf(&s->attn, B * QD)) || (rc = fbuf(&s->ffn, B * ff)) ||
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
@@ -715,6 +716,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) {
             if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }          // straight into the output projection's input layout
             aa.chunk_kv16 = reinterpret_cast<_Float16 *>(s->chunk_kv16);
+            aa.part_rows = s->attn_part_rows;
             rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
         }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {

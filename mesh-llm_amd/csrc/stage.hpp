@@ -89,6 +89,7 @@ struct mesh_session {
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr;
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
+    size_t attn_part_rows = 0;                          // (token, split) rows they hold
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
     uint16_t *xn16 = nullptr, *ffn16 = nullptr;
     uint16_t *chunk_kv16 = nullptr;      // quantised KV caches: f16 rows of one sequence and layer for long prefill chunks (attn.hpp)

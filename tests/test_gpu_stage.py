@@ -431,6 +431,33 @@ def test_long_chunk_with_an_odd_number_of_head_rows(tmp_path):
     ses.close(); st.close()
 
 
+def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path, monkeypatch):
+    """A chunk with few query tiles and a long history splits every tile's walk over several workgroups and merges the
+    partials (the split-KV combine kernel): 96 tokens on top of 448 (two splits), then 48 on top of 2000 (eight splits;
+    the last split holds the diagonal, where the chunk's earlier queries see no key at all).  Against the oracle, and
+    against the same calls with the splitting switched off."""
+    n_ctx = 2112
+    m, cfg, tensors, st = _open(tmp_path, "tiny-qwen2", [0], 0, 1, n_ctx=n_ctx, n_seq=1, n_batch=1024)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(46))
+    orc = StageOracle(cfg, tensors, 0, 1, n_ctx, n_seq_max=1)
+    calls = [(448, 0), (96, 448), (976, 544), (480, 1520), (48, 2000)]
+    xs = [rng.standard_normal((T, E)).astype(np.float32) for T, _ in calls]
+    outs = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("MESH_ATTN_CHUNK_KSPLIT", mode)
+        ses = st.session()
+        outs[mode] = [ses.decode(x, np.arange(p0, p0 + T)).view(np.float32).reshape(T, E).copy() for x, (T, p0) in zip(xs, calls)]
+        ses.close()
+    monkeypatch.delenv("MESH_ATTN_CHUNK_KSPLIT")
+    for x, (T, p0), got, alt in zip(xs, calls, outs["1"], outs["0"]):
+        ref = orc.forward(x, np.arange(p0, p0 + T))
+        assert rel_l2(got, ref) <= 3e-3, (T, p0)
+        assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 1e-2, (T, p0)
+        assert rel_l2(got, alt) <= 2e-3, (T, p0)
+    st.close()
+
+
 def test_prefill_chunks_of_a_model_with_one_query_head_per_kv_head(tmp_path):
     """Groups of fewer than four query heads fill a chunk attention workgroup with several consecutive query tiles (four for
     one head per KV head): 300 tokens from position 0 (ragged: 9 full tiles + 12 tokens, so the last workgroup has a tile
