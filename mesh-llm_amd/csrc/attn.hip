@@ -282,8 +282,14 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float *p_part, 
     for (int s2 = 0; s2 < p_n_splits; ++s2) {
         const float ms = s_m[s2];
         const float w = ms == -INFINITY ? 0.f : exp2f(ms - mh);      // maxima are in log2 units
-        num = fmaf(pp[(size_t)s2 * p_head_dim], w, num);
-        den = fmaf(s_l[s2], w, den);
+        // A split that saw no key has weight 0 and must contribute nothing, whatever its partial row holds: the clamp
+        // turns NaN and infinities into finite values (fmaxf / fminf return the other operand for NaN) and is the
+        // identity otherwise.  (A select on `ms` instead is compiled into a branch around the load, and the 32 loads of
+        // a thread then go out one after the other: measured, 9 us per layer at batch 1.)
+        const float pv = fminf(fmaxf(pp[(size_t)s2 * p_head_dim], -3.4028234664e38f), 3.4028234664e38f);
+        const float lv = fminf(fmaxf(s_l[s2], 0.f), 3.4028234664e38f);
+        num = fmaf(pv, w, num);
+        den = fmaf(lv, w, den);
     }
     if (p_out_q16) {
         q16_store_block32(p_out_q16, p_n_head * p_head_dim, t, h * p_head_dim + dd, num / den);

@@ -232,7 +232,10 @@ __global__ __launch_bounds__(512) void attn_chunk_kernel(const AttnArgs a, int T
         // query, so after the first step m is finite for every live column.)
         if (__builtin_amdgcn_ballot_w64(mx > m + PF_RESCALE_STEP) != 0ull) {
             const float m_new = mx > m + PF_RESCALE_STEP ? mx : m;
-            const float corr = exp2f(m - m_new);                    // exp2(-inf) = 0 while nothing is accumulated; 1 for lanes that stay
+            // 1 for lanes that stay, exp2(-inf) = 0 while nothing is accumulated.  A query that has seen no key yet and
+            // sees none in this step either (a key split that begins inside the tile's position range) has m = m_new =
+            // -inf: its l and o are still zero, and -inf - -inf must not reach them as NaN.
+            const float corr = m_new == -INFINITY ? 1.f : exp2f(m - m_new);
             l *= corr;
             m = m_new;
 #pragma unroll

@@ -104,8 +104,12 @@ class StageOracle:
                 out[t] += float(we) * O.mul_mat(dt, ddata[e * d_sz:(e + 1) * d_sz], E, FE, h)[0].astype(np.float64)
         return out.astype(np.float32)
 
-    def forward(self, x, pos, seq=None):
-        """x: [T, n_embd] f32 -> [T, n_embd] f32 after layers [lb, le); updates the KV cache."""
+    def forward(self, x, pos, seq=None, kv_rows=None):
+        """x: [T, n_embd] f32 -> [T, n_embd] f32 after layers [lb, le); updates the KV cache.
+        kv_rows: {local layer index: (k [T, n_head_kv, head_dim] f32, v likewise)}: rows to put into the cache for this
+        call's tokens in place of the ones computed here.  A test hands in the rows the device under test wrote, which
+        separates its attention arithmetic from the sensitivity of a 4-bit cache quantiser to rounding upstream of it
+        (a value near a decision threshold lands on the neighbouring code)."""
         c = self.c
         x = np.array(x, dtype=np.float32).reshape(-1, c["n_embd"])
         T = x.shape[0]
@@ -129,6 +133,10 @@ class StageOracle:
                 kh, vh = O.kv_round(self.kv_types[0], k), O.kv_round(self.kv_types[1], v)
             else:
                 kh, vh = O.fp32_to_fp16(k), O.fp32_to_fp16(v)
+            if kv_rows is not None and li in kv_rows:
+                kh, vh = (np.asarray(r, np.float32).reshape(T, HK, hd) for r in kv_rows[li])
+                if not self.kv_f32:
+                    kh, vh = O.fp32_to_fp16(kh).reshape(T, HK, hd), O.fp32_to_fp16(vh).reshape(T, HK, hd)
             for t in range(T):
                 self.k[li, seq[t], :, pos[t], :] = kh[t]
                 self.v[li, seq[t], :, pos[t], :] = vh[t]

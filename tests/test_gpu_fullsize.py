@@ -64,11 +64,14 @@ def test_c3_sixteen_layer_stage_decode_at_kv_depth_4095(c3_model):
     orc = StageOracle(cfg, tensors, 0, 16, n_ctx, n_seq_max=n_seq)
     rng = np.random.Generator(np.random.PCG64(4095))
     for il in range(16):
-        k, v = random_kv(rng, depth), random_kv(rng, depth)       # every sequence holds the same context
+        # every sequence holds its own context (a sequence-index mix-up in a batched kernel must show): sequence s is the
+        # layer's random rows rotated by 251 s positions, K and V in opposite directions
+        k, v = random_kv(rng, depth), random_kv(rng, depth)
         for s in range(n_seq):
-            ses.kv_write(il, s, 0, k, v)
-        orc.k[il, :, :, :depth] = np.ascontiguousarray(k.transpose(1, 0, 2))[None]
-        orc.v[il, :, :, :depth] = np.ascontiguousarray(v.transpose(1, 0, 2))[None]
+            ks, vs = np.roll(k, 251 * s, axis=0), np.roll(v, -251 * s, axis=0)
+            ses.kv_write(il, s, 0, ks, vs)
+            orc.k[il, s, :, :depth] = ks.transpose(1, 0, 2)
+            orc.v[il, s, :, :depth] = vs.transpose(1, 0, 2)
     for seqs in ([0], [1, 2, 3, 4], list(range(16))):
         T = len(seqs)
         x = rng.standard_normal((T, 4096)).astype(np.float32)
@@ -212,6 +215,51 @@ def test_c4_qwen25_32b_layers_wide_batches_and_prefill(tmp_path, kv):
         r = rel_l2(got, ref)
         report("C4 layers 7-8, %s KV, decode batch %d" % (kv, T), r)
         assert r <= NORTH_STAR, T
+    ses.close(); st.close()
+
+
+@pytest.mark.parametrize("kv", ["f16", "q8_0/q4_0", "q4_0/q4_0"])
+def test_c4_decode_at_kv_depth_8191(tmp_path, kv):
+    """The context the Qwen2.5-32B-shaped configuration is stated on: layers 7 (q6_K attn_v / ffn_down) and 8 at KV depth
+    8191 of an 8192-token context, decode batch 1, 8 and 32, every sequence with its own cache rows, over an f16 cache and
+    over the two quantised tiers the reference's launcher picks by model size (mesh-llm/src/inference/launch.rs:568-591:
+    K q8_0 / V q4_0, and q4_0 / q4_0).  5 query heads per KV head, 32 key splits at batch 1."""
+    m = mesh()
+    cfg = models.CONFIGS["qwen2.5-32b"]
+    path = os.path.join(str(tmp_path), "c4d.gguf")
+    tensors = models.write_model(path, cfg, [7, 8], seed=42, fast=True)
+    n_ctx, n_seq, depth, E = 8192, 32, 8191, 5120
+    kv_m = {"f16": (m.F16, m.F16), "q8_0/q4_0": (m.Q8_0, m.Q4_0), "q4_0/q4_0": (m.Q4_0, m.Q4_0)}[kv]
+    kv_o = {"f16": None, "q8_0/q4_0": (oracle.Q8_0, oracle.Q4_0), "q4_0/q4_0": (oracle.Q4_0, oracle.Q4_0)}[kv]
+    st = m.Stage(path, 7, 9, n_ctx=n_ctx, n_seq_max=n_seq, n_batch_max=32, kv_types=kv_m)
+    os.unlink(path)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, 7, 9, n_ctx, n_seq_max=n_seq, kv_types=kv_o)
+    rng = np.random.Generator(np.random.PCG64(8191))
+    for il in (7, 8):
+        k, v = random_kv(rng, depth), random_kv(rng, depth)
+        if kv_o:
+            kq = oracle.kv_round(kv_o[0], k.view(np.float16).astype(np.float32))
+            vq = oracle.kv_round(kv_o[1], v.view(np.float16).astype(np.float32))
+        for s in range(n_seq):
+            ks, vs = np.roll(k, 509 * s, axis=0), np.roll(v, -509 * s, axis=0)
+            ses.kv_write(il, s, 0, ks, vs)
+            if kv_o:        # (a row's quantisation depends on that row alone, so rounding commutes with the rotation)
+                orc.k[il - 7, s, :, :depth] = np.roll(kq, 509 * s, axis=0).transpose(1, 0, 2)
+                orc.v[il - 7, s, :, :depth] = np.roll(vq, -509 * s, axis=0).transpose(1, 0, 2)
+            else:
+                orc.k[il - 7, s, :, :depth] = ks.transpose(1, 0, 2)
+                orc.v[il - 7, s, :, :depth] = vs.transpose(1, 0, 2)
+    for seqs in ([5], list(range(8, 16)), list(range(32))):
+        T = len(seqs)
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        pos = [depth] * T
+        got = ses.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos, seq=seqs)
+        r = rel_l2(got, ref)
+        report("C4 layers 7-8, %s KV, depth 8191, decode batch %d" % (kv, T), r)
+        assert r <= NORTH_STAR, T
+        assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR, T
     ses.close(); st.close()
 
 

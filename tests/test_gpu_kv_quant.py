@@ -2,6 +2,7 @@
 mesh-llm/src/inference/launch.rs:568-591) against the CPU oracle: the cache rows bit-exactly, the stage output within
 the stage tolerance (1e-2 rel-L2; the quantisation itself is part of both sides)."""
 import os
+import sys
 
 import numpy as np
 import pytest
@@ -22,6 +23,13 @@ def rel_l2(a, b):
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
 
 PAIRS = [(oracle.Q8_0, oracle.Q4_0), (oracle.Q4_0, oracle.Q4_0)]
+# A prefill chunk that starts an EMPTY sequence over a quantised cache, whole chunk and worst token.  The f16-activation
+# GEMMs move the K / V rows entering the cache by ~1e-3 relative, which lands a fraction of a percent of the 4-bit codes
+# on the neighbouring step (an eighth of the block maximum); the first tokens of a sequence attend to a handful of rows,
+# so nothing averages that out: measured 1.3e-2 (q8_0 / q4_0) and 2.1e-2 (q4_0 / q4_0) for the chunk, 3.9e-2 for its worst token.  This bound is
+# therefore about the quantiser's discontinuity, not the kernels: those are held to 2e-3 by the same test with the
+# device's own cache rows handed to the oracle (measured 8e-4, worst token 9e-4), and the codes that moved are counted.
+CHUNK_TOL, CHUNK_TOL_TOKEN = 3e-2, 6e-2
 
 
 def _open(tmp_path, name, layers, lb, le, kv_types, n_ctx=64, n_seq=2, n_batch=16, seed=5):
@@ -146,15 +154,41 @@ def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types, monk
     xp = rng.standard_normal((T, 4096)).astype(np.float32)
     got = ses.decode(xp, np.arange(T), seq=np.full(T, 9, np.int32)).view(np.float32).reshape(T, 4096)
     ref = orc.forward(xp, np.arange(T), seq=np.full(T, 9, np.int32))
-    assert rel_l2(got, ref) <= 3e-2
-    assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 8e-2
+    r, r_tok = rel_l2(got, ref), max(rel_l2(got[i], ref[i]) for i in range(T))
+    # (a) the rows the chunk left in the cache against the oracle's: the same blocks up to a few codes that sat near a
+    # decision threshold; (b) the oracle run again with the device's rows in its cache: what is left is the arithmetic
+    dev_rows = {}
+    for il in (3, 4):
+        kd, vd = ses.kv_read(il, 9, 0, T)
+        dev_rows[il - 3] = (_f16(kd), _f16(vd))
+        ko, vo = orc.k[il - 3, 9, :, :T].transpose(1, 0, 2), orc.v[il - 3, 9, :, :T].transpose(1, 0, 2)
+        for name, d_, o_, typ in (("K", dev_rows[il - 3][0], ko, kv_types[0]), ("V", dev_rows[il - 3][1], vo, kv_types[1])):
+            blk_max = np.abs(o_).reshape(-1, 32).max(axis=1, keepdims=True) + 1e-30
+            step = blk_max / (7.0 if typ == oracle.Q4_0 else 127.0)
+            off = np.abs(d_.reshape(-1, 32) - o_.reshape(-1, 32)) / step
+            moved = float((off > 0.5).mean())
+            print("[kv-quant] layer %d %s rows: %.3f%% of the codes differ from the oracle's, largest distance %.2f steps" % (il, name, 100 * moved, off.max()),
+                  file=sys.stderr, flush=True)
+            # the first layer's rows come from identical inputs: a code and, rarely, a block scale's rounding on top.  (The
+            # next layer's input already carries the first layer's moved codes, so its rows are only reported.)
+            if il == 3:
+                assert moved <= 0.03 and off.max() <= 2.6
+    ref_same = orc.forward(xp, np.arange(T), seq=np.full(T, 9, np.int32), kv_rows=dev_rows)
+    r_same, r_same_tok = rel_l2(got, ref_same), max(rel_l2(got[i], ref_same[i]) for i in range(T))
+    print("[kv-quant] %s prefill chunk of 200: rel-L2 %.3e, worst token %.3e; with the device's cache rows in the oracle %.3e, %.3e"
+          % (kv_types, r, r_tok, r_same, r_same_tok), file=sys.stderr, flush=True)
+    assert r_same <= 2e-3 and r_same_tok <= 3e-3
+    assert r <= CHUNK_TOL
+    assert r_tok <= CHUNK_TOL_TOKEN
     # a second chunk on top of the first (136 tokens at positions 200 .. 335): chunks this long decode the cache rows
     # they attend to once, into an f16 scratch, before the walk; that has to cover the first chunk's rows too
     T2 = 136
     xp2 = rng.standard_normal((T2, 4096)).astype(np.float32)
     got2 = ses.decode(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32)).view(np.float32).reshape(T2, 4096)
     ref2 = orc.forward(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32))
-    assert rel_l2(got2, ref2) <= 3e-2
+    r2 = rel_l2(got2, ref2)
+    print("[kv-quant] %s second chunk of 136: rel-L2 %.3e" % (kv_types, r2), file=sys.stderr, flush=True)
+    assert r2 <= CHUNK_TOL
     ses.close()
     # the same two chunks with the scratch switched off (every query tile decodes the rows itself): the same values
     # reach the matrix cores in the same order, so the hidden states are bit-identical

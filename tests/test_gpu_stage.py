@@ -458,6 +458,44 @@ def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path, monkeypa
     st.close()
 
 
+def test_key_split_boundary_inside_a_query_tile(tmp_path, monkeypatch):
+    """Chunks whose first position is not a multiple of 32: a key split then begins strictly inside a query tile's
+    position range, so that in the split's first step the tile's earlier queries still see no key while the later ones
+    do.  40 tokens on top of 3560 (eight splits of 512 keys; the last begins at key 3584, inside positions 3560..3591)
+    and 512 tokens on top of 10; finite, against the oracle, and against the same calls with the splitting switched off."""
+    n_ctx = 3712
+    m, cfg, tensors, st = _open(tmp_path, "tiny-qwen2", [0], 0, 1, n_ctx=n_ctx, n_seq=2, n_batch=1024)
+    E = cfg["n_embd"]
+    rng = np.random.Generator(np.random.PCG64(3560))
+    orc = StageOracle(cfg, tensors, 0, 1, n_ctx, n_seq_max=2)
+    hist = {0: 3560, 1: 10}
+    kv = {}
+    for s, n_past in hist.items():
+        k = (rng.standard_normal((n_past, 1, 128)) * 0.5).astype(np.float16).view(np.uint16)
+        v = (rng.standard_normal((n_past, 1, 128)) * 0.5).astype(np.float16).view(np.uint16)
+        kv[s] = (k, v)
+        orc.k[0, s, :, :n_past] = np.ascontiguousarray(k.transpose(1, 0, 2))
+        orc.v[0, s, :, :n_past] = np.ascontiguousarray(v.transpose(1, 0, 2))
+    calls = [(40, 3560, 0), (512, 10, 1)]
+    xs = [rng.standard_normal((T, E)).astype(np.float32) for T, _, _ in calls]
+    outs = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("MESH_ATTN_CHUNK_KSPLIT", mode)
+        ses = st.session()
+        for s, (k, v) in kv.items():
+            ses.kv_write(0, s, 0, k, v)
+        outs[mode] = [ses.decode(x, np.arange(p0, p0 + T), seq=[s] * T).view(np.float32).reshape(T, E).copy() for x, (T, p0, s) in zip(xs, calls)]
+        ses.close()
+    monkeypatch.delenv("MESH_ATTN_CHUNK_KSPLIT")
+    for x, (T, p0, s), got, alt in zip(xs, calls, outs["1"], outs["0"]):
+        assert np.isfinite(got).all(), (T, p0)
+        ref = orc.forward(x, np.arange(p0, p0 + T), seq=[s] * T)
+        assert rel_l2(got, ref) <= 3e-3, (T, p0)
+        assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= 1e-2, (T, p0)
+        assert rel_l2(got, alt) <= 2e-3, (T, p0)
+    st.close()
+
+
 def test_prefill_chunks_of_a_model_with_one_query_head_per_kv_head(tmp_path):
     """Groups of fewer than four query heads fill a chunk attention workgroup with several consecutive query tiles (four for
     one head per KV head): 300 tokens from position 0 (ragged: 9 full tiles + 12 tokens, so the last workgroup has a tile
