@@ -55,6 +55,7 @@ struct GemvKernelArgs {
     const int32_t *items, *n_items;
     GemvRope rope;         // rope.pos / rope.seq already point at the launch's first column
     int kind[3];
+    uint8_t *xq_out;       // EPI_SWIGLU, one column: the output in the xq layout instead of f32 (gemv.hpp)
 };
 
 
@@ -86,7 +87,8 @@ struct GemvKernelArgs {
 // total tile-rows | tile-rows per workgroup << 16, p_begins = first tile-row of matrix 1 | of matrix 2 << 16,
 // p_r_nsb_ks = workgroups with one tile-row more | K / 256 << 16 | waves along K << 24), and whether the launch uses the per-pair expert
 // indirection is a template parameter, so that the dense kernel does not wait for a pointer only to find it null.
-template <int TYPE, int NB, int NU, bool EXPERT>
+// XQ: p_x points at activations in the xq layout (gemv.hpp) instead of an f32 vector.
+template <int TYPE, int NB, int NU, bool EXPERT, bool XQ>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x, const float *p_norm_w, const uint8_t *p_wbase0,
                                                                 const uint8_t *p_wbase1, const uint8_t *p_wbase2, unsigned p_ldx_grid,
                                                                 unsigned p_rows_q, unsigned p_begins, unsigned p_r_nsb_ks,
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dot_kernel(const float *p_x
     const size_t h_expert_stride = EXPERT ? a.expert_stride : 0;
     (void)h_rows;
     const int bid = blockIdx.x;      // (the workgroup count is folded into h_q / h_r: gridDim.x would be one more load from the argument block)
-    constexpr bool GROUPED = false;
+    constexpr bool GROUPED = false, XQ_IN = XQ;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
 #include "gemv_body.inc"
 }
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(GROUPED_THREADS) void gemv_grouped_kernel(const int
     const int p_ldx = (int)(p_ldx_xdiv & 0xFFFFu);
     if ((int)blockIdx.y >= p_n_items[0]) return;
     const int bid = blockIdx.x, nblk = gridDim.x;
-    constexpr bool GROUPED = true;
+    constexpr bool GROUPED = true, XQ_IN = false;
     constexpr int THREADS = GROUPED_THREADS, WAVES = GROUPED_THREADS / 64;
     const int n = __builtin_amdgcn_readfirstlane(p_items[(size_t)blockIdx.y * MOE_ITEM_INTS + 1]);
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_dual_kernel(const float *p_
                                                                  const uint8_t *p_w6, unsigned p_ldx_n4, unsigned p_rows, unsigned p_begin_grid,
                                                                  unsigned p_nsb_ks, const GemvKernelArgs a4, const GemvKernelArgs a6) {
     constexpr int NU = 1;
-    constexpr bool GROUPED = false;
+    constexpr bool GROUPED = false, XQ_IN = false;
     constexpr int THREADS = GEMV_THREADS, WAVES = GEMV_WAVES;
     const int n4 = (int)(p_ldx_n4 >> 16);
     const float *const h_x = p_x, *const h_norm_w = p_norm_w;
@@ -192,7 +194,7 @@ static size_t dot_smem_bytes(int type, int NB, int K, int rows_here, int KS, int
            sizeof(float) * ((size_t)KS * rows_here * NU * 16 * NB + waves * NB);
 }
 
-template <int TYPE, int NB, int NU, bool EXPERT = false>
+template <int TYPE, int NB, int NU, bool EXPERT = false, bool XQ = false>
 static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStream_t stream) {
     if (ka.tile_begin[3] > 0xFFFF || ka.ldx > 0xFFFF || grid.x > 0xFFFFu || ka.K / QK_K > 0xFF)
         return fail(MESH_ERR_UNSUPPORTED, "gemv: %d tile-rows / activation stride %d / %u workgroups / row length %d in one launch",
@@ -200,11 +202,11 @@ static int launch_dot(const GemvKernelArgs &ka, dim3 grid, size_t smem, hipStrea
     const unsigned rows = (unsigned)ka.tile_begin[3], q = rows / grid.x, r = rows % grid.x;
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dot_kernel<TYPE, NB, NU, EXPERT>),
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dot_kernel<TYPE, NB, NU, EXPERT, XQ>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_LIMIT));
         attr_set = true;
     }
-    MESH_LAUNCH((gemv_dot_kernel<TYPE, NB, NU, EXPERT>), grid, dim3(GEMV_THREADS), smem, stream, 
+    MESH_LAUNCH((gemv_dot_kernel<TYPE, NB, NU, EXPERT, XQ>), grid, dim3(GEMV_THREADS), smem, stream, 
         ka.x, ka.norm_w, ka.wbase[0], ka.wbase[1], ka.wbase[2], (unsigned)ka.ldx | (grid.x << 16), rows | (q << 16),
         (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16), r | ((unsigned)(ka.K / QK_K) << 16) | ((unsigned)ka.ks << 24), ka);
     MESH_LAUNCH_CHECK();
@@ -340,6 +342,20 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
         if (type == MESH_Q4_K) return NU == 2 ? launch_dot<MESH_Q4_K, 1, 2, true>(ka, g, smem, stream) : launch_dot<MESH_Q4_K, 1, 1, true>(ka, g, smem, stream);
         return NU == 2 ? launch_dot<MESH_Q6_K, 1, 2, true>(ka, g, smem, stream) : launch_dot<MESH_Q6_K, 1, 1, true>(ka, g, smem, stream);
     }
+    if (a.xq_out) {
+        if (!gemv_xq_out_supported(a)) return fail(MESH_ERR_INVALID, "gemv: xq output asked of a launch that cannot produce it");
+        ka.xq_out = a.xq_out;
+    }
+    if (a.xq_in) {
+        // one column from a quantised vector: the activations argument is that buffer
+        if (!gemv_xq_in_supported(a)) return fail(MESH_ERR_INVALID, "gemv: xq input asked of a launch that cannot read it");
+        GemvKernelArgs kb = ka;
+        kb.x = reinterpret_cast<const float *>(a.xq_in);
+        kb.residual = a.residual;
+        const size_t smem = dot_smem_bytes(type, 1, a.K, rows_max, KS, NU);
+        const dim3 g((unsigned)grid);
+        return type == MESH_Q4_K ? launch_dot<MESH_Q4_K, 1, 1, false, true>(kb, g, smem, stream) : launch_dot<MESH_Q6_K, 1, 1, false, true>(kb, g, smem, stream);
+    }
     int t = 0;
     while (t < a.T) {
         const int left = a.T - t;
@@ -415,6 +431,28 @@ static int gemv_dual(const GemvArgs &a4, const GemvArgs &a6, hipStream_t stream)
     return MESH_OK;
 }
 
+static bool all_tiled_one_type(const GemvArgs &a) {
+    for (int i = 0; i < a.n_mat; ++i)
+        if (!type_is_tiled(a.mat[i].type) || a.mat[i].type != a.mat[0].type) return false;
+    return a.n_mat >= 1;
+}
+
+// The SwiGLU launch of one column can leave its output quantised when every workgroup owns whole 32-element blocks
+// of it: an even number of 16-row tile-rows each, the same for all.
+bool gemv_xq_out_supported(const GemvArgs &a) {
+    if (a.epi != EPI_SWIGLU || a.n_mat != 2 || a.T != 1 || a.expert_ids || !all_tiled_one_type(a) || a.mat[0].M != a.mat[1].M) return false;
+    if (a.mat[0].M % 32 || a.mat[0].M % QK_K || a.K % QK_K) return false;
+    KquantPlan p;
+    if (plan_kquant(a, n_compute_units(), p) != MESH_OK) return false;
+    const int total = a.mat[0].M / TILE_ROWS;
+    return total % p.grid == 0 && (total / p.grid) % 2 == 0;
+}
+
+bool gemv_xq_in_supported(const GemvArgs &a) {
+    return a.T == 1 && a.n_mat == 1 && !a.expert_ids && !a.norm_w && !a.rope.pos && all_tiled_one_type(a) && a.K % QK_K == 0 &&
+           (a.epi == EPI_STORE || a.epi == EPI_RESIDUAL);
+}
+
 bool gemv_can_fuse_rope(const GemvArgs &a) {
     if (!a.rope.pos || a.epi != EPI_STORE || a.expert_ids || a.rope.head_dim % 2 || a.rope.n_rot % 2) return false;
     for (int i = 0; i < a.n_mat; ++i)
@@ -424,12 +462,13 @@ bool gemv_can_fuse_rope(const GemvArgs &a) {
 
 int gemv(const GemvArgs &a, hipStream_t stream) {
     if (a.rope.pos && !gemv_can_fuse_rope(a)) return fail(MESH_ERR_INVALID, "gemv: rope epilogue asked for a launch that cannot carry it");
-    if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.K <= 0 || a.T < 0)
+    if (a.n_mat < 1 || a.n_mat > 3 || (!a.x && !a.xq_in) || a.K <= 0 || a.T < 0)
         return fail(MESH_ERR_INVALID, "gemv: bad arguments (n_mat %d, K %d, T %d)", a.n_mat, a.K, a.T);
     if (a.epi == EPI_SWIGLU && a.n_mat != 2) return fail(MESH_ERR_INVALID, "gemv: swiglu needs exactly gate and up");
     if (a.epi == EPI_SWIGLU && a.mat[0].M != a.mat[1].M) return fail(MESH_ERR_INVALID, "gemv: gate and up differ in rows");
     if (a.epi == EPI_RESIDUAL && !a.residual) return fail(MESH_ERR_INVALID, "gemv: residual epilogue without residual");
-    if ((a.ldx % 4) || (reinterpret_cast<uintptr_t>(a.x) & 15)) return fail(MESH_ERR_INVALID, "gemv: x must be 16-byte aligned");
+    if (!a.xq_in && ((a.ldx % 4) || (reinterpret_cast<uintptr_t>(a.x) & 15))) return fail(MESH_ERR_INVALID, "gemv: x must be 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(a.xq_in) & 15) || (reinterpret_cast<uintptr_t>(a.xq_out) & 15)) return fail(MESH_ERR_INVALID, "gemv: xq buffers must be 16-byte aligned");
     bool uniform = true;
     for (int i = 0; i < a.n_mat; ++i) {
         const GemvMat &m = a.mat[i];

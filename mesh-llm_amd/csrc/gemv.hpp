@@ -95,7 +95,19 @@ struct GemvArgs {
     // Fused RoPE / KV append: kind[i] says what matrix i produces (tiled K-quant matrices, EPI_STORE, no experts only)
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+    // Activations quantised by their producer (T == 1).  xq_out: an EPI_SWIGLU launch also leaves its output vector in
+    // the "xq" layout below (the 16-bit fixed-point form every mat-vec workgroup otherwise derives from the f32 vector for
+    // itself, the same bits) and skips the f32 store.  xq_in: the launch reads its activations from such a buffer
+    // instead of x (no norm).  Callers ask gemv_xq_out_supported / gemv_xq_in_supported first.
+    uint8_t *xq_out = nullptr;
+    const uint8_t *xq_in = nullptr;
 };
+// "xq" layout of a vector of K elements (K a multiple of 256): int8 hi[K] | int8 lo[K] | f32 d[K / 32] | f32 s[K / 32] |
+// int32 i16[K / 16]: element k ~ d[k / 32] * (256 * hi[k] + lo[k]), s = d * (sum of the block's 32 fixed-point values),
+// i16 = sum of 16 of them (what the q6_K kernels need)
+inline size_t xq_bytes(int K) { return (size_t)K * 2 + (size_t)(K / 32) * 8 + (size_t)(K / 16) * 4; }
+bool gemv_xq_out_supported(const GemvArgs &a);
+bool gemv_xq_in_supported(const GemvArgs &a);
 // whether gemv() will honour a.rope for this argument set (otherwise the caller runs rope_kv itself)
 bool gemv_can_fuse_rope(const GemvArgs &a);
 

@@ -128,6 +128,32 @@ __device__ __forceinline__ void x_quantise(const XRegs<NB> &X, int K, const XSta
     }
 }
 
+// Producer side of the "xq" layout (gemv.hpp): called by 32 consecutive lanes (an aligned half of a wave, all active) that
+// hold elements kk .. kk + 31 of a vector of K elements, one each (kk: this lane's element).  The same arithmetic as
+// x_quantise on the same 32 values, hence the same bits.
+__device__ __forceinline__ void xq_store_block32(uint8_t *xq, int K, int kk, float v) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const float inv = amax > 0.f ? XQ_LEVELS / amax : 0.f;
+    const int q = __float2int_rn(v * inv);
+    const int lo = ((q + 128) & 0xFF) - 128, hi = (q - lo) >> 8;
+    int isum = q;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) isum += __shfl_xor(isum, o);
+    const int isum32 = isum + __shfl_xor(isum, 16);
+    xq[kk] = (uint8_t)hi;
+    xq[K + kk] = (uint8_t)lo;
+    float *xd = reinterpret_cast<float *>(xq + 2 * (size_t)K), *xs = xd + (K >> 5);
+    int *xi16 = reinterpret_cast<int *>(xs + (K >> 5));
+    if ((kk & 15) == 0) xi16[kk >> 4] = isum;
+    if ((kk & 31) == 0) {
+        const float d = amax / XQ_LEVELS;
+        xd[kk >> 5] = d;
+        xs[kk >> 5] = d * (float)isum32;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ tiles
 template <int TYPE> struct TileRegs;
 

@@ -385,6 +385,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
+    if (const char *e = getenv("MESH_XQ_HANDOVER")) s->xq_handover = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_FUSE_QUANT")) s->moe_fuse_quant = e[0] != '0';
     if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
@@ -415,6 +416,10 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->v, B * KD)) || (rc = fbuf(&s->attn, B * QD)) || (rc = fbuf(&s->ffn, B * ff)) ||
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
+    if (hp.n_ff && hp.n_ff % QK_K == 0) {
+        if ((rc = sess_alloc(s.get(), &p, xq_bytes((int)hp.n_ff))) != MESH_OK) return rc;
+        s->ffn_xq = static_cast<uint8_t *>(p);
+    }
     if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens())) {
         const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
@@ -1051,15 +1056,21 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         ga.x = s->x; ga.ldx = E; ga.K = E; ga.T = T;
         ga.norm_w = static_cast<const float *>(L.ffn_norm.data); ga.eps = hp.rms_eps;
         ga.epi = EPI_SWIGLU;
-        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ga, stream); }
-        if (rc != MESH_OK) return rc;
-
         // x += Wdown . ffn
         GemvArgs da;
         da.n_mat = 1;
         da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
         da.x = s->ffn; da.ldx = (int)hp.n_ff; da.K = (int)hp.n_ff; da.T = T;
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        // a single token: the gate / up launch leaves the FFN vector in the fixed-point form the down projection's
+        // workgroups would each derive from it again (the same bits), and the down projection copies that
+        if (s->ffn_xq && s->xq_handover && gemv_xq_out_supported(ga) && gemv_xq_in_supported(da)) {
+            ga.xq_out = s->ffn_xq;
+            da.xq_in = s->ffn_xq;
+        }
+        { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ga, stream); }
+        if (rc != MESH_OK) return rc;
+
         { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(da, stream); }
         if (rc != MESH_OK) return rc;
     }

@@ -88,6 +88,8 @@ struct mesh_session {
     size_t k_layer_bytes = 0, v_layer_bytes = 0;
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr;
+    uint8_t *ffn_xq = nullptr;                          // single-token decode: the FFN vector as its producer quantised it (gemv.hpp: xq layout)
+    bool xq_handover = true;                            // MESH_XQ_HANDOVER=0 at session creation: the down projection quantises the f32 vector itself
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     size_t attn_part_rows = 0;                          // (token, split) rows they hold
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer

@@ -622,6 +622,30 @@ def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
         st.close()
 
 
+def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path, monkeypatch):
+    """At one token per call the gate / up launch leaves the FFN vector in the 16-bit fixed-point form the down projection
+    consumes (whole 32-element blocks per workgroup), and the down projection copies it instead of quantising the f32
+    vector in every workgroup.  The same arithmetic on the same values: bit-identical outputs with the hand-over switched
+    off, through a q6_K and a q4_K down projection (real shape) and on a small model whose FFN rows do not split into
+    whole blocks per workgroup (where the hand-over must not be taken)."""
+    for name, layers in (("llama3-8b", [3, 4]), ("tiny-llama", [0, 1])):
+        m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=64, n_seq=2, n_batch=4)
+        E = cfg["n_embd"]
+        rng = np.random.Generator(np.random.PCG64(77))
+        xs = [rng.standard_normal((1, E)).astype(np.float32) * (50.0 if i == 2 else 1.0) for i in range(4)]
+        runs = []
+        for flag in ("1", "0"):
+            monkeypatch.setenv("MESH_XQ_HANDOVER", flag)
+            ses = st.session()
+            runs.append([ses.decode(x, [i]).copy() for i, x in enumerate(xs)])
+            ses.close()
+        monkeypatch.delenv("MESH_XQ_HANDOVER")
+        for a, b in zip(*runs):
+            assert np.isfinite(a.view(np.float32)).all()
+            assert np.array_equal(a, b)
+        st.close()
+
+
 @pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-moe", [0, 1])])
 def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers):
     """Decode-sized batches replay their layer launches from a captured graph (first use of a shape eager, second
