@@ -161,6 +161,10 @@ typedef struct mesh_session mesh_session;
 /* Pseudo-formats for the two ends of the pipeline. */
 #define MESH_TOKENS 100   /* input: int32 token ids (stage must start at layer 0 and the file hold token_embd) */
 #define MESH_LOGITS 101   /* output: f32 [n_tokens][n_vocab] after output_norm and the output projection */
+/* Most tokens one mesh_stage_decode call (host pointers) returns logits for: its pinned staging holds that many rows of the
+ * vocabulary.  More tokens in one call fail with MESH_ERR_INVALID; mesh_stage_decode_dev writes straight into the caller's
+ * device buffer and has no such limit. */
+#define MESH_LOGITS_TOKENS_MAX 128
 
 typedef struct mesh_stage_opts {
     const char *device;     /* "ROCm0" / "HIP0" / "0"; NULL = current device               (-d, launch.rs:920-952) */

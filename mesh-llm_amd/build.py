@@ -55,7 +55,7 @@ RPC_SERVER = os.path.join(HERE, "rpc-server")
 def build_rpc_server():
     """Links mesh-llm_amd/rpc-server: the rpc-server-compatible front end over libmeshstage.so (host code only; its
     buffers are HBM through the HIP runtime)."""
-    srcs = [os.path.join(RPC_SRC, f) for f in ("rpc_main.cpp", "rpc_server.cpp", "rpc_buffers_hip.cpp")]
+    srcs = [os.path.join(RPC_SRC, f) for f in ("rpc_main.cpp", "rpc_server.cpp", "rpc_graph.cpp", "rpc_graph_runner.cpp", "rpc_buffers_hip.cpp")]
     cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-pthread", *srcs, "-L" + HERE, "-lmeshstage", "-Wl,-rpath,$ORIGIN", "-o", RPC_SERVER]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -67,7 +67,8 @@ def build_rpc_server_hostmem(out_path):
     """The same server with tests/rpc_hostmem/buffers_host.cpp in place of the HIP buffers (g++ only): what the protocol
     tests run on a machine without a GPU.  Test infrastructure, never shipped."""
     root = os.path.dirname(HERE)
-    srcs = [os.path.join(RPC_SRC, "rpc_main.cpp"), os.path.join(RPC_SRC, "rpc_server.cpp"), os.path.join(root, "tests", "rpc_hostmem", "buffers_host.cpp")]
+    srcs = [os.path.join(RPC_SRC, "rpc_main.cpp"), os.path.join(RPC_SRC, "rpc_server.cpp"), os.path.join(RPC_SRC, "rpc_graph.cpp"),
+            os.path.join(root, "tests", "rpc_hostmem", "buffers_host.cpp"), os.path.join(root, "tests", "rpc_hostmem", "runner_host.cpp")]
     cmd = [os.environ.get("CXX", "g++"), "-O1", "-std=c++17", "-Wall", "-pthread", "-I" + RPC_SRC, *srcs, "-L" + HERE, "-lmeshstage", "-L/opt/rocm/lib",
            "-Wl,-rpath," + HERE, "-Wl,-rpath,/opt/rocm/lib", "-o", out_path]
     r = subprocess.run(cmd, capture_output=True, text=True)

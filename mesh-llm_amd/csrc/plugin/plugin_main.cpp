@@ -234,6 +234,9 @@ static void handle_decode(int fd, State &st, const std::string &head, const std:
     const int in_fmt = format_id(header_value(head, "X-Mesh-In-Format"), MESH_Q8_0), out_fmt = format_id(header_value(head, "X-Mesh-Out-Format"), MESH_Q8_0);
     if (T < 1 || T > st.cfg.n_batch_max || pos0 < 0 || pos0 > (1 << 30) || seq < 0 || in_fmt < 0 || out_fmt < 0 || in_fmt == MESH_LOGITS || out_fmt == MESH_TOKENS)
         return http_error(fd, "400 Bad Request", "X-Mesh-Tokens / X-Mesh-Pos0 / formats out of range", "invalid_request_error");
+    // (refused before anything is allocated for it: a row of logits is the whole vocabulary)
+    if (out_fmt == MESH_LOGITS && T > MESH_LOGITS_TOKENS_MAX)
+        return http_error(fd, "400 Bad Request", "logits of at most " + std::to_string(MESH_LOGITS_TOKENS_MAX) + " tokens per request", "invalid_request_error");
     const size_t want = in_fmt == MESH_TOKENS ? (size_t)T * 4 : mesh_act_packed_size(in_fmt, T, st.info.n_embd);
     if (body.size() != want) return http_error(fd, "400 Bad Request", "body has " + std::to_string(body.size()) + " bytes, " + std::to_string(want) + " expected", "invalid_request_error");
     std::vector<int32_t> pos((size_t)T), seqs((size_t)T, seq);
@@ -245,6 +248,7 @@ static void handle_decode(int fd, State &st, const std::string &head, const std:
     int rc;
     {
         std::lock_guard<std::mutex> lk(st.decode_mu);
+        if (st.stopping || !st.session) return http_error(fd, "503 Service Unavailable", "the plugin is shutting down", "stage_unavailable");
         rc = mesh_stage_decode(st.session, &b, body.data(), in_fmt, &out[0], out_fmt, cap, &len);
     }
     if (rc != MESH_OK) return http_error(fd, rc == MESH_ERR_INVALID ? "400 Bad Request" : "500 Internal Server Error", mesh_last_error(), "stage_error");
@@ -389,7 +393,13 @@ int main(int argc, char **argv) {
     st.stopping = true;
     ::close(fd);
     if (st.http_fd >= 0) { ::shutdown(st.http_fd, SHUT_RDWR); ::close(st.http_fd); }
-    if (st.session) mesh_stage_session_free(st.session);
-    if (st.stage) mesh_stage_close(st.stage);
+    {
+        // a request thread may be inside a decode call: wait for it, and let later ones find the session gone
+        std::lock_guard<std::mutex> lk(st.decode_mu);
+        if (st.session) mesh_stage_session_free(st.session);
+        st.session = nullptr;
+        if (st.stage) mesh_stage_close(st.stage);
+        st.stage = nullptr;
+    }
     return rc;
 }

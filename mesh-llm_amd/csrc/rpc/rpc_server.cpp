@@ -19,6 +19,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <chrono>
 #include <fstream>
 #include <thread>
 
@@ -154,18 +155,23 @@ int Server::listen_on() {
 }
 
 void Server::stop() {
-    if (listen_fd_ >= 0) {
-        ::shutdown(listen_fd_, SHUT_RDWR);
-        ::close(listen_fd_);
-        listen_fd_ = -1;
+    const int fd = listen_fd_.exchange(-1);
+    if (fd >= 0) {
+        ::shutdown(fd, SHUT_RDWR);
+        ::close(fd);
     }
+    std::unique_lock<std::mutex> lk(clients_mu_);
+    for (int cfd : client_fds_) ::shutdown(cfd, SHUT_RDWR);       // their blocking reads return; the threads close the sockets themselves
+    clients_cv_.wait_for(lk, std::chrono::seconds(10), [this]() { return client_fds_.empty(); });
 }
 
 void Server::serve() {
-    while (listen_fd_ >= 0) {
-        const int fd = ::accept(listen_fd_, nullptr, nullptr);
+    for (;;) {
+        const int lfd = listen_fd_.load();
+        if (lfd < 0) break;
+        const int fd = ::accept(lfd, nullptr, nullptr);
         if (fd < 0) {
-            if (listen_fd_ < 0) break;
+            if (listen_fd_.load() < 0) break;
             if (errno == EINTR || errno == ECONNABORTED) continue;
             log("accept failed: %s", strerror(errno));
             break;
@@ -173,11 +179,20 @@ void Server::serve() {
         tune_socket(fd);
         printf("Accepted client connection\n");
         fflush(stdout);
+        {
+            std::lock_guard<std::mutex> lk(clients_mu_);
+            client_fds_.insert(fd);
+        }
         std::thread([this, fd]() {
-            Conn conn(fd);
-            serve_client(conn);
-            printf("Client connection closed\n");
-            fflush(stdout);
+            {
+                Conn conn(fd);
+                serve_client(conn);
+                printf("Client connection closed\n");
+                fflush(stdout);
+                std::lock_guard<std::mutex> lk(clients_mu_);      // (before the socket closes: the number cannot be reused while it is listed)
+                client_fds_.erase(fd);
+                clients_cv_.notify_all();                         // under the lock: the last thing this thread does with the server
+            }
         }).detach();
     }
 }
@@ -289,37 +304,47 @@ bool Server::register_peer(const RegisterPeerReq &req) {
         return false;
     }
     std::lock_guard<std::mutex> lk(peers_mu_);
-    peers_[req.peer_id] = Peer{endpoint, nullptr};
+    peers_[req.peer_id] = Peer{endpoint, nullptr};      // (a re-registration drops the old link)
     debug("registered peer %u at %s", req.peer_id, endpoint.c_str());
     return true;
 }
 
-// caller holds peers_mu_
-std::shared_ptr<Conn> Server::peer_conn(uint32_t peer_id) {
-    auto it = peers_.find(peer_id);
-    if (it == peers_.end()) {
-        log("push: unknown peer %u", peer_id);
-        return nullptr;
+// The link to a registered peer, connected on first use.  The registry lock is held only to look the peer up and to publish
+// a new link: connecting and the HELLO exchange happen outside it (the reference releases its lock before it talks to the
+// peer, patches/0002:589-621), so one slow or dead peer does not stall pushes to the others.
+std::shared_ptr<Server::PeerLink> Server::peer_link(uint32_t peer_id) {
+    std::string endpoint;
+    {
+        std::lock_guard<std::mutex> lk(peers_mu_);
+        auto it = peers_.find(peer_id);
+        if (it == peers_.end()) {
+            log("push: unknown peer %u", peer_id);
+            return nullptr;
+        }
+        if (it->second.link) return it->second.link;
+        endpoint = it->second.endpoint;
     }
-    Peer &p = it->second;
-    if (p.conn) return p.conn;
-    const size_t colon = p.endpoint.rfind(':');
-    const std::string host = p.endpoint.substr(0, colon);
-    const int port = atoi(p.endpoint.c_str() + colon + 1);
-    std::shared_ptr<Conn> c(Conn::connect_to(host, port).release());
-    if (!c) {
-        log("push: cannot connect to peer %u at %s", peer_id, p.endpoint.c_str());
+    const size_t colon = endpoint.rfind(':');
+    const std::string host = endpoint.substr(0, colon);
+    const int port = atoi(endpoint.c_str() + colon + 1);
+    std::shared_ptr<PeerLink> link(new PeerLink());
+    link->conn = Conn::connect_to(host, port);
+    if (!link->conn) {
+        log("push: cannot connect to peer %u at %s", peer_id, endpoint.c_str());
         return nullptr;
     }
     const uint8_t cmd = CMD_HELLO;
     HelloReq hreq{};
     HelloRsp hrsp{};
-    if (!c->send_all(&cmd, 1) || !c->send_msg(&hreq, sizeof hreq) || !c->recv_msg(&hrsp, sizeof hrsp) || hrsp.major != PROTO_MAJOR) {
-        log("push: peer %u at %s does not speak protocol %d.x", peer_id, p.endpoint.c_str(), PROTO_MAJOR);
+    if (!link->conn->send_all(&cmd, 1) || !link->conn->send_msg(&hreq, sizeof hreq) || !link->conn->recv_msg(&hrsp, sizeof hrsp) || hrsp.major != PROTO_MAJOR) {
+        log("push: peer %u at %s does not speak protocol %d.x", peer_id, endpoint.c_str(), PROTO_MAJOR);
         return nullptr;
     }
-    p.conn = c;
-    return c;
+    std::lock_guard<std::mutex> lk(peers_mu_);
+    auto it = peers_.find(peer_id);
+    if (it == peers_.end() || it->second.endpoint != endpoint) return link;      // re-registered meanwhile: use this link once
+    if (!it->second.link) it->second.link = link;                                // (another thread may have connected first: keep its link)
+    return it->second.link;
 }
 
 bool Server::push_tensor_to_peer(const PushTensorToPeerReq &req) {
@@ -340,19 +365,93 @@ bool Server::push_tensor_to_peer(const PushTensorToPeerReq &req) {
                                             reinterpret_cast<const void *>((uintptr_t)(req.src.data + req.offset)), req.size))
             return false;
     }
-    std::lock_guard<std::mutex> lk(peers_mu_);
-    std::shared_ptr<Conn> c = peer_conn(req.peer_id);
-    if (!c) return false;
+    std::shared_ptr<PeerLink> link = peer_link(req.peer_id);
+    if (!link) return false;
     const uint8_t cmd = CMD_PEER_TENSOR_DATA;
     uint8_t result = 0;
-    if (!c->send_all(&cmd, 1) || !c->send_msg(payload.data(), payload.size()) || !c->recv_msg(&result, 1)) {
+    bool sent;
+    {
+        std::lock_guard<std::mutex> io(link->io);          // this peer's connection only
+        sent = link->conn->send_all(&cmd, 1) && link->conn->send_msg(payload.data(), payload.size()) && link->conn->recv_msg(&result, 1);
+    }
+    if (!sent) {
         log("push: lost the connection to peer %u", req.peer_id);
-        peers_[req.peer_id].conn = nullptr;
+        std::lock_guard<std::mutex> lk(peers_mu_);
+        auto it = peers_.find(req.peer_id);
+        if (it != peers_.end() && it->second.link == link) it->second.link = nullptr;       // the next push connects again
         return false;
     }
     if (result != 1) log("push: peer %u rejected the tensor data", req.peer_id);
     return result == 1;
 }
+
+// ------------------------------------------------------------------------------------------------ graphs
+// mu_ held.  The three tensors the run touches must lie inside live buffers of the graph's device.
+bool Server::run_graph(const ParsedGraph &g) {
+    if (g.device >= cfg_.devices.size()) {
+        log("graph: device %u of %zu", g.device, cfg_.devices.size());
+        return false;
+    }
+    const int dev = cfg_.devices[g.device];
+    StagePlan plan;
+    std::string why;
+    if (!recognise_layer_range(g, &plan, &why)) {
+        log("graph of %zu nodes refused: %s", g.nodes.size(), why.c_str());
+        return false;
+    }
+    const Tensor *io[3] = {&plan.input, &plan.positions, &plan.output};
+    const char *what[3] = {"graph (hidden-state input)", "graph (positions)", "graph (result)"};
+    for (int i = 0; i < 3; ++i) {
+        const Buffer *b = locate(*io[i], 0, tensor_nbytes(*io[i]), what[i]);
+        if (!b) return false;
+        if (b->dev != dev) {
+            log("%s: tensor lives on another device than the graph's", what[i]);
+            return false;
+        }
+    }
+    // contiguous rows are what the stage reads and writes
+    if (plan.input.nb[0] != 4 || plan.input.nb[1] != 4ull * plan.input.ne[0] || plan.output.nb[0] != 4 || plan.output.nb[1] != 4ull * plan.output.ne[0] ||
+        plan.positions.nb[0] != 4) {
+        log("graph refused: input, positions or result tensor is not contiguous");
+        return false;
+    }
+    if (!graph_runner()->run(dev, cfg_.gguf_path, plan, &why)) {
+        log("graph of layers [%d, %d), %d tokens failed: %s", plan.layer_begin, plan.layer_end, plan.n_tokens, why.c_str());
+        return false;
+    }
+    debug("graph: layers [%d, %d), %d tokens%s", plan.layer_begin, plan.layer_end, plan.n_tokens, plan.logits ? ", logits" : "");
+    return true;
+}
+
+bool Server::graph_compute(const std::vector<uint8_t> &input) {
+    ParsedGraph g;
+    std::string why;
+    if (!parse_graph(input.data(), input.size(), &g, &why)) {
+        log("graph_compute: malformed payload: %s", why.c_str());
+        return false;
+    }
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!run_graph(g)) return false;
+    stored_graphs_[g.device] = input;
+    return true;
+}
+
+bool Server::graph_recompute(uint32_t device) {
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = stored_graphs_.find(device);
+    if (it == stored_graphs_.end()) {
+        log("graph_recompute: device %u has no stored graph", device);
+        return false;
+    }
+    ParsedGraph g;
+    std::string why;
+    // parsed and checked again: buffers may have been freed since the graph ran
+    if (!parse_graph(it->second.data(), it->second.size(), &g, &why)) return false;
+    return run_graph(g);
+}
+
+// a serialized graph: 296 bytes per tensor; a 64-layer range has a few thousand
+constexpr uint64_t GRAPH_PAYLOAD_LIMIT = (uint64_t)256 << 20;
 
 void Server::serve_client(Conn &conn) {
     // a tensor payload cannot be larger than the largest live buffer it could land in
@@ -557,10 +656,16 @@ void Server::serve_client(Conn &conn) {
                 if (!conn.send_msg(&result, 1)) return;
                 break;
             }
-            case CMD_GRAPH_COMPUTE:
-            case CMD_GRAPH_RECOMPUTE:
-                log("graph execution over RPC is not served by this build (command %u); use the stage library's decode call", cmd);
-                return;
+            case CMD_GRAPH_COMPUTE: {
+                std::vector<uint8_t> input;
+                if (!conn.recv_msg(input, GRAPH_PAYLOAD_LIMIT) || !graph_compute(input)) return;
+                break;                  // no reply (patches/0002: the client does not wait for one)
+            }
+            case CMD_GRAPH_RECOMPUTE: {
+                GraphRecomputeReq req;
+                if (!conn.recv_msg(&req, sizeof req) || !graph_recompute(req.device)) return;
+                break;                  // no reply
+            }
             default:
                 return;
         }

@@ -1,17 +1,22 @@
 // rpc-server-compatible front end of the stage library: the process mesh-llm starts per serving node
 // (mesh-llm/src/inference/launch.rs:887-1030) and the peer of llama-server's RPC backend.  Buffer, tensor-transfer,
-// local-GGUF load and server-to-server push commands are served; graph execution is not part of this build and ends the
-// connection with a message, as an unknown command would.
+// local-GGUF load and server-to-server push commands are served; of graphs, the decoder sub-graph of a contiguous layer
+// range is recognised and run as one stage decode call (rpc_graph.hpp), any other graph ends the connection with a logged
+// reason, as a failing request does in the reference.
 #pragma once
 
+#include <atomic>
+#include <condition_variable>
 #include <cstdint>
 #include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "rpc_buffers.hpp"
+#include "rpc_graph.hpp"
 #include "rpc_wire.hpp"
 
 namespace mesh_rpc {
@@ -53,6 +58,8 @@ class Server {
     int listen_on();
     // accept loop: one thread per client; returns when stop() closes the listening socket
     void serve();
+    // closes the listening socket, shuts the clients' sockets down and waits for their threads to leave (they touch the
+    // buffers the destructor frees)
     void stop();
     // one client connection until it closes or sends something this build does not serve
     void serve_client(Conn &conn);
@@ -63,9 +70,14 @@ class Server {
         uint64_t size;
         int dev;                         // backend device index
     };
+    // a connection to a peer server and the lock that keeps two pushes to that peer from interleaving on it
+    struct PeerLink {
+        std::unique_ptr<Conn> conn;
+        std::mutex io;
+    };
     struct Peer {
         std::string endpoint;
-        std::shared_ptr<Conn> conn;      // connected on first push
+        std::shared_ptr<PeerLink> link;  // connected on first push
     };
 
     // the byte range [t.data + offset, + size) of a live buffer; nullptr with a logged reason otherwise
@@ -76,16 +88,24 @@ class Server {
     bool set_tensor_gguf(const SetTensorGgufReq &req);
     bool register_peer(const RegisterPeerReq &req);
     bool push_tensor_to_peer(const PushTensorToPeerReq &req);
-    std::shared_ptr<Conn> peer_conn(uint32_t peer_id);
+    std::shared_ptr<PeerLink> peer_link(uint32_t peer_id);
+    // GRAPH_COMPUTE: parse, recognise, run, remember for GRAPH_RECOMPUTE (patches/0001:163-174: one stored graph per device)
+    bool graph_compute(const std::vector<uint8_t> &input);
+    bool graph_recompute(uint32_t device);
+    bool run_graph(const ParsedGraph &g);
     void log(const char *fmt, ...) __attribute__((format(printf, 2, 3)));
     void debug(const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 
     BufferBackend *backend_;
     ServerConfig cfg_;
-    int listen_fd_ = -1;
+    std::atomic<int> listen_fd_{-1};                         // read by the accept loop while stop() closes it
+    std::mutex clients_mu_;
+    std::condition_variable clients_cv_;
+    std::unordered_set<int> client_fds_;                     // sockets of the running client threads
     std::mutex mu_;                                          // guards buffers_ and every backend call, like the reference's backend_mutex
     std::unordered_map<uint64_t, std::unique_ptr<Buffer>> buffers_;   // handle -> buffer
-    std::mutex peers_mu_;
+    std::unordered_map<uint32_t, std::vector<uint8_t>> stored_graphs_;  // RPC device -> payload of its last graph that ran (under mu_)
+    std::mutex peers_mu_;                                    // guards the registry only, never held across network traffic
     std::unordered_map<uint32_t, Peer> peers_;
 };
 

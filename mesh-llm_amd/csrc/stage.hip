@@ -340,7 +340,7 @@ static int sess_alloc(mesh_session *s, void **p, size_t bytes) {
 constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
-constexpr int LOGITS_TOKENS_MAX = 128;        // logits rows the host-pointer entry point stages per call
+constexpr int LOGITS_TOKENS_MAX = MESH_LOGITS_TOKENS_MAX;        // logits rows the host-pointer entry point stages per call
 // calls with at least this many tokens take the MFMA GEMM path (MESH_GEMM_MIN_TOKENS overrides, for tuning)
 static int gemm_min_tokens() {
     static int v = 0;

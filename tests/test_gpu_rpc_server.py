@@ -65,3 +65,70 @@ def test_device_memory_and_gguf_load_into_hbm(server_bin, tmp_path):
             at += (len(raw) + 255) // 256 * 256
         assert c.free_buffer(h)
         c.close()
+
+
+@pytest.mark.parametrize("name,lb,le,with_output", [("tiny-llama", 1, 3, False), ("tiny-qwen2", 1, 3, True), ("tiny-moe", 0, 2, False)])
+def test_graph_compute_of_a_layer_range_equals_the_stage_library(server_bin, tmp_path, name, lb, le, with_output):
+    """GRAPH_COMPUTE with the decoder sub-graph of a layer range, tensors in HBM buffers of the server: a 5-token prompt
+    chunk, then single-token steps replayed with GRAPH_RECOMPUTE (same graph, new input and position).  The hidden states
+    (or, through the last layer, the logits) the client reads back are bit for bit what mesh_stage_decode of the same
+    range returns, and within the stage tolerance of the CPU oracle."""
+    import models
+    import rpc_graph_util as GU
+    from oracle.stage import StageOracle
+    from util import mesh
+    m = mesh()
+    cfg = models.CONFIGS[name]
+    path = str(tmp_path / (name + ".gguf"))
+    extra = ("output",) if with_output else ()
+    tensors = models.write_model(path, cfg, range(lb, le), seed=11, **({"with_output": True} if with_output else {}))
+    E, n_ctx = cfg["n_embd"], 64
+    weights = {n: (t, list(d)) for n, (t, d, _) in tensors.items() if n.startswith("blk.") or (with_output and n in ("output_norm.weight", "output.weight", "token_embd.weight"))}
+    if with_output and "output.weight" in weights:
+        weights.pop("token_embd.weight", None)
+    st = m.Stage(path, lb, le, n_ctx=n_ctx, n_seq_max=1, n_batch_max=512)
+    ses = st.session()
+    orc = StageOracle(cfg, tensors, lb, le, n_ctx)
+    rng = np.random.Generator(np.random.PCG64(5))
+    with ServerProcess(server_bin, extra=["-d", "ROCm0", "--gguf", path]) as s:
+        c = Client(s.port)
+        steps = [(5, 0), (1, 5), (1, 6)]
+        graphs = {}
+        for T, p0 in steps:
+            if T not in graphs:
+                h, _ = c.alloc_buffer(64 << 20)
+                gb = GU.GraphBuilder(h, c.buffer_get_base(h))
+                graphs[T] = (gb,) + GU.layer_range_graph(gb, weights, list(range(lb, le)), T, cfg["n_head"], cfg["n_head_kv"], cfg["head_dim"], n_ctx,
+                                                         with_output=with_output)
+                fresh = True
+            else:
+                fresh = False
+            gb, inp, pos, out = graphs[T]
+            x = rng.standard_normal((T, E)).astype(np.float32)
+            positions = np.arange(p0, p0 + T, dtype=np.int32)
+            c.set_tensor(gb.descriptor(inp), 0, x.tobytes())
+            c.set_tensor(gb.descriptor(pos), 0, positions.tobytes())
+            if fresh:
+                c.send(R_GRAPH_COMPUTE, gb.payload())
+            else:
+                c.send(R_GRAPH_RECOMPUTE, (0).to_bytes(4, "little"))
+            rows = struct_ne0(gb.descriptor(out))
+            got = np.frombuffer(c.get_tensor(gb.descriptor(out), 0, T * rows * 4), np.float32).reshape(T, rows)
+            want = ses.decode(x, positions, out_fmt=m.LOGITS if with_output else m.F32).view(np.float32).reshape(T, rows)
+            assert np.array_equal(got, want), (T, p0)
+            ref = orc.logits(orc.forward(x, positions)) if with_output else orc.forward(x, positions)
+            rel = float(np.linalg.norm(got.astype(np.float64) - ref) / np.linalg.norm(ref))
+            assert rel <= 1e-2, (T, p0, rel)
+        c.close()
+        log = s.stop()
+        assert "opened as a stage" in log
+    ses.close(); st.close()
+
+
+R_GRAPH_COMPUTE, R_GRAPH_RECOMPUTE = 10, 16
+
+
+def struct_ne0(descriptor):
+    import struct
+    from rpc_client import TENSOR_FMT
+    return struct.unpack(TENSOR_FMT, descriptor)[3]

@@ -230,13 +230,175 @@ def test_register_peer_frame_of_the_tunnel(server_bin):
         c.close()
 
 
-def test_graph_compute_is_refused_not_ignored(server_bin):
-    with ServerProcess(server_bin) as s:
+# ---- GRAPH_COMPUTE / GRAPH_RECOMPUTE (patches/0002:443-459, patches/0001:163-174)
+def _fake_weights(layers, E=64, H=2, HK=1, hd=32, FF=96, extra=None, drop=()):
+    """GGUF names and shapes of decoder layers (shapes only: the host-memory build's stand-in runner never reads weights)."""
+    w = {}
+    for il in layers:
+        p = "blk.%d." % il
+        w.update({p + "attn_norm.weight": (F32, [E]), p + "attn_q.weight": (Q4_K, [E * 4, H * hd]), p + "attn_k.weight": (Q4_K, [E * 4, HK * hd]),
+                  p + "attn_v.weight": (Q6_K, [E * 4, HK * hd]), p + "attn_output.weight": (Q4_K, [H * hd * 4, E]), p + "ffn_norm.weight": (F32, [E]),
+                  p + "ffn_gate.weight": (Q4_K, [E * 4, FF]), p + "ffn_up.weight": (Q4_K, [E * 4, FF]), p + "ffn_down.weight": (Q6_K, [FF * 8 // 3, E])})
+    # (row lengths of the quantised matrices are multiples of 256 so that their descriptors are well-formed; the attention
+    # norm fixes the hidden size the recogniser reads)
+    for k in drop:
+        del w[k]
+    w.update(extra or {})
+    return w
+
+
+def _graph_case(c, layers, T=3, device=0, **kw):
+    import rpc_graph_util as GU
+    h, _ = c.alloc_buffer(8 << 20, device)
+    base = c.buffer_get_base(h)
+    gb = GU.GraphBuilder(h, base, device)
+    weights = kw.pop("weights", None) or _fake_weights(layers)
+    inp, pos, out = GU.layer_range_graph(gb, weights, layers, T, 2, 1, 32, 128, **kw)
+    return gb, inp, pos, out
+
+
+def _expected(x, pos, b, e, rows):
+    T, E = x.shape
+    cols = np.arange(rows) % E
+    return x[:, cols] + np.asarray(pos, np.float32)[:, None] + 100.0 * b + 10000.0 * e
+
+
+def _any_gguf(tmp_path):
+    path = str(tmp_path / "m.gguf")
+    G.write_gguf(path, [("general.architecture", G.T_STR, "llama")], [("a", F32, (8,), np.arange(8, dtype=np.float32))])
+    return path
+
+
+def test_graph_compute_runs_a_layer_range_and_recompute_replays_it(server_bin, tmp_path):
+    """The decoder sub-graph of layers 1-2 is parsed, recognised by its weight names and handed to the runner (here the
+    host-memory stand-in, whose result shows which range ran on which data); GRAPH_RECOMPUTE replays the stored graph on
+    the inputs as they are then; a second device keeps its own stored graph."""
+    with ServerProcess(server_bin, extra=["--gguf", _any_gguf(tmp_path)]) as s:
         c = Client(s.port)
-        c.send(R.GRAPH_COMPUTE, struct.pack("<II", 0, 0))
-        assert c.closed_by_server()
+        gb, inp, pos, out = _graph_case(c, [1, 2], T=3)
+        rng = np.random.Generator(np.random.PCG64(1))
+        x = rng.standard_normal((3, 64)).astype(np.float32)
+        c.set_tensor(gb.descriptor(inp), 0, x.tobytes())
+        c.set_tensor(gb.descriptor(pos), 0, np.array([7, 8, 9], np.int32).tobytes())
+        c.send(R.GRAPH_COMPUTE, gb.payload())                    # no reply
+        got = np.frombuffer(c.get_tensor(gb.descriptor(out), 0, 3 * 64 * 4), np.float32).reshape(3, 64)
+        assert np.array_equal(got, _expected(x, [7, 8, 9], 1, 3, 64).astype(np.float32))
+        # new data, same graph
+        x2 = rng.standard_normal((3, 64)).astype(np.float32)
+        c.set_tensor(gb.descriptor(inp), 0, x2.tobytes())
+        c.set_tensor(gb.descriptor(pos), 0, np.array([10, 11, 12], np.int32).tobytes())
+        c.send(R.GRAPH_RECOMPUTE, struct.pack("<I", 0))
+        got = np.frombuffer(c.get_tensor(gb.descriptor(out), 0, 3 * 64 * 4), np.float32).reshape(3, 64)
+        assert np.array_equal(got, _expected(x2, [10, 11, 12], 1, 3, 64).astype(np.float32))
+        # the other device: its own graph (one layer, one token, logits out), and the first device's stored graph is untouched
+        gb1, inp1, pos1, out1 = _graph_case(c, [3], T=1, device=1, with_output=True,
+                                            weights=_fake_weights([3], extra={"output_norm.weight": (F32, [64]), "output.weight": (Q6_K, [256, 80])}))
+        x3 = rng.standard_normal((1, 64)).astype(np.float32)
+        c.set_tensor(gb1.descriptor(inp1), 0, x3.tobytes())
+        c.set_tensor(gb1.descriptor(pos1), 0, np.array([5], np.int32).tobytes())
+        c.send(R.GRAPH_COMPUTE, gb1.payload())
+        got = np.frombuffer(c.get_tensor(gb1.descriptor(out1), 0, 80 * 4), np.float32).reshape(1, 80)
+        assert np.array_equal(got, _expected(x3, [5], 3, 4, 80).astype(np.float32))
+        c.send(R.GRAPH_RECOMPUTE, struct.pack("<I", 0))
+        got = np.frombuffer(c.get_tensor(gb.descriptor(out), 0, 3 * 64 * 4), np.float32).reshape(3, 64)
+        assert np.array_equal(got, _expected(x2, [10, 11, 12], 1, 3, 64).astype(np.float32))
         c.close()
-        assert "graph execution" in s.stop()
+
+
+def test_graph_of_a_mixture_of_experts_range_with_biases_and_head_norms(server_bin, tmp_path):
+    w = _fake_weights([0, 1], drop=["blk.%d.ffn_%s.weight" % (il, k) for il in (0, 1) for k in ("gate", "up", "down")])
+    for il in (0, 1):
+        p = "blk.%d." % il
+        w.update({p + "ffn_gate_inp.weight": (F32, [64, 4]), p + "ffn_gate_exps.weight": (Q4_K, [256, 32, 4]), p + "ffn_up_exps.weight": (Q4_K, [256, 32, 4]),
+                  p + "ffn_down_exps.weight": (Q6_K, [256, 64, 4]), p + "attn_q.bias": (F32, [64]), p + "attn_k.bias": (F32, [32]), p + "attn_v.bias": (F32, [32]),
+                  p + "attn_q_norm.weight": (F32, [32]), p + "attn_k_norm.weight": (F32, [32])})
+    with ServerProcess(server_bin, extra=["--gguf", _any_gguf(tmp_path)]) as s:
+        c = Client(s.port)
+        gb, inp, pos, out = _graph_case(c, [0, 1], T=2, weights=w)
+        x = np.arange(128, dtype=np.float32).reshape(2, 64)
+        c.set_tensor(gb.descriptor(inp), 0, x.tobytes())
+        c.set_tensor(gb.descriptor(pos), 0, np.array([0, 1], np.int32).tobytes())
+        c.send(R.GRAPH_COMPUTE, gb.payload())
+        got = np.frombuffer(c.get_tensor(gb.descriptor(out), 0, 2 * 64 * 4), np.float32).reshape(2, 64)
+        assert np.array_equal(got, _expected(x, [0, 1], 0, 2, 64).astype(np.float32))
+        c.close()
+
+
+@pytest.mark.parametrize("case", ["empty", "truncated", "trailing", "dangling-source", "duplicate-id", "not-a-layer-graph", "layers-1-and-3", "fused-qkv",
+                                  "layer-without-ffn", "result-outside-buffer", "row-selection", "two-inputs", "recompute-without-a-graph", "no-model-file"])
+def test_graphs_this_build_cannot_run_end_the_connection_with_a_reason(server_bin, tmp_path, case):
+    """A malformed payload, a graph that is not the decoder sub-graph of one contiguous layer range, or one that needs
+    something the stage has no kernel for: the request fails, which ends the connection (what a failing request does in
+    the reference), and the log says why."""
+    import rpc_graph_util as GU
+    extra = [] if case == "no-model-file" else ["--gguf", _any_gguf(tmp_path)]
+    with ServerProcess(server_bin, extra=extra) as s:
+        c = Client(s.port)
+        reason = None
+        if case == "empty":
+            payload, reason = struct.pack("<II", 0, 0), "malformed"
+        elif case == "recompute-without-a-graph":
+            c.send(R.GRAPH_RECOMPUTE, struct.pack("<I", 0))
+            payload, reason = None, "no stored graph"
+        elif case == "not-a-layer-graph":
+            h, _ = c.alloc_buffer(1 << 16)
+            gb = GU.GraphBuilder(h, c.buffer_get_base(h))
+            a, b = gb.leaf("a", F32, [8]), gb.leaf("b", F32, [8])
+            gb.node("sum", "ADD", [8], [a, b])
+            payload, reason = gb.payload(), "not a decoder layer sub-graph"
+        else:
+            kw, layers = {}, [1, 2]
+            if case == "layers-1-and-3":
+                layers, reason = [1, 3], "contiguous"
+            if case == "fused-qkv":
+                kw["weights"], reason = _fake_weights(layers, extra={"blk.1.attn_qkv.weight": (Q4_K, [256, 128])}), "no kernel for this weight"
+            if case == "layer-without-ffn":
+                kw["weights"], reason = _fake_weights(layers, drop=["blk.2.ffn_up.weight"]), "feed-forward"
+            gb, inp, pos, out = _graph_case(c, layers, T=3, **kw) if case not in ("fused-qkv", "layer-without-ffn") else (None, None, None, None)
+            if gb is None:
+                # these two cannot be built by the layer builder (it would dereference the odd weight set): assemble by hand
+                h, _ = c.alloc_buffer(8 << 20)
+                gb = GU.GraphBuilder(h, c.buffer_get_base(h))
+                w = {n: gb.leaf(n, t, d) for n, (t, d) in kw["weights"].items()}
+                x = gb.leaf("RPC0#l_out-0#0", F32, [64, 3])
+                gb.leaf("RPC0#inp_pos#0", GU.I32, [3])
+                cur = x
+                for n, wid in w.items():
+                    cur = gb.node("use-" + n, "MUL_MAT", [64, 3], [wid, cur])
+            payload = gb.payload()
+            if case == "truncated":
+                payload, reason = payload[:-100], "malformed"
+            elif case == "trailing":
+                payload, reason = payload + b"\0" * 8, "malformed"
+            elif case == "dangling-source":
+                payload, reason = gb.payload(drop=[inp]), "malformed"
+            elif case == "duplicate-id":
+                first = next(iter(gb.tensors.values()))
+                payload = gb.payload()
+                payload = payload[:-len(first)] + first                    # the last descriptor replaced by a copy of the first
+                reason = "malformed"
+            elif case == "result-outside-buffer":
+                t = list(struct.unpack(R.TENSOR_FMT, gb.tensors[out]))
+                t[-3] += 64 << 20
+                gb.tensors[out] = struct.pack(R.TENSOR_FMT, *t)
+                payload, reason = gb.payload(), "does not lie inside its buffer"
+            elif case == "row-selection":
+                t = list(struct.unpack(R.TENSOR_FMT, gb.tensors[out]))
+                t[4] = 1                                                    # ne[1]: one output row for three tokens
+                gb.tensors[out] = struct.pack(R.TENSOR_FMT, *t)
+                payload, reason = gb.payload(), "row selection"
+            elif case == "two-inputs":
+                extra_in = gb.leaf("RPC0#other#0", F32, [64, 3])
+                gb.node("mix", "ADD", [64, 3], [extra_in, out])
+                payload, reason = gb.payload(), "candidates for the hidden-state input"
+            elif case == "no-model-file":
+                reason = "--gguf"
+        if payload is not None:
+            c.send(R.GRAPH_COMPUTE, payload)
+        assert c.closed_by_server(), case
+        c.close()
+        log = s.stop()
+        assert reason in log, (case, log[-600:])
 
 
 # ---- SET_TENSOR_GGUF (patches/0001:179-266)
