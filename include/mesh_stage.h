@@ -239,6 +239,14 @@ int mesh_session_set_expert_mask(mesh_session *session, const uint8_t *allowed, 
  * ids[n_tokens][n_expert_used].  For tests and for counting distinct experts touched. */
 int mesh_session_moe_last_ids(mesh_session *session, int32_t *ids, int32_t n_tokens);
 
+/* Values the session's f16 producers clamped to the f16 range (+-65504) since the session was created.  Calls of 5 or more
+ * tokens hand activations to the matrix cores as f16 (normalised hidden state, attention output, SwiGLU product); a value
+ * beyond the range is stored as the largest finite f16 instead of infinity and counted here, so a caller can tell a
+ * saturated step from an exact one.  Single-token calls use 16-bit fixed point with a scale per 32 values and never
+ * count.  Waits for the session's stream.  No counterpart in the reference (ggml's f16 conversions saturate silently to
+ * infinity). */
+int mesh_session_f16_saturations(mesh_session *session, uint64_t *count);
+
 /* KV cache import/export for one sequence and one (absolute) layer: n_pos positions starting at pos0, host
  * buffers of f16 bits laid out [n_pos][n_head_kv][head_dim].  (The reference has no KV hand-over; a restarted
  * stage refills from the prompt -- mesh-llm/src/inference/election.rs:1894-1910.) */

@@ -107,6 +107,7 @@ SIGNATURES.update({
     "mesh_session_profile_read": (_i32, [_vp, ctypes.POINTER(Profile)]),
     "mesh_session_set_expert_mask": (_i32, [_vp, _vp, _i32]),
     "mesh_session_moe_last_ids": (_i32, [_vp, _vp, _i32]),
+    "mesh_session_f16_saturations": (_i32, [_vp, ctypes.POINTER(ctypes.c_uint64)]),
     "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_op_q16_bytes": (_sz, [_i64, _i64]),
@@ -399,6 +400,12 @@ class Session:
         out = np.empty((n_tokens, self.stage.info.n_expert_used), dtype=np.int32)
         check(lib().mesh_session_moe_last_ids(self._h, _np_ptr(out), n_tokens))
         return out
+
+    def f16_saturations(self):
+        """Values clamped to the f16 range by the batched paths since the session was created."""
+        n = ctypes.c_uint64(0)
+        check(lib().mesh_session_f16_saturations(self._h, ctypes.byref(n)))
+        return int(n.value)
 
     def kv_write(self, layer, seq_id, pos0, k, v):
         """k, v: uint16 arrays [n_pos, n_head_kv, head_dim] of f16 bits."""

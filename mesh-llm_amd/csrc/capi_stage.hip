@@ -209,6 +209,19 @@ int mesh_session_moe_last_ids(mesh_session *session, int32_t *ids, int32_t n_tok
     return MESH_OK;
 }
 
+int mesh_session_f16_saturations(mesh_session *session, uint64_t *count) {
+    if (!session || !count) return fail(MESH_ERR_INVALID, "mesh_session_f16_saturations: null argument");
+    unsigned v = 0;
+    MESH_HIP_TRY(hipSetDevice(session->stage->device));
+    MESH_HIP_TRY(hipStreamSynchronize(session->stream));
+    MESH_HIP_TRY(hipMemcpy(&v, session->f16_sat, sizeof(v), hipMemcpyDeviceToHost));
+    // the device counter is 32 bits wide and wraps; the host keeps the running total
+    session->f16_sat_total += (uint32_t)(v - session->f16_sat_seen);
+    session->f16_sat_seen = v;
+    *count = session->f16_sat_total;
+    return MESH_OK;
+}
+
 static int kv_xfer(mesh_session *s, int layer, int seq_id, int pos0, int n_pos, uint16_t *k, uint16_t *v, bool write) {
     if (!s || !k || !v) return fail(MESH_ERR_INVALID, "mesh_session_kv: null argument");
     const mesh_stage *st = s->stage;

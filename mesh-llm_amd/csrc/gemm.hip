@@ -445,6 +445,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kq_kernel(GemmArgs a) {
                         const float g = acc[i][j][4 * e4 + c], u = xch[((pair + i * 2 + j) * 16 + 4 * e4 + c) * 64 + lane];
                         o[c] = t < t_end ? g / (1.0f + expf(-g)) * u : 0.f;       // padding columns of the last token block hold zeros
                     }
+                    note_f16_clamp(a.sat, o[0], o[1], o[2], o[3]);
                     *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
                         make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
                 }
@@ -636,6 +637,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_big_kernel(GemmArgs a) {
                         const float g = acc[i][j][4 * e4 + c], u = acc[i + 2][j][4 * e4 + c];
                         o[c] = t < a.T ? g / (1.0f + expf(-g)) * u : 0.f;
                     }
+                    note_f16_clamp(a.sat, o[0], o[1], o[2], o[3]);
                     *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
                         make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
                 }
@@ -731,6 +733,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_epilogue_kernel(GemmArgs a, i
                 o[0] = g.x / (1.0f + expf(-g.x)) * u.x; o[1] = g.y / (1.0f + expf(-g.y)) * u.y;
                 o[2] = g.z / (1.0f + expf(-g.z)) * u.z; o[3] = g.w / (1.0f + expf(-g.w)) * u.w;
             }
+            note_f16_clamp(a.sat, o[0], o[1], o[2], o[3]);
             *reinterpret_cast<uint2 *>(a.y16_k8 + (size_t)(t >> 4) * 16 * a.M + ((size_t)(m >> 3) * 16 + (t & 15)) * 8 + (m & 7)) =
                 make_uint2(pack_h2(o[0], o[1]), pack_h2(o[2], o[3]));
             continue;
@@ -975,7 +978,7 @@ int gemm_pack_pair(int type, const void *gate_tiled, const void *up_tiled, void 
 // ---- small elementwise companions of the prefill path ---------------------------------------------------------
 // y16[t] = f16( x[t] * rsqrt(mean(x[t]^2) + eps) * w ), one workgroup per token
 __global__ __launch_bounds__(256) void rmsnorm_f16_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps,
-                                                          int n, _Float16 *__restrict__ y, int ldy) {
+                                                          int n, _Float16 *__restrict__ y, int ldy, unsigned *sat) {
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     const float *xt = x + (size_t)t * n;
@@ -992,34 +995,36 @@ __global__ __launch_bounds__(256) void rmsnorm_f16_kernel(const float *__restric
     for (int i = tid * 4; i < n; i += 1024) {
         const float4 v = *reinterpret_cast<const float4 *>(xt + i);
         const float4 g = *reinterpret_cast<const float4 *>(w + i);
+        note_f16_clamp(sat, v.x * scale * g.x, v.y * scale * g.y, v.z * scale * g.z, v.w * scale * g.w);
         *reinterpret_cast<uint2 *>(y + (size_t)t * ldy + i) =
             make_uint2(pack_h2(v.x * scale * g.x, v.y * scale * g.y), pack_h2(v.z * scale * g.z, v.w * scale * g.w));
     }
 }
 
-int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream) {
+int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream, unsigned *sat) {
     if (T <= 0) return MESH_OK;
     if (n % 4 || ldy % 4) return fail(MESH_ERR_INVALID, "rmsnorm: row length %d not a multiple of 4", n);
-    MESH_LAUNCH(rmsnorm_f16_kernel, dim3((unsigned)T), dim3(256), 0, stream, x, w, eps, n, y, ldy);
+    MESH_LAUNCH(rmsnorm_f16_kernel, dim3((unsigned)T), dim3(256), 0, stream, x, w, eps, n, y, ldy, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
 // out16 = f16( silu(gate) * up )
 __global__ __launch_bounds__(256) void swiglu_f16_kernel(const float *__restrict__ g, const float *__restrict__ u,
-                                                         _Float16 *__restrict__ o, int64_t n4) {
+                                                         _Float16 *__restrict__ o, int64_t n4, unsigned *sat) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
     const float4 a = reinterpret_cast<const float4 *>(g)[i], b = reinterpret_cast<const float4 *>(u)[i];
     const float r0 = a.x / (1.0f + expf(-a.x)) * b.x, r1 = a.y / (1.0f + expf(-a.y)) * b.y;
     const float r2 = a.z / (1.0f + expf(-a.z)) * b.z, r3 = a.w / (1.0f + expf(-a.w)) * b.w;
+    note_f16_clamp(sat, r0, r1, r2, r3);
     reinterpret_cast<uint2 *>(o)[i] = make_uint2(pack_h2(r0, r1), pack_h2(r2, r3));
 }
 
-int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream) {
+int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream, unsigned *sat) {
     if (n <= 0) return MESH_OK;
     if (n % 4) return fail(MESH_ERR_INVALID, "swiglu: count not a multiple of 4");
-    MESH_LAUNCH(swiglu_f16_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream, gate, up, out, n / 4);
+    MESH_LAUNCH(swiglu_f16_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, stream, gate, up, out, n / 4, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }

@@ -31,6 +31,7 @@ struct GemmArgs {
     // SwiGLU pair: Wp is a gate/up pair packed by gemm_pack_pair (every row block 64 gate rows, then the same 64 up
     // rows), M their common row count; the launch writes f16(silu(gate) * up) in the k8-major layout to y16_k8 (Y unused).
     _Float16 *y16_k8 = nullptr;
+    unsigned *sat = nullptr;         // optional device counter of SwiGLU outputs clamped to the f16 range (mesh_common.hpp: note_f16_clamp)
     // Optional scratch for launches too narrow to fill the chip (few row blocks x token blocks): K is then split over
     // blockIdx.z, every slice writes its f32 partial tile to `part` ([slice][token][row of the launch]) and a second
     // kernel adds the slices in slice order and applies the epilogue.  Null: never split.  ksplit / k_per_split are
@@ -109,14 +110,34 @@ bool moe_combine_quant16_supported(int n);
 int moe_combine_quant16(float *x, const float *y, const float *w, int T, int n, int top_k, const float *norm_w, float eps, uint8_t *yq, hipStream_t stream);
 // The "k8-major" f16 layout the large-tile GEMM reads: blocks of 16 tokens, element (t, k) of block t / 16 at
 // ((k / 8) * 16 + t % 16) * 8 + k % 8 within the block of 16 * K halfs; columns beyond T hold zeros.
-// y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
-int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream);
-int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream);
-// the same as rmsnorm_f16_k8 for n_slots (a multiple of 16) gathered rows: slot i holds row row_of_slot[i] / row_div of x, zeros when negative
-int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream);
-int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream);
+// The same launches on the f16 matrix cores (gemm_skinny_f16.hip): activations in the k8-major f16 layout below, weights
+// dequantised to f16 with one rounding each.  Faster than the integer kernel, less precise (f16 activations).
+struct SkinnyF16Args {
+    GemvMat mat[3];
+    int n_mat = 1;                   // for EPI_SWIGLU exactly 2 (gate, up), written through mat[0].y and/or y16
+    const _Float16 *x = nullptr;     // k8-major, ceil(T / 16) blocks of 16 * K halfs, 16-byte aligned
+    int K = 0, T = 0;
+    int epi = EPI_STORE;
+    const float *residual = nullptr; // EPI_RESIDUAL: [T][ldres]; may alias y
+    int ldres = 0;
+    _Float16 *y16 = nullptr;         // optional f16 copy of matrix 0's output in the k8-major layout (feeds the next GEMM)
+    unsigned *sat = nullptr;         // optional device counter of y16 values clamped to the f16 range
+    // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
+    GemvRope rope;
+    int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+};
+int gemm_skinny_f16(const SkinnyF16Args &a, hipStream_t stream);
 
-int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream);
-int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream);
+// y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
+// (sat: optional device counter of values clamped to the f16 range, in all of these)
+int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat = nullptr);
+int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat = nullptr);
+// the same as rmsnorm_f16_k8 for n_slots (a multiple of 16) gathered rows: slot i holds row row_of_slot[i] / row_div of x, zeros when negative
+int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream,
+                          unsigned *sat = nullptr);
+int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat = nullptr);
+
+int rmsnorm_f16(const float *x, const float *w, float eps, int T, int n, _Float16 *y, int ldy, hipStream_t stream, unsigned *sat = nullptr);
+int swiglu_f16(const float *gate, const float *up, _Float16 *out, int64_t n, hipStream_t stream, unsigned *sat = nullptr);
 
 }  // namespace mesh

@@ -710,7 +710,9 @@ int moe_combine_quant16(float *x, const float *y, const float *w, int T, int n, 
 // Tokens are grouped in blocks of 16 columns, and within a block the 8 consecutive k of every column sit together:
 // element (t, k) of block b = t / 16 is at ((b * K/8 + k/8) * 16 + t % 16) * 8 + k % 8.
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {       // saturating, like gemm.hip's pack_h2
+// saturating, like gemm.hip's pack_h2; a clamped pair is noted in the caller's counter (mesh_common.hpp), if it has one
+__device__ __forceinline__ uint32_t sk_pack_h2(unsigned *sat, float a, float b) {
+    note_f16_clamp(sat, a, b);
     const h2_t h = {(_Float16)__builtin_amdgcn_fmed3f(a, -65504.f, 65504.f), (_Float16)__builtin_amdgcn_fmed3f(b, -65504.f, 65504.f)};
     return __builtin_bit_cast(uint32_t, h);
 }
@@ -718,7 +720,7 @@ __device__ __forceinline__ uint32_t sk_pack_h2(float a, float b) {       // satu
 // y = f16(x[t] * rsqrt(mean(x[t]^2) + eps) * w), or with w == null just f16(x[t]); one workgroup per token slot of the
 // padded batch (slots >= T write zeros).
 __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int T, int n,
-                                                    _Float16 *__restrict__ y) {
+                                                    _Float16 *__restrict__ y, unsigned *sat) {
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     _Float16 *yb = y + (size_t)(t / 16) * 16 * n + (size_t)(t % 16) * 8;        // element (t, k) at yb + (k / 8) * 128 + k % 8
@@ -760,8 +762,8 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
             if (i >= n) continue;
             const float4 v0 = v[j][0], v1 = v[j][1], g0 = g[j][0], g1 = g[j][1];
             *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) =
-                make_uint4(sk_pack_h2(v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(v0.z * sc * g0.z, v0.w * sc * g0.w),
-                           sk_pack_h2(v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(v1.z * sc * g1.z, v1.w * sc * g1.w));
+                make_uint4(sk_pack_h2(sat, v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(sat, v0.z * sc * g0.z, v0.w * sc * g0.w),
+                           sk_pack_h2(sat, v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(sat, v1.z * sc * g1.z, v1.w * sc * g1.w));
         }
         return;
     }
@@ -783,15 +785,15 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
         float4 g0 = make_float4(1.f, 1.f, 1.f, 1.f), g1 = g0;
         if (w) { g0 = *reinterpret_cast<const float4 *>(w + i); g1 = *reinterpret_cast<const float4 *>(w + i + 4); }
         *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) =
-            make_uint4(sk_pack_h2(v0.x * scale * g0.x, v0.y * scale * g0.y), sk_pack_h2(v0.z * scale * g0.z, v0.w * scale * g0.w),
-                       sk_pack_h2(v1.x * scale * g1.x, v1.y * scale * g1.y), sk_pack_h2(v1.z * scale * g1.z, v1.w * scale * g1.w));
+            make_uint4(sk_pack_h2(sat, v0.x * scale * g0.x, v0.y * scale * g0.y), sk_pack_h2(sat, v0.z * scale * g0.z, v0.w * scale * g0.w),
+                       sk_pack_h2(sat, v1.x * scale * g1.x, v1.y * scale * g1.y), sk_pack_h2(sat, v1.z * scale * g1.z, v1.w * scale * g1.w));
     }
 }
 
-int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream) {
+int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
-    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y);
+    MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
@@ -801,7 +803,7 @@ int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Flo
 // run of the block.  The sum of squares is taken in another order than in to_k8_kernel (one wave per row instead of four),
 // so the scale can differ from that kernel's in its last bit.
 __global__ __launch_bounds__(256) void gather_k8_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int n,
-                                                        _Float16 *__restrict__ y, const int32_t *__restrict__ row_of_slot, int row_div) {
+                                                        _Float16 *__restrict__ y, const int32_t *__restrict__ row_of_slot, int row_div, unsigned *sat) {
     __shared__ float s_scale[16];
     __shared__ int s_row[16];
     const int blk = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -835,24 +837,25 @@ __global__ __launch_bounds__(256) void gather_k8_kernel(const float *__restrict_
             const float *xt = x + (size_t)row * n + k8 * 8;
             const float4 v0 = *reinterpret_cast<const float4 *>(xt), v1 = *reinterpret_cast<const float4 *>(xt + 4);
             const float4 g0 = *reinterpret_cast<const float4 *>(w + k8 * 8), g1 = *reinterpret_cast<const float4 *>(w + k8 * 8 + 4);
-            o = make_uint4(sk_pack_h2(v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(v0.z * sc * g0.z, v0.w * sc * g0.w),
-                           sk_pack_h2(v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(v1.z * sc * g1.z, v1.w * sc * g1.w));
+            o = make_uint4(sk_pack_h2(sat, v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(sat, v0.z * sc * g0.z, v0.w * sc * g0.w),
+                           sk_pack_h2(sat, v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(sat, v1.z * sc * g1.z, v1.w * sc * g1.w));
         }
         *reinterpret_cast<uint4 *>(yb + (size_t)k8 * 128) = o;
     }
 }
 
-int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream) {
+int rmsnorm_f16_k8_gather(const float *x, const float *w, float eps, const int32_t *row_of_slot, int row_div, int n_slots, int n, _Float16 *y, hipStream_t stream,
+                          unsigned *sat) {
     if (n_slots <= 0) return MESH_OK;
     if (n % 8 || n_slots % 16 || !row_of_slot || row_div < 1 || !w) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8_gather: bad arguments (row length %d, %d slots)", n, n_slots);
-    MESH_LAUNCH(gather_k8_kernel, dim3((unsigned)(n_slots / 16)), dim3(256), 0, stream, x, w, eps, n, y, row_of_slot, row_div);
+    MESH_LAUNCH(gather_k8_kernel, dim3((unsigned)(n_slots / 16)), dim3(256), 0, stream, x, w, eps, n, y, row_of_slot, row_div, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
 // out (k8-major) = f16( silu(gate) * up ): one workgroup per token, padding tokens of the last block write zeros
 __global__ __launch_bounds__(256) void swiglu_k8_kernel(const float *__restrict__ g, const float *__restrict__ u, int T, int n,
-                                                        _Float16 *__restrict__ y) {
+                                                        _Float16 *__restrict__ y, unsigned *sat) {
     const int t = blockIdx.x, tid = threadIdx.x;
     _Float16 *yb = y + (size_t)(t >> 4) * 16 * n + (size_t)(t & 15) * 8;
     if (t >= T) {
@@ -865,24 +868,24 @@ __global__ __launch_bounds__(256) void swiglu_k8_kernel(const float *__restrict_
         const float4 b0 = *reinterpret_cast<const float4 *>(ut + i), b1 = *reinterpret_cast<const float4 *>(ut + i + 4);
         auto f = [](float a, float b) { return a / (1.0f + expf(-a)) * b; };
         uint4 o;
-        o.x = sk_pack_h2(f(a0.x, b0.x), f(a0.y, b0.y));
-        o.y = sk_pack_h2(f(a0.z, b0.z), f(a0.w, b0.w));
-        o.z = sk_pack_h2(f(a1.x, b1.x), f(a1.y, b1.y));
-        o.w = sk_pack_h2(f(a1.z, b1.z), f(a1.w, b1.w));
+        o.x = sk_pack_h2(sat, f(a0.x, b0.x), f(a0.y, b0.y));
+        o.y = sk_pack_h2(sat, f(a0.z, b0.z), f(a0.w, b0.w));
+        o.z = sk_pack_h2(sat, f(a1.x, b1.x), f(a1.y, b1.y));
+        o.w = sk_pack_h2(sat, f(a1.z, b1.z), f(a1.w, b1.w));
         *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) = o;
     }
 }
 
-int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream) {
+int swiglu_f16_k8(const float *gate, const float *up, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "swiglu_f16_k8: row length %d not a multiple of 8", n);
-    MESH_LAUNCH(swiglu_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, gate, up, T, n, y);
+    MESH_LAUNCH(swiglu_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, gate, up, T, n, y, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
-int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream) {
-    return rmsnorm_f16_k8(x, nullptr, 0.f, T, n, y, stream);
+int pack_f16_k8(const float *x, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat) {
+    return rmsnorm_f16_k8(x, nullptr, 0.f, T, n, y, stream, sat);
 }
 
 int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {

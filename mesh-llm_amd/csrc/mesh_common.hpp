@@ -113,6 +113,13 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
     return (w & 0x7FFFFFFFu) > 0x7F800000u ? (uint16_t)(((w >> 16) & 0x8000u) | 0x7E00u) : h;
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
+// The f16 producers of the batched paths clamp what f16 cannot hold to +-65504.  A caller can ask how often that happened
+// (mesh_session_f16_saturations): every producer that can meet such a value is handed the session's counter and notes each
+// group of values it clamps.  `sat` may be null (no counting).
+__device__ __forceinline__ void note_f16_clamp(unsigned *sat, float a, float b, float c = 0.f, float d = 0.f) {
+    if (sat && fmaxf(fmaxf(fabsf(a), fabsf(b)), fmaxf(fabsf(c), fabsf(d))) > 65504.f) atomicAdd(sat, 1u);
+}
 #endif
 
 }  // namespace mesh

@@ -386,6 +386,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
     if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
     if (const char *e = getenv("MESH_XQ_HANDOVER")) s->xq_handover = e[0] != '0';
+    if (const char *e = getenv("MESH_SKINNY_F16")) s->skinny_f16 = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
     if (const char *e = getenv("MESH_MOE_FUSE_QUANT")) s->moe_fuse_quant = e[0] != '0';
     if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
@@ -416,6 +417,9 @@ int session_new(mesh_stage *st, mesh_session **out) {
         (rc = fbuf(&s->v, B * KD)) || (rc = fbuf(&s->attn, B * QD)) || (rc = fbuf(&s->ffn, B * ff)) ||
         (rc = fbuf(&s->attn_part, part_rows * QD)) || (rc = fbuf(&s->attn_ml, part_rows * hp.n_head * 2)))
         return rc;
+    if ((rc = sess_alloc(s.get(), &p, 256)) != MESH_OK) return rc;
+    s->f16_sat = static_cast<unsigned *>(p);
+    MESH_HIP_TRY(hipMemsetAsync(p, 0, 256, s->stream));
     if (hp.n_ff && hp.n_ff % QK_K == 0) {
         if ((rc = sess_alloc(s.get(), &p, xq_bytes((int)hp.n_ff))) != MESH_OK) return rc;
         s->ffn_xq = static_cast<uint8_t *>(p);
@@ -629,16 +633,43 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     int rc;
     bool rope_fused = false, attn_is_k8 = false;
     const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
-    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; return g; };
+    // the batched-decode GEMM on the f16 matrix cores (k8-major f16 activations) instead of the integer ones (q16 activations);
+    // a mixture-of-experts stage keeps the integer kernel, whose activation layout its expert launches share
+    const bool sk16 = skinny && s->skinny_f16 && L.w_gate.present() && f16ffn;
+    const bool sk8 = skinny && !sk16;
+    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; g.sat = s->f16_sat; return g; };
+    auto rope_of = [&]() {
+        GemvRope r;
+        r.pos = s->d_pos; r.seq = s->d_seq; r.inv_freq = st->rope_inv_freq;
+        r.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
+        r.vcache = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
+        r.head_dim = (int)hp.head_dim; r.n_rot = (int)hp.n_rot; r.n_kv = (int)hp.n_head_kv; r.n_ctx = st->n_ctx;
+        return r;
+    };
     {
         ProfScope ps(s, MESH_PROF_PREP);
-        if (skinny && s->xq_layer == (int)il) rc = MESH_OK;     // the previous layer's combine step has left them in s->xq
-        else if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
-        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream);
-        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+        if (sk8 && s->xq_layer == (int)il) rc = MESH_OK;     // the previous layer's combine step has left them in s->xq
+        else if (sk8) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream, s->f16_sat);
+        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream, s->f16_sat);
     }
     if (rc != MESH_OK) return rc;
-    if (skinny) {
+    if (sk16) {
+        SkinnyF16Args qa;
+        qa.n_mat = 3;
+        qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
+        qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
+        qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
+        qa.x = xn; qa.K = E; qa.T = T;
+        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+            !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
+            qa.rope = rope_of();
+            qa.kind[0] = GEMV_KIND_Q; qa.kind[1] = GEMV_KIND_K; qa.kind[2] = GEMV_KIND_V;
+            rope_fused = true;
+        }
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny_f16(qa, stream)) != MESH_OK) return rc;
+    } else if (skinny) {
         SkinnyArgs qa;
         qa.n_mat = 3;
         qa.mat[0] = mat_of(L.wq, s->q, QD, &L.bq);
@@ -726,7 +757,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         }
         else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
             // straight into the output projection's input layout
-            if (skinny) { aa.out_q16 = s->xq; attn_is_k8 = true; }
+            if (sk8) { aa.out_q16 = s->xq; attn_is_k8 = true; }
             else if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }
             rc = attention_mma(aa, T, stream);
         } else rc = attention(aa, T, stream);
@@ -735,12 +766,20 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     {
         ProfScope ps(s, MESH_PROF_PREP);
         if (attn_is_k8) rc = MESH_OK;
-        else if (skinny) rc = quant16_k8(s->attn, nullptr, 0.f, T, QD, s->xq, stream);
-        else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream);
+        else if (sk8) rc = quant16_k8(s->attn, nullptr, 0.f, T, QD, s->xq, stream);
+        else if (k8) rc = pack_f16_k8(s->attn, T, QD, xn, stream, s->f16_sat);
         else rc = act_pack_dev(MESH_F16, s->attn, s->xn16, (int64_t)T * QD, stream);
     }
     if (rc != MESH_OK) return rc;
-    if (skinny) {
+    if (sk16) {
+        SkinnyF16Args oa;
+        oa.n_mat = 1;
+        oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
+        oa.x = xn; oa.K = QD; oa.T = T;
+        oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny_f16(oa, stream)) != MESH_OK) return rc;
+    } else if (skinny) {
         SkinnyArgs oa;
         oa.n_mat = 1;
         oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
@@ -757,11 +796,29 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     if (attn_only) return MESH_OK;
     {
         ProfScope ps(s, MESH_PROF_PREP);
-        if (skinny) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
-        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream);
-        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream);
+        if (sk8) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream, s->f16_sat);
+        else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream, s->f16_sat);
     }
     if (rc != MESH_OK) return rc;
+    if (sk16) {
+        // gate and up in one pass with the SwiGLU epilogue, written as f16 straight into the down projection's input
+        SkinnyF16Args ga;
+        ga.n_mat = 2;
+        ga.mat[0] = mat_of(L.w_gate, nullptr, FF, nullptr);
+        ga.mat[1] = mat_of(L.w_up, nullptr, FF, nullptr);
+        ga.x = xn; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
+        ga.y16 = f16ffn;
+        ga.sat = s->f16_sat;
+        SkinnyF16Args da;
+        da.n_mat = 1;
+        da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
+        da.x = f16ffn; da.K = FF; da.T = T;
+        da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        ProfScope ps(s, MESH_PROF_GEMV);
+        if ((rc = gemm_skinny_f16(ga, stream)) != MESH_OK) return rc;
+        return gemm_skinny_f16(da, stream);
+    }
     if (skinny) {
         // gate and up in one pass with the SwiGLU epilogue; its f32 output is quantised for the down projection
         SkinnyArgs ga;
@@ -797,8 +854,8 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         }
         {
             ProfScope ps(s, MESH_PROF_PREP);
-            if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream);
-            else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream);
+            if (k8) rc = swiglu_f16_k8(s->ffn, s->ffn_up, T, FF, f16ffn, stream, s->f16_sat);
+            else rc = swiglu_f16(s->ffn, s->ffn_up, f16ffn, (int64_t)T * FF, stream, s->f16_sat);
         }
         if (rc != MESH_OK) return rc;
     }
@@ -952,13 +1009,14 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                     ProfScope ps(s, MESH_PROF_PREP);
                     if ((rc = moe_sort(s->moe_ids, T * k, ne, s->moe_sorted, stream)) != MESH_OK) return rc;
                     if ((rc = rmsnorm_f16_k8_gather(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, s->moe_sorted.pair_of_slot, k, slots, E,
-                                                    reinterpret_cast<_Float16 *>(s->moe_x16), stream)) != MESH_OK) return rc;
+                                                    reinterpret_cast<_Float16 *>(s->moe_x16), stream, s->f16_sat)) != MESH_OK) return rc;
                 }
                 GemmArgs g;
                 g.W = L.gate_exps.data; g.Wp = L.exps_gate_up_gemm; g.type = L.gate_exps.type;
                 g.M = ffe; g.K = E; g.T = slots;
                 g.X = reinterpret_cast<const _Float16 *>(s->moe_x16); g.ldx = E; g.x_k8 = true;
                 g.y16_k8 = reinterpret_cast<_Float16 *>(s->moe_ffn16);
+                g.sat = s->f16_sat;
                 g.tiles = s->moe_sorted.tiles; g.n_tiles = s->moe_sorted.counts; g.max_tiles = max_tiles; g.expert_stride = L.exps_gate_up_stride;
                 { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_kquant(g, stream); }
                 if (rc != MESH_OK) return rc;

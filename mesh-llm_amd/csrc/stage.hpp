@@ -89,6 +89,10 @@ struct mesh_session {
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr;
     uint8_t *ffn_xq = nullptr;                          // single-token decode: the FFN vector as its producer quantised it (gemv.hpp: xq layout)
+    unsigned *f16_sat = nullptr;                        // device counter: values the f16 producers of the batched paths clamped to +-65504
+    uint32_t f16_sat_seen = 0;                          // device counter at its last read
+    uint64_t f16_sat_total = 0;                         // running total the ABI reports
+    bool skinny_f16 = true;                             // MESH_SKINNY_F16=0 at session creation: batched decode on the integer matrix cores (16-bit activations)
     bool xq_handover = true;                            // MESH_XQ_HANDOVER=0 at session creation: the down projection quantises the f32 vector itself
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     size_t attn_part_rows = 0;                          // (token, split) rows they hold

@@ -1,8 +1,10 @@
-"""Activation range of the projection paths.  Decode batches (mat-vec kernels, integer-MFMA skinny GEMM) quantise
-activations to 16-bit fixed point per 32-element block with an f32 block scale: any f32 magnitude is representable, and
-an outlier channel costs precision only inside its own block.  Calls of 17+ tokens (large-tile GEMM) round activations
-to f16: relative precision 2^-11 whatever the magnitude, up to +-65504, beyond which the producers SATURATE (a finite,
-wrong-by-clamping value) rather than emit an infinity that the next norm would turn into NaN for the whole token.
+"""Activation range of the projection paths.  The mat-vec kernels (calls of up to 4 tokens) and the integer-MFMA skinny
+GEMM quantise activations to 16-bit fixed point per 32-element block with an f32 block scale: any f32 magnitude is
+representable, and an outlier channel costs precision only inside its own block.  The f16 skinny GEMM (calls of 5 to 16
+tokens, the default) and the large-tile GEMM (17+ tokens) round activations to f16: relative precision 2^-11 whatever the
+magnitude, up to +-65504, beyond which the producers SATURATE (a finite, wrong-by-clamping value) rather than emit an
+infinity that the next norm would turn into NaN for the whole token, and count the value in the session's saturation
+counter.
 
 Checked here against the oracle: hidden states with the boundary codec's x50 outlier channels through every path, and
 SwiGLU products beyond the f16 range (exact on the decode paths, finite on the f16 path)."""
@@ -47,16 +49,21 @@ def _stage(tmp_path, scale_ffn_norm=None, n_seq=24, n_batch=208):
     return m, cfg, {n: (t, d, x) for n, t, d, x in tl}, st
 
 
-def test_outlier_channels_through_every_projection_path(tmp_path):
+@pytest.mark.parametrize("skinny", ["f16", "integer"])
+def test_outlier_channels_through_every_projection_path(tmp_path, monkeypatch, skinny):
+    """Batches of 5..16 tokens once on the f16 matrix cores (the default: f16 activations, one rounding per weight) and once
+    on the integer ones (16-bit fixed-point activations, MESH_SKINNY_F16=0 at session creation)."""
     m, cfg, tensors, st = _stage(tmp_path)
     E = cfg["n_embd"]
+    monkeypatch.setenv("MESH_SKINNY_F16", "1" if skinny == "f16" else "0")
     ses = st.session()
+    monkeypatch.delenv("MESH_SKINNY_F16")
     orc = StageOracle(cfg, tensors, 3, 5, 256, n_seq_max=24, blas=True)
     rng = np.random.Generator(np.random.PCG64(50))
     nxt = {}
     # 200-token prefill chunk (large-tile GEMM, f16 activations), then decode batches on top of it and on fresh sequences
     for T, seqs, what in ((200, [0] * 200, "prefill 200 (f16 large-tile GEMM)"), (1, [0], "decode 1 (mat-vec)"), (3, [0, 1, 2], "decode 3 (mat-vec)"),
-                          (8, list(range(8)), "decode 8 (integer skinny GEMM)"), (16, list(range(16)), "decode 16 (integer skinny GEMM)"),
+                          (8, list(range(8)), "decode 8 (%s skinny GEMM)" % skinny), (16, list(range(16)), "decode 16 (%s skinny GEMM)" % skinny),
                           (24, list(range(24)), "decode 24 (f16 large-tile GEMM, split K)")):
         x = outlier_input(rng, T, E)
         pos = []
@@ -88,19 +95,35 @@ def test_swiglu_products_beyond_the_f16_range(tmp_path):
     t, d, w = tensors["blk.3.ffn_up.weight"]
     u = O.mul_mat(t, w, d[1], d[0], n)
     assert np.abs(O.swiglu(g, u)).max() > 65504
-    # decode paths: exact arithmetic range, same tolerance as ever
-    for T in (1, 8):
+    def run(ses, T, pos0, seq0):
         xs = rng.standard_normal((T, E)).astype(np.float32)
-        seqs = list(range(T))
-        got = ses.decode(xs, [0] * T, seq=seqs).view(np.float32).reshape(T, E)
-        ref = orc.forward(xs, [0] * T, seq=seqs)
-        r = rel_l2(got, ref)
-        print("[outliers] SwiGLU beyond f16, decode %d: rel-L2 %.3e" % (T, r))
+        seqs = [seq0 + i for i in range(T)] if pos0 == 0 else [seq0] * T
+        pos = [0] * T if pos0 == 0 else list(range(pos0, pos0 + T))
+        got = ses.decode(xs, pos, seq=seqs).view(np.float32).reshape(T, E)
+        return got, rel_l2(got, orc.forward(xs, pos, seq=seqs))
+
+    # integer paths (the single-token mat-vec, and the 16-bit fixed-point matrix-core kernel for small batches): exact
+    # arithmetic range, same tolerance as ever, and nothing counted as saturated
+    os.environ["MESH_SKINNY_F16"] = "0"
+    try:
+        ses_int = st.session()
+    finally:
+        del os.environ["MESH_SKINNY_F16"]
+    for T in (1, 8):
+        got, r = run(ses_int, T, 0, 0)
+        print("[outliers] SwiGLU beyond f16, decode %d (integer kernels): rel-L2 %.3e" % (T, r))
         assert r <= 5e-4, T
-    # f16 path: saturates, stays finite (and is therefore off by what the clamp removed)
-    xs = rng.standard_normal((64, E)).astype(np.float32)
-    got = ses.decode(xs, np.arange(64) + 1, seq=[20] * 64).view(np.float32).reshape(64, E)
-    ref = orc.forward(xs, np.arange(64) + 1, seq=[20] * 64)
-    print("[outliers] SwiGLU beyond f16, prefill 64 (saturating f16): rel-L2 %.3e" % rel_l2(got, ref))
-    assert np.isfinite(got).all()
+    assert ses_int.f16_saturations() == 0
+    ses_int.close()
+    # f16 paths: saturate, stay finite (and are therefore off by what the clamp removed), and say so through the counter
+    got, r = run(ses, 1, 0, 0)
+    assert r <= 5e-4 and ses.f16_saturations() == 0
+    seen = 0
+    for T, pos0, seq0, what in ((8, 0, 8, "f16 skinny GEMM"), (64, 1, 20, "prefill")):
+        got, r = run(ses, T, pos0, seq0)
+        n = ses.f16_saturations()
+        print("[outliers] SwiGLU beyond f16, %s of %d tokens (saturating f16): rel-L2 %.3e, %d values clamped so far" % (what, T, r, n))
+        assert np.isfinite(got).all()
+        assert n > seen, what
+        seen = n
     ses.close(); st.close()
