@@ -174,6 +174,8 @@ typedef struct mesh_stage_opts {
     int32_t kv_type;        /* K cache rows: 0 or MESH_F16, MESH_Q8_0, MESH_Q4_0            (--cache-type-k, launch.rs:639-644) */
     int32_t kv_type_v;      /* V cache rows: 0 = MESH_F16 when kv_type is f16, else MESH_Q4_0 (--cache-type-v).  The pairs of
                                KvCacheQuant::for_model_size (launch.rs:568-591) are supported: f16/f16, q8_0/q4_0, q4_0/q4_0 */
+    const char *tuning;     /* kernel-selection switches as "name=value,name=value"; NULL = the defaults.  See
+                               mesh_session_set_option for the names.  No counterpart in the reference. */
 } mesh_stage_opts;
 
 typedef struct mesh_batch {
@@ -209,8 +211,8 @@ int mesh_stage_decode_dev(mesh_session *session, const mesh_batch *batch, const 
 void *mesh_session_stream(mesh_session *session);
 int mesh_session_synchronize(mesh_session *session);
 /* Number of decode steps of this session whose layer launches were replayed from a captured HIP graph (batches of up to
- * 32 tokens, from the third call with the same token count and KV split count on; environment MESH_STAGE_GRAPHS=1 at
- * session creation turns graphs on: they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
+ * 32 tokens, from the third call with the same token count and KV split count on; the switch graphs=1 turns them on:
+ * they save the host the submission of ~80 launches per step).  -1 for a null session.  No counterpart in the reference. */
 int64_t mesh_session_graph_replays(const mesh_session *session);
 
 /* Per-kernel-class timing of a session: every kernel launched for the session while profiling is on carries its own
@@ -246,6 +248,41 @@ int mesh_session_moe_last_ids(mesh_session *session, int32_t *ids, int32_t n_tok
  * count.  Waits for the session's stream.  No counterpart in the reference (ggml's f16 conversions saturate silently to
  * infinity). */
 int mesh_session_f16_saturations(mesh_session *session, uint64_t *count);
+
+/* Kernel-selection switches.  Every choice between two kernels for the same arithmetic and every dispatch threshold has
+ * a name; the defaults are what the benchmarks run.  A stage takes the defaults, then the environment variable
+ * MESH_TUNING ("name=value,...", read once per process, for A/B runs of an unmodified host), then
+ * mesh_stage_opts.tuning; a session starts from its stage's values, and mesh_session_set_option changes a
+ * session-level switch between decode calls (it waits for the session's stream and drops captured graphs).
+ *
+ *   stage level (decide what is allocated; mesh_stage_opts.tuning / MESH_TUNING only):
+ *     gemm_layout=1        keep a GEMM-layout copy of the projections when n_batch_max reaches gemm_min_tokens
+ *     gemm_min_tokens=17   calls of at least this many tokens run the large-tile MFMA GEMM
+ *     skinny_min_tokens=0  calls of at least this many (and fewer than the above) run the skinny MFMA GEMM;
+ *                          0 = 4 with skinny_f16, 5 without
+ *   session level:
+ *     gemm_splitk=1        GEMM launches too narrow to fill the chip split K over workgroups
+ *     chunk_kv16=1         long prefill chunks over a quantised cache decode a layer's rows once into an f16 copy
+ *     gemv_rope=1          RoPE and the KV append in the q/k/v projection's epilogue
+ *     xq_handover=1        single-token calls: gate/up leaves the FFN vector quantised for the down projection
+ *     skinny_f16=1         the skinny GEMM on the f16 matrix cores (0: integer matrix cores, 16-bit activations)
+ *     gemm_fused=1         q/k/v and gate/up of a prefill call as one launch each
+ *     gemm_xdirect=1       the prefill GEMM reads k8-major activations directly
+ *     gemm_big=1           256-row tiles for wide projections of long calls
+ *     gemm_narrow=1        64-token tiles for calls of at most 64 tokens
+ *     attn_chunk_ksplit=1  a prefill chunk's key walks split over workgroups when the grid would not fill the chip
+ *     attn_mma_min_tokens=1  decode attention on the matrix cores from this many tokens
+ *     attn_split_target=0  workgroups a decode attention launch aims at (0 = 256, or 512 for quantised rows)
+ *     moe_group=1          (token, slot) pairs grouped by expert
+ *     moe_fuse_quant=1     the expert combine step quantises for the next layer
+ *     moe_gemm=1, moe_gemm_min_pairs=4   prefill-sized expert products on the large-tile GEMM
+ *     grouped_oversub=8    grouped expert mat-vec: workgroups per compute unit and item
+ *     graphs=0             decode steps of up to 32 tokens replayed from captured HIP graphs
+ *
+ * MESH_ERR_INVALID: unknown name, value out of range, or a stage-level switch passed to set_option.  No counterpart in
+ * the reference (llama.cpp picks kernels by compile-time flags and GGML_* environment variables). */
+int mesh_session_set_option(mesh_session *session, const char *name, int32_t value);
+int mesh_session_get_option(const mesh_session *session, const char *name, int32_t *value);
 
 /* KV cache import/export for one sequence and one (absolute) layer: n_pos positions starting at pos0, host
  * buffers of f16 bits laid out [n_pos][n_head_kv][head_dim].  (The reference has no KV hand-over; a restarted

@@ -65,7 +65,8 @@ class TensorInfo(ctypes.Structure):
 class StageOpts(ctypes.Structure):
     """mesh_stage_opts"""
     _fields_ = [("device", ctypes.c_char_p), ("n_ctx", ctypes.c_int32), ("n_seq_max", ctypes.c_int32),
-                ("n_batch_max", ctypes.c_int32), ("kv_type", ctypes.c_int32), ("kv_type_v", ctypes.c_int32)]
+                ("n_batch_max", ctypes.c_int32), ("kv_type", ctypes.c_int32), ("kv_type_v", ctypes.c_int32),
+                ("tuning", ctypes.c_char_p)]
 
 
 class Batch(ctypes.Structure):
@@ -108,6 +109,8 @@ SIGNATURES.update({
     "mesh_session_set_expert_mask": (_i32, [_vp, _vp, _i32]),
     "mesh_session_moe_last_ids": (_i32, [_vp, _vp, _i32]),
     "mesh_session_f16_saturations": (_i32, [_vp, ctypes.POINTER(ctypes.c_uint64)]),
+    "mesh_session_set_option": (_i32, [_vp, ctypes.c_char_p, _i32]),
+    "mesh_session_get_option": (_i32, [_vp, ctypes.c_char_p, ctypes.POINTER(_i32)]),
     "mesh_session_kv_write": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_session_kv_read": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "mesh_op_q16_bytes": (_sz, [_i64, _i64]),
@@ -295,10 +298,13 @@ def gguf_tensor(path, name):
 class Stage:
     """Layers [layer_begin, layer_end) of a GGUF model resident on the GPU (mesh_stage)."""
 
-    def __init__(self, gguf_path, layer_begin, layer_end=-1, n_ctx=0, n_seq_max=0, n_batch_max=0, device=None, kv_types=None):
-        """kv_types: (K, V) cache row types, one of (F16, F16), (Q8_0, Q4_0), (Q4_0, Q4_0); None = f16 / f16."""
+    def __init__(self, gguf_path, layer_begin, layer_end=-1, n_ctx=0, n_seq_max=0, n_batch_max=0, device=None, kv_types=None, tuning=None):
+        """kv_types: (K, V) cache row types, one of (F16, F16), (Q8_0, Q4_0), (Q4_0, Q4_0); None = f16 / f16.
+        tuning: kernel-selection switches, {"name": value} or "name=value,..." (mesh_stage_opts.tuning)."""
         kt, vt = kv_types if kv_types else (0, 0)
-        opts = StageOpts(device.encode() if device else None, n_ctx, n_seq_max, n_batch_max, kt, vt)
+        if isinstance(tuning, dict):
+            tuning = ",".join("%s=%d" % (k, int(v)) for k, v in tuning.items())
+        opts = StageOpts(device.encode() if device else None, n_ctx, n_seq_max, n_batch_max, kt, vt, tuning.encode() if tuning else None)
         self._h = ctypes.c_void_p()
         check(lib().mesh_stage_open(os.fsencode(gguf_path), layer_begin, layer_end, ctypes.byref(opts), ctypes.byref(self._h)))
         self.info = ModelInfo()
@@ -308,8 +314,12 @@ class Stage:
     def weight_bytes(self):
         return int(lib().mesh_stage_weight_bytes(self._h))
 
-    def session(self):
-        return Session(self)
+    def session(self, **options):
+        """options: session-level kernel-selection switches (mesh_session_set_option), e.g. session(skinny_f16=0)."""
+        ses = Session(self)
+        for name, value in options.items():
+            ses.set_option(name, value)
+        return ses
 
     def close(self):
         if self._h:
@@ -400,6 +410,14 @@ class Session:
         out = np.empty((n_tokens, self.stage.info.n_expert_used), dtype=np.int32)
         check(lib().mesh_session_moe_last_ids(self._h, _np_ptr(out), n_tokens))
         return out
+
+    def set_option(self, name, value):
+        check(lib().mesh_session_set_option(self._h, name.encode(), int(value)))
+
+    def get_option(self, name):
+        v = ctypes.c_int32(0)
+        check(lib().mesh_session_get_option(self._h, name.encode(), ctypes.byref(v)))
+        return int(v.value)
 
     def f16_saturations(self):
         """Values clamped to the f16 range by the batched paths since the session was created."""

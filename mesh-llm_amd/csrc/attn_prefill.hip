@@ -352,12 +352,6 @@ static int pf_n_cu() {
     return n;
 }
 
-// MESH_ATTN_CHUNK_KSPLIT=0: a chunk's walks are never split over workgroups (for comparison)
-static bool pf_ksplit_on() {
-    const char *e = getenv("MESH_ATTN_CHUNK_KSPLIT");
-    return !(e && e[0] == '0');
-}
-
 int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t stream) {
     if (T <= 0) return MESH_OK;
     AttnArgs a = a_in;
@@ -396,7 +390,7 @@ int attention_chunk(const AttnArgs &a_in, int T, int pos0, int seq, hipStream_t 
     int n_ksplit = 1;
     {
         const int wgs = (int)(grid.x * grid.y * grid.z), n_keys = pos0 + T;
-        if (a.part && a.ml && pf_ksplit_on() && wgs < pf_n_cu())
+        if (a.part && a.ml && a.part_rows > 0 && wgs < pf_n_cu())
             n_ksplit = std::max(1, std::min(std::min(pf_n_cu() / wgs, 8), std::min(n_keys / 256, (int)(a.part_rows / (size_t)T))));
         if (n_ksplit > ATTN_SPLITS_CAP) n_ksplit = ATTN_SPLITS_CAP;
     }

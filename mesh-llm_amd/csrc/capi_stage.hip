@@ -222,6 +222,29 @@ int mesh_session_f16_saturations(mesh_session *session, uint64_t *count) {
     return MESH_OK;
 }
 
+int mesh_session_set_option(mesh_session *session, const char *name, int32_t value) {
+    if (!session || !name) return fail(MESH_ERR_INVALID, "mesh_session_set_option: null argument");
+    Tuning t = session->tune;
+    const int rc = tuning_set(t, name, value, true);
+    if (rc != MESH_OK) return rc;
+    // launches captured under the old value would replay it
+    MESH_HIP_TRY(hipSetDevice(session->stage->device));
+    MESH_HIP_TRY(hipStreamSynchronize(session->stream));
+    for (auto &g : session->graphs)
+        if (g.second.exec) (void)hipGraphExecDestroy(g.second.exec);
+    session->graphs.clear();
+    session->tune = t;
+    return MESH_OK;
+}
+
+int mesh_session_get_option(const mesh_session *session, const char *name, int32_t *value) {
+    if (!session || !name || !value) return fail(MESH_ERR_INVALID, "mesh_session_get_option: null argument");
+    int v = 0;
+    const int rc = tuning_get(session->tune, name, &v);
+    if (rc == MESH_OK) *value = v;
+    return rc;
+}
+
 static int kv_xfer(mesh_session *s, int layer, int seq_id, int pos0, int n_pos, uint16_t *k, uint16_t *v, bool write) {
     if (!s || !k || !v) return fail(MESH_ERR_INVALID, "mesh_session_kv: null argument");
     const mesh_stage *st = s->stage;

@@ -692,12 +692,6 @@ static int launch_gemm_big(const GemmArgs &k, int row_blocks, int t_blocks, hipS
     return MESH_OK;
 }
 
-// MESH_GEMM_BIG=0: every call keeps the 128 x 128 tile (for comparison)
-static bool gemm_big_on() {
-    const char *e = getenv("MESH_GEMM_BIG");
-    return !(e && e[0] == '0');
-}
-
 // Second kernel of a split launch: adds the slices of part[slice][token][row] in slice order and applies the epilogue
 // of the unsplit kernel.  One thread per (token, four consecutive rows); rows run fastest, so partial reads and output
 // writes are contiguous.
@@ -812,13 +806,6 @@ static int launch_gemm_kernel(const GemmArgs &k, dim3 grid, hipStream_t stream) 
     return MESH_OK;
 }
 
-// MESH_GEMM_NARROW=0: calls of at most 64 tokens use the 128-token tile like the others (for comparison)
-static bool gemm_narrow_on() {
-    static int v = -1;
-    if (v < 0) { const char *e = getenv("MESH_GEMM_NARROW"); v = !(e && e[0] == '0'); }
-    return v != 0;
-}
-
 static int gemm_n_cu() {
     static int n = 0;
     if (!n) {
@@ -834,7 +821,7 @@ template <int TYPE, bool PACKED, bool XDIRECT>
 static int launch_gemm(const GemmArgs &k, dim3 grid, hipStream_t stream) {
     // calls of at most 64 tokens on the production layout (GEMM-layout weights, k8-major activations): narrow tile
     if constexpr (PACKED && XDIRECT) {
-        if (k.T <= GN / 2 && gemm_narrow_on())
+        if (k.T <= GN / 2 && k.narrow_tile)
             return k.ksplit > 1 ? launch_gemm_kernel<TYPE, true, true, true, true>(k, grid, stream) : launch_gemm_kernel<TYPE, true, true, false, true>(k, grid, stream);
     }
     return k.ksplit > 1 ? launch_gemm_kernel<TYPE, PACKED, XDIRECT, true, false>(k, grid, stream) : launch_gemm_kernel<TYPE, PACKED, XDIRECT, false, false>(k, grid, stream);
@@ -900,7 +887,7 @@ int gemm_kquant(const GemmArgs &a, hipStream_t stream) {
     if (a.type != MESH_Q4_K && a.type != MESH_Q6_K) return fail(MESH_ERR_UNSUPPORTED, "gemm: no MFMA kernel for ggml type %d", a.type);
     const bool q4 = a.type == MESH_Q4_K, packed = a.Wp != nullptr;
     // enough workgroups of the 256 x 128 tile to give every CU one: the big tile (gemm_big_kernel)
-    if (a.x_k8 && packed && k.ksplit <= 1 && !a.rope.pos && row_blocks % 2 == 0 && gemm_big_on() &&
+    if (a.x_k8 && packed && k.ksplit <= 1 && !a.rope.pos && row_blocks % 2 == 0 && a.big_tile &&
         (row_blocks / 2) * (int)grid.y >= gemm_n_cu())
         return q4 ? launch_gemm_big<MESH_Q4_K>(k, row_blocks, (int)grid.y, stream) : launch_gemm_big<MESH_Q6_K>(k, row_blocks, (int)grid.y, stream);
     if (a.x_k8) {

@@ -32,6 +32,8 @@ struct GemmArgs {
     // rows), M their common row count; the launch writes f16(silu(gate) * up) in the k8-major layout to y16_k8 (Y unused).
     _Float16 *y16_k8 = nullptr;
     unsigned *sat = nullptr;         // optional device counter of SwiGLU outputs clamped to the f16 range (mesh_common.hpp: note_f16_clamp)
+    bool big_tile = true;            // wide projections of long calls may take the 256-row tile
+    bool narrow_tile = true;         // calls of at most 64 tokens may take the 64-token tile
     // Optional scratch for launches too narrow to fill the chip (few row blocks x token blocks): K is then split over
     // blockIdx.z, every slice writes its f32 partial tile to `part` ([slice][token][row of the launch]) and a second
     // kernel adds the slices in slice order and applies the epilogue.  Null: never split.  ksplit / k_per_split are

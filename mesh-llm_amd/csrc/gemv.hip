@@ -311,7 +311,7 @@ static int gemv_kquant(const GemvArgs &a, hipStream_t stream) {
     if (a.items && (!a.expert_ids || !a.n_items || a.max_items <= 0)) return fail(MESH_ERR_INVALID, "gemv: bad grouped-expert arguments");
     KquantPlan plan;
     // (grouped launches: workgroups of a quarter of the size, several times as many per item)
-    static const int oversub = getenv("MESH_GROUPED_OVERSUB") ? std::max(1, atoi(getenv("MESH_GROUPED_OVERSUB"))) : 8;
+    const int oversub = std::max(1, a.grouped_oversub);
     int rc0 = a.items ? plan_kquant(a, std::max(1, oversub * n_compute_units() / n_pairs), plan, GROUPED_THREADS / 64)
                       : plan_kquant(a, std::max(1, n_compute_units() / n_pairs), plan);
     if (rc0 != MESH_OK) return rc0;

@@ -92,6 +92,7 @@ struct GemvArgs {
     const int32_t *items = nullptr;
     const int32_t *n_items = nullptr;
     int max_items = 0;
+    int grouped_oversub = 8;        // grouped launches: workgroups per compute unit and item
     // Fused RoPE / KV append: kind[i] says what matrix i produces (tiled K-quant matrices, EPI_STORE, no experts only)
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};

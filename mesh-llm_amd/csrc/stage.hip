@@ -71,7 +71,6 @@ int hparams_from_gguf(const GgufFile &g, HParams &hp) {
     return MESH_OK;
 }
 
-static int gemm_min_tokens();
 
 // ------------------------------------------------------------------------------------------------ loading
 namespace {
@@ -229,6 +228,8 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
         return fail(MESH_ERR_INVALID, "mesh_stage_open: layer range [%d,%d) does not fit a %u-layer model", layer_begin, layer_end, hp.n_layer);
     st->layer_begin = layer_begin;
     st->layer_end = layer_end;
+    if ((rc = tuning_process_default(st->tune)) != MESH_OK) return rc;
+    if (opts && opts->tuning && (rc = tuning_parse(st->tune, opts->tuning, "mesh_stage_opts.tuning")) != MESH_OK) return rc;
     st->n_ctx = opts && opts->n_ctx > 0 ? opts->n_ctx : 4096;
     st->n_seq_max = opts && opts->n_seq_max > 0 ? opts->n_seq_max : 1;
     st->n_batch_max = opts && opts->n_batch_max > 0 ? opts->n_batch_max : 512;
@@ -245,12 +246,9 @@ int stage_open(const char *path, int layer_begin, int layer_end, const mesh_stag
         return fail(MESH_ERR_UNSUPPORTED, "mesh_stage_open: head_dim %u has no attention kernel (64 and 128 do)", hp.head_dim);
 
     Loader ld{g, *st};
-    // stages that can be handed prefill-sized calls keep a GEMM-layout copy of their projections (MESH_GEMM_LAYOUT=0:
-    // no copy, the GEMM reads the mat-vec tiles)
-    {
-        const char *e = getenv("MESH_GEMM_LAYOUT");
-        ld.gemm_layout = st->n_batch_max >= gemm_min_tokens() && !(e && e[0] == '0');
-    }
+    // stages that can be handed prefill-sized calls keep a GEMM-layout copy of their projections (gemm_layout=0: no
+    // copy, the GEMM reads the mat-vec tiles)
+    ld.gemm_layout = st->n_batch_max >= st->tune.gemm_min_tokens && st->tune.gemm_layout;
     const int64_t E = hp.n_embd, QD = (int64_t)hp.n_head * hp.head_dim, KD = (int64_t)hp.n_head_kv * hp.head_dim;
     const bool moe = hp.arch == "qwen3moe";
     st->layers.resize((size_t)(layer_end - layer_begin));
@@ -341,39 +339,12 @@ constexpr int ATTN_SPLITS_MAX = ATTN_SPLITS_CAP;
 constexpr int ATTN_PART_ROWS_MIN = 512;     // rows of (token, split) the partial buffers always hold
 constexpr int META_SLOTS = 8;
 constexpr int LOGITS_TOKENS_MAX = MESH_LOGITS_TOKENS_MAX;        // logits rows the host-pointer entry point stages per call
-// calls with at least this many tokens take the MFMA GEMM path (MESH_GEMM_MIN_TOKENS overrides, for tuning)
-static int gemm_min_tokens() {
-    static int v = 0;
-    if (!v) {
-        const char *e = getenv("MESH_GEMM_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 17;
-    }
-    return v;
-}
-#define PREFILL_MIN_TOKENS gemm_min_tokens()
-// mixture of experts: calls with at least this many (token, slot) pairs per expert on average run the expert products as
-// tiles of the large-tile GEMM (measured against the other kernels on a 64-expert shard with top-8 routing, four layers:
-// 0.607 against 0.659 ms at 4 pairs per expert, 0.536 against 0.485 at 2; MESH_MOE_GEMM_MIN_PAIRS moves it).  Below that the
-// mat-vec kernel; the 16-pair integer matrix-core kernel covers stages without GEMM-layout copies of the experts.
-static size_t moe_gemm_min_pairs() {
-    static const size_t v = getenv("MESH_MOE_GEMM_MIN_PAIRS") ? (size_t)std::max(1, atoi(getenv("MESH_MOE_GEMM_MIN_PAIRS"))) : 4;
-    return v;
-}
-#define MOE_GEMM_MIN_PAIRS_PER_EXPERT moe_gemm_min_pairs()
-// MESH_MOE_GEMM=0: never (for comparison)
-static bool moe_gemm_on() {
-    const char *e = getenv("MESH_MOE_GEMM");
-    return !(e && e[0] == '0');
-}
-// calls with at least this many tokens (and fewer than the above) take the skinny MFMA GEMM (MESH_SKINNY_MIN_TOKENS)
-static int skinny_min_tokens() {
-    static int v = 0;
-    if (!v) {
-        const char *e = getenv("MESH_SKINNY_MIN_TOKENS");
-        v = e && atoi(e) > 0 ? atoi(e) : 5;
-    }
-    return v;
-}
+// Mixture of experts: calls with at least moe_gemm_min_pairs (token, slot) pairs per expert on average run the expert
+// products as tiles of the large-tile GEMM (measured against the other kernels on a 64-expert shard with top-8 routing,
+// four layers: 0.607 against 0.659 ms at 4 pairs per expert, 0.536 against 0.485 at 2).  Below that the mat-vec kernel;
+// the 16-pair integer matrix-core kernel covers stages without GEMM-layout copies of the experts.
+#define PREFILL_MIN_TOKENS (s->tune.gemm_min_tokens)
+#define MOE_GEMM_MIN_PAIRS_PER_EXPERT ((size_t)s->tune.moe_gemm_min_pairs)
 
 int session_new(mesh_stage *st, mesh_session **out) {
     if (!st || !out) return fail(MESH_ERR_INVALID, "mesh_stage_session_new: null argument");
@@ -384,14 +355,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     const HParams &hp = st->hp;
     const size_t nl = st->layers.size(), B = (size_t)st->n_batch_max;
     MESH_HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
-    if (const char *e = getenv("MESH_GEMV_ROPE")) s->rope_in_gemv = e[0] != '0';
-    if (const char *e = getenv("MESH_XQ_HANDOVER")) s->xq_handover = e[0] != '0';
-    if (const char *e = getenv("MESH_SKINNY_F16")) s->skinny_f16 = e[0] != '0';
-    if (const char *e = getenv("MESH_MOE_GROUP")) s->moe_grouped = e[0] != '0';
-    if (const char *e = getenv("MESH_MOE_FUSE_QUANT")) s->moe_fuse_quant = e[0] != '0';
-    if (const char *e = getenv("MESH_GEMM_XDIRECT")) s->gemm_x_k8 = e[0] != '0';
-    if (const char *e = getenv("MESH_GEMM_FUSED")) s->gemm_fused = e[0] != '0';
-    if (const char *e = getenv("MESH_STAGE_GRAPHS")) s->graphs_on = e[0] != '0';
+    s->tune = st->tune;
     const size_t kv_rows = (size_t)st->n_seq_max * hp.n_head_kv * (size_t)st->n_ctx;
     s->k_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->k_type, (int)hp.head_dim);
     s->v_layer_bytes = kv_rows * (size_t)kv_row_bytes(st->v_type, (int)hp.head_dim);
@@ -424,7 +388,9 @@ int session_new(mesh_stage *st, mesh_session **out) {
         if ((rc = sess_alloc(s.get(), &p, xq_bytes((int)hp.n_ff))) != MESH_OK) return rc;
         s->ffn_xq = static_cast<uint8_t *>(p);
     }
-    if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_min_tokens())) {
+    // (either skinny kernel may be picked per call, so the buffers are there from the smaller of their thresholds on)
+    const int skinny_alloc_from = s->tune.skinny_min_tokens > 0 ? s->tune.skinny_min_tokens : 4;
+    if (B >= (size_t)std::min(PREFILL_MIN_TOKENS, skinny_alloc_from)) {
         const size_t B16 = (B + 15) / 16 * 16;       // the skinny GEMM reads whole blocks of 16 tokens
         if ((rc = sess_alloc(s.get(), &p, B16 * std::max<size_t>(hp.n_embd, QD) * 2)) != MESH_OK) return rc;
         s->xn16 = static_cast<uint16_t *>(p);
@@ -441,8 +407,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
             if ((rc = sess_alloc(s.get(), &p, bytes)) != MESH_OK) return rc;
             s->xq = static_cast<uint8_t *>(p);
         }
-        const char *ckv = getenv("MESH_CHUNK_KV16");      // =0 at session creation: every query tile decodes the quantised rows itself
-        if (st->k_type != MESH_F16 && hp.head_dim == 128 && B >= 128 && !(ckv && atoi(ckv) == 0)) {
+        if (st->k_type != MESH_F16 && hp.head_dim == 128 && B >= 128) {
             // f16 copy of one sequence's K and V rows of one layer: a long prefill chunk decodes the quantised cache once
             // per layer into it (attn.hpp: chunk_kv16).  Zeroed, so that rows past a chunk's last key are finite.
             const size_t bytes = 2 * (size_t)hp.n_head_kv * st->n_ctx * hp.head_dim * 2;
@@ -455,8 +420,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
             s->ffn16 = static_cast<uint16_t *>(p);
             if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
         }
-        const char *sk = getenv("MESH_GEMM_SPLITK");
-        if (B >= (size_t)PREFILL_MIN_TOKENS && !(sk && sk[0] == '0')) {
+        if (B >= (size_t)PREFILL_MIN_TOKENS) {
             // a split launch holds at most one 128 x 128 f32 tile per CU: 16.8 MB on 256 CUs
             s->gemm_part_bytes = (size_t)32 << 20;
             if ((rc = sess_alloc(s.get(), &p, s->gemm_part_bytes)) != MESH_OK) return rc;
@@ -521,27 +485,18 @@ static GemvMat mat_of(const DevTensor &w, float *y, int ldy, const DevTensor *bi
     return m;
 }
 
-// Batches of at least this many tokens take the matrix-core decode attention (Q and the probabilities rounded to f16;
-// faster at every batch size, so the default is 1).  MESH_ATTN_MMA_MIN_TOKENS raises it for callers that want the
-// all-f32 vector-ALU kernel at small batches.
-static int attn_mma_min_tokens() {
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("MESH_ATTN_MMA_MIN_TOKENS");
-        v = e ? std::max(1, atoi(e)) : 1;
-    }
-    return v;
-}
-
+// Batches of at least attn_mma_min_tokens tokens take the matrix-core decode attention (Q and the probabilities rounded
+// to f16; faster at every batch size, so the default is 1).  Callers that want the all-f32 vector-ALU kernel at small
+// batches raise it.
 // quantised: the cache rows are q8_0 / q4_0
-static int attn_splits_for(int T, int n_kv, int max_keys, bool quantised) {
+static int attn_splits_for(const Tuning &tune, int T, int n_kv, int max_keys, bool quantised) {
     // One workgroup per compute unit (256 on gfx950) measured best from batch 1 to 16 with f16 rows, which that many
     // workgroups stream at the memory's rate.  Quantised rows are bound by the instructions that decode them, and two
     // workgroups per CU hide each other's waits: 3-7% of the step at batch 8-32 (Qwen2.5-32B shape, q8_0 / q4_0 cache:
     // 9.86 -> 9.18 ms at batch 32, which otherwise runs unsplit); four per CU lose again, and so do 64 splits of a single
     // token's walk (from 64 (token, KV head) pairs on).
-    // (MESH_ATTN_SPLIT_TARGET: the workgroup count aimed at, for experiments)
-    static const int forced = getenv("MESH_ATTN_SPLIT_TARGET") ? std::max(1, atoi(getenv("MESH_ATTN_SPLIT_TARGET"))) : 0;
+    // (attn_split_target: the workgroup count aimed at, for experiments)
+    const int forced = tune.attn_split_target;
     const int target = forced ? forced : (quantised && T * n_kv >= 64) ? 512 : 256;
     int s = target / std::max(1, T * n_kv);
     s = std::min(s, (max_keys + 63) / 64);
@@ -632,12 +587,12 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
     bool rope_fused = false, attn_is_k8 = false;
-    const bool k8 = skinny || s->gemm_x_k8;      // activations in the k8-major layout (both GEMMs can read it)
+    const bool k8 = skinny || s->tune.gemm_xdirect;      // activations in the k8-major layout (both GEMMs can read it)
     // the batched-decode GEMM on the f16 matrix cores (k8-major f16 activations) instead of the integer ones (q16 activations);
     // a mixture-of-experts stage keeps the integer kernel, whose activation layout its expert launches share
-    const bool sk16 = skinny && s->skinny_f16 && L.w_gate.present() && f16ffn;
+    const bool sk16 = skinny && s->tune.skinny_f16 && L.w_gate.present() && f16ffn;
     const bool sk8 = skinny && !sk16;
-    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->gemm_part; g.part_bytes = s->gemm_part_bytes; g.sat = s->f16_sat; return g; };
+    auto gemm_k8 = [&](GemmArgs g) { g.x_k8 = k8; g.part = s->tune.gemm_splitk ? s->gemm_part : nullptr; g.part_bytes = s->gemm_part_bytes; g.sat = s->f16_sat; g.big_tile = s->tune.gemm_big; g.narrow_tile = s->tune.gemm_narrow; return g; };
     auto rope_of = [&]() {
         GemvRope r;
         r.pos = s->d_pos; r.seq = s->d_seq; r.inv_freq = st->rope_inv_freq;
@@ -661,7 +616,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = xn; qa.K = E; qa.T = T;
-        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+        if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
             !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
             qa.rope = rope_of();
             qa.kind[0] = GEMV_KIND_Q; qa.kind[1] = GEMV_KIND_K; qa.kind[2] = GEMV_KIND_V;
@@ -676,7 +631,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.xq = s->xq; qa.K = E; qa.T = T;
-        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+        if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
             !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
             qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;
             qa.rope.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
@@ -689,7 +644,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         if ((rc = gemm_skinny(qa, stream)) != MESH_OK) return rc;
     } else {
         ProfScope ps(s, MESH_PROF_GEMV);
-        if (L.qkv_fused >= 2 && s->gemm_fused) {
+        if (L.qkv_fused >= 2 && s->tune.gemm_fused) {
             // q, k (and v when it is of the same K-quant type) as one launch over their back-to-back GEMM-layout copies
             const DevTensor *w[3] = {&L.wq, &L.wk, &L.wv}, *b[3] = {&L.bq, &L.bk, &L.bv};
             float *y[3] = {s->q, s->k, s->v};
@@ -704,7 +659,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
             }
             GemmArgs gv = gemm_k8(gemm_of(L.wv, s->xn16, E, T, s->v, KD, &L.bv));
             // RoPE and the KV append ride in the second kernel of split launches (both launches must be split)
-            if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
+            if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
                 !L.k_norm.present() && hp.head_dim % 4 == 0 && hp.n_rot % 2 == 0 && gemm_split_count(g) > 1 &&
                 (L.qkv_fused == 3 || gemm_split_count(gv) > 1)) {
                 GemvRope r;
@@ -746,16 +701,16 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;     // a batch of decode steps still splits the long KV
+    aa.n_splits = T < 64 ? attn_splits_for(s->tune, T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;     // a batch of decode steps still splits the long KV
     {
         ProfScope ps(s, MESH_PROF_ATTN);
         if (!skinny && s->chunk_pos0 >= 0 && hp.head_dim == 128) {
             if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }          // straight into the output projection's input layout
-            aa.chunk_kv16 = reinterpret_cast<_Float16 *>(s->chunk_kv16);
-            aa.part_rows = s->attn_part_rows;
+            aa.chunk_kv16 = s->tune.chunk_kv16 ? reinterpret_cast<_Float16 *>(s->chunk_kv16) : nullptr;     // 0: every query tile decodes the quantised rows itself
+            aa.part_rows = s->tune.attn_chunk_ksplit ? s->attn_part_rows : 0;
             rc = attention_chunk(aa, T, s->chunk_pos0, s->chunk_seq, stream);
         }
-        else if (T >= attn_mma_min_tokens() && attention_mma_supported(aa)) {
+        else if (T >= s->tune.attn_mma_min_tokens && attention_mma_supported(aa)) {
             // straight into the output projection's input layout
             if (sk8) { aa.out_q16 = s->xq; attn_is_k8 = true; }
             else if (k8) { aa.out16_k8 = xn; attn_is_k8 = true; }
@@ -838,7 +793,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         ProfScope ps(s, MESH_PROF_GEMV);
         return gemm_skinny(da, stream);
     }
-    if (L.gate_up_gemm && k8 && s->gemm_fused) {
+    if (L.gate_up_gemm && k8 && s->tune.gemm_fused) {
         // gate and up as one launch whose epilogue writes f16(silu(gate) * up) straight into the down projection's input
         ProfScope ps(s, MESH_PROF_GEMV);
         GemmArgs g = gemm_k8(gemm_of(L.w_gate, s->xn16, E, T, nullptr, FF, nullptr));
@@ -878,13 +833,13 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     s->xq_layer = -1;
     // a mixture-of-experts layer whose attention block runs on the batched-decode (integer matrix-core) path
     auto moe_attn_skinny = [&](const LayerWeights &Ln) {
-        return !Ln.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && T < PREFILL_MIN_TOKENS && s->xn16 && layer_attn_is_kquant(Ln) &&
+        return !Ln.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, s->tune.skinny_from()) && T < PREFILL_MIN_TOKENS && s->xn16 && layer_attn_is_kquant(Ln) &&
                hp.n_embd % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0;
     };
     // the combine step at the end of a mixture-of-experts layer; when the next layer starts by quantising the new hidden
     // state for its projections, the same launch does that too (the same bits) and the layer finds them in s->xq
     auto combine = [&](size_t il, int top_k) {
-        if (s->moe_fuse_quant && il + 1 < st->layers.size() && moe_attn_skinny(st->layers[il + 1]) && moe_combine_quant16_supported(E)) {
+        if (s->tune.moe_fuse_quant && il + 1 < st->layers.size() && moe_attn_skinny(st->layers[il + 1]) && moe_combine_quant16_supported(E)) {
             const int r = moe_combine_quant16(s->x, s->moe_out, s->moe_w, T, E, top_k, static_cast<const float *>(st->layers[il + 1].attn_norm.data), hp.rms_eps,
                                               s->xq, stream);
             if (r == MESH_OK) s->xq_layer = (int)il + 1;
@@ -894,7 +849,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     };
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
-        if (T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
+        if (T >= std::min(PREFILL_MIN_TOKENS, s->tune.skinny_from()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
             const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0 &&
                                 L.w_gate.type == L.w_up.type;
             if (skinny || T >= PREFILL_MIN_TOKENS) {
@@ -904,7 +859,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         }
         // a mixture-of-experts layer with many tokens: its attention block on the matrix cores, experts below
         bool attn_done = false;
-        if (!L.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, skinny_min_tokens()) && s->xn16 && layer_attn_is_kquant(L) &&
+        if (!L.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, s->tune.skinny_from()) && s->xn16 && layer_attn_is_kquant(L) &&
             hp.n_embd % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0) {
             if ((rc = run_layer_prefill(s, L, il, T, max_keys, T < PREFILL_MIN_TOKENS, true)) != MESH_OK) return rc;
             attn_done = true;
@@ -921,7 +876,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         // neighbouring-pair RoPE into an f16 cache without per-head norms: rotation and KV append ride in the
         // projection's epilogue (the same arithmetic as rope_kv_kernel), one launch fewer per layer
         bool rope_fused = false;
-        if (s->rope_in_gemv && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() && !L.k_norm.present()) {
+        if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() && !L.k_norm.present()) {
             qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;
             qa.rope.kcache = reinterpret_cast<uint16_t *>(s->kcache + il * s->k_layer_bytes);
             qa.rope.vcache = reinterpret_cast<uint16_t *>(s->vcache + il * s->v_layer_bytes);
@@ -955,10 +910,10 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         aa.scale = 1.0f / sqrtf((float)hp.head_dim);
         aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
         aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-        aa.n_splits = attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16);
+        aa.n_splits = attn_splits_for(s->tune, T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16);
         {
             ProfScope ps(s, MESH_PROF_ATTN);
-            rc = T >= attn_mma_min_tokens() && attention_mma_supported(aa) ? attention_mma(aa, T, stream) : attention(aa, T, stream);
+            rc = T >= s->tune.attn_mma_min_tokens && attention_mma_supported(aa) ? attention_mma(aa, T, stream) : attention(aa, T, stream);
         }
         if (rc != MESH_OK) return rc;
 
@@ -978,7 +933,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             MoeRouteArgs mr;
             mr.logits = s->moe_logits; mr.mask = s->expert_mask_on ? s->expert_mask : nullptr;
             mr.ids = s->moe_ids; mr.weights = s->moe_w; mr.n_expert = ne; mr.top_k = k; mr.norm_w = 1;
-            const bool want_groups = s->moe_grouped && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
+            const bool want_groups = s->tune.moe_group && moe_group_supported(T * k, ne) && moe_max_items(T * k, ne) <= 65535;
             // a batch of decode steps over K-quant experts: the expert products on the matrix cores, 16 pairs of an expert per pass
             // (worth it from about four pairs per expert: below that the mat-vec kernel, which only computes the columns an
             // item has, is as fast)
@@ -987,8 +942,8 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                               moe_max_items(T * k, ne, SKINNY_ITEM_PAIRS) <= 65535;
             // a prefill chunk (from MOE_GEMM_MIN_PAIRS_PER_EXPERT pairs per expert on average): the pairs sorted by expert and
             // the expert products as tiles of the large-tile GEMM, up to 128 pairs of an expert per pass over its weights
-            const bool big = s->moe_sorted.tiles && s->moe_grouped && (size_t)T * k >= (size_t)MOE_GEMM_MIN_PAIRS_PER_EXPERT * ne &&
-                             moe_gemm_on() && E % 256 == 0 && ffe % 256 == 0;
+            const bool big = s->moe_sorted.tiles && s->tune.moe_group && (size_t)T * k >= (size_t)MOE_GEMM_MIN_PAIRS_PER_EXPERT * ne &&
+                             s->tune.moe_gemm && E % 256 == 0 && ffe % 256 == 0;
             if (big) {
                 if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
                     ProfScope ps(s, MESH_PROF_GEMV);
@@ -1011,12 +966,14 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                     if ((rc = rmsnorm_f16_k8_gather(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, s->moe_sorted.pair_of_slot, k, slots, E,
                                                     reinterpret_cast<_Float16 *>(s->moe_x16), stream, s->f16_sat)) != MESH_OK) return rc;
                 }
+                const bool d_big = s->tune.gemm_big, d_narrow = s->tune.gemm_narrow;
                 GemmArgs g;
                 g.W = L.gate_exps.data; g.Wp = L.exps_gate_up_gemm; g.type = L.gate_exps.type;
                 g.M = ffe; g.K = E; g.T = slots;
                 g.X = reinterpret_cast<const _Float16 *>(s->moe_x16); g.ldx = E; g.x_k8 = true;
                 g.y16_k8 = reinterpret_cast<_Float16 *>(s->moe_ffn16);
                 g.sat = s->f16_sat;
+                g.big_tile = d_big; g.narrow_tile = d_narrow;
                 g.tiles = s->moe_sorted.tiles; g.n_tiles = s->moe_sorted.counts; g.max_tiles = max_tiles; g.expert_stride = L.exps_gate_up_stride;
                 { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_kquant(g, stream); }
                 if (rc != MESH_OK) return rc;
@@ -1025,6 +982,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                 d.M = E; d.K = ffe; d.T = slots;
                 d.X = reinterpret_cast<const _Float16 *>(s->moe_ffn16); d.ldx = ffe; d.x_k8 = true;
                 d.Y = s->moe_out_slots; d.ldy = E;
+                d.big_tile = d_big; d.narrow_tile = d_narrow;
                 d.tiles = s->moe_sorted.tiles; d.n_tiles = s->moe_sorted.counts; d.max_tiles = max_tiles; d.expert_stride = L.exps_down_stride;
                 { ProfScope ps(s, MESH_PROF_GEMV); rc = gemm_kquant(d, stream); }
                 if (rc != MESH_OK) return rc;
@@ -1092,7 +1050,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             ea.norm_w = static_cast<const float *>(L.ffn_norm.data); ea.eps = hp.rms_eps;
             ea.epi = EPI_SWIGLU;
             ea.expert_ids = s->moe_ids; ea.n_pairs = T * k; ea.x_div = k;
-            if (grouped) { ea.items = s->moe_items; ea.n_items = s->moe_n_items; ea.max_items = moe_max_items(T * k, ne); }
+            if (grouped) { ea.grouped_oversub = s->tune.grouped_oversub; ea.items = s->moe_items; ea.n_items = s->moe_n_items; ea.max_items = moe_max_items(T * k, ne); }
             { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(ea, stream); }
             if (rc != MESH_OK) return rc;
             GemvArgs xa;
@@ -1100,7 +1058,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
             xa.mat[0] = mat_of(L.down_exps, s->moe_out, E, nullptr);
             xa.x = s->ffn; xa.ldx = ffe; xa.K = ffe; xa.T = 1;
             xa.expert_ids = s->moe_ids; xa.n_pairs = T * k; xa.x_div = 1;
-            if (grouped) { xa.items = s->moe_items; xa.n_items = s->moe_n_items; xa.max_items = ea.max_items; }
+            if (grouped) { xa.grouped_oversub = s->tune.grouped_oversub; xa.items = s->moe_items; xa.n_items = s->moe_n_items; xa.max_items = ea.max_items; }
             { ProfScope ps(s, MESH_PROF_GEMV); rc = gemv(xa, stream); }
             if (rc != MESH_OK) return rc;
             if ((rc = combine(il, k)) != MESH_OK) return rc;
@@ -1122,7 +1080,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
         // a single token: the gate / up launch leaves the FFN vector in the fixed-point form the down projection's
         // workgroups would each derive from it again (the same bits), and the down projection copies that
-        if (s->ffn_xq && s->xq_handover && gemv_xq_out_supported(ga) && gemv_xq_in_supported(da)) {
+        if (s->ffn_xq && s->tune.xq_handover && gemv_xq_out_supported(ga) && gemv_xq_in_supported(da)) {
             ga.xq_out = s->ffn_xq;
             da.xq_in = s->ffn_xq;
         }
@@ -1157,13 +1115,13 @@ static int validate_batch(const mesh_session *s, const mesh_batch *b, int *max_k
 constexpr int GRAPH_MAX_TOKENS = 32;
 constexpr size_t GRAPH_MAX_ENTRIES = 96;
 static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
-    if (!s->graphs_on || s->profile || T > GRAPH_MAX_TOKENS) return run_layers(s, T, max_keys);
+    if (!s->tune.graphs || s->graphs_failed || s->profile || T > GRAPH_MAX_TOKENS) return run_layers(s, T, max_keys);
     // A prefill chunk (consecutive positions of one sequence, enough tokens for the large-tile GEMM) runs the chunk
     // attention kernel, whose first position and sequence are launch arguments: a replay would carry the captured
     // chunk's.  Such calls are always launched eagerly.
     if (s->chunk_pos0 >= 0 && T >= PREFILL_MIN_TOKENS) return run_layers(s, T, max_keys);
     const mesh_stage *st = s->stage;
-    const int n_splits = attn_splits_for(T, (int)st->hp.n_head_kv, max_keys, st->k_type != MESH_F16);
+    const int n_splits = attn_splits_for(s->tune, T, (int)st->hp.n_head_kv, max_keys, st->k_type != MESH_F16);
     const uint64_t key = (uint64_t)T | ((uint64_t)n_splits << 8) | ((uint64_t)(s->expert_mask_on ? 1 : 0) << 20);
     auto it = s->graphs.find(key);
     if (it == s->graphs.end()) {
@@ -1175,7 +1133,7 @@ static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
         if (e.uses++ == 0) return run_layers(s, T, max_keys);
         if (hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
             (void)hipGetLastError();
-            s->graphs_on = false;
+            s->graphs_failed = true;
             return run_layers(s, T, max_keys);
         }
         const int rc = run_layers(s, T, max_keys);           // records, does not execute
@@ -1186,7 +1144,7 @@ static int run_layers_graphed(mesh_session *s, int T, int max_keys) {
         if (rc != MESH_OK || err != hipSuccess || !e.exec) {
             (void)hipGetLastError();
             e.exec = nullptr;
-            s->graphs_on = false;
+            s->graphs_failed = true;
             return rc != MESH_OK ? rc : run_layers(s, T, max_keys);      // nothing has run yet
         }
     }
@@ -1327,7 +1285,7 @@ int session_attention(mesh_session *s, int layer, const float *d_q, const mesh_b
     aa.scale = 1.0f / sqrtf((float)hp.head_dim);
     aa.n_head = (int)hp.n_head; aa.n_kv = (int)hp.n_head_kv; aa.group = (int)(hp.n_head / hp.n_head_kv);
     aa.head_dim = (int)hp.head_dim; aa.n_ctx = st->n_ctx;
-    aa.n_splits = T < 64 ? attn_splits_for(T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;
+    aa.n_splits = T < 64 ? attn_splits_for(s->tune, T, (int)hp.n_head_kv, max_keys, st->k_type != MESH_F16) : 1;
     if (matrix_cores) {
         if (!attention_mma_supported(aa)) return fail(MESH_ERR_UNSUPPORTED, "mesh_session_attn_dev: the matrix-core kernel does not cover this shape");
         return attention_mma(aa, T, s->stream);

@@ -9,6 +9,7 @@
 #include "gguf.hpp"
 #include "mesh_common.hpp"
 #include "moe.hpp"
+#include "tuning.hpp"
 
 namespace mesh {
 
@@ -70,6 +71,7 @@ struct mesh_stage {
     int k_type = MESH_F16, v_type = MESH_F16;          // KV cache row types
     int layer_begin = 0, layer_end = 0;
     int n_ctx = 0, n_seq_max = 1, n_batch_max = 0;
+    mesh::Tuning tune;            // process default, then mesh_stage_opts.tuning; fixed from here on
     std::vector<mesh::LayerWeights> layers;
     mesh::DevTensor tok_embd, output_norm, output;
     std::vector<void *> allocations;
@@ -82,9 +84,10 @@ struct mesh_stage {
 struct mesh_session {
     mesh_stage *stage = nullptr;
     hipStream_t stream = nullptr;
+    mesh::Tuning tune;            // starts as the stage's copy; mesh_session_set_option changes the session-level switches
+    bool graphs_failed = false;   // a failed capture turns graph replay off for the rest of the session
     // KV cache: per local layer, K and V as f16 [n_seq_max][n_head_kv][n_ctx][head_dim]
     uint8_t *kcache = nullptr, *vcache = nullptr;       // rows of the stage's k_type / v_type (kv_cache.hpp)
-    bool rope_in_gemv = true;        // MESH_GEMV_ROPE=0 at session creation keeps RoPE / KV append in their own kernel
     size_t k_layer_bytes = 0, v_layer_bytes = 0;
     // activations (f32), sized for n_batch_max tokens
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *ffn = nullptr;
@@ -92,8 +95,6 @@ struct mesh_session {
     unsigned *f16_sat = nullptr;                        // device counter: values the f16 producers of the batched paths clamped to +-65504
     uint32_t f16_sat_seen = 0;                          // device counter at its last read
     uint64_t f16_sat_total = 0;                         // running total the ABI reports
-    bool skinny_f16 = true;                             // MESH_SKINNY_F16=0 at session creation: batched decode on the integer matrix cores (16-bit activations)
-    bool xq_handover = true;                            // MESH_XQ_HANDOVER=0 at session creation: the down projection quantises the f32 vector itself
     float *attn_part = nullptr, *attn_ml = nullptr;     // split-KV partial outputs and (max, sum) pairs
     size_t attn_part_rows = 0;                          // (token, split) rows they hold
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
@@ -112,10 +113,6 @@ struct mesh_session {
     mesh::MoeSorted moe_sorted;
     uint16_t *moe_x16 = nullptr, *moe_ffn16 = nullptr;          // k8-major f16: normalised inputs, SwiGLU outputs
     float *moe_out_slots = nullptr;                            // down-projection rows
-    bool gemm_fused = true;          // MESH_GEMM_FUSED=0 at session creation: q / k / v and gate / up as separate prefill GEMM launches
-    bool gemm_x_k8 = true;           // MESH_GEMM_XDIRECT=0 at session creation: the prefill GEMM stages row-major activations through LDS
-    bool moe_grouped = true;         // MESH_MOE_GROUP=0 at session creation runs every pair as its own product
-    bool moe_fuse_quant = true;      // MESH_MOE_FUSE_QUANT=0 at session creation: the combine step never quantises for the next layer
     int xq_layer = -1;               // layer whose attention-norm activations the previous layer's combine step has left in xq (-1: none)
     int32_t *d_pos = nullptr, *d_seq = nullptr, *d_tok = nullptr;
     int32_t *h_meta = nullptr;      // pinned staging for pos/seq/token ids (ring of slots)
@@ -136,7 +133,6 @@ struct mesh_session {
     struct LayerGraph { hipGraphExec_t exec = nullptr; int uses = 0; };
     std::unordered_map<uint64_t, LayerGraph> graphs;
     int64_t graph_replays = 0;
-    bool graphs_on = false;          // MESH_STAGE_GRAPHS=1 at session creation turns them on; a failed capture turns them off
     std::vector<hipEvent_t> prof_events;      // pairs (begin, end)
     std::vector<int> prof_kinds;
     size_t prof_used = 0;

@@ -88,7 +88,7 @@ def test_c3_sixteen_layer_stage_decode_at_kv_depth_4095(c3_model):
     ses.close(); st.close()
 
 
-def test_c3_prefill_2048_tokens_two_layers(c3_model, monkeypatch):
+def test_c3_prefill_2048_tokens_two_layers(c3_model):
     m = mesh()
     cfg, tensors, path = c3_model
     T = 2048
@@ -103,11 +103,11 @@ def test_c3_prefill_2048_tokens_two_layers(c3_model, monkeypatch):
     report("C3 layers 3-4, prefill 2048 tokens", r)
     assert r <= NORTH_STAR
     assert max(rel_l2(got[i], ref[i]) for i in range(T)) <= NORTH_STAR
-    # launches that fill the chip with 256 x 128 tiles take the big-tile kernel; with MESH_GEMM_BIG=0 all keep the
+    # launches that fill the chip with 256 x 128 tiles take the big-tile kernel; with gemm_big=0 all keep the
     # 128 x 128 one.  Same fragments, same order along K: the same bits.
-    monkeypatch.setenv("MESH_GEMM_BIG", "0")
+    ses.set_option("gemm_big", 0)
     small = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, 4096)
-    monkeypatch.delenv("MESH_GEMM_BIG")
+    ses.set_option("gemm_big", 1)
     assert np.array_equal(got, small)
     # one decode token on top of the 2048 cached positions
     x1 = rng.standard_normal((1, 4096)).astype(np.float32)
@@ -139,7 +139,7 @@ def test_c3_prefill_256_tokens_sixteen_layers(c3_model):
     ses.close(); st.close()
 
 
-def test_c4_long_prefill_takes_the_big_tile_with_biases(tmp_path, monkeypatch):
+def test_c4_long_prefill_takes_the_big_tile_with_biases(tmp_path):
     """1664 tokens through one Qwen2.5-32B-shaped layer: every projection launch has enough 256-row tiles to fill the chip,
     so the fused q / k / v launch (three matrices, biases, 40 + 8 + 8 row blocks) and the q6_K down projection run on the
     256 x 128 tile; against the oracle, and bit for bit against the 128 x 128 kernel."""
@@ -159,9 +159,8 @@ def test_c4_long_prefill_takes_the_big_tile_with_biases(tmp_path, monkeypatch):
     r = rel_l2(got, ref)
     report("C4 layer 7, prefill 1664 tokens (big tile)", r)
     assert r <= NORTH_STAR
-    monkeypatch.setenv("MESH_GEMM_BIG", "0")
+    ses.set_option("gemm_big", 0)
     small = ses.decode(x, np.arange(T)).view(np.float32).reshape(T, E)
-    monkeypatch.delenv("MESH_GEMM_BIG")
     assert np.array_equal(got, small)
     ses.close(); st.close()
 
@@ -301,12 +300,11 @@ def test_c5_expert_shard_layer_zipf_router_on_filled_cache(tmp_path):
 
 
 @pytest.mark.parametrize("expert_gemm", ["1", "0"])
-def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, monkeypatch, expert_gemm):
+def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, expert_gemm):
     """The same shard with enough tokens per expert for the matrix cores (from four pairs per expert on average: 32
     tokens x top-8 over 64 experts): a 96-token prompt chunk of one sequence, then a decode batch of 40 sequences, Zipf
     router, against the oracle; routing decisions identical.  Once with the expert products as tiles of the large-tile
-    f16 GEMM (the default), once through the 16-pair integer kernel (MESH_MOE_GEMM=0)."""
-    monkeypatch.setenv("MESH_MOE_GEMM", expert_gemm)
+    f16 GEMM (the default), once through the 16-pair integer kernel (moe_gemm=0)."""
     m = mesh()
     cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
     path = os.path.join(str(tmp_path), "shard.gguf")
@@ -314,7 +312,7 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, monkey
     n_ctx, E = 128, 2048
     st = m.Stage(path, 5, 7, n_ctx=n_ctx, n_seq_max=40, n_batch_max=96)
     os.unlink(path)
-    ses = st.session()
+    ses = st.session(moe_gemm=int(expert_gemm))
     orc = StageOracle(cfg, tensors, 5, 7, n_ctx, n_seq_max=40)
     rng = np.random.Generator(np.random.PCG64(56))
     # prompt chunk
@@ -324,7 +322,7 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, monkey
     got = ses.decode(x, pos).view(np.float32).reshape(T, E)
     ref = orc.forward(x, pos)
     r = rel_l2(got - x, ref - x)
-    report("C5 shard layers 5-6, 96-token prefill (matrix-core expert products, MESH_MOE_GEMM=%s; of the layers' contribution)" % expert_gemm, r)
+    report("C5 shard layers 5-6, 96-token prefill (matrix-core expert products, moe_gemm=%s; of the layers' contribution)" % expert_gemm, r)
     assert r <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     # wide decode batch: sequence 0 continues its prompt, the others start
@@ -336,17 +334,17 @@ def test_c5_expert_shard_prefill_and_wide_batch_on_matrix_cores(tmp_path, monkey
     got = ses.decode(x, pos, seq=seq).view(np.float32).reshape(T, E)
     ref = orc.forward(x, pos, seq=seq)
     r = rel_l2(got - x, ref - x)
-    report("C5 shard layers 5-6, decode batch 40 (matrix-core expert products, MESH_MOE_GEMM=%s)" % expert_gemm, r)
+    report("C5 shard layers 5-6, decode batch 40 (matrix-core expert products, moe_gemm=%s)" % expert_gemm, r)
     assert r <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     ses.close(); st.close()
 
 
-def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch):
+def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path):
     """The same shard with a 272-token prompt chunk (34 pairs per expert on average; ragged: 272 = 2 * 128 + 16): the
     pairs are sorted by expert and the expert products run as tiles of the large-tile f16 GEMM.  Against the oracle, the
     routing decisions identical; then a second chunk on top; then the first chunk again through the 16-pair
-    integer matrix-core kernel (MESH_MOE_GEMM=0), which has to agree to within both paths' distance from the oracle."""
+    integer matrix-core kernel (moe_gemm=0), which has to agree to within both paths' distance from the oracle."""
     m = mesh()
     cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
     path = os.path.join(str(tmp_path), "shard.gguf")
@@ -386,10 +384,8 @@ def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch
     assert r3 <= NORTH_STAR
     assert np.array_equal(np.sort(ses.moe_last_ids(T3), axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     ses.close()
-    monkeypatch.setenv("MESH_MOE_GEMM", "0")
-    ses = st.session()
+    ses = st.session(moe_gemm=0)
     alt = ses.decode(x, pos).view(np.float32).reshape(T, E)
-    monkeypatch.delenv("MESH_MOE_GEMM")
     ra = rel_l2(alt - x, ref - x)
     report("C5 shard layers 5-6, the same 272 tokens through the 16-pair integer kernel", ra)
     assert ra <= NORTH_STAR
@@ -397,10 +393,10 @@ def test_c5_expert_shard_long_prefill_as_expert_gemm_tiles(tmp_path, monkeypatch
     ses.close(); st.close()
 
 
-def test_c5_combine_step_quantises_for_the_next_layer_bit_identically(tmp_path, monkeypatch):
+def test_c5_combine_step_quantises_for_the_next_layer_bit_identically(tmp_path):
     """Decode batch 16 over three shard layers: the combine step at the end of a mixture-of-experts layer also writes the
     quantised activations the next layer's q / k / v launch reads.  The same bits as with the two separate launches
-    (MESH_MOE_FUSE_QUANT=0), step after step."""
+    (moe_fuse_quant=0), step after step."""
     m = mesh()
     cfg = dict(models.CONFIGS["qwen3-30b-a3b"])
     path = os.path.join(str(tmp_path), "shard.gguf")
@@ -412,14 +408,12 @@ def test_c5_combine_step_quantises_for_the_next_layer_bit_identically(tmp_path, 
     xs = [models.zipf_hidden_state(rng, 16, E) for _ in range(3)]
     outs = []
     for fuse in ("1", "0"):
-        monkeypatch.setenv("MESH_MOE_FUSE_QUANT", fuse)
-        ses = st.session()
+        ses = st.session(moe_fuse_quant=int(fuse))
         got = []
         for step, x in enumerate(xs):
             got.append(ses.decode(x, np.full(16, step, np.int32), seq=np.arange(16, dtype=np.int32)).view(np.uint32).copy())
         outs.append(got)
         ses.close()
-    monkeypatch.delenv("MESH_MOE_FUSE_QUANT")
     for a, b in zip(*outs):
         assert np.array_equal(a, b)
     st.close()

@@ -116,7 +116,7 @@ def test_stage_with_quantised_kv_matches_oracle(tmp_path, name, kv_types):
 
 
 @pytest.mark.parametrize("kv_types", PAIRS)
-def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types, monkeypatch):
+def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types):
     """Two real-shape layers over a 300-deep quantised cache: split-KV decode at batch 1 and 4, the batched (skinny
     GEMM) path at batch 9, and a 200-token prefill chunk through the matrix-core attention kernel."""
     name = "llama3-8b"
@@ -192,9 +192,7 @@ def test_llama3_8b_shaped_layers_quantised_kv_all_paths(tmp_path, kv_types, monk
     ses.close()
     # the same two chunks with the scratch switched off (every query tile decodes the rows itself): the same values
     # reach the matrix cores in the same order, so the hidden states are bit-identical
-    monkeypatch.setenv("MESH_CHUNK_KV16", "0")
-    ses = st.session()
-    monkeypatch.delenv("MESH_CHUNK_KV16")
+    ses = st.session(chunk_kv16=0)
     got_b = ses.decode(xp, np.arange(T), seq=np.full(T, 9, np.int32)).view(np.float32).reshape(T, 4096)
     got2_b = ses.decode(xp2, np.arange(T, T + T2), seq=np.full(T2, 9, np.int32)).view(np.float32).reshape(T2, 4096)
     assert np.array_equal(got_b.view(np.uint32), got.view(np.uint32))

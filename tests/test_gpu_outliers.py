@@ -50,14 +50,12 @@ def _stage(tmp_path, scale_ffn_norm=None, n_seq=24, n_batch=208):
 
 
 @pytest.mark.parametrize("skinny", ["f16", "integer"])
-def test_outlier_channels_through_every_projection_path(tmp_path, monkeypatch, skinny):
+def test_outlier_channels_through_every_projection_path(tmp_path, skinny):
     """Batches of 5..16 tokens once on the f16 matrix cores (the default: f16 activations, one rounding per weight) and once
-    on the integer ones (16-bit fixed-point activations, MESH_SKINNY_F16=0 at session creation)."""
+    on the integer ones (16-bit fixed-point activations, the session switch skinny_f16=0)."""
     m, cfg, tensors, st = _stage(tmp_path)
     E = cfg["n_embd"]
-    monkeypatch.setenv("MESH_SKINNY_F16", "1" if skinny == "f16" else "0")
-    ses = st.session()
-    monkeypatch.delenv("MESH_SKINNY_F16")
+    ses = st.session(skinny_f16=int(skinny == "f16"))
     orc = StageOracle(cfg, tensors, 3, 5, 256, n_seq_max=24, blas=True)
     rng = np.random.Generator(np.random.PCG64(50))
     nxt = {}
@@ -104,11 +102,7 @@ def test_swiglu_products_beyond_the_f16_range(tmp_path):
 
     # integer paths (the single-token mat-vec, and the 16-bit fixed-point matrix-core kernel for small batches): exact
     # arithmetic range, same tolerance as ever, and nothing counted as saturated
-    os.environ["MESH_SKINNY_F16"] = "0"
-    try:
-        ses_int = st.session()
-    finally:
-        del os.environ["MESH_SKINNY_F16"]
+    ses_int = st.session(skinny_f16=0)
     for T in (1, 8):
         got, r = run(ses_int, T, 0, 0)
         print("[outliers] SwiGLU beyond f16, decode %d (integer kernels): rel-L2 %.3e" % (T, r))

@@ -245,9 +245,9 @@ def test_moe_stage_matches_oracle_with_and_without_mask(tmp_path):
     ses.close(); ses2.close(); st.close()
 
 
-def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path, monkeypatch):
+def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path):
     """The expert launches walk (token, slot) pairs grouped by expert, up to four pairs of an expert per pass over its
-    weights (mat-vec kernel, fewer than 5 tokens) or up to sixteen (matrix-core kernel); MESH_MOE_GROUP=0 runs every pair
+    weights (mat-vec kernel, fewer than 5 tokens) or up to sixteen (matrix-core kernel); the switch moe_group=0 runs every pair
     as its own product.  A column's arithmetic does not depend on its neighbours, so the mat-vec groups give the same
     bits as pair-by-pair, whatever the group sizes (8 experts, top-2: 1 to 30 tokens make groups of every size and
     experts with more than one group)."""
@@ -255,9 +255,7 @@ def test_moe_pairs_grouped_by_expert_equal_pair_by_pair(tmp_path, monkeypatch):
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(77))
     ses = st.session()
-    monkeypatch.setenv("MESH_MOE_GROUP", "0")
-    ses0 = st.session()
-    monkeypatch.delenv("MESH_MOE_GROUP")
+    ses0 = st.session(moe_group=0)
     orc = StageOracle(cfg, tensors, 0, 2, 64)
     pos0 = 0
     for T in (1, 2, 4, 3, 5, 23, 26):           # the bit-exact cases first: afterwards the two caches differ in the last bits
@@ -321,14 +319,14 @@ def test_prefill_gemm_token_counts_and_head_layouts(tmp_path, name, T):
 
 
 @pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-llama", [0, 1])])
-def test_prefill_gemm_variants_agree(tmp_path, monkeypatch, name, layers):
+def test_prefill_gemm_variants_agree(tmp_path, name, layers):
     """Stages that can take prefill-sized calls keep a second copy of their projections arranged for the GEMM's
-    staging threads, with the per-sub-block f16 scale products precomputed; MESH_GEMM_LAYOUT=0 makes the GEMM read the
+    staging threads, with the per-sub-block f16 scale products precomputed; the stage switch gemm_layout=0 makes the GEMM read the
     mat-vec tiles instead.  Same arithmetic on the same values: bit-identical outputs (q4_K and q6_K matrices, row
     counts that are and are not multiples of the 128-row tile), both when the matrix-core waves take their activation
     fragments straight from the k8-major layout and when row-major activations are staged through LDS
-    (MESH_GEMM_XDIRECT=0).  Across producers of the f16 activations -- the two activation layouts, or the SwiGLU
-    epilogue of the fused gate / up launch against the separate kernel (MESH_GEMM_FUSED=0) -- the f32 expressions are
+    (gemm_xdirect=0).  Across producers of the f16 activations -- the two activation layouts, or the SwiGLU
+    epilogue of the fused gate / up launch against the separate kernel (gemm_fused=0) -- the f32 expressions are
     the same but compiled in different kernels, so a few values differ by an f16 rounding step: those agree to 1e-3."""
     m = mesh()
     cfg = models.CONFIGS[name]
@@ -336,29 +334,23 @@ def test_prefill_gemm_variants_agree(tmp_path, monkeypatch, name, layers):
     models.write_model(path, cfg, layers, seed=5)
     lb, le = layers[0], layers[-1] + 1
     st1 = m.Stage(path, lb, le, n_ctx=256, n_seq_max=1, n_batch_max=208)
-    monkeypatch.setenv("MESH_GEMM_LAYOUT", "0")
-    st0 = m.Stage(path, lb, le, n_ctx=256, n_seq_max=1, n_batch_max=208)
-    monkeypatch.delenv("MESH_GEMM_LAYOUT")
+    st0 = m.Stage(path, lb, le, n_ctx=256, n_seq_max=1, n_batch_max=208, tuning={"gemm_layout": 0})
     os.unlink(path)
     E = cfg["n_embd"]
     T = 200
     x = np.random.Generator(np.random.PCG64(3)).standard_normal((T, E)).astype(np.float32)
 
-    def run(st, **env):
-        for k, v in env.items():
-            monkeypatch.setenv(k, v)
-        ses = st.session()
-        for k in env:
-            monkeypatch.delenv(k)
+    def run(st, **options):
+        ses = st.session(**options)
         out = ses.decode(x, np.arange(T)).view(np.uint32)
         ses.close()
         return out
 
     fused = run(st1)
-    split = run(st1, MESH_GEMM_FUSED="0")
+    split = run(st1, gemm_fused=0)
     assert np.array_equal(split, run(st0))
-    staged = run(st1, MESH_GEMM_FUSED="0", MESH_GEMM_XDIRECT="0")
-    assert np.array_equal(staged, run(st0, MESH_GEMM_XDIRECT="0"))
+    staged = run(st1, gemm_fused=0, gemm_xdirect=0)
+    assert np.array_equal(staged, run(st0, gemm_xdirect=0))
     f = lambda a: a.view(np.float32)
     assert rel_l2(f(fused), f(split)) <= 1e-3
     assert rel_l2(f(staged), f(split)) <= 1e-3
@@ -431,7 +423,7 @@ def test_long_chunk_with_an_odd_number_of_head_rows(tmp_path):
     ses.close(); st.close()
 
 
-def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path, monkeypatch):
+def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path):
     """A chunk with few query tiles and a long history splits every tile's walk over several workgroups and merges the
     partials (the split-KV combine kernel): 96 tokens on top of 448 (two splits), then 48 on top of 2000 (eight splits;
     the last split holds the diagonal, where the chunk's earlier queries see no key at all).  Against the oracle, and
@@ -445,11 +437,9 @@ def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path, monkeypa
     xs = [rng.standard_normal((T, E)).astype(np.float32) for T, _ in calls]
     outs = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("MESH_ATTN_CHUNK_KSPLIT", mode)
-        ses = st.session()
+        ses = st.session(attn_chunk_ksplit=int(mode))
         outs[mode] = [ses.decode(x, np.arange(p0, p0 + T)).view(np.float32).reshape(T, E).copy() for x, (T, p0) in zip(xs, calls)]
         ses.close()
-    monkeypatch.delenv("MESH_ATTN_CHUNK_KSPLIT")
     for x, (T, p0), got, alt in zip(xs, calls, outs["1"], outs["0"]):
         ref = orc.forward(x, np.arange(p0, p0 + T))
         assert rel_l2(got, ref) <= 3e-3, (T, p0)
@@ -458,7 +448,7 @@ def test_short_chunks_on_a_long_history_split_their_key_walks(tmp_path, monkeypa
     st.close()
 
 
-def test_key_split_boundary_inside_a_query_tile(tmp_path, monkeypatch):
+def test_key_split_boundary_inside_a_query_tile(tmp_path):
     """Chunks whose first position is not a multiple of 32: a key split then begins strictly inside a query tile's
     position range, so that in the split's first step the tile's earlier queries still see no key while the later ones
     do.  40 tokens on top of 3560 (eight splits of 512 keys; the last begins at key 3584, inside positions 3560..3591)
@@ -480,13 +470,11 @@ def test_key_split_boundary_inside_a_query_tile(tmp_path, monkeypatch):
     xs = [rng.standard_normal((T, E)).astype(np.float32) for T, _, _ in calls]
     outs = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("MESH_ATTN_CHUNK_KSPLIT", mode)
-        ses = st.session()
+        ses = st.session(attn_chunk_ksplit=int(mode))
         for s, (k, v) in kv.items():
             ses.kv_write(0, s, 0, k, v)
         outs[mode] = [ses.decode(x, np.arange(p0, p0 + T), seq=[s] * T).view(np.float32).reshape(T, E).copy() for x, (T, p0, s) in zip(xs, calls)]
         ses.close()
-    monkeypatch.delenv("MESH_ATTN_CHUNK_KSPLIT")
     for x, (T, p0, s), got, alt in zip(xs, calls, outs["1"], outs["0"]):
         assert np.isfinite(got).all(), (T, p0)
         ref = orc.forward(x, np.arange(p0, p0 + T), seq=[s] * T)
@@ -548,18 +536,16 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
     ses.close(); ses4.close(); st.close()
 
 
-def test_wide_decode_batch_takes_large_tile_gemm(tmp_path, monkeypatch):
+def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
     """From 17 tokens a call takes the large-tile MFMA GEMM whatever its shape: here 70 single-token sequences at ragged
     positions (not a prefill chunk, so the split-KV decode attention runs behind the GEMM's q/k/v).  One token block
     and 32..224 row blocks per projection: the launches split K over workgroups and add the slices in a second
     kernel.  Real-shape layers, against the oracle, against the same tokens fed 16 at a time (skinny GEMM) and against
-    the unsplit launches (MESH_GEMM_SPLITK=0: same products, another summation order)."""
+    the unsplit launches (gemm_splitk=0: same products, another summation order)."""
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=64, n_seq=70, n_batch=70)
     ses, ses16 = st.session(), st.session()
-    monkeypatch.setenv("MESH_GEMM_SPLITK", "0")
-    ses_whole = st.session()
-    monkeypatch.delenv("MESH_GEMM_SPLITK")
+    ses_whole = st.session(gemm_splitk=0)
     orc = StageOracle(cfg, tensors, 3, 5, 64, n_seq_max=70)
     rng = np.random.Generator(np.random.PCG64(21))
     depth = [int(d) for d in rng.integers(1, 40, size=70)]
@@ -589,9 +575,9 @@ def test_wide_decode_batch_takes_large_tile_gemm(tmp_path, monkeypatch):
     ses.close(); ses16.close(); ses_whole.close(); st.close()
 
 
-def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
+def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path):
     """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
-    1-3 tokens (mat-vec kernels) and of 4+ tokens (batched MFMA GEMM); with MESH_GEMV_ROPE=0 the separate kernel does
+    1-3 tokens (mat-vec kernels) and of 4+ tokens (batched MFMA GEMM); with gemv_rope=0 the separate kernel does
     them.  Outputs and cache contents must agree bit for bit (the arithmetic is the same), through the single-type
     and the mixed q4_K/q6_K launches."""
     for name, layers in (("llama3-8b", [3, 4]), ("tiny-llama", [0, 1])):
@@ -601,8 +587,7 @@ def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
         xs = [rng.standard_normal((T, E)).astype(np.float32) for T in (1, 2, 3, 4, 1, 6, 9, 5)]
         runs = []
         for flag in ("1", "0"):
-            monkeypatch.setenv("MESH_GEMV_ROPE", flag)
-            ses = st.session()
+            ses = st.session(gemv_rope=int(flag))
             outs, nxt = [], [0] * 9
             for x in xs:
                 T = x.shape[0]
@@ -622,7 +607,7 @@ def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path, monkeypatch):
         st.close()
 
 
-def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path, monkeypatch):
+def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path):
     """At one token per call the gate / up launch leaves the FFN vector in the 16-bit fixed-point form the down projection
     consumes (whole 32-element blocks per workgroup), and the down projection copies it instead of quantising the f32
     vector in every workgroup.  The same arithmetic on the same values: bit-identical outputs with the hand-over switched
@@ -635,11 +620,9 @@ def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path,
         xs = [rng.standard_normal((1, E)).astype(np.float32) * (50.0 if i == 2 else 1.0) for i in range(4)]
         runs = []
         for flag in ("1", "0"):
-            monkeypatch.setenv("MESH_XQ_HANDOVER", flag)
-            ses = st.session()
+            ses = st.session(xq_handover=int(flag))
             runs.append([ses.decode(x, [i]).copy() for i, x in enumerate(xs)])
             ses.close()
-        monkeypatch.delenv("MESH_XQ_HANDOVER")
         for a, b in zip(*runs):
             assert np.isfinite(a.view(np.float32)).all()
             assert np.array_equal(a, b)
@@ -647,7 +630,7 @@ def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path,
 
 
 @pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-moe", [0, 1])])
-def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers):
+def test_graph_replays_equal_eager_launches(tmp_path, name, layers):
     """Decode-sized batches replay their layer launches from a captured graph (first use of a shape eager, second
     captured, then replays).  Every replay must give the bits the eager launches give: two sessions, graphs on and
     off, walk the same sequence of steps -- repeated shapes, other shapes and host synchronisations in between, KV
@@ -661,8 +644,7 @@ def test_graph_replays_equal_eager_launches(tmp_path, monkeypatch, name, layers)
     chunk_xs = [rng.standard_normal((25, E)).astype(np.float32) for _ in range(8)]
     runs = []
     for flag in ("1", "0"):
-        monkeypatch.setenv("MESH_STAGE_GRAPHS", flag)
-        ses = st.session()
+        ses = st.session(graphs=int(flag))
         nxt = [0] * 20
         outs = []
         for x in xs:
