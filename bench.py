@@ -45,17 +45,41 @@ def codec_input(T, h=4096):
     return x
 
 
-def profiled_ratio(fname, key):
-    """The number on the line `<key> = <number>` of profiles/<fname> (HBM traffic measured with rocprofv3 counters, as
-    a multiple of the algorithmic bytes); None when the file or the line is not there."""
+def kernel_sources_digest(files):
+    """sha256 over the named files of mesh-llm_amd/csrc (the sources of one kernel family), first 16 hex digits."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, "mesh-llm_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+GEMV_SOURCES = ("gemv.hip", "gemv_body.inc", "gemv_device.hpp", "gemv.hpp")
+CODEC_SOURCES = ("codec.hip",)
+
+
+def profiled_ratio(fname, key, sources):
+    """(ratio, note): the number on the line `<key> = <number>` of profiles/<fname> (HBM traffic measured with rocprofv3
+    counters, as a multiple of the algorithmic bytes).  The profile names the digest of the kernel sources it was taken
+    with (`sources_sha256 = ...`); when the sources have changed since, the ratio describes another kernel and is not
+    used: (None, "stale ...").  (None, "absent") when the file or the line is not there."""
+    ratio = digest = None
     try:
         with open(os.path.join(ROOT, "profiles", fname)) as f:
             for line in f:
                 if line.startswith(key + " ="):
-                    return float(line.split("=", 1)[1].split()[0])
+                    ratio = float(line.split("=", 1)[1].split()[0])
+                if line.startswith("sources_sha256 ="):
+                    digest = line.split("=", 1)[1].split()[0]
     except (OSError, ValueError):
-        pass
-    return None
+        return None, "absent"
+    if ratio is None:
+        return None, "absent"
+    now = kernel_sources_digest(sources)
+    if digest != now:
+        return None, "stale: profiles/%s was taken with kernel sources %s, the tree holds %s" % (fname, digest, now)
+    return ratio, "profiles/" + fname
 
 
 def time_on_stream(torch, stream, fn, steps, warmup):
@@ -151,7 +175,7 @@ def bench_codec(args):
     m.lib()
     res = run_codec(torch, m, args.steps, args.warmup)
     gbs, ms = res["pack_q8_0"]["GBps"], res["pack_q8_0"]["ms"]
-    codec_ratio = profiled_ratio(CODEC_TRAFFIC_PROFILE, "pack_q8_0_traffic_over_algorithmic")
+    codec_ratio, codec_src = profiled_ratio(CODEC_TRAFFIC_PROFILE, "pack_q8_0_traffic_over_algorithmic", CODEC_SOURCES)
     out = {
         "metric": "activation pack GB/s (q8_0, [4096,4096] f32)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -160,7 +184,7 @@ def bench_codec(args):
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": int(round(codec_ratio * 4096 * 4096 * Q8_BPE)) if codec_ratio else None,
-                     "traffic_source": "profiles/" + CODEC_TRAFFIC_PROFILE if codec_ratio else None,
+                     "traffic_source": codec_src,
                      "plain_stream_GBps": res["pack_q8_0"]["plain_stream_GBps"], "frac_of_plain_stream": res["pack_q8_0"]["frac_of_plain_stream"],
                      "measured_stream_read_GBps": hbm_probe(m)},
         "codec": res,
@@ -357,7 +381,7 @@ def bench_stage(args):
     g_ms = b1["kernel_ms_per_step"]["gemv"]
     g_n = b1["kernel_launches_per_step"]["gemv"]
     gemv_gbs = weight_bytes / g_ms / 1e6
-    traffic_ratio = profiled_ratio(TRAFFIC_PROFILE, "gemv_batch1_traffic_over_algorithmic")
+    traffic_ratio, traffic_src = profiled_ratio(TRAFFIC_PROFILE, "gemv_batch1_traffic_over_algorithmic", GEMV_SOURCES)
     codec = run_codec(torch, m, max(10, args.steps // 2), args.warmup)
     probe = hbm_probe(m)
     vendor_matvec = vendor_f16_matvec(torch, cfg)
@@ -373,7 +397,7 @@ def bench_stage(args):
                      # HBM bytes per average launch: the ratio of counted (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated
                      # on a copy of known size) to algorithmic bytes recorded in the committed profile summary
                      "traffic": int(round(traffic_ratio * weight_bytes / g_n)) if traffic_ratio else None,
-                     "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic_ratio else None, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
+                     "traffic_source": traffic_src, "launches_per_step": g_n, "avg_launch_us": round(g_ms / g_n * 1e3, 2),
                      "algorithmic_bytes_per_launch": weight_bytes // g_n,
                      "measured_stream_read_GBps": probe, "frac_of_measured_p90": round(gemv_gbs / probe["p90"], 4),
                      "vendor_f16_matvec_same_shapes": vendor_matvec},
@@ -392,7 +416,8 @@ def bench_stage(args):
 
 # ------------------------------------------------------------------------------------------------ other shapes
 SHAPES = {
-    "c4": dict(model="qwen2.5-32b", layers=32, n_ctx=8192, batches=[1, 8, 32], prefill=4096, n_expert_local=None, kv="q8_0/q4_0",
+    # (the reference's table quotes this shape on an f16 cache and its launcher picks q8_0 / q4_0 for a 32B model: both are measured)
+    "c4": dict(model="qwen2.5-32b", layers=32, n_ctx=8192, batches=[1, 8, 32], prefill=4096, n_expert_local=None, kv="q8_0/q4_0", also_kv="f16",
                metric="stage decode tok/s @32B Q4_K_M, layers 0-31 of 64"),
     "c5": dict(model="qwen3-30b-a3b", layers=48, n_ctx=4096, batches=[16], prefill=1024, n_expert_local=64, kv="q8_0/q4_0", router="zipf",
                metric="expert-shard decode tok/s @Qwen3-30B-A3B Q4_K_M, 64 of 128 experts, batch 16"),
@@ -522,6 +547,15 @@ def bench_shape(args):
            "setup_s": {"generate_gguf": round(t_gen, 1), "open_stage": round(t_load, 1), "fill_kv": round(t_kv, 1)}}
     ses.close()
     st.close()
+    del ses, st
+    if sp.get("also_kv") and not args.kv_given:
+        # the same decode batches once more on the other cache type (a stage of its own: the cache rows are fixed at open)
+        import copy
+        a2 = copy.copy(args)
+        a2.kv, a2.kv_given, a2.prefill = sp["also_kv"], True, False
+        torch.cuda.empty_cache()
+        second = bench_shape(a2)
+        out["decode_%s_kv" % sp["also_kv"].replace("/", "_")] = {"kv_bytes_per_seq": second["config"]["kv_bytes_per_seq"], **second["decode"]}
     return out
 
 

@@ -60,7 +60,16 @@ struct SkinnyKernelArgs {
     int ks;                       // waves along K
     GemvRope rope;                // rope.pos / rope.seq point at the launch's first column
     int kind[3];
+    // RMS-norm hand-over (gemm.hpp: SkinnyF16Args::NormOut / NormIn)
+    const float *no_w;            // producer: weight of the norm that follows
+    _Float16 *no_x16;
+    float *no_part;
+    const float *ni_part;         // consumer: [ni_parts][16] partial sums of squares
+    int ni_parts;
+    float ni_eps;
 };
+constexpr int SK_NORM_GROUPS = SK_THREADS / SK_NT;      // threads sharing a token column in the epilogue
+constexpr int SK_NORM_SHARE = SKINNY_F16_NORM_PARTS_MAX / SK_NORM_GROUPS;      // partial sums a thread fetches
 
 // four bytes (values < 64) -> four f16 holding 1024 + value
 __device__ __forceinline__ void bytes_to_h1024(uint32_t v, h2_t &lo, h2_t &hi) {
@@ -199,6 +208,9 @@ __device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_la
     R.d = lane_gather(R.d, src_lane4);
 }
 
+// most tile-rows a workgroup of the launch has (p_split = tile-rows per workgroup | workgroups with one more << 16)
+__device__ __forceinline__ int rows_here_max(unsigned p_split) { return (int)(p_split & 0xFFFFu) + ((p_split >> 16) ? 1 : 0); }
+
 template <int TYPE, int NU, int SEGS>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
                                                                  int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
@@ -269,6 +281,23 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
         B[0].load(p_x, lane_off, ks);
         B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
+    }
+    // norm hand-over, consumer side: this thread's share of the partial sums of squares of its epilogue column.  Issued
+    // behind the first weight tiles (loads return in order: waiting for a tile never waits for these) and not touched
+    // before the weight stream is through.  Branch-free: a share past the end re-reads the last one and is not added.
+    // (and unconditional: without a hand-over they read the start of the activations, so that no load sits under a
+    // branch and the compiler's count of loads in flight stays exact)
+    float ni_v[SK_NORM_SHARE];
+    {
+        const float *np = a.ni_part ? a.ni_part : reinterpret_cast<const float *>(p_x);
+        const int np_n = a.ni_part ? a.ni_parts : 1;
+#pragma unroll
+        for (int q = 0; q < SK_NORM_SHARE; ++q) {
+            const int p = tid / SK_NT + q * SK_NORM_GROUPS;
+            ni_v[q] = np[(size_t)(p < np_n ? p : np_n - 1) * SK_NT + tid % SK_NT];
+        }
+    }
+    if (total > 0) {
         if (n_i <= 2 && total <= SK_DEPTH) {
             // short walk: everything it needs is already in flight
 #pragma unroll
@@ -302,7 +331,23 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
             for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + 4 * g + i) * 16 + m] = D[seg][i];
         }
     }
+    // (after the reduction buffer: [SK_NORM_GROUPS][16] sums of the consumer side, [SK_WAVES][16] of the producer side)
+    float *nrm = red + (size_t)KS * rows_here_max(p_split) * NU * 16 * SK_NT;
+    if (a.ni_part) {
+        float ni_sum = 0.f;
+#pragma unroll
+        for (int q = 0; q < SK_NORM_SHARE; ++q) ni_sum += tid / SK_NT + q * SK_NORM_GROUPS < a.ni_parts ? ni_v[q] : 0.f;
+        nrm[tid] = ni_sum;                             // tid = group * 16 + column
+    }
     __syncthreads();
+    // 1 / rms of this thread's column (every output of a thread is of column tid % 16): groups added in order
+    float inv_rms = 1.0f;
+    if (a.ni_part) {
+        float ss = 0.f;
+        for (int q = 0; q < SK_NORM_GROUPS; ++q) ss += nrm[q * SK_NT + tid % SK_NT];
+        inv_rms = 1.0f / sqrtf(ss / (float)K + a.ni_eps);
+    }
+    float no_ss = 0.f;         // producer side: sum of squares of this thread's outputs (one column)
     // outputs of this workgroup: rows_here x 16 rows x T columns
     for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
@@ -313,6 +358,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         if (row >= a.M[mi]) continue;
         if (t >= a.T) {                                    // unused columns of the f16 output block stay finite
             if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
+            if (a.no_x16) a.no_x16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
             continue;
         }
         float s0 = 0.f, s1 = 0.f;
@@ -320,6 +366,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
             s0 += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + r) * 16 + t];
             if (NU == 2) s1 += red[((((size_t)k2 * rows_here + j) * NU + 1) * 16 + r) * 16 + t];
         }
+        s0 *= inv_rms;
+        if (NU == 2) s1 *= inv_rms;
         if (a.bias[mi]) s0 += a.bias[mi][row];
         if (NU == 1 && a.rope.pos && a.kind[mi] != GEMV_KIND_PLAIN) {
             // q / k / v row of a token (see gemv.hpp): rotate q and k with the neighbouring row, k and v go to the cache
@@ -330,6 +378,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
             if (kind != GEMV_KIND_V && dd < a.rope.n_rot) {
                 float sp = 0.f;
                 for (int k2 = 0; k2 < KS; ++k2) sp += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + (r ^ 1)) * 16 + t];
+                sp *= inv_rms;
                 if (a.bias[mi]) sp += a.bias[mi][row ^ 1];
                 float sn, cs;
                 sincosf((float)pos * a.rope.inv_freq[dd >> 1], &sn, &cs);
@@ -357,6 +406,25 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         if (a.y16 && mi == 0) {
             note_f16_clamp(a.sat, out, 0.f);
             a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)__builtin_amdgcn_fmed3f(out, -65504.f, 65504.f);
+        }
+        if (a.no_x16) {
+            const float v = out * a.no_w[row];
+            note_f16_clamp(a.sat, v, 0.f);
+            a.no_x16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)__builtin_amdgcn_fmed3f(v, -65504.f, 65504.f);
+            no_ss = fmaf(out, out, no_ss);
+        }
+    }
+    if (a.no_part) {
+        // this workgroup's sum of squares per column: the four lanes of a wave that share a column, then the waves in order
+        no_ss += __shfl_xor(no_ss, 16);
+        no_ss += __shfl_xor(no_ss, 32);
+        float *wsum = nrm + SK_NORM_GROUPS * SK_NT;
+        if (lane < SK_NT) wsum[wave * SK_NT + lane] = no_ss;
+        __syncthreads();
+        if (tid < SK_NT) {
+            float ss = 0.f;
+            for (int w = 0; w < SK_WAVES; ++w) ss += wsum[w * SK_NT + tid];
+            a.no_part[(size_t)blockIdx.x * SK_NT + tid] = ss;
         }
     }
 }
@@ -394,6 +462,22 @@ static int skinny_n_cu() {
     return n;
 }
 
+// waves along K: a power of two (the kernel splits its waves with shifts)
+static int skinny_ks(int nsb) {
+    int KS = 1;
+    while (KS * 2 <= nsb && KS * 2 <= SK_WAVES) KS *= 2;
+    return KS;
+}
+// workgroups of a launch over total_rows tile-rows: spread over the CUs, bounded by the segments a wave can hold
+static int skinny_grid(int total_rows, int NU, int KS) {
+    const int RS = SK_WAVES / KS;
+    const int rows_cap = std::max(1, SK_SEGS_MAX / NU) * RS;
+    const int ncu = skinny_n_cu();
+    int rows_per_wg = std::min((total_rows + ncu - 1) / ncu, rows_cap);
+    rows_per_wg = std::max(1, rows_per_wg);
+    return (total_rows + rows_per_wg - 1) / rows_per_wg;
+}
+
 // all matrices of `a` are tiled K-quants of one type
 static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
     const int type = a.mat[0].type;
@@ -419,21 +503,17 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
     ka.rope = a.rope;
     ka.M16 = a.mat[0].M;
     ka.sat = a.sat;
-    int KS = 1;
-    while (KS * 2 <= nsb && KS * 2 <= SK_WAVES) KS *= 2;      // a power of two: the kernel splits its waves with shifts
+    ka.no_w = a.norm_out.norm_w; ka.no_x16 = a.norm_out.x16; ka.no_part = a.norm_out.part;
+    ka.ni_part = a.norm_in.part; ka.ni_parts = a.norm_in.n_parts; ka.ni_eps = a.norm_in.eps;
+    const int KS = skinny_ks(nsb);
     const int RS = SK_WAVES / KS;
     ka.ks = KS;
-    // tile-rows per workgroup: spread over the CUs, bounded by the segments a wave can hold
-    const int rows_cap = std::max(1, SK_SEGS_MAX / NU) * RS;
-    const int ncu = skinny_n_cu();
-    int rows_per_wg = std::min((total_rows + ncu - 1) / ncu, rows_cap);
-    rows_per_wg = std::max(1, rows_per_wg);
-    const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
+    const int grid = skinny_grid(total_rows, NU, KS);
     const int rows_max = (total_rows + grid - 1) / grid;
     const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
     if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", segs);
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d tile-rows in one launch", total_rows);
-    const size_t smem = sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
+    const size_t smem = sizeof(float) * ((size_t)KS * rows_max * NU * 16 * SK_NT + (size_t)(SK_NORM_GROUPS + SK_WAVES) * SK_NT);
     if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: reduction buffer of %zu bytes does not fit LDS", smem);
     for (int t = 0; t < a.T; t += SK_NT) {
         SkinnyKernelArgs kb = ka;
@@ -454,8 +534,21 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
 
 }  // namespace f16sk
 
+int gemm_skinny_f16_workgroups(const SkinnyF16Args &a) {
+    using namespace f16sk;
+    if (a.n_mat != 1 || a.K <= 0 || a.K % QK_K || a.mat[0].M <= 0) return 0;
+    return skinny_grid((a.mat[0].M + TILE_ROWS - 1) / TILE_ROWS, 1, skinny_ks(a.K / QK_K));
+}
+
 int gemm_skinny_f16(const SkinnyF16Args &a, hipStream_t stream) {
     using namespace f16sk;
+    if (a.norm_out.x16 || a.norm_out.part || a.norm_out.norm_w) {
+        if (!a.norm_out.x16 || !a.norm_out.part || !a.norm_out.norm_w || a.n_mat != 1 || a.epi != EPI_RESIDUAL || a.T > SK_NT || a.mat[0].M % 8 ||
+            gemm_skinny_f16_workgroups(a) > SKINNY_F16_NORM_PARTS_MAX)
+            return fail(MESH_ERR_INVALID, "gemm_skinny_f16: the norm hand-over needs one matrix with a residual epilogue, at most 16 tokens and a row count that is a multiple of 8");
+    }
+    if (a.norm_in.part && (a.norm_in.n_parts < 1 || a.norm_in.n_parts > SKINNY_F16_NORM_PARTS_MAX || a.T > SK_NT))
+        return fail(MESH_ERR_INVALID, "gemm_skinny_f16: bad norm hand-over input (%d partial sums, %d tokens)", a.norm_in.n_parts, a.T);
     if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.T <= 0 || a.K <= 0) return fail(MESH_ERR_INVALID, "gemm_skinny_f16: bad arguments");
     if (a.K % QK_K || (reinterpret_cast<uintptr_t>(a.x) & 15))
         return fail(MESH_ERR_INVALID, "gemm_skinny_f16: K %d must be a multiple of 256 and the activations 16-byte aligned", a.K);

@@ -416,6 +416,11 @@ int session_new(mesh_stage *st, mesh_session **out) {
             MESH_HIP_TRY(hipMemsetAsync(p, 0, bytes, s->stream));
         }
         if (hp.n_ff > 0) {
+            // (one block of 16 tokens: the hand-over is for calls the skinny GEMM takes)
+            if ((rc = sess_alloc(s.get(), &p, 16 * (size_t)hp.n_embd * 2)) != MESH_OK) return rc;
+            s->norm16 = static_cast<uint16_t *>(p);
+            MESH_HIP_TRY(hipMemsetAsync(p, 0, 16 * (size_t)hp.n_embd * 2, s->stream));
+            if ((rc = fbuf(&s->norm_part, (size_t)SKINNY_F16_NORM_PARTS_MAX * 16)) != MESH_OK) return rc;
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
             if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
@@ -586,7 +591,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim), FF = (int)hp.n_ff;
     _Float16 *xn = reinterpret_cast<_Float16 *>(s->xn16), *f16ffn = reinterpret_cast<_Float16 *>(s->ffn16);
     int rc;
-    bool rope_fused = false, attn_is_k8 = false;
+    bool rope_fused = false, attn_is_k8 = false, ffn_norm_fused = false;
     const bool k8 = skinny || s->tune.gemm_xdirect;      // activations in the k8-major layout (both GEMMs can read it)
     // the batched-decode GEMM on the f16 matrix cores (k8-major f16 activations) instead of the integer ones (q16 activations);
     // a mixture-of-experts stage keeps the integer kernel, whose activation layout its expert launches share
@@ -601,9 +606,17 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         r.head_dim = (int)hp.head_dim; r.n_rot = (int)hp.n_rot; r.n_kv = (int)hp.n_head_kv; r.n_ctx = st->n_ctx;
         return r;
     };
+    // f16 skinny GEMM, at most 16 tokens: the two RMS norms of the layer ride in the launches around them.  The output
+    // projection and the down projection also write their result times the next norm's weight as f16 (norm16) and the sums
+    // of squares their workgroups saw; q/k/v and gate/up read that and divide their products by the token's rms.
+    const bool nf = sk16 && T <= 16 && s->tune.skinny_norm_fused && s->norm16 && s->norm_part && E % 8 == 0;
+    _Float16 *const nx = reinterpret_cast<_Float16 *>(s->norm16);
+    const bool norm_ready = nf && s->norm_layer == (int)il;
+    s->norm_layer = -1;
     {
         ProfScope ps(s, MESH_PROF_PREP);
-        if (sk8 && s->xq_layer == (int)il) rc = MESH_OK;     // the previous layer's combine step has left them in s->xq
+        if (norm_ready) rc = MESH_OK;                        // the previous layer's down projection has left them in norm16
+        else if (sk8 && s->xq_layer == (int)il) rc = MESH_OK;     // the previous layer's combine step has left them in s->xq
         else if (sk8) rc = quant16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, s->xq, stream);
         else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, stream, s->f16_sat);
         else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.attn_norm.data), hp.rms_eps, T, E, xn, E, stream, s->f16_sat);
@@ -616,6 +629,10 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = xn; qa.K = E; qa.T = T;
+        if (norm_ready) {
+            qa.x = nx;
+            qa.norm_in.part = s->norm_part; qa.norm_in.n_parts = s->norm_parts; qa.norm_in.eps = hp.rms_eps;
+        }
         if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
             !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
             qa.rope = rope_of();
@@ -732,6 +749,12 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         oa.mat[0] = mat_of(L.wo, s->x, E, nullptr);
         oa.x = xn; oa.K = QD; oa.T = T;
         oa.residual = s->x; oa.ldres = E; oa.epi = EPI_RESIDUAL;
+        oa.sat = s->f16_sat;
+        ffn_norm_fused = nf && !attn_only && gemm_skinny_f16_workgroups(oa) >= 1 && gemm_skinny_f16_workgroups(oa) <= SKINNY_F16_NORM_PARTS_MAX;
+        if (ffn_norm_fused) {
+            oa.norm_out.norm_w = static_cast<const float *>(L.ffn_norm.data); oa.norm_out.x16 = nx; oa.norm_out.part = s->norm_part;
+            s->norm_parts = gemm_skinny_f16_workgroups(oa);
+        }
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny_f16(oa, stream)) != MESH_OK) return rc;
     } else if (skinny) {
@@ -751,7 +774,8 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
     if (attn_only) return MESH_OK;
     {
         ProfScope ps(s, MESH_PROF_PREP);
-        if (sk8) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
+        if (ffn_norm_fused) rc = MESH_OK;
+        else if (sk8) rc = quant16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, s->xq, stream);
         else if (k8) rc = rmsnorm_f16_k8(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, stream, s->f16_sat);
         else rc = rmsnorm_f16(s->x, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps, T, E, xn, E, stream, s->f16_sat);
     }
@@ -765,14 +789,28 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         ga.x = xn; ga.K = E; ga.T = T; ga.epi = EPI_SWIGLU;
         ga.y16 = f16ffn;
         ga.sat = s->f16_sat;
+        if (ffn_norm_fused) {
+            ga.x = nx;
+            ga.norm_in.part = s->norm_part; ga.norm_in.n_parts = s->norm_parts; ga.norm_in.eps = hp.rms_eps;
+        }
         SkinnyF16Args da;
         da.n_mat = 1;
         da.mat[0] = mat_of(L.w_down, s->x, E, nullptr);
         da.x = f16ffn; da.K = FF; da.T = T;
         da.residual = s->x; da.ldres = E; da.epi = EPI_RESIDUAL;
+        da.sat = s->f16_sat;
+        // the next layer's attention norm, when that layer takes this path too
+        const LayerWeights *Ln = il + 1 < st->layers.size() ? &st->layers[il + 1] : nullptr;
+        const bool next_fused = nf && Ln && layer_is_kquant_dense(*Ln) && Ln->w_gate.type == Ln->w_up.type &&
+                                gemm_skinny_f16_workgroups(da) >= 1 && gemm_skinny_f16_workgroups(da) <= SKINNY_F16_NORM_PARTS_MAX;
         ProfScope ps(s, MESH_PROF_GEMV);
         if ((rc = gemm_skinny_f16(ga, stream)) != MESH_OK) return rc;
-        return gemm_skinny_f16(da, stream);
+        if (next_fused) {
+            da.norm_out.norm_w = static_cast<const float *>(Ln->attn_norm.data); da.norm_out.x16 = nx; da.norm_out.part = s->norm_part;
+        }
+        if ((rc = gemm_skinny_f16(da, stream)) != MESH_OK) return rc;
+        if (next_fused) { s->norm_parts = gemm_skinny_f16_workgroups(da); s->norm_layer = (int)il + 1; }
+        return MESH_OK;
     }
     if (skinny) {
         // gate and up in one pass with the SwiGLU epilogue; its f32 output is quantised for the down projection
@@ -831,6 +869,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     const int E = (int)hp.n_embd, QD = (int)(hp.n_head * hp.head_dim), KD = (int)(hp.n_head_kv * hp.head_dim);
     int rc;
     s->xq_layer = -1;
+    s->norm_layer = -1;
     // a mixture-of-experts layer whose attention block runs on the batched-decode (integer matrix-core) path
     auto moe_attn_skinny = [&](const LayerWeights &Ln) {
         return !Ln.w_gate.present() && T >= std::min(PREFILL_MIN_TOKENS, s->tune.skinny_from()) && T < PREFILL_MIN_TOKENS && s->xn16 && layer_attn_is_kquant(Ln) &&

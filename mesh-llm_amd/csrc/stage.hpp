@@ -99,6 +99,12 @@ struct mesh_session {
     size_t attn_part_rows = 0;                          // (token, split) rows they hold
     // prefill path (many tokens per call): f16 copies of the GEMM inputs and a second FFN buffer
     uint16_t *xn16 = nullptr, *ffn16 = nullptr;
+    // f16 skinny GEMM with the RMS norms handed over between launches (gemm.hpp: SkinnyF16Args::NormOut): the next norm's
+    // input as its producer wrote it, the producer's partial sums of squares, and whose input that is
+    uint16_t *norm16 = nullptr;
+    float *norm_part = nullptr;
+    int norm_parts = 0;              // partial sums per token the last producer wrote
+    int norm_layer = -1;             // layer whose attention norm norm16 / norm_part hold (-1: none)
     uint16_t *chunk_kv16 = nullptr;      // quantised KV caches: f16 rows of one sequence and layer for long prefill chunks (attn.hpp)
     size_t xq_tokens = 0;               // tokens the q16 buffer below is sized for
     uint8_t *xq = nullptr;               // 16-bit fixed-point activations of the skinny GEMM (gemm.hpp: q16 layout)

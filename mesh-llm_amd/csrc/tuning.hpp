@@ -24,6 +24,7 @@ struct Tuning {
     int gemv_rope = 1;             // RoPE and the KV append in the q/k/v projection's epilogue (0: their own kernel)
     int xq_handover = 1;           // the gate/up mat-vec leaves the FFN vector quantised for the down projection
     int skinny_f16 = 1;            // calls of skinny_min_tokens..gemm_min_tokens-1 tokens on the f16 matrix cores (0: integer, 16-bit activations)
+    int skinny_norm_fused = 1;     // f16 skinny GEMM: the RMS norms ride in the launches around them (0: a norm launch of their own)
     int gemm_fused = 1;            // q/k/v and gate/up of a prefill call as one GEMM launch each
     int gemm_xdirect = 1;          // the prefill GEMM reads k8-major activations directly (0: row-major staged through LDS)
     int gemm_big = 1;              // the 256-row tile for wide projections of long calls

@@ -575,6 +575,40 @@ def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
     ses.close(); ses16.close(); ses_whole.close(); st.close()
 
 
+def test_skinny_gemm_norms_ride_in_the_neighbouring_launches(tmp_path):
+    """Batches of 4 to 16 tokens on the f16 skinny GEMM: the output projection and the down projection also write their
+    result times the next RMS norm's weight as f16 plus per-workgroup sums of squares, and q/k/v and gate/up divide their
+    products by the token's rms -- W . (y w / rms) = (W . (y w)) / rms -- instead of a norm launch in between
+    (skinny_norm_fused=0).  Three real-shape layers (the middle one with q6_K attn_v / ffn_down), with a x40 outlier
+    channel in one step so that the unnormalised f16 values are large: both ways against the oracle and against each
+    other; the rounding points differ (f16 of y w against f16 of y w / rms), nothing else."""
+    m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [2, 3, 4], 2, 5, n_ctx=64, n_seq=16, n_batch=16)
+    E = cfg["n_embd"]
+    fused, plain = st.session(), st.session(skinny_norm_fused=0)
+    assert fused.get_option("skinny_norm_fused") == 1
+    orc = StageOracle(cfg, tensors, 2, 5, 64, n_seq_max=16)
+    rng = np.random.Generator(np.random.PCG64(91))
+    nxt = [0] * 16
+    for step, T in enumerate((16, 5, 9, 16, 4, 13)):
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        if step == 2:
+            x[:, 1234] *= 40.0
+        seqs = list(range(T))
+        pos = [nxt[q] for q in seqs]
+        for q in seqs:
+            nxt[q] += 1
+        a = fused.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        b = plain.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos, seq=seqs)
+        ra, rb, rab = rel_l2(a, ref), rel_l2(b, ref), rel_l2(a, b)
+        print("[skinny norms] step %d, %d tokens: fused %.3e, separate %.3e of the oracle, %.3e apart" % (step, T, ra, rb, rab))
+        assert np.isfinite(a).all()
+        assert ra <= 3e-3 and rb <= 3e-3 and rab <= 3e-3, (step, T)
+        assert max(rel_l2(a[i], ref[i]) for i in range(T)) <= 1e-2
+    assert fused.f16_saturations() == 0
+    fused.close(); plain.close(); st.close()
+
+
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path):
     """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
     1-3 tokens (mat-vec kernels) and of 4+ tokens (batched MFMA GEMM); with gemv_rope=0 the separate kernel does
