@@ -69,7 +69,6 @@ struct SkinnyKernelArgs {
     float ni_eps;
 };
 constexpr int SK_NORM_GROUPS = SK_THREADS / SK_NT;      // threads sharing a token column in the epilogue
-constexpr int SK_NORM_SHARE = SKINNY_F16_NORM_PARTS_MAX / SK_NORM_GROUPS;      // partial sums a thread fetches
 
 // four bytes (values < 64) -> four f16 holding 1024 + value
 __device__ __forceinline__ void bytes_to_h1024(uint32_t v, h2_t &lo, h2_t &hi) {
@@ -281,23 +280,6 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
         B[0].load(p_x, lane_off, ks);
         B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
-    }
-    // norm hand-over, consumer side: this thread's share of the partial sums of squares of its epilogue column.  Issued
-    // behind the first weight tiles (loads return in order: waiting for a tile never waits for these) and not touched
-    // before the weight stream is through.  Branch-free: a share past the end re-reads the last one and is not added.
-    // (and unconditional: without a hand-over they read the start of the activations, so that no load sits under a
-    // branch and the compiler's count of loads in flight stays exact)
-    float ni_v[SK_NORM_SHARE];
-    {
-        const float *np = a.ni_part ? a.ni_part : reinterpret_cast<const float *>(p_x);
-        const int np_n = a.ni_part ? a.ni_parts : 1;
-#pragma unroll
-        for (int q = 0; q < SK_NORM_SHARE; ++q) {
-            const int p = tid / SK_NT + q * SK_NORM_GROUPS;
-            ni_v[q] = np[(size_t)(p < np_n ? p : np_n - 1) * SK_NT + tid % SK_NT];
-        }
-    }
-    if (total > 0) {
         if (n_i <= 2 && total <= SK_DEPTH) {
             // short walk: everything it needs is already in flight
 #pragma unroll
@@ -334,9 +316,10 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     // (after the reduction buffer: [SK_NORM_GROUPS][16] sums of the consumer side, [SK_WAVES][16] of the producer side)
     float *nrm = red + (size_t)KS * rows_here_max(p_split) * NU * 16 * SK_NT;
     if (a.ni_part) {
+        // norm hand-over, consumer side: this thread's share of the partial sums of squares of its epilogue column
+        // (fetched after the weight stream: before it, the wave would wait for them ahead of its first tile loads)
         float ni_sum = 0.f;
-#pragma unroll
-        for (int q = 0; q < SK_NORM_SHARE; ++q) ni_sum += tid / SK_NT + q * SK_NORM_GROUPS < a.ni_parts ? ni_v[q] : 0.f;
+        for (int p = tid / SK_NT; p < a.ni_parts; p += SK_NORM_GROUPS) ni_sum += a.ni_part[(size_t)p * SK_NT + tid % SK_NT];
         nrm[tid] = ni_sum;                             // tid = group * 16 + column
     }
     __syncthreads();
