@@ -275,6 +275,7 @@ int mesh_session_f16_saturations(mesh_session *session, uint64_t *count);
  *     attn_mma_min_tokens=1  decode attention on the matrix cores from this many tokens
  *     attn_split_target=0  workgroups a decode attention launch aims at (0 = 256, or 512 for quantised rows)
  *     moe_group=1          (token, slot) pairs grouped by expert
+ *     moe_router_tail=1    small decode batches: the router launch's last workgroup routes and groups the pairs
  *     moe_fuse_quant=1     the expert combine step quantises for the next layer
  *     moe_gemm=1, moe_gemm_min_pairs=4   prefill-sized expert products on the large-tile GEMM
  *     grouped_oversub=8    grouped expert mat-vec: workgroups per compute unit and item

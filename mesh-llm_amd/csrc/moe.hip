@@ -133,13 +133,11 @@ constexpr int ROUTER_THREADS = 1024, ROUTER_WAVES = ROUTER_THREADS / 64;
 // (RT: threads of the workgroup.  A decode batch has few tokens and wants every wave it can get on a token's expert rows;
 // a prefill chunk has a workgroup per token anyway, and small workgroups, eight to a CU, hide each other's row loads.)
 constexpr int ROUTER_THREADS_WIDE = 256, ROUTER_WIDE_MIN_TOKENS = 512;
-template <int NV, int RT = ROUTER_THREADS>      // float4 groups per lane = E / 256
-// (scalar arguments first: preloaded into SGPRs, see gemv.hip)
-__global__ __launch_bounds__(RT) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
-                                                                          const float *__restrict__ W, float *__restrict__ logits_out,
-                                                                          int ldx, float eps, int p_n_expert, const MoeRouteArgs a) {
+// the logits of this workgroup's token and expert slice (blockIdx.y of gridDim.y), into s_logits and logits_out
+template <int NV, int RT>      // float4 groups per lane = E / 256
+__device__ __forceinline__ void router_logits(const float *__restrict__ x, const float *__restrict__ norm_w, const float *__restrict__ W,
+                                              float *__restrict__ logits_out, int ldx, float eps, int p_n_expert, float *s_logits) {
     constexpr int E = NV * 256, ROUTER_WAVES = RT / 64;
-    __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // element index of a lane's values: 4 * (lane + 64 * i) + c
     const float *xt = x + (size_t)t * ldx;
@@ -189,9 +187,18 @@ __global__ __launch_bounds__(RT) void moe_router_fused_kernel(const float *__res
             }
         }
     }
+}
+
+template <int NV, int RT = ROUTER_THREADS>
+// (scalar arguments first: preloaded into SGPRs, see gemv.hip)
+__global__ __launch_bounds__(RT) void moe_router_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+                                                                          const float *__restrict__ W, float *__restrict__ logits_out,
+                                                                          int ldx, float eps, int p_n_expert, const MoeRouteArgs a) {
+    __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
+    router_logits<NV, RT>(x, norm_w, W, logits_out, ldx, eps, p_n_expert, s_logits);
     if (gridDim.y > 1) return;
     __syncthreads();
-    if (wave == 0) route_wave_any(s_logits, a, t, lane);
+    if ((threadIdx.x >> 6) == 0) route_wave_any(s_logits, a, blockIdx.x, threadIdx.x & 63);
 }
 
 // The same for a prefill chunk, four tokens per workgroup of eight waves: every wave keeps the four normalised hidden
@@ -393,14 +400,68 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(const fl
     group_pairs(p_ids, T * p_top_k, p_n_expert, items, n_items, g_lds, ipairs);
 }
 
+// The two launches above as one: every workgroup computes its slice of the logits; the one that arrives last (a device-wide
+// counter, release fence before the increment, acquire fence after it) then routes all tokens and groups the pairs, as
+// moe_route_group_kernel does.  The counter is back at zero when the launch ends.  No workgroup waits for another.
+template <int NV>
+__global__ __launch_bounds__(GROUP_THREADS) void moe_router_group_fused_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+                                                                               const float *__restrict__ W, float *logits, int ldx, float eps,
+                                                                               int p_n_expert, const MoeRouteArgs a, int T, int32_t *items, int32_t *n_items,
+                                                                               int ipairs, int *arrive) {
+    static_assert(GROUP_THREADS == ROUTER_THREADS, "the routing tail runs in a router workgroup");
+    extern __shared__ int32_t g_lds[];
+    __shared__ float s_logits[64 * ROUTE_MAX_PER_LANE];
+    __shared__ int s_last;
+    router_logits<NV, ROUTER_THREADS>(x, norm_w, W, logits, ldx, eps, p_n_expert, s_logits);
+    // One release per workgroup, by one thread: the barrier orders the other waves' logits stores before it, and a
+    // release at device scope covers what the releasing thread has observed.  (A __threadfence() in every wave measured
+    // 35 us for this tail: sixteen cache write-backs and invalidations per workgroup.)
+    __syncthreads();
+    if (threadIdx.x == 0)
+        s_last = __hip_atomic_fetch_add(arrive, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == (int)(gridDim.x * gridDim.y) - 1;
+    __syncthreads();
+    if (!s_last) return;
+    if (threadIdx.x == 0) __hip_atomic_store(arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int t = wave; t < T; t += GROUP_WAVES) {
+        // the token's logits through LDS: route_wave reads plain floats
+        float *row = reinterpret_cast<float *>(g_lds) + (size_t)wave * 64 * ROUTE_MAX_PER_LANE;
+        // (device-scope loads: written by other workgroups of this launch, possibly on another die)
+        for (int e = lane; e < p_n_expert; e += 64) row[e] = __hip_atomic_load(logits + (size_t)t * p_n_expert + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        route_wave_any(row, a, t, lane);
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    group_pairs(a.ids, T * a.top_k, p_n_expert, items, n_items, g_lds, ipairs);
+}
+
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
-                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream) {
+                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream, int *arrive) {
     if (T <= 0) return MESH_OK;
     if (!moe_router_group_supported(E, a.n_expert, a.top_k, T) || !logits)
         return fail(MESH_ERR_UNSUPPORTED, "moe: split router for hidden size %d / %d experts / %d tokens", E, a.n_expert, T);
     const int split = (a.n_expert + ROUTER_WAVES - 1) / ROUTER_WAVES;      // one expert row per wave
     const dim3 grid((unsigned)T, (unsigned)split), block(ROUTER_THREADS);
     MoeRouteArgs la = a;
+    if (arrive) {
+        // one launch: the last workgroup to finish its logits routes and groups
+        la.logits = logits;
+        // LDS of the tail: a logits row per wave while routing, then the grouping's pair list and counters
+        const size_t smem = std::max((size_t)GROUP_WAVES * 64 * ROUTE_MAX_PER_LANE * sizeof(float),
+                                     ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t));
+        switch (E / 256) {
+            case 2: MESH_LAUNCH(moe_router_group_fused_kernel<2>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
+            case 4: MESH_LAUNCH(moe_router_group_fused_kernel<4>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
+            case 8: MESH_LAUNCH(moe_router_group_fused_kernel<8>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
+            case 16: MESH_LAUNCH(moe_router_group_fused_kernel<16>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
+            default: return fail(MESH_ERR_UNSUPPORTED, "moe: fused router for hidden size %d", E);
+        }
+        MESH_LAUNCH_CHECK();
+        return MESH_OK;
+    }
     switch (E / 256) {
         case 2: MESH_LAUNCH(moe_router_fused_kernel<2>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;
         case 4: MESH_LAUNCH(moe_router_fused_kernel<4>, grid, block, 0, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la); break;

@@ -31,8 +31,10 @@ int moe_group(const int32_t *ids, int n_pairs, int n_expert, int32_t *items, int
 // grouping in one single-workgroup launch.  Same results as moe_router_fused followed by moe_group; `logits`
 // ([T][n_expert]) is required.
 bool moe_router_group_supported(int E, int n_expert, int top_k, int T);
+// arrive (optional): a device int that is zero between launches; with it the two launches become one, whose last-arriving
+// workgroup routes and groups (same results)
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
-                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream);
+                     float *logits, int T, int32_t *items, int32_t *n_items, int item_pairs, hipStream_t stream, int *arrive = nullptr);
 // x[t] += sum_s weights[t][s] * y[t*top_k + s]
 int moe_combine(float *x, const float *y, const float *w, int T, int n_embd, int top_k, hipStream_t stream);
 

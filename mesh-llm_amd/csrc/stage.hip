@@ -442,10 +442,12 @@ int session_new(mesh_stage *st, mesh_session **out) {
         // work items: 4 pairs each for the mat-vec kernel, 16 for the matrix-core one; the buffer fits either
         const size_t items = (size_t)std::max(moe_max_items((int)(B * k), (int)ne) * MOE_ITEM_INTS,
                                               moe_max_items((int)(B * k), (int)ne, SKINNY_ITEM_PAIRS) * moe_item_ints(SKINNY_ITEM_PAIRS)) / MOE_ITEM_INTS + 1;
-        if ((rc = sess_alloc(s.get(), &p, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t))) != MESH_OK) return rc;
+        // (+ the item count, + the arrival counter of the router launch whose last workgroup routes and groups)
+        if ((rc = sess_alloc(s.get(), &p, (items * MOE_ITEM_INTS + 2) * sizeof(int32_t))) != MESH_OK) return rc;
         s->moe_items = static_cast<int32_t *>(p);
         s->moe_n_items = s->moe_items + items * MOE_ITEM_INTS;
-        MESH_HIP_TRY(hipMemsetAsync(s->moe_items, 0, (items * MOE_ITEM_INTS + 1) * sizeof(int32_t), s->stream));
+        s->moe_arrive = reinterpret_cast<int *>(s->moe_n_items + 1);
+        MESH_HIP_TRY(hipMemsetAsync(s->moe_items, 0, (items * MOE_ITEM_INTS + 2) * sizeof(int32_t), s->stream));
         MESH_HIP_TRY(hipMemsetAsync(s->expert_mask, 0, ne * sizeof(float), s->stream));
         if (st->layers[0].exps_gate_up_gemm && s->xn16 && B * k >= MOE_GEMM_MIN_PAIRS_PER_EXPERT * ne) {
             // prefill chunks: the pairs sorted by expert, their inputs / SwiGLU outputs in the k8-major f16 layout and their
@@ -1035,7 +1037,7 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
                 ProfScope ps(s, MESH_PROF_GEMV);
                 if ((rc = moe_router_group(mr, s->x, E, static_cast<const float *>(L.ffn_norm.data), hp.rms_eps,
                                            static_cast<const float *>(L.gate_inp.data), E, s->moe_logits, T, s->moe_items, s->moe_n_items,
-                                           item_pairs, stream)) != MESH_OK) return rc;
+                                           item_pairs, stream, s->tune.moe_router_tail ? s->moe_arrive : nullptr)) != MESH_OK) return rc;
                 grouped_done = true;
             } else if (L.gate_inp.type == MESH_F32 && moe_router_fused_supported(E, ne, k)) {
                 // the router matrix is small and f32: logits and routing in one launch

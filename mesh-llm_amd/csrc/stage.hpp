@@ -115,6 +115,7 @@ struct mesh_session {
     bool expert_mask_on = false;
     int32_t *moe_ids = nullptr;
     int32_t *moe_items = nullptr, *moe_n_items = nullptr;      // (token, slot) pairs grouped by expert, see moe_group
+    int *moe_arrive = nullptr;                                 // arrival counter of the fused router launch (zero between launches)
     // prefill chunks: the pairs sorted by expert (moe_sort) and their buffers, rows indexed by slot
     mesh::MoeSorted moe_sorted;
     uint16_t *moe_x16 = nullptr, *moe_ffn16 = nullptr;          // k8-major f16: normalised inputs, SwiGLU outputs

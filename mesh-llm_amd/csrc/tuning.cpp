@@ -29,6 +29,7 @@ const TuningField *tuning_fields() {
         {"attn_mma_min_tokens", &Tuning::attn_mma_min_tokens, 1, 1 << 20, TUNE_SESSION},
         {"attn_split_target", &Tuning::attn_split_target, 0, 1 << 16, TUNE_SESSION},
         {"moe_group", &Tuning::moe_group, 0, 1, TUNE_SESSION},
+        {"moe_router_tail", &Tuning::moe_router_tail, 0, 1, TUNE_SESSION},
         {"moe_fuse_quant", &Tuning::moe_fuse_quant, 0, 1, TUNE_SESSION},
         {"moe_gemm", &Tuning::moe_gemm, 0, 1, TUNE_SESSION},
         {"moe_gemm_min_pairs", &Tuning::moe_gemm_min_pairs, 1, 1 << 20, TUNE_SESSION},

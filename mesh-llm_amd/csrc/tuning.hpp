@@ -33,6 +33,7 @@ struct Tuning {
     int attn_mma_min_tokens = 1;   // decode attention on the matrix cores from this many tokens (below: the all-f32 kernel)
     int attn_split_target = 0;     // workgroups a decode attention launch aims at; 0 = 256, 512 for quantised rows of 64+ (token, head) pairs
     int moe_group = 1;             // (token, slot) pairs grouped by expert (0: every pair its own product)
+    int moe_router_tail = 1;       // small decode batches: the router launch's last workgroup routes and groups (0: a second launch)
     int moe_fuse_quant = 1;        // the expert combine step quantises for the next layer's projections
     int moe_gemm = 1;              // prefill-sized expert products as tiles of the large-tile GEMM
     int moe_gemm_min_pairs = 4;    // ... from this many pairs per expert on average

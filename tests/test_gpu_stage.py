@@ -295,7 +295,23 @@ def test_qwen3_30b_a3b_shaped_expert_shard_layer(tmp_path):
     ids = ses.moe_last_ids(16)
     assert np.array_equal(np.sort(ids, axis=1), np.sort(np.stack(orc.last_expert_ids), axis=1))
     assert len(set(ids.reshape(-1))) > 8
-    ses.close(); st.close()
+    ses.close()
+    # the router launch's last-arriving workgroup routes and groups the pairs (the default), or a second launch does
+    # (moe_router_tail=0): the same bits and the same routing, step after step (the arrival counter returns to zero)
+    runs = []
+    for tail in (1, 0):
+        q = st.session(moe_router_tail=tail)
+        r2 = np.random.Generator(np.random.PCG64(32))
+        outs = []
+        for step, T in enumerate((16, 11, 6, 16, 1, 16)):
+            xs = r2.standard_normal((T, 2048)).astype(np.float32)
+            outs.append((q.decode(xs, np.full(T, step, np.int32), seq=np.arange(T, dtype=np.int32)).copy(), q.moe_last_ids(T).copy()))
+        runs.append(outs)
+        q.close()
+    for (a, ia), (b, ib) in zip(*runs):
+        assert np.array_equal(ia, ib)
+        assert np.array_equal(a, b)
+    st.close()
 
 
 @pytest.mark.parametrize("name,T", [("tiny-llama", 192), ("tiny-llama", 257), ("tiny-qwen2", 256), ("tiny-qwen3", 300), ("tiny-g7", 193)])
