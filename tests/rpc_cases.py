@@ -42,6 +42,9 @@ def direct_push(binary):
         assert cb.get_tensor(tb, 0, size) == src
         # partial
         cb.set_tensor(tb, 0, bytes(size))
+        # SET_TENSOR has no reply and the push reaches B on another connection: a command with a reply on this
+        # connection first, so that the zeroing has been processed before the push can arrive
+        assert cb.get_tensor(tb, 0, 16) == bytes(16)
         assert ca.push_tensor_to_peer(1, ta, tb, 1024, 2048) == 1
         got = cb.get_tensor(tb, 0, size)
         assert got[:1024] == bytes(1024) and got[1024:3072] == src[1024:3072] and got[3072:] == bytes(1024)
