@@ -425,7 +425,7 @@ SHAPES = {
 
 
 def bench_shape(args):
-    """The larger BASELINE shapes at full size on one GPU: same timing as the default workload, fewer extras."""
+    """The larger configurations (32B dense stage, 64-expert shard) at full size on one GPU: same timing as the default workload, fewer extras."""
     import torch
     import __graft_entry__ as graft
     import models
