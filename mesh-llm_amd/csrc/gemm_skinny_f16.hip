@@ -31,7 +31,7 @@ namespace f16sk {
 
 constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
-constexpr int SK_DEPTH_Q4 = 4;            // weight tiles a wave keeps in flight (2304 B each)
+constexpr int SK_DEPTH_Q4 = 2;            // weight tiles a wave keeps in flight (2304 B each; four measured 2% slower: 250+ registers)
 constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B and their fragments need more registers
 constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA N)
 constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
