@@ -64,6 +64,30 @@ def test_bad_tuning_text_is_refused_before_any_device_call(tmp_path, text, fragm
     assert "mesh_stage_opts.tuning" in e.value.message and fragment in e.value.message, e.value.message
 
 
+def test_environment_string_is_read_once_per_process_and_checked(tmp_path):
+    """MESH_TUNING holds the same text as mesh_stage_opts.tuning; a bad one makes mesh_stage_open fail with a message that
+    names the variable (a process of its own: the library reads it once)."""
+    import subprocess
+    import sys
+    cfg = models.CONFIGS["tiny-llama"]
+    path = os.path.join(str(tmp_path), "t.gguf")
+    models.write_model(path, cfg, [0], seed=1)
+    prog = ("import sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+            "from util import mesh\n"
+            "m = mesh()\n"
+            "try:\n"
+            "    m.Stage(%r, 0, 1, n_ctx=32)\n"
+            "    print('opened')\n"
+            "except m.MeshError as e:\n"
+            "    print(e.code, e.message)\n") % (ROOT, os.path.join(ROOT, "tests"), path)
+    for text, expect in (("skinny_f16=3", "MESH_TUNING: tuning: skinny_f16=3 outside [0, 1]"), ("nonsense", "MESH_TUNING: 'nonsense' is not name=integer")):
+        out = subprocess.run([sys.executable, "-c", prog], env=dict(os.environ, MESH_TUNING=text), capture_output=True, text=True, timeout=120).stdout
+        assert out.startswith("-1 ") and expect in out, out
+    # a good one gets past the parser: what stops the call on a machine without a GPU is the device, not the text
+    out = subprocess.run([sys.executable, "-c", prog], env=dict(os.environ, MESH_TUNING=" graphs=1 , skinny_f16=0 "), capture_output=True, text=True, timeout=120).stdout
+    assert "MESH_TUNING" not in out, out
+
+
 @pytest.mark.gpu
 def test_session_options_round_trip_and_levels(tmp_path):
     m = mesh()
