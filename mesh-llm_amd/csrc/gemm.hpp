@@ -127,10 +127,10 @@ struct SkinnyF16Args {
     // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
-    // RMS-norm hand-over between two launches (T <= 16), in place of a norm kernel of its own between them.  The producer
+    // RMS-norm hand-over between two launches (T <= 32: one launch each), in place of a norm kernel of its own between them.  The producer
     // (EPI_RESIDUAL, one matrix) also writes f16(y * norm_w) -- scaled by the next norm's weight but not yet by the
     // token's 1 / rms -- in the k8-major layout to norm_out.x16, and per workgroup the sum of y^2 of its rows for every
-    // token to norm_out.part ([workgroups][16]); *norm_out.n_parts_host receives the workgroup count.  The consumer reads
+    // token to norm_out.part ([workgroups][16], or [workgroups][32] for a call of more than 16 tokens); gemm_skinny_f16_workgroups gives the workgroup count.  The consumer reads
     // those activations as its x, adds the partial sums in workgroup order and multiplies every accumulated product by
     // 1 / sqrt(sum / K + eps) before bias and epilogue: W . (y w / rms) = (W . (y w)) / rms.
     struct NormOut { const float *norm_w = nullptr; _Float16 *x16 = nullptr; float *part = nullptr; } norm_out;
@@ -140,6 +140,7 @@ int gemm_skinny_f16(const SkinnyF16Args &a, hipStream_t stream);
 // workgroups a producer launch of `a` will have (= partial sums per token it writes); 0 when the launch is not valid
 int gemm_skinny_f16_workgroups(const SkinnyF16Args &a);
 constexpr int SKINNY_F16_NORM_PARTS_MAX = 256;
+constexpr int SKINNY_F16_NORM_TOKENS_MAX = 32;
 
 // y (k8-major) = f16(rms_norm(x) * w) for T rows of n floats; pack_f16_k8: plain conversion
 // (sat: optional device counter of values clamped to the f16 range, in all of these)

@@ -1,4 +1,4 @@
-// Skinny GEMM for batched decode on the f16 matrix cores: Y[T][M] = W[M][K] . X[T][K] with 5 <= T <= 16 tokens per
+// Skinny GEMM for batched decode on the f16 matrix cores: Y[T][M] = W[M][K] . X[T][K] with up to 16 or up to 32 tokens per
 // pass, W a tiled q4_K / q6_K matrix, X in f16 (the k8-major layout of gemm.hpp).
 //
 // The alternative to the integer kernel of gemm_skinny.hip for the same launches: the weight stream is organised as in
@@ -33,7 +33,7 @@ constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
 constexpr int SK_DEPTH_Q4 = 2;            // weight tiles a wave keeps in flight (2304 B each; four measured 2% slower: 250+ registers)
 constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B and their fragments need more registers
-constexpr int SK_NT = 16;                 // activation columns per launch (one MFMA N)
+constexpr int SK_NT = 16;                 // activation columns of one MFMA (a launch takes one or two such blocks)
 constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
 constexpr size_t SK_LDS_LIMIT = 160 * 1024;
 
@@ -68,7 +68,6 @@ struct SkinnyKernelArgs {
     int ni_parts;
     float ni_eps;
 };
-constexpr int SK_NORM_GROUPS = SK_THREADS / SK_NT;      // threads sharing a token column in the epilogue
 
 // four bytes (values < 64) -> four f16 holding 1024 + value
 __device__ __forceinline__ void bytes_to_h1024(uint32_t v, h2_t &lo, h2_t &hi) {
@@ -207,10 +206,14 @@ __device__ __forceinline__ void to_mfma_lanes(TileRegs<MESH_Q6_K> &R, int src_la
     R.d = lane_gather(R.d, src_lane4);
 }
 
+// element (row k, column t) of k8-major f16 activations with K rows per column: block t / 16 of 16 * K halfs
+__device__ __forceinline__ size_t k8_at(int K, int k, int t) { return (size_t)(t >> 4) * 16 * K + ((size_t)(k >> 3) * 16 + (t & 15)) * 8 + (k & 7); }
+
 // most tile-rows a workgroup of the launch has (p_split = tile-rows per workgroup | workgroups with one more << 16)
 __device__ __forceinline__ int rows_here_max(unsigned p_split) { return (int)(p_split & 0xFFFFu) + ((p_split >> 16) ? 1 : 0); }
 
-template <int TYPE, int NU, int SEGS>
+// NC: blocks of 16 activation columns one pass over the weights multiplies with (1: up to 16 tokens, 2: up to 32).
+template <int TYPE, int NU, int SEGS, int NC>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
                                                                  int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
                                                                  const SkinnyKernelArgs a) {
@@ -252,11 +255,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
     // segment has nothing at all
     const int total = seg_valid(0) ? n_i * SEGS : 0;
 
+    constexpr int NT = SK_NT * NC;                        // activation columns of this launch
     TileRegs<TYPE> ring[SK_DEPTH];
-    BFrags<TYPE> B[2];
-    f4_t D[SEGS];
+    f4_t D[SEGS][NC];
 #pragma unroll
-    for (int s = 0; s < SEGS; ++s) D[s] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < SEGS; ++s)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) D[s][c] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     // Loads are never under a branch of their own: an index past the end or an invalid segment is clamped to a tile
     // the wave owns (a cache hit).  The compiler then knows exactly how many loads are in flight at every point
@@ -266,40 +271,98 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         const bool ok = f < total && seg_valid(seg);
         dst.load(tile_ptr(ok ? f / SEGS : n_i - 1, ok ? seg : 0), lane);
     };
-    auto compute = [&](const TileRegs<TYPE> &loaded, const BFrags<TYPE> &bf, f4_t &acc) {
-        TileRegs<TYPE> tile = loaded;
-        to_mfma_lanes(tile, src_lane4);
-        TileFrags<TYPE> F;
-        F.prepare(tile, g);
+    if constexpr (NC == 1) {
+        // one column block: the activation fragments of two super-blocks in registers, a whole super-block ahead
+        BFrags<TYPE> B[2];
+        auto compute = [&](const TileRegs<TYPE> &loaded, const BFrags<TYPE> &bf, f4_t &acc) {
+            TileRegs<TYPE> tile = loaded;
+            to_mfma_lanes(tile, src_lane4);
+            TileFrags<TYPE> F;
+            F.prepare(tile, g);
 #pragma unroll
-        for (int t = 0; t < 8; ++t)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
-    };
-    if (total > 0) {
+            for (int t = 0; t < 8; ++t)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
+        };
+        if (total > 0) {
 #pragma unroll
-        for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
-        B[0].load(p_x, lane_off, ks);
-        B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
-        if (n_i <= 2 && total <= SK_DEPTH) {
-            // short walk: everything it needs is already in flight
+            for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
+            B[0].load(p_x, lane_off, ks);
+            B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
+            if (n_i <= 2 && total <= SK_DEPTH) {
+                // short walk: everything it needs is already in flight
 #pragma unroll
-            for (int q = 0; q < SK_DEPTH; ++q)
-                if (q < total && seg_valid(q % SEGS)) compute(ring[q], B[(q / SEGS) % 2], D[q % SEGS]);
-        } else {
-            constexpr int RB = SEGS >= 2 ? 2 : 4;            // super-block rounds per unrolled block (even: B parity is static)
-            constexpr int UB = RB * SEGS;                    // tiles per block, a multiple of the ring depth
+                for (int q = 0; q < SK_DEPTH; ++q)
+                    if (q < total && seg_valid(q % SEGS)) compute(ring[q], B[(q / SEGS) % 2], D[q % SEGS][0]);
+            } else {
+                constexpr int RB = SEGS >= 2 ? 2 : 4;            // super-block rounds per unrolled block (even: B parity is static)
+                constexpr int UB = RB * SEGS;                    // tiles per block, a multiple of the ring depth
+                static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
+                for (int blk = 0; blk * RB < n_i; ++blk) {
+#pragma unroll
+                    for (int q = 0; q < UB; ++q) {
+                        const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
+                        const int ii = blk * RB + r, f = ii * SEGS + seg;
+                        if (ii < n_i && seg_valid(seg)) compute(ring[slot], B[r % 2], D[seg][0]);
+                        // refill this slot with the tile DEPTH positions ahead
+                        load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
+                        // last segment of a super-block: its activation buffer is free for the one after next
+                        if (seg == SEGS - 1) B[r % 2].load(p_x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
+                        __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
+                    }
+                }
+            }
+        }
+    } else {
+        // two column blocks: 16 KB of activation fragments per super-block and wave, so only ONE super-block is held (64
+        // registers, as many as the two of a single block) and every fragment is fetched again, for the next super-block,
+        // right behind the last MFMAs that read it: one tile's time ahead of its use.  A tile that is not computed (past the
+        // end, invalid segment) issues the same loads in the same order, so that the compiler's count of loads in flight
+        // is the same along both paths.
+        BFrags<TYPE> Bw[NC];
+        auto frag_koff = [](int t) { return (TYPE == MESH_Q4_K ? 32 * (t >> 2) + 8 * (t & 3) : 32 * (t >> 1) + 8 * (t & 1)) * 16; };
+        auto b_base = [&](int sb, int c) { return p_x + (size_t)c * SK_NT * K + (size_t)sb * (QK_K * 16) + lane_off; };
+        auto step = [&](const TileRegs<TYPE> &loaded, f4_t (&acc)[NC], bool valid, bool refill, int next_sb) {
+            const _Float16 *nb[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) nb[c] = b_base(next_sb, c);
+            if (valid) {
+                TileRegs<TYPE> tile = loaded;
+                to_mfma_lanes(tile, src_lane4);
+                TileFrags<TYPE> F;
+                F.prepare(tile, g);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const h8_t af = F.frag(t);
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(h8_t, Bw[c].b[t]), acc[c], 0, 0, 0);
+                    if (refill) {
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) Bw[c].b[t] = ldg<uint4>(nb[c] + frag_koff(t));
+                    }
+                }
+            } else if (refill) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) Bw[c].b[t] = ldg<uint4>(nb[c] + frag_koff(t));
+            }
+        };
+        if (total > 0) {
+#pragma unroll
+            for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) Bw[c].load(p_x + (size_t)c * SK_NT * K, lane_off, ks);
+            constexpr int RB = SEGS % SK_DEPTH == 0 ? 1 : SK_DEPTH;      // rounds per unrolled block: ring slots static inside it
+            constexpr int UB = RB * SEGS;
             static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
             for (int blk = 0; blk * RB < n_i; ++blk) {
 #pragma unroll
                 for (int q = 0; q < UB; ++q) {
                     const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
                     const int ii = blk * RB + r, f = ii * SEGS + seg;
-                    if (ii < n_i && seg_valid(seg)) compute(ring[slot], B[r % 2], D[seg]);
-                    // refill this slot with the tile DEPTH positions ahead
+                    step(ring[slot], D[seg], ii < n_i && seg_valid(seg), seg == SEGS - 1, ks + KS * (ii + 1 < n_i ? ii + 1 : n_i - 1));
                     load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
-                    // last segment of a super-block: its activation buffer is free for the one after next
-                    if (seg == SEGS - 1) B[r % 2].load(p_x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
-                    __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -310,44 +373,47 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         if (total > 0 && seg_valid(seg)) {
             const int j = rs + RS * (seg / NU), u = seg % NU;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + 4 * g + i) * 16 + m] = D[seg][i];
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((((size_t)ks * rows_here + j) * NU + u) * 16 + 4 * g + i) * NT + c * SK_NT + m] = D[seg][c][i];
         }
     }
-    // (after the reduction buffer: [SK_NORM_GROUPS][16] sums of the consumer side, [SK_WAVES][16] of the producer side)
-    float *nrm = red + (size_t)KS * rows_here_max(p_split) * NU * 16 * SK_NT;
+    // (after the reduction buffer: [NORM_GROUPS][NT] sums of the consumer side, [SK_WAVES][NT] of the producer side)
+    constexpr int NORM_GROUPS = SK_THREADS / NT;          // threads sharing a token column in the epilogue
+    float *nrm = red + (size_t)KS * rows_here_max(p_split) * NU * 16 * NT;
     if (a.ni_part) {
         // norm hand-over, consumer side: this thread's share of the partial sums of squares of its epilogue column
         // (fetched after the weight stream: before it, the wave would wait for them ahead of its first tile loads)
         float ni_sum = 0.f;
-        for (int p = tid / SK_NT; p < a.ni_parts; p += SK_NORM_GROUPS) ni_sum += a.ni_part[(size_t)p * SK_NT + tid % SK_NT];
-        nrm[tid] = ni_sum;                             // tid = group * 16 + column
+        for (int p = tid / NT; p < a.ni_parts; p += NORM_GROUPS) ni_sum += a.ni_part[(size_t)p * NT + tid % NT];
+        nrm[tid] = ni_sum;                             // tid = group * NT + column
     }
     __syncthreads();
-    // 1 / rms of this thread's column (every output of a thread is of column tid % 16): groups added in order
+    // 1 / rms of this thread's column (every output of a thread is of column tid % NT): groups added in order
     float inv_rms = 1.0f;
     if (a.ni_part) {
         float ss = 0.f;
-        for (int q = 0; q < SK_NORM_GROUPS; ++q) ss += nrm[q * SK_NT + tid % SK_NT];
+        for (int q = 0; q < NORM_GROUPS; ++q) ss += nrm[q * NT + tid % NT];
         inv_rms = 1.0f / sqrtf(ss / (float)K + a.ni_eps);
     }
     float no_ss = 0.f;         // producer side: sum of squares of this thread's outputs (one column)
-    // outputs of this workgroup: rows_here x 16 rows x T columns
-    for (int o = tid; o < rows_here * 16 * SK_NT; o += SK_THREADS) {
-        const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
+    // outputs of this workgroup: rows_here x 16 rows x T columns; column t is column t % 16 of the f16 layouts' block t / 16
+    for (int o = tid; o < rows_here * 16 * NT; o += SK_THREADS) {
+        const int t = o % NT, r = (o / NT) % 16, j = o / (NT * 16);
         const int tr = tr0 + j;
         int mi = 0;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
         const int row = (tr - a.tile_begin[mi]) * TILE_ROWS + r;
         if (row >= a.M[mi]) continue;
         if (t >= a.T) {                                    // unused columns of the f16 output block stay finite
-            if (a.y16 && mi == 0) a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
-            if (a.no_x16) a.no_x16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)0.f;
+            if (a.y16 && mi == 0) a.y16[k8_at(a.M16, row, t)] = (_Float16)0.f;
+            if (a.no_x16) a.no_x16[k8_at(a.M[0], row, t)] = (_Float16)0.f;
             continue;
         }
         float s0 = 0.f, s1 = 0.f;
         for (int k2 = 0; k2 < KS; ++k2) {
-            s0 += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + r) * 16 + t];
-            if (NU == 2) s1 += red[((((size_t)k2 * rows_here + j) * NU + 1) * 16 + r) * 16 + t];
+            s0 += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + r) * NT + t];
+            if (NU == 2) s1 += red[((((size_t)k2 * rows_here + j) * NU + 1) * 16 + r) * NT + t];
         }
         s0 *= inv_rms;
         if (NU == 2) s1 *= inv_rms;
@@ -360,7 +426,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
             float val = s0;
             if (kind != GEMV_KIND_V && dd < a.rope.n_rot) {
                 float sp = 0.f;
-                for (int k2 = 0; k2 < KS; ++k2) sp += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + (r ^ 1)) * 16 + t];
+                for (int k2 = 0; k2 < KS; ++k2) sp += red[((((size_t)k2 * rows_here + j) * NU + 0) * 16 + (r ^ 1)) * NT + t];
                 sp *= inv_rms;
                 if (a.bias[mi]) sp += a.bias[mi][row ^ 1];
                 float sn, cs;
@@ -388,50 +454,54 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         // (saturating: a SwiGLU product beyond the f16 range becomes +-65504, not an infinity the next GEMM would spread)
         if (a.y16 && mi == 0) {
             note_f16_clamp(a.sat, out, 0.f);
-            a.y16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)__builtin_amdgcn_fmed3f(out, -65504.f, 65504.f);
+            a.y16[k8_at(a.M16, row, t)] = (_Float16)__builtin_amdgcn_fmed3f(out, -65504.f, 65504.f);
         }
         if (a.no_x16) {
             const float v = out * a.no_w[row];
             note_f16_clamp(a.sat, v, 0.f);
-            a.no_x16[((size_t)(row >> 3) * 16 + t) * 8 + (row & 7)] = (_Float16)__builtin_amdgcn_fmed3f(v, -65504.f, 65504.f);
+            a.no_x16[k8_at(a.M[0], row, t)] = (_Float16)__builtin_amdgcn_fmed3f(v, -65504.f, 65504.f);
             no_ss = fmaf(out, out, no_ss);
         }
     }
     if (a.no_part) {
-        // this workgroup's sum of squares per column: the four lanes of a wave that share a column, then the waves in order
-        no_ss += __shfl_xor(no_ss, 16);
+        // this workgroup's sum of squares per column: the lanes of a wave that share a column, then the waves in order
+        if (NT == 16) no_ss += __shfl_xor(no_ss, 16);
         no_ss += __shfl_xor(no_ss, 32);
-        float *wsum = nrm + SK_NORM_GROUPS * SK_NT;
-        if (lane < SK_NT) wsum[wave * SK_NT + lane] = no_ss;
+        float *wsum = nrm + NORM_GROUPS * NT;
+        if (lane < NT) wsum[wave * NT + lane] = no_ss;
         __syncthreads();
-        if (tid < SK_NT) {
+        if (tid < NT) {
             float ss = 0.f;
-            for (int w = 0; w < SK_WAVES; ++w) ss += wsum[w * SK_NT + tid];
-            a.no_part[(size_t)blockIdx.x * SK_NT + tid] = ss;
+            for (int w = 0; w < SK_WAVES; ++w) ss += wsum[w * NT + tid];
+            a.no_part[(size_t)blockIdx.x * NT + tid] = ss;
         }
     }
 }
 
-template <int TYPE, int NU, int SEGS>
+template <int TYPE, int NU, int SEGS, int NC>
 static int launch_skinny(const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
-        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_kernel<TYPE, NU, SEGS>),
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_kernel<TYPE, NU, SEGS, NC>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)SK_LDS_LIMIT));
         attr_set = true;
     }
-    MESH_LAUNCH((gemm_skinny_kernel<TYPE, NU, SEGS>), dim3((unsigned)grid), dim3(SK_THREADS), smem, stream, ka.x, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0],
+    MESH_LAUNCH((gemm_skinny_kernel<TYPE, NU, SEGS, NC>), dim3((unsigned)grid), dim3(SK_THREADS), smem, stream, ka.x, ka.wbase[0], ka.wbase[1] ? ka.wbase[1] : ka.wbase[0],
                 ka.wbase[2] ? ka.wbase[2] : ka.wbase[0], ka.K, ka.ks, ka.tile_begin[3], (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16),
                 (unsigned)(ka.tile_begin[3] / grid) | ((unsigned)(ka.tile_begin[3] % grid) << 16), ka);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
 }
 
-template <int TYPE, int NU>
+template <int TYPE, int NU, int NC>
 static int launch_skinny_segs(int segs, const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
-    if (segs <= 1) return launch_skinny<TYPE, NU, NU>(ka, grid, smem, stream);       // NU == 2 needs two segments at least
-    if (segs <= 2) return launch_skinny<TYPE, NU, 2>(ka, grid, smem, stream);
-    return launch_skinny<TYPE, NU, 4>(ka, grid, smem, stream);
+    if (segs <= 1) return launch_skinny<TYPE, NU, NU, NC>(ka, grid, smem, stream);   // NU == 2 needs two segments at least
+    if (segs <= 2) return launch_skinny<TYPE, NU, 2, NC>(ka, grid, smem, stream);
+    return launch_skinny<TYPE, NU, 4, NC>(ka, grid, smem, stream);
+}
+template <int TYPE, int NU>
+static int launch_skinny_cols(int nc, int segs, const SkinnyKernelArgs &ka, int grid, size_t smem, hipStream_t stream) {
+    return nc == 2 ? launch_skinny_segs<TYPE, NU, 2>(segs, ka, grid, smem, stream) : launch_skinny_segs<TYPE, NU, 1>(segs, ka, grid, smem, stream);
 }
 
 static int skinny_n_cu() {
@@ -496,11 +566,13 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
     const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
     if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", segs);
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d tile-rows in one launch", total_rows);
-    const size_t smem = sizeof(float) * ((size_t)KS * rows_max * NU * 16 * SK_NT + (size_t)(SK_NORM_GROUPS + SK_WAVES) * SK_NT);
-    if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: reduction buffer of %zu bytes does not fit LDS", smem);
-    for (int t = 0; t < a.T; t += SK_NT) {
+    // a pass over the weights takes 32 columns while more than 16 remain, else 16 (a call of up to 32 tokens is one launch)
+    for (int t = 0; t < a.T;) {
+        const int nc = a.T - t > SK_NT ? 2 : 1, nt = nc * SK_NT;
+        const size_t smem = sizeof(float) * ((size_t)KS * rows_max * NU * 16 * nt + (size_t)SK_THREADS + (size_t)SK_WAVES * nt);
+        if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: reduction buffer of %zu bytes does not fit LDS", smem);
         SkinnyKernelArgs kb = ka;
-        kb.T = std::min(SK_NT, a.T - t);
+        kb.T = std::min(nt, a.T - t);
         if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
         kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
         kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
@@ -508,9 +580,10 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
         for (int i = 0; i < a.n_mat; ++i)
             if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
         int rc;
-        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, grid, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, grid, smem, stream);
-        else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, grid, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, grid, smem, stream);
+        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_cols<MESH_Q4_K, 2>(nc, segs, kb, grid, smem, stream) : launch_skinny_cols<MESH_Q4_K, 1>(nc, segs, kb, grid, smem, stream);
+        else rc = NU == 2 ? launch_skinny_cols<MESH_Q6_K, 2>(nc, segs, kb, grid, smem, stream) : launch_skinny_cols<MESH_Q6_K, 1>(nc, segs, kb, grid, smem, stream);
         if (rc != MESH_OK) return rc;
+        t += nt;
     }
     return MESH_OK;
 }
@@ -526,11 +599,11 @@ int gemm_skinny_f16_workgroups(const SkinnyF16Args &a) {
 int gemm_skinny_f16(const SkinnyF16Args &a, hipStream_t stream) {
     using namespace f16sk;
     if (a.norm_out.x16 || a.norm_out.part || a.norm_out.norm_w) {
-        if (!a.norm_out.x16 || !a.norm_out.part || !a.norm_out.norm_w || a.n_mat != 1 || a.epi != EPI_RESIDUAL || a.T > SK_NT || a.mat[0].M % 8 ||
+        if (!a.norm_out.x16 || !a.norm_out.part || !a.norm_out.norm_w || a.n_mat != 1 || a.epi != EPI_RESIDUAL || a.T > SKINNY_F16_NORM_TOKENS_MAX || a.mat[0].M % 8 ||
             gemm_skinny_f16_workgroups(a) > SKINNY_F16_NORM_PARTS_MAX)
-            return fail(MESH_ERR_INVALID, "gemm_skinny_f16: the norm hand-over needs one matrix with a residual epilogue, at most 16 tokens and a row count that is a multiple of 8");
+            return fail(MESH_ERR_INVALID, "gemm_skinny_f16: the norm hand-over needs one matrix with a residual epilogue, at most 32 tokens and a row count that is a multiple of 8");
     }
-    if (a.norm_in.part && (a.norm_in.n_parts < 1 || a.norm_in.n_parts > SKINNY_F16_NORM_PARTS_MAX || a.T > SK_NT))
+    if (a.norm_in.part && (a.norm_in.n_parts < 1 || a.norm_in.n_parts > SKINNY_F16_NORM_PARTS_MAX || a.T > SKINNY_F16_NORM_TOKENS_MAX))
         return fail(MESH_ERR_INVALID, "gemm_skinny_f16: bad norm hand-over input (%d partial sums, %d tokens)", a.norm_in.n_parts, a.T);
     if (a.n_mat < 1 || a.n_mat > 3 || !a.x || a.T <= 0 || a.K <= 0) return fail(MESH_ERR_INVALID, "gemm_skinny_f16: bad arguments");
     if (a.K % QK_K || (reinterpret_cast<uintptr_t>(a.x) & 15))

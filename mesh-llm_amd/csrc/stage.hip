@@ -416,11 +416,11 @@ int session_new(mesh_stage *st, mesh_session **out) {
             MESH_HIP_TRY(hipMemsetAsync(p, 0, bytes, s->stream));
         }
         if (hp.n_ff > 0) {
-            // (one block of 16 tokens: the hand-over is for calls the skinny GEMM takes)
-            if ((rc = sess_alloc(s.get(), &p, 16 * (size_t)hp.n_embd * 2)) != MESH_OK) return rc;
+            // (two blocks of 16 tokens: the hand-over is for calls the skinny GEMM takes in one launch)
+            if ((rc = sess_alloc(s.get(), &p, SKINNY_F16_NORM_TOKENS_MAX * (size_t)hp.n_embd * 2)) != MESH_OK) return rc;
             s->norm16 = static_cast<uint16_t *>(p);
-            MESH_HIP_TRY(hipMemsetAsync(p, 0, 16 * (size_t)hp.n_embd * 2, s->stream));
-            if ((rc = fbuf(&s->norm_part, (size_t)SKINNY_F16_NORM_PARTS_MAX * 16)) != MESH_OK) return rc;
+            MESH_HIP_TRY(hipMemsetAsync(p, 0, SKINNY_F16_NORM_TOKENS_MAX * (size_t)hp.n_embd * 2, s->stream));
+            if ((rc = fbuf(&s->norm_part, (size_t)SKINNY_F16_NORM_PARTS_MAX * SKINNY_F16_NORM_TOKENS_MAX)) != MESH_OK) return rc;
             if ((rc = sess_alloc(s.get(), &p, B16 * (size_t)hp.n_ff * 2)) != MESH_OK) return rc;
             s->ffn16 = static_cast<uint16_t *>(p);
             if ((rc = fbuf(&s->ffn_up, B * (size_t)hp.n_ff)) != MESH_OK) return rc;
@@ -608,10 +608,10 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         r.head_dim = (int)hp.head_dim; r.n_rot = (int)hp.n_rot; r.n_kv = (int)hp.n_head_kv; r.n_ctx = st->n_ctx;
         return r;
     };
-    // f16 skinny GEMM, at most 16 tokens: the two RMS norms of the layer ride in the launches around them.  The output
+    // f16 skinny GEMM, calls it takes in one launch: the two RMS norms of the layer ride in the launches around them.  The output
     // projection and the down projection also write their result times the next norm's weight as f16 (norm16) and the sums
     // of squares their workgroups saw; q/k/v and gate/up read that and divide their products by the token's rms.
-    const bool nf = sk16 && T <= 16 && s->tune.skinny_norm_fused && s->norm16 && s->norm_part && E % 8 == 0;
+    const bool nf = sk16 && T <= SKINNY_F16_NORM_TOKENS_MAX && s->tune.skinny_norm_fused && s->norm16 && s->norm_part && E % 8 == 0;
     _Float16 *const nx = reinterpret_cast<_Float16 *>(s->norm16);
     const bool norm_ready = nf && s->norm_layer == (int)il;
     s->norm_layer = -1;
@@ -891,7 +891,10 @@ static int run_layers(mesh_session *s, int T, int max_keys) {
     for (size_t il = 0; il < st->layers.size(); ++il) {
         const LayerWeights &L = st->layers[il];
         if (T >= std::min(PREFILL_MIN_TOKENS, s->tune.skinny_from()) && s->xn16 && layer_is_kquant_dense(L) && hp.n_embd % 8 == 0 && hp.n_ff % 8 == 0) {
-            const bool skinny = T < PREFILL_MIN_TOKENS && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0 &&
+            // batches of decode steps of up to 32 tokens stay on the f16 skinny GEMM, two blocks of 16 columns per pass over
+            // the weights (a prefill chunk of that length goes to the large-tile GEMM and the chunk attention)
+            const bool wide = T >= PREFILL_MIN_TOKENS && T <= 32 && s->tune.skinny_f16 && s->tune.skinny_f16_wide && s->ffn16 && s->chunk_pos0 < 0;
+            const bool skinny = (T < PREFILL_MIN_TOKENS || wide) && hp.n_embd % 256 == 0 && hp.n_ff % 256 == 0 && (hp.n_head * hp.head_dim) % 256 == 0 &&
                                 L.w_gate.type == L.w_up.type;
             if (skinny || T >= PREFILL_MIN_TOKENS) {
                 if ((rc = run_layer_prefill(s, L, il, T, max_keys, skinny, false)) != MESH_OK) return rc;

@@ -625,6 +625,60 @@ def test_skinny_gemm_norms_ride_in_the_neighbouring_launches(tmp_path):
     fused.close(); plain.close(); st.close()
 
 
+def test_decode_batches_of_17_to_32_stay_on_the_skinny_gemm(tmp_path):
+    """Batches of 17 to 32 decode steps: one pass of the f16 skinny GEMM over the weights multiplies with two blocks of 16
+    activation columns (the activation fragments of one super-block are held and refilled behind the MFMAs that used
+    them), RoPE / KV append and the norm hand-over as for smaller batches.  Three real-shape layers (the middle one
+    with q6_K attn_v / ffn_down) at ragged KV depths, a x40 outlier channel in one step: against the oracle, against the
+    large-tile GEMM (skinny_f16_wide=0) and against norm launches of their own (skinny_norm_fused=0); then a smaller batch
+    on the same sessions, so that the hand-over buffers of a 32-column call are followed by a 16-column one."""
+    m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [2, 3, 4], 2, 5, n_ctx=64, n_seq=32, n_batch=32)
+    E = cfg["n_embd"]
+    wide, gemm, plain = st.session(), st.session(skinny_f16_wide=0), st.session(skinny_norm_fused=0)
+    assert wide.get_option("skinny_f16_wide") == 1 and gemm.get_option("skinny_f16_wide") == 0
+    orc = StageOracle(cfg, tensors, 2, 5, 64, n_seq_max=32)
+    rng = np.random.Generator(np.random.PCG64(177))
+    depth = [int(d) for d in rng.integers(0, 30, size=32)]
+    for il in (2, 3, 4):
+        for q in range(32):
+            if depth[q] == 0:
+                continue
+            k = (rng.standard_normal((depth[q], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
+            v = (rng.standard_normal((depth[q], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
+            for x_ in (wide, gemm, plain):
+                x_.kv_write(il, q, 0, k, v)
+            orc.k[il - 2, q, :, :depth[q]] = k.transpose(1, 0, 2)
+            orc.v[il - 2, q, :, :depth[q]] = v.transpose(1, 0, 2)
+    nxt = list(depth)
+    for step, T in enumerate((32, 17, 25, 32, 9, 20)):
+        seqs = [int(q) for q in sorted(rng.permutation(32)[:T])]
+        x = rng.standard_normal((T, E)).astype(np.float32)
+        if step == 2:
+            x[:, 1234] *= 40.0
+        pos = [nxt[q] for q in seqs]
+        for q in seqs:
+            nxt[q] += 1
+        a = wide.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        b = gemm.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        c = plain.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        ref = orc.forward(x, pos, seq=seqs)
+        ra, rb, rc = rel_l2(a, ref), rel_l2(b, ref), rel_l2(c, ref)
+        print("[wide skinny] step %d, %d tokens: %.3e (large-tile GEMM %.3e, own norm launches %.3e) of the oracle, %.3e / %.3e apart"
+              % (step, T, ra, rb, rc, rel_l2(a, b), rel_l2(a, c)))
+        assert np.isfinite(a).all()
+        assert ra <= 3e-3 and rb <= 3e-3 and rc <= 3e-3, (step, T)
+        assert rel_l2(a, b) <= 3e-3 and rel_l2(a, c) <= 3e-3, (step, T)
+        assert max(rel_l2(a[i], ref[i]) for i in range(T)) <= 1e-2
+        # the K / V rows this step appended, last layer: both paths round the same f32 values to f16
+        for q, p_ in ((seqs[0], pos[0]), (seqs[-1], pos[-1])):
+            ka, va = wide.kv_read(4, q, p_, 1)
+            kb, vb = gemm.kv_read(4, q, p_, 1)
+            assert rel_l2(ka.view(np.float16).astype(np.float32), kb.view(np.float16).astype(np.float32)) <= 5e-3
+            assert rel_l2(va.view(np.float16).astype(np.float32), vb.view(np.float16).astype(np.float32)) <= 5e-3
+    assert wide.f16_saturations() == 0
+    wide.close(); gemm.close(); plain.close(); st.close()
+
+
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path):
     """Llama-style (neighbouring-pair) RoPE and the KV append ride in the q/k/v projection's epilogue at batches of
     1-3 tokens (mat-vec kernels) and of 4+ tokens (batched MFMA GEMM); with gemv_rope=0 the separate kernel does
