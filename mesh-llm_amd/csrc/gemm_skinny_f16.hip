@@ -2,7 +2,7 @@
 // pass, W a tiled q4_K / q6_K matrix, X in f16 (the k8-major layout of gemm.hpp).
 //
 // The alternative to the integer kernel of gemm_skinny.hip for the same launches: the weight stream is organised as in
-// the mat-vec kernel -- a workgroup owns a few tile-rows (16 rows each), its waves split K and each keeps up to four
+// the mat-vec kernel -- a workgroup owns a few tile-rows (16 rows each), its waves split K and each keeps two
 // weight tiles in flight -- and a tile is dequantised in registers to f16 and multiplied with 16 activation columns at
 // once (v_mfma_f32_16x16x32_f16).  It issues about a third of the integer kernel's vector instructions per tile, so it
 // streams weights faster; what it gives up is precision: activations are rounded to f16 (11 significant bits against the
@@ -31,7 +31,7 @@ namespace f16sk {
 
 constexpr int SK_THREADS = 512;
 constexpr int SK_WAVES = SK_THREADS / 64;
-constexpr int SK_DEPTH_Q4 = 2;            // weight tiles a wave keeps in flight (2304 B each; four measured 2% slower: 250+ registers)
+constexpr int SK_DEPTH_Q4 = 2;            // weight tiles a wave keeps in flight (2304 B each; three and four measured 8% slower)
 constexpr int SK_DEPTH_Q6 = 2;            // q6_K tiles are 3360 B and their fragments need more registers
 constexpr int SK_NT = 16;                 // activation columns of one MFMA (a launch takes one or two such blocks)
 constexpr int SK_SEGS_MAX = 4;            // (tile-row, matrix) segments one wave may own (8 spills registers)
@@ -214,7 +214,7 @@ __device__ __forceinline__ int rows_here_max(unsigned p_split) { return (int)(p_
 
 // NC: blocks of 16 activation columns one pass over the weights multiplies with (1: up to 16 tokens, 2: up to 32).
 template <int TYPE, int NU, int SEGS, int NC>
-__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+__global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
                                                                  int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
                                                                  const SkinnyKernelArgs a) {
     // (p_begins = first tile-row of matrix 1 | of matrix 2 << 16; p_split = tile-rows per workgroup | workgroups with one
@@ -271,53 +271,13 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const _Float16 
         const bool ok = f < total && seg_valid(seg);
         dst.load(tile_ptr(ok ? f / SEGS : n_i - 1, ok ? seg : 0), lane);
     };
-    if constexpr (NC == 1) {
-        // one column block: the activation fragments of two super-blocks in registers, a whole super-block ahead
-        BFrags<TYPE> B[2];
-        auto compute = [&](const TileRegs<TYPE> &loaded, const BFrags<TYPE> &bf, f4_t &acc) {
-            TileRegs<TYPE> tile = loaded;
-            to_mfma_lanes(tile, src_lane4);
-            TileFrags<TYPE> F;
-            F.prepare(tile, g);
-#pragma unroll
-            for (int t = 0; t < 8; ++t)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(F.frag(t), __builtin_bit_cast(h8_t, bf.b[t]), acc, 0, 0, 0);
-        };
-        if (total > 0) {
-#pragma unroll
-            for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
-            B[0].load(p_x, lane_off, ks);
-            B[1].load(p_x, lane_off, ks + KS * (n_i > 1 ? 1 : 0));
-            if (n_i <= 2 && total <= SK_DEPTH) {
-                // short walk: everything it needs is already in flight
-#pragma unroll
-                for (int q = 0; q < SK_DEPTH; ++q)
-                    if (q < total && seg_valid(q % SEGS)) compute(ring[q], B[(q / SEGS) % 2], D[q % SEGS][0]);
-            } else {
-                constexpr int RB = SEGS >= 2 ? 2 : 4;            // super-block rounds per unrolled block (even: B parity is static)
-                constexpr int UB = RB * SEGS;                    // tiles per block, a multiple of the ring depth
-                static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
-                for (int blk = 0; blk * RB < n_i; ++blk) {
-#pragma unroll
-                    for (int q = 0; q < UB; ++q) {
-                        const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
-                        const int ii = blk * RB + r, f = ii * SEGS + seg;
-                        if (ii < n_i && seg_valid(seg)) compute(ring[slot], B[r % 2], D[seg][0]);
-                        // refill this slot with the tile DEPTH positions ahead
-                        load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
-                        // last segment of a super-block: its activation buffer is free for the one after next
-                        if (seg == SEGS - 1) B[r % 2].load(p_x, lane_off, ks + KS * (ii + 2 < n_i ? ii + 2 : n_i - 1));
-                        __builtin_amdgcn_sched_barrier(0);      // tiles stay in program order: hoisted loads would only cost registers
-                    }
-                }
-            }
-        }
-    } else {
-        // two column blocks: 16 KB of activation fragments per super-block and wave, so only ONE super-block is held (64
-        // registers, as many as the two of a single block) and every fragment is fetched again, for the next super-block,
-        // right behind the last MFMAs that read it: one tile's time ahead of its use.  A tile that is not computed (past the
-        // end, invalid segment) issues the same loads in the same order, so that the compiler's count of loads in flight
-        // is the same along both paths.
+    {
+        // Activation fragments: 8 KB per super-block, column block and wave.  Only ONE super-block is held (32 registers per
+        // column block) and every fragment is fetched again, for the next super-block, right behind the last MFMAs that read
+        // it: one tile's time ahead of its use, enough for a hit in L2.  (Two whole super-blocks in registers, fetched a
+        // super-block ahead, cost 32 more registers per column block and measured 6% slower at 16 columns.)  A tile that
+        // is not computed (past the end, invalid segment) issues the same loads in the same order, so that the compiler's
+        // count of loads in flight is the same along both paths.
         BFrags<TYPE> Bw[NC];
         auto frag_koff = [](int t) { return (TYPE == MESH_Q4_K ? 32 * (t >> 2) + 8 * (t & 3) : 32 * (t >> 1) + 8 * (t & 1)) * 16; };
         auto b_base = [&](int sb, int c) { return p_x + (size_t)c * SK_NT * K + (size_t)sb * (QK_K * 16) + lane_off; };
@@ -561,14 +521,14 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
     const int KS = skinny_ks(nsb);
     const int RS = SK_WAVES / KS;
     ka.ks = KS;
-    const int grid = skinny_grid(total_rows, NU, KS);
-    const int rows_max = (total_rows + grid - 1) / grid;
-    const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
-    if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", segs);
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d tile-rows in one launch", total_rows);
     // a pass over the weights takes 32 columns while more than 16 remain, else 16 (a call of up to 32 tokens is one launch)
     for (int t = 0; t < a.T;) {
         const int nc = a.T - t > SK_NT ? 2 : 1, nt = nc * SK_NT;
+        const int grid = skinny_grid(total_rows, NU, KS);
+        const int rows_max = (total_rows + grid - 1) / grid;
+        const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
+        if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", segs);
         const size_t smem = sizeof(float) * ((size_t)KS * rows_max * NU * 16 * nt + (size_t)SK_THREADS + (size_t)SK_WAVES * nt);
         if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: reduction buffer of %zu bytes does not fit LDS", smem);
         SkinnyKernelArgs kb = ka;
