@@ -14,9 +14,10 @@ namespace mesh {
 constexpr int ROUTE_MAX_PER_LANE = MOE_EXPERTS_MAX / 64;
 
 // softmax -> (+mask) -> top-k of one token's logits by one wave; NPL = experts per lane (n_expert <= 64 * NPL)
+// (ids_copy: optional second destination of the expert ids, e.g. the workgroup's LDS)
 template <int NPL>
 __device__ __forceinline__ void route_wave(const float *lg, const float *mask, int n_expert, int top_k, int norm_w,
-                                           int32_t *ids, float *weights, int lane) {
+                                           int32_t *ids, float *weights, int lane, int32_t *ids_copy = nullptr) {
     float p[NPL], sel[NPL];
     float mx = -INFINITY;
 #pragma unroll
@@ -106,16 +107,18 @@ __device__ __forceinline__ void route_wave(const float *lg, const float *mask, i
     }
     if (lane < top_k) {
         ids[lane] = my_id;
+        if (ids_copy) ids_copy[lane] = my_id;
         weights[lane] = norm_w && wsum > 0.f ? my_w / wsum : my_w;
     }
 }
 
-__device__ __forceinline__ void route_wave_any(const float *lg, const MoeRouteArgs &a, int t, int lane) {
+__device__ __forceinline__ void route_wave_any(const float *lg, const MoeRouteArgs &a, int t, int lane, int32_t *ids_copy = nullptr) {
     int32_t *ids = a.ids + (size_t)t * a.top_k;
     float *w = a.weights + (size_t)t * a.top_k;
-    if (a.n_expert <= 64) route_wave<1>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane);
-    else if (a.n_expert <= 128) route_wave<2>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane);
-    else route_wave<ROUTE_MAX_PER_LANE>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane);
+    if (ids_copy) ids_copy += (size_t)t * a.top_k;
+    if (a.n_expert <= 64) route_wave<1>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane, ids_copy);
+    else if (a.n_expert <= 128) route_wave<2>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane, ids_copy);
+    else route_wave<ROUTE_MAX_PER_LANE>(lg, a.mask, a.n_expert, a.top_k, a.norm_w, ids, w, lane, ids_copy);
 }
 
 // one wave per token
@@ -322,13 +325,16 @@ int moe_route(const MoeRouteArgs &a, int T, hipStream_t stream) {
 constexpr int GROUP_THREADS = 1024, GROUP_WAVES = GROUP_THREADS / 64;
 // (whole workgroup; lds: n_pairs + 2 * n_expert ints)
 // ipairs: most pairs per item; an item takes iints = moe_item_ints(ipairs) int32
+// ids == nullptr: the pair list is in lds[0 .. n_pairs) already and a barrier has been passed since it was written
 __device__ __forceinline__ void group_pairs(const int32_t *__restrict__ ids, int n_pairs, int n_expert, int32_t *__restrict__ items,
                                             int32_t *__restrict__ n_items, int32_t *lds, int ipairs) {
     const int iints = moe_item_ints(ipairs);
     int32_t *s_ids = lds, *s_cnt = lds + n_pairs, *s_base = s_cnt + n_expert;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int p = tid; p < n_pairs; p += GROUP_THREADS) s_ids[p] = ids[p];
-    __syncthreads();
+    if (ids) {
+        for (int p = tid; p < n_pairs; p += GROUP_THREADS) s_ids[p] = ids[p];
+        __syncthreads();
+    }
     for (int e = wave; e < n_expert; e += GROUP_WAVES) {
         int c = 0;
         for (int p0 = 0; p0 < n_pairs; p0 += 64) {
@@ -395,9 +401,10 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_route_group_kernel(const fl
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     MoeRouteArgs a;
     a.logits = p_logits; a.mask = p_mask; a.ids = p_ids; a.weights = p_weights; a.n_expert = p_n_expert; a.top_k = p_top_k; a.norm_w = p_norm_w;
-    for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(p_logits + (size_t)t * p_n_expert, a, t, lane);
+    // (the ids also go to the pair list in LDS: the grouping does not wait for them to come back from memory)
+    for (int t = wave; t < T; t += GROUP_WAVES) route_wave_any(p_logits + (size_t)t * p_n_expert, a, t, lane, g_lds);
     __syncthreads();
-    group_pairs(p_ids, T * p_top_k, p_n_expert, items, n_items, g_lds, ipairs);
+    group_pairs(nullptr, T * p_top_k, p_n_expert, items, n_items, g_lds, ipairs);
 }
 
 // The two launches above as one: every workgroup computes its slice of the logits; the one that arrives last (a device-wide
@@ -423,19 +430,21 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_router_group_fused_kernel(c
     if (!s_last) return;
     if (threadIdx.x == 0) __hip_atomic_store(arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // LDS of the tail: the pair list and the grouping's counters, then a logits row per wave
+    const int n_group_ints = T * a.top_k + 2 * p_n_expert;
     for (int t = wave; t < T; t += GROUP_WAVES) {
         // the token's logits through LDS: route_wave reads plain floats
-        float *row = reinterpret_cast<float *>(g_lds) + (size_t)wave * 64 * ROUTE_MAX_PER_LANE;
+        float *row = reinterpret_cast<float *>(g_lds + n_group_ints) + (size_t)wave * 64 * ROUTE_MAX_PER_LANE;
         // (device-scope loads: written by other workgroups of this launch, possibly on another die)
         for (int e = lane; e < p_n_expert; e += 64) row[e] = __hip_atomic_load(logits + (size_t)t * p_n_expert + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        route_wave_any(row, a, t, lane);
+        route_wave_any(row, a, t, lane, g_lds);        // (ids to memory and to the pair list in LDS)
         __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
-    group_pairs(a.ids, T * a.top_k, p_n_expert, items, n_items, g_lds, ipairs);
+    group_pairs(nullptr, T * a.top_k, p_n_expert, items, n_items, g_lds, ipairs);
 }
 
 int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float *norm_w, float eps, const float *W, int E,
@@ -449,9 +458,8 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
     if (arrive) {
         // one launch: the last workgroup to finish its logits routes and groups
         la.logits = logits;
-        // LDS of the tail: a logits row per wave while routing, then the grouping's pair list and counters
-        const size_t smem = std::max((size_t)GROUP_WAVES * 64 * ROUTE_MAX_PER_LANE * sizeof(float),
-                                     ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t));
+        // LDS of the tail: the grouping's pair list and counters, then a logits row per wave
+        const size_t smem = (size_t)GROUP_WAVES * 64 * ROUTE_MAX_PER_LANE * sizeof(float) + ((size_t)T * a.top_k + 2 * (size_t)a.n_expert) * sizeof(int32_t);
         switch (E / 256) {
             case 2: MESH_LAUNCH(moe_router_group_fused_kernel<2>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
             case 4: MESH_LAUNCH(moe_router_group_fused_kernel<4>, grid, block, smem, stream, x, norm_w, W, logits, ldx, eps, la.n_expert, la, T, items, n_items, item_pairs, arrive); break;
@@ -479,7 +487,7 @@ int moe_router_group(const MoeRouteArgs &a, const float *x, int ldx, const float
 }
 bool moe_router_group_supported(int E, int n_expert, int top_k, int T) {
     return moe_router_fused_supported(E, n_expert, top_k) && n_expert > ROUTER_WAVES && T >= 1 && T <= 64 &&
-           ((size_t)T * top_k + 2 * (size_t)n_expert) * sizeof(int32_t) <= 48 * 1024;
+           ((size_t)T * top_k + 2 * (size_t)n_expert) * sizeof(int32_t) <= 28 * 1024;      // (plus 32 KB of logits rows in the same workgroup)
 }
 
 bool moe_group_supported(int n_pairs, int n_expert) {
