@@ -1,7 +1,7 @@
 """Activation range of the projection paths.  The mat-vec kernels (calls of up to 4 tokens) and the integer-MFMA skinny
 GEMM quantise activations to 16-bit fixed point per 32-element block with an f32 block scale: any f32 magnitude is
-representable, and an outlier channel costs precision only inside its own block.  The f16 skinny GEMM (calls of 5 to 16
-tokens, the default) and the large-tile GEMM (17+ tokens) round activations to f16: relative precision 2^-11 whatever the
+representable, and an outlier channel costs precision only inside its own block.  The f16 skinny GEMM (calls of 4 to 16
+tokens and batches of up to 32 decode steps, the default) and the large-tile GEMM (longer calls, prefill chunks) round activations to f16: relative precision 2^-11 whatever the
 magnitude, up to +-65504, beyond which the producers SATURATE (a finite, wrong-by-clamping value) rather than emit an
 infinity that the next norm would turn into NaN for the whole token, and count the value in the session's saturation
 counter.
@@ -62,7 +62,7 @@ def test_outlier_channels_through_every_projection_path(tmp_path, skinny):
     # 200-token prefill chunk (large-tile GEMM, f16 activations), then decode batches on top of it and on fresh sequences
     for T, seqs, what in ((200, [0] * 200, "prefill 200 (f16 large-tile GEMM)"), (1, [0], "decode 1 (mat-vec)"), (3, [0, 1, 2], "decode 3 (mat-vec)"),
                           (8, list(range(8)), "decode 8 (%s skinny GEMM)" % skinny), (16, list(range(16)), "decode 16 (%s skinny GEMM)" % skinny),
-                          (24, list(range(24)), "decode 24 (f16 large-tile GEMM, split K)")):
+                          (24, list(range(24)), "decode 24 (f16 skinny GEMM, two column blocks)" if skinny == "f16" else "decode 24 (f16 large-tile GEMM, split K)")):
         x = outlier_input(rng, T, E)
         pos = []
         for q in seqs:                      # every sequence continues where it stands
@@ -113,7 +113,7 @@ def test_swiglu_products_beyond_the_f16_range(tmp_path):
     got, r = run(ses, 1, 0, 0)
     assert r <= 5e-4 and ses.f16_saturations() == 0
     seen = 0
-    for T, pos0, seq0, what in ((8, 0, 8, "f16 skinny GEMM"), (64, 1, 20, "prefill")):
+    for T, pos0, seq0, what in ((8, 0, 8, "f16 skinny GEMM"), (24, 0, 0, "f16 skinny GEMM, two column blocks"), (64, 1, 20, "prefill")):
         got, r = run(ses, T, pos0, seq0)
         n = ses.f16_saturations()
         print("[outliers] SwiGLU beyond f16, %s of %d tokens (saturating f16): rel-L2 %.3e, %d values clamped so far" % (what, T, r, n))

@@ -733,8 +733,8 @@ def test_ffn_vector_quantised_by_its_producer_equals_the_f32_hand_over(tmp_path)
         st.close()
 
 
-@pytest.mark.parametrize("name,layers", [("llama3-8b", [3, 4]), ("tiny-qwen2", [0, 1, 2]), ("tiny-moe", [0, 1])])
-def test_graph_replays_equal_eager_launches(tmp_path, name, layers):
+@pytest.mark.parametrize("name,layers,wide", [("llama3-8b", [3, 4], 1), ("llama3-8b", [3, 4], 0), ("tiny-qwen2", [0, 1, 2], 1), ("tiny-moe", [0, 1], 1)])
+def test_graph_replays_equal_eager_launches(tmp_path, name, layers, wide):
     """Decode-sized batches replay their layer launches from a captured graph (first use of a shape eager, second
     captured, then replays).  Every replay must give the bits the eager launches give: two sessions, graphs on and
     off, walk the same sequence of steps -- repeated shapes, other shapes and host synchronisations in between, KV
@@ -742,13 +742,14 @@ def test_graph_replays_equal_eager_launches(tmp_path, name, layers):
     m, cfg, tensors, st = _open(tmp_path, name, layers, layers[0], layers[-1] + 1, n_ctx=256, n_seq=20, n_batch=32)
     E = cfg["n_embd"]
     rng = np.random.Generator(np.random.PCG64(17))
-    # (20 tokens: the large-tile GEMM with K split over workgroups, two kernels per projection, inside a graph)
+    # (20 tokens on real-shape layers: the f16 skinny GEMM with two column blocks; with skinny_f16_wide=0, and on the small
+    # models, the large-tile GEMM with K split over workgroups, two kernels per projection, inside a graph)
     plan = [1, 1, 1, 4, 1, 4, 6, 1, 4, 6, 6, 1, 20, 1, 20] + [1] * 70 + [4, 4, 1, 6, 20]
     xs = [rng.standard_normal((T, E)).astype(np.float32) for T in plan]
     chunk_xs = [rng.standard_normal((25, E)).astype(np.float32) for _ in range(8)]
     runs = []
     for flag in ("1", "0"):
-        ses = st.session(graphs=int(flag))
+        ses = st.session(graphs=int(flag), skinny_f16_wide=wide)
         nxt = [0] * 20
         outs = []
         for x in xs:
