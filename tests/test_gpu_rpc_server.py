@@ -125,6 +125,67 @@ def test_graph_compute_of_a_layer_range_equals_the_stage_library(server_bin, tmp
     ses.close(); st.close()
 
 
+def test_graph_recompute_step_through_the_server_costs_little_more_than_the_library_call(server_bin, tmp_path):
+    """What the front end adds to a decode step: two real-shape layers (Llama-3-8B shape), single-token steps as a client
+    drives them -- SET_TENSOR of the hidden state and of the position, GRAPH_RECOMPUTE, GET_TENSOR of the result -- against
+    mesh_stage_decode of the same layers on host buffers in this process.  Bit-identical results; the difference in wall
+    time per step is the four messages over loopback, their handling in the server and this Python client."""
+    import time
+    import models
+    import rpc_graph_util as GU
+    from util import mesh
+    m = mesh()
+    name, lb, le = "llama3-8b", 3, 5
+    cfg = models.CONFIGS[name]
+    path = str(tmp_path / (name + ".gguf"))
+    tensors = models.write_model(path, cfg, range(lb, le), seed=11)
+    E, n_ctx = cfg["n_embd"], 256
+    weights = {n: (t, list(d)) for n, (t, d, _) in tensors.items() if n.startswith("blk.")}
+    st = m.Stage(path, lb, le, n_ctx=n_ctx, n_seq_max=1, n_batch_max=16)
+    ses = st.session()
+    rng = np.random.Generator(np.random.PCG64(6))
+    n_steps = 120
+    xs = rng.standard_normal((n_steps, 1, E)).astype(np.float32)
+    with ServerProcess(server_bin, extra=["-d", "ROCm0", "--gguf", path]) as s:
+        c = Client(s.port)
+        h, _ = c.alloc_buffer(512 << 20)       # (the graph's weight leaves lie in the client's buffer too: 2 x 218 MB)
+        gb = GU.GraphBuilder(h, c.buffer_get_base(h))
+        inp, pos, out = GU.layer_range_graph(gb, weights, list(range(lb, le)), 1, cfg["n_head"], cfg["n_head_kv"], cfg["head_dim"], n_ctx)
+        d_in, d_pos, d_out = gb.descriptor(inp), gb.descriptor(pos), gb.descriptor(out)
+        got, want = [], []
+        t_rpc = t_lib = 0.0
+        for i in range(n_steps):
+            p = np.array([i], np.int32)
+            t0 = time.perf_counter()
+            c.set_tensor(d_in, 0, xs[i].tobytes())
+            c.set_tensor(d_pos, 0, p.tobytes())
+            if i == 0:
+                c.send(R_GRAPH_COMPUTE, gb.payload())
+            else:
+                c.send(R_GRAPH_RECOMPUTE, (0).to_bytes(4, "little"))
+            try:
+                r = c.get_tensor(d_out, 0, E * 4)
+            except ConnectionError:
+                raise AssertionError("the server closed the connection: " + s.stop()[-2000:])
+            t1 = time.perf_counter()
+            w = ses.decode(xs[i], p).copy()
+            t2 = time.perf_counter()
+            got.append(np.frombuffer(r, np.float32))
+            want.append(w.view(np.float32).reshape(-1))
+            if i >= 20:                     # (the first steps open the stage and warm both paths)
+                t_rpc += t1 - t0
+                t_lib += t2 - t1
+        c.close()
+        s.stop()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert np.array_equal(a, b), i
+    n = n_steps - 20
+    print("[rpc] decode step of 2 real-shape layers: %.1f us through rpc-server (4 messages), %.1f us through the library; the front end adds %.1f us"
+          % (t_rpc / n * 1e6, t_lib / n * 1e6, (t_rpc - t_lib) / n * 1e6))
+    assert (t_rpc - t_lib) / n < 2e-3          # a loose bound: loopback round trips and a Python client, not a regression gate for microseconds
+    ses.close(); st.close()
+
+
 R_GRAPH_COMPUTE, R_GRAPH_RECOMPUTE = 10, 16
 
 
