@@ -127,6 +127,8 @@ struct SkinnyF16Args {
     // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+    // q4_K matrices followed by one q6_K matrix (q, k and a q6_K v): one launch for both types instead of two
+    bool pair_launch = true;
     // RMS-norm hand-over between two launches (T <= 32: one launch each), in place of a norm kernel of its own between them.  The producer
     // (EPI_RESIDUAL, one matrix) also writes f16(y * norm_w) -- scaled by the next norm's weight but not yet by the
     // token's 1 / rms -- in the k8-major layout to norm_out.x16, and per workgroup the sum of y^2 of its rows for every

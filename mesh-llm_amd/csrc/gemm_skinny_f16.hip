@@ -213,10 +213,10 @@ __device__ __forceinline__ size_t k8_at(int K, int k, int t) { return (size_t)(t
 __device__ __forceinline__ int rows_here_max(unsigned p_split) { return (int)(p_split & 0xFFFFu) + ((p_split >> 16) ? 1 : 0); }
 
 // NC: blocks of 16 activation columns one pass over the weights multiplies with (1: up to 16 tokens, 2: up to 32).
+// bx: the workgroup's index among those of its launch part (the whole launch, or one side of a pair launch).
 template <int TYPE, int NU, int SEGS, int NC>
-__global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
-                                                                 int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
-                                                                 const SkinnyKernelArgs a) {
+__device__ __forceinline__ void skinny_workgroup(int bx, const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+                                                 int p_ks, unsigned p_begins, unsigned p_split, const SkinnyKernelArgs &a) {
     // (p_begins = first tile-row of matrix 1 | of matrix 2 << 16; p_split = tile-rows per workgroup | workgroups with one
     // more << 16, computed on the host: no division and no grid-size load stand before the first weight load)
     const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
@@ -232,8 +232,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_kernel(const _Float
     const int src_lane4 = 4 * (4 * m + g);                // byte address, for ds_bpermute, of the lane that loaded row m, quarter g
     const int KS = p_ks, LK = __builtin_ctz((unsigned)KS), RS = SK_WAVES >> LK;      // KS is a power of two
     const int ks = wave & (KS - 1), rs = wave >> LK;
-    (void)p_rows;
-    const int sq = (int)(p_split & 0xFFFFu), sr = (int)(p_split >> 16), bx = blockIdx.x;
+    const int sq = (int)(p_split & 0xFFFFu), sr = (int)(p_split >> 16);
     const int tr0 = bx * sq + (bx < sr ? bx : sr);
     const int rows_here = sq + (bx < sr ? 1 : 0);
     const int n_i = rs < RS ? (nsb - ks + KS - 1) >> LK : 0;        // super-blocks of this wave (ks < KS <= nsb)
@@ -433,9 +432,29 @@ __global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_kernel(const _Float
         if (tid < NT) {
             float ss = 0.f;
             for (int w = 0; w < SK_WAVES; ++w) ss += wsum[w * NT + tid];
-            a.no_part[(size_t)blockIdx.x * NT + tid] = ss;
+            a.no_part[(size_t)bx * NT + tid] = ss;
         }
     }
+}
+
+template <int TYPE, int NU, int SEGS, int NC>
+__global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+                                                                 int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
+                                                                 const SkinnyKernelArgs a) {
+    (void)p_rows;
+    skinny_workgroup<TYPE, NU, SEGS, NC>((int)blockIdx.x, p_x, p_w0, p_w1, p_w2, p_K, p_ks, p_begins, p_split, a);
+}
+
+// Two launches that read the same activations as one: the first grid_a workgroups run a q4_K launch, the others a q6_K launch
+// (the q and k projections of a layer next to a q6_K v projection: 160 + 64 workgroups at Llama-3-8B shape, one wave of
+// workgroups instead of two dependent launches).  Same arithmetic per workgroup as the separate launches.
+template <int SEGS_A, int SEGS_B, int NC>
+__global__ __launch_bounds__(SK_THREADS, 2) void gemm_skinny_pair_kernel(const _Float16 *p_x, const uint8_t *p_w0, const uint8_t *p_w1, int p_K, int p_ks,
+                                                                      int grid_a, unsigned p_begins, unsigned p_split_a, unsigned p_split_b,
+                                                                      const uint8_t *p_wb, const SkinnyKernelArgs a, const SkinnyKernelArgs b) {
+    const int bx = (int)blockIdx.x;
+    if (bx < grid_a) skinny_workgroup<MESH_Q4_K, 1, SEGS_A, NC>(bx, p_x, p_w0, p_w1, p_w1, p_K, p_ks, p_begins, p_split_a, a);
+    else skinny_workgroup<MESH_Q6_K, 1, SEGS_B, NC>(bx - grid_a, p_x, p_wb, p_wb, p_wb, p_K, p_ks, 0xFFFFFFFFu, p_split_b, b);
 }
 
 template <int TYPE, int NU, int SEGS, int NC>
@@ -491,12 +510,19 @@ static int skinny_grid(int total_rows, int NU, int KS) {
     return (total_rows + rows_per_wg - 1) / rows_per_wg;
 }
 
-// all matrices of `a` are tiled K-quants of one type
-static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
-    const int type = a.mat[0].type;
+// What a launch over the matrices of `a` (tiled K-quants of one type) needs, before the token chunk is chosen
+struct SkinnyLaunch {
+    SkinnyKernelArgs ka;
+    int type, NU, KS, total_rows, grid, rows_max, segs;
+    size_t smem(int nt) const { return sizeof(float) * ((size_t)KS * rows_max * NU * 16 * nt + (size_t)SK_THREADS + (size_t)SK_WAVES * nt); }
+};
+static int skinny_prepare(const SkinnyF16Args &a, SkinnyLaunch &L) {
+    L.type = a.mat[0].type;
     const int nsb = a.K / QK_K, NU = a.epi == EPI_SWIGLU ? 2 : 1;
-    const size_t row_stride = (size_t)nsb * (type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES);
-    SkinnyKernelArgs ka{};
+    L.NU = NU;
+    const size_t row_stride = (size_t)nsb * (L.type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES);
+    SkinnyKernelArgs &ka = L.ka;
+    ka = SkinnyKernelArgs{};
     int total_rows = 0;
     for (int i = 0; i < a.n_mat; ++i) {
         const int begin = (NU == 2 && i == 1) ? 0 : total_rows;     // gate and up share tile-row indices
@@ -518,30 +544,92 @@ static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
     ka.sat = a.sat;
     ka.no_w = a.norm_out.norm_w; ka.no_x16 = a.norm_out.x16; ka.no_part = a.norm_out.part;
     ka.ni_part = a.norm_in.part; ka.ni_parts = a.norm_in.n_parts; ka.ni_eps = a.norm_in.eps;
-    const int KS = skinny_ks(nsb);
-    const int RS = SK_WAVES / KS;
-    ka.ks = KS;
+    L.KS = skinny_ks(nsb);
+    const int RS = SK_WAVES / L.KS;
+    ka.ks = L.KS;
+    L.total_rows = total_rows;
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d tile-rows in one launch", total_rows);
+    L.grid = skinny_grid(total_rows, NU, L.KS);
+    L.rows_max = (total_rows + L.grid - 1) / L.grid;
+    L.segs = ((L.rows_max + RS - 1) / RS) * NU;         // per wave
+    if (L.segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", L.segs);
+    return MESH_OK;
+}
+// the kernel arguments of the launch for columns t .. t + nt - 1 of the call
+static SkinnyKernelArgs skinny_chunk(const SkinnyF16Args &a, const SkinnyLaunch &L, int t, int nt) {
+    SkinnyKernelArgs kb = L.ka;
+    kb.T = std::min(nt, a.T - t);
+    if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
+    kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
+    kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
+    kb.y16 = a.y16 ? a.y16 + (size_t)t * a.mat[0].M : nullptr;
+    for (int i = 0; i < a.n_mat; ++i)
+        if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
+    return kb;
+}
+
+// all matrices of `a` are tiled K-quants of one type
+static int skinny_one_type(const SkinnyF16Args &a, hipStream_t stream) {
+    SkinnyLaunch L;
+    int rc = skinny_prepare(a, L);
+    if (rc != MESH_OK) return rc;
     // a pass over the weights takes 32 columns while more than 16 remain, else 16 (a call of up to 32 tokens is one launch)
     for (int t = 0; t < a.T;) {
         const int nc = a.T - t > SK_NT ? 2 : 1, nt = nc * SK_NT;
-        const int grid = skinny_grid(total_rows, NU, KS);
-        const int rows_max = (total_rows + grid - 1) / grid;
-        const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
-        if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: %d segments per wave", segs);
-        const size_t smem = sizeof(float) * ((size_t)KS * rows_max * NU * 16 * nt + (size_t)SK_THREADS + (size_t)SK_WAVES * nt);
+        const size_t smem = L.smem(nt);
         if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny_f16: reduction buffer of %zu bytes does not fit LDS", smem);
-        SkinnyKernelArgs kb = ka;
-        kb.T = std::min(nt, a.T - t);
-        if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
-        kb.x = a.x + (size_t)t * a.K;                  // block t / 16 of the k8-major activations
-        kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
-        kb.y16 = a.y16 ? a.y16 + (size_t)t * a.mat[0].M : nullptr;
-        for (int i = 0; i < a.n_mat; ++i)
-            if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
-        int rc;
-        if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_cols<MESH_Q4_K, 2>(nc, segs, kb, grid, smem, stream) : launch_skinny_cols<MESH_Q4_K, 1>(nc, segs, kb, grid, smem, stream);
-        else rc = NU == 2 ? launch_skinny_cols<MESH_Q6_K, 2>(nc, segs, kb, grid, smem, stream) : launch_skinny_cols<MESH_Q6_K, 1>(nc, segs, kb, grid, smem, stream);
+        const SkinnyKernelArgs kb = skinny_chunk(a, L, t, nt);
+        if (L.type == MESH_Q4_K) rc = L.NU == 2 ? launch_skinny_cols<MESH_Q4_K, 2>(nc, L.segs, kb, L.grid, smem, stream) : launch_skinny_cols<MESH_Q4_K, 1>(nc, L.segs, kb, L.grid, smem, stream);
+        else rc = L.NU == 2 ? launch_skinny_cols<MESH_Q6_K, 2>(nc, L.segs, kb, L.grid, smem, stream) : launch_skinny_cols<MESH_Q6_K, 1>(nc, L.segs, kb, L.grid, smem, stream);
+        if (rc != MESH_OK) return rc;
+        t += nt;
+    }
+    return MESH_OK;
+}
+
+template <int SEGS_A, int SEGS_B, int NC>
+static int launch_pair(const SkinnyKernelArgs &ka, const SkinnyKernelArgs &kb, int grid_a, int grid_b, size_t smem, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_pair_kernel<SEGS_A, SEGS_B, NC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)SK_LDS_LIMIT));
+        attr_set = true;
+    }
+    MESH_LAUNCH((gemm_skinny_pair_kernel<SEGS_A, SEGS_B, NC>), dim3((unsigned)(grid_a + grid_b)), dim3(SK_THREADS), smem, stream, ka.x, ka.wbase[0],
+                ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.K, ka.ks, grid_a, (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16),
+                (unsigned)(ka.tile_begin[3] / grid_a) | ((unsigned)(ka.tile_begin[3] % grid_a) << 16),
+                (unsigned)(kb.tile_begin[3] / grid_b) | ((unsigned)(kb.tile_begin[3] % grid_b) << 16), kb.wbase[0], ka, kb);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+template <int NC>
+static int launch_pair_segs(int segs_a, int segs_b, const SkinnyKernelArgs &ka, const SkinnyKernelArgs &kb, int grid_a, int grid_b, size_t smem, hipStream_t stream) {
+    const int sa = segs_a <= 1 ? 1 : segs_a <= 2 ? 2 : 4;
+    if (segs_b <= 1) {
+        if (sa == 1) return launch_pair<1, 1, NC>(ka, kb, grid_a, grid_b, smem, stream);
+        if (sa == 2) return launch_pair<2, 1, NC>(ka, kb, grid_a, grid_b, smem, stream);
+        return launch_pair<4, 1, NC>(ka, kb, grid_a, grid_b, smem, stream);
+    }
+    if (sa == 1) return launch_pair<1, 2, NC>(ka, kb, grid_a, grid_b, smem, stream);
+    if (sa == 2) return launch_pair<2, 2, NC>(ka, kb, grid_a, grid_b, smem, stream);
+    return launch_pair<4, 2, NC>(ka, kb, grid_a, grid_b, smem, stream);
+}
+
+// `qa`: one or two q4_K matrices, `qb`: one q6_K matrix, same activations, plain-store epilogues (with or without RoPE):
+// one launch whose first workgroups are qa's and whose last are qb's.  MESH_ERR_UNSUPPORTED when the shapes do not fit
+// (the caller then launches them one after the other).
+static int skinny_pair(const SkinnyF16Args &qa, const SkinnyF16Args &qb, hipStream_t stream) {
+    SkinnyLaunch A, B;
+    int rc = skinny_prepare(qa, A);
+    if (rc != MESH_OK) return rc;
+    if ((rc = skinny_prepare(qb, B)) != MESH_OK) return rc;
+    if (B.segs > 2 || A.KS != B.KS) return MESH_ERR_UNSUPPORTED;
+    for (int t = 0; t < qa.T;) {
+        const int nc = qa.T - t > SK_NT ? 2 : 1, nt = nc * SK_NT;
+        const size_t smem = std::max(A.smem(nt), B.smem(nt));
+        if (smem > SK_LDS_LIMIT) return MESH_ERR_UNSUPPORTED;
+        const SkinnyKernelArgs ka = skinny_chunk(qa, A, t, nt), kb = skinny_chunk(qb, B, t, nt);
+        rc = nc == 2 ? launch_pair_segs<2>(A.segs, B.segs, ka, kb, A.grid, B.grid, smem, stream) : launch_pair_segs<1>(A.segs, B.segs, ka, kb, A.grid, B.grid, smem, stream);
         if (rc != MESH_OK) return rc;
         t += nt;
     }
@@ -580,7 +668,20 @@ int gemm_skinny_f16(const SkinnyF16Args &a, hipStream_t stream) {
     bool same = true;
     for (int i = 1; i < a.n_mat; ++i) same = same && a.mat[i].type == a.mat[0].type;
     if (same) return skinny_one_type(a, stream);
-    // mixed types (q/k in q4_K, v in q6_K): one launch per run of equal type
+    // mixed types (q/k in q4_K, v in q6_K): q4_K matrices followed by one q6_K matrix share a launch ...
+    if (a.pair_launch && a.epi == EPI_STORE && !a.y16 && a.mat[a.n_mat - 1].type == MESH_Q6_K) {
+        bool lead_q4 = true;
+        for (int k2 = 0; k2 + 1 < a.n_mat; ++k2) lead_q4 = lead_q4 && a.mat[k2].type == MESH_Q4_K;
+        if (lead_q4) {
+            SkinnyF16Args qa = a, qb = a;
+            qa.n_mat = a.n_mat - 1;
+            qb.n_mat = 1;
+            qb.mat[0] = a.mat[a.n_mat - 1]; qb.kind[0] = a.kind[a.n_mat - 1];
+            const int rc = skinny_pair(qa, qb, stream);
+            if (rc != MESH_ERR_UNSUPPORTED) return rc;
+        }
+    }
+    // ... anything else: one launch per run of equal type
     int i = 0;
     while (i < a.n_mat) {
         int j = i + 1;

@@ -631,6 +631,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.x = xn; qa.K = E; qa.T = T;
+        qa.pair_launch = s->tune.skinny_pair != 0;
         if (norm_ready) {
             qa.x = nx;
             qa.norm_in.part = s->norm_part; qa.norm_in.n_parts = s->norm_parts; qa.norm_in.eps = hp.rms_eps;

@@ -21,6 +21,7 @@ const TuningField *tuning_fields() {
         {"xq_handover", &Tuning::xq_handover, 0, 1, TUNE_SESSION},
         {"skinny_f16", &Tuning::skinny_f16, 0, 1, TUNE_SESSION},
         {"skinny_norm_fused", &Tuning::skinny_norm_fused, 0, 1, TUNE_SESSION},
+        {"skinny_pair", &Tuning::skinny_pair, 0, 1, TUNE_SESSION},
         {"skinny_f16_wide", &Tuning::skinny_f16_wide, 0, 1, TUNE_SESSION},
         {"gemm_fused", &Tuning::gemm_fused, 0, 1, TUNE_SESSION},
         {"gemm_xdirect", &Tuning::gemm_xdirect, 0, 1, TUNE_SESSION},

@@ -526,6 +526,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=512, n_seq=16, n_batch=16)
     ses, ses4 = st.session(), st.session()
+    ses_two = st.session(skinny_pair=0)        # q/k (q4_K) and v (q6_K) as two launches instead of one: the same bits
     orc = StageOracle(cfg, tensors, 3, 5, 512, n_seq_max=16)
     rng = np.random.Generator(np.random.PCG64(12))
     n_past = 300
@@ -533,7 +534,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         for s in range(16):
             k = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
             v = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
-            for x_ in (ses, ses4):
+            for x_ in (ses, ses4, ses_two):
                 x_.kv_write(il, s, 0, k, v)
             orc.k[il - 3, s, :, :n_past] = k.transpose(1, 0, 2)
             orc.v[il - 3, s, :, :n_past] = v.transpose(1, 0, 2)
@@ -549,7 +550,14 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         alt = np.concatenate([ses4.decode(x[i:i + 3], pos[i:i + 3], seq=seqs[i:i + 3]).view(np.float32) for i in range(0, T, 3)]).reshape(T, 4096)
         assert rel_l2(got, ref) <= 3e-3, T
         assert rel_l2(got, alt) <= 3e-3, T
-    ses.close(); ses4.close(); st.close()
+        two = ses_two.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
+        assert np.array_equal(got, two), T
+        for q, p_ in ((seqs[0], pos[0]), (seqs[-1], pos[-1])):
+            for il in (3, 4):
+                ka, va = ses.kv_read(il, q, p_, 1)
+                kb, vb = ses_two.kv_read(il, q, p_, 1)
+                assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+    ses.close(); ses4.close(); ses_two.close(); st.close()
 
 
 def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
@@ -635,6 +643,7 @@ def test_decode_batches_of_17_to_32_stay_on_the_skinny_gemm(tmp_path):
     m, cfg, tensors, st = _open(tmp_path, "llama3-8b", [2, 3, 4], 2, 5, n_ctx=64, n_seq=32, n_batch=32)
     E = cfg["n_embd"]
     wide, gemm, plain = st.session(), st.session(skinny_f16_wide=0), st.session(skinny_norm_fused=0)
+    two = st.session(skinny_pair=0)            # one launch per weight type in the q/k/v group: the same bits
     assert wide.get_option("skinny_f16_wide") == 1 and gemm.get_option("skinny_f16_wide") == 0
     orc = StageOracle(cfg, tensors, 2, 5, 64, n_seq_max=32)
     rng = np.random.Generator(np.random.PCG64(177))
@@ -645,7 +654,7 @@ def test_decode_batches_of_17_to_32_stay_on_the_skinny_gemm(tmp_path):
                 continue
             k = (rng.standard_normal((depth[q], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
             v = (rng.standard_normal((depth[q], 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
-            for x_ in (wide, gemm, plain):
+            for x_ in (wide, gemm, plain, two):
                 x_.kv_write(il, q, 0, k, v)
             orc.k[il - 2, q, :, :depth[q]] = k.transpose(1, 0, 2)
             orc.v[il - 2, q, :, :depth[q]] = v.transpose(1, 0, 2)
@@ -661,6 +670,7 @@ def test_decode_batches_of_17_to_32_stay_on_the_skinny_gemm(tmp_path):
         a = wide.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
         b = gemm.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
         c = plain.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)
+        assert np.array_equal(a, two.decode(x, pos, seq=seqs).view(np.float32).reshape(T, E)), (step, T)
         ref = orc.forward(x, pos, seq=seqs)
         ra, rb, rc = rel_l2(a, ref), rel_l2(b, ref), rel_l2(c, ref)
         print("[wide skinny] step %d, %d tokens: %.3e (large-tile GEMM %.3e, own norm launches %.3e) of the oracle, %.3e / %.3e apart"
@@ -676,7 +686,7 @@ def test_decode_batches_of_17_to_32_stay_on_the_skinny_gemm(tmp_path):
             assert rel_l2(ka.view(np.float16).astype(np.float32), kb.view(np.float16).astype(np.float32)) <= 5e-3
             assert rel_l2(va.view(np.float16).astype(np.float32), vb.view(np.float16).astype(np.float32)) <= 5e-3
     assert wide.f16_saturations() == 0
-    wide.close(); gemm.close(); plain.close(); st.close()
+    wide.close(); gemm.close(); plain.close(); two.close(); st.close()
 
 
 def test_rope_in_projection_epilogue_equals_rope_kernel(tmp_path):
