@@ -267,7 +267,7 @@ int mesh_session_f16_saturations(mesh_session *session, uint64_t *count);
  *     xq_handover=1        single-token calls: gate/up leaves the FFN vector quantised for the down projection
  *     skinny_f16=1         the skinny GEMM on the f16 matrix cores (0: integer matrix cores, 16-bit activations)
  *     skinny_norm_fused=1  f16 skinny GEMM: the RMS norms ride in the launches around them
- *     skinny_pair=1        f16 skinny GEMM: q4_K q/k and a q6_K v projection as one launch (0: one launch per type)
+ *     skinny_pair=1        skinny GEMMs: q4_K q/k and a q6_K v projection as one launch (0: one launch per type)
  *     skinny_f16_wide=1    batches of gemm_min_tokens..32 decode steps stay on the f16 skinny GEMM (0: large-tile GEMM)
  *     gemm_fused=1         q/k/v and gate/up of a prefill call as one launch each
  *     gemm_xdirect=1       the prefill GEMM reads k8-major activations directly

@@ -93,6 +93,7 @@ struct SkinnyArgs {
     // RoPE + KV append in the epilogue of a q/k/v launch, as in the mat-vec kernel (gemv.hpp); EPI_STORE only
     GemvRope rope;
     int kind[3] = {GEMV_KIND_PLAIN, GEMV_KIND_PLAIN, GEMV_KIND_PLAIN};
+    bool pair_launch = true;         // q4_K matrices followed by one q6_K matrix (q, k and a q6_K v): one launch for both types
     // Expert launch (mixture of experts): mat[] describe expert 0 of stacked, equally shaped tiled matrices; work
     // item i (blockIdx.y) = {expert, n, pair[0..n)} in the grouping kernel's format with SKINNY_ITEM_PAIRS pairs per item
     // (moe.hpp); slot j of an item reads activation column pair[j] / x_div of xq (any block of 16) and writes output row

@@ -255,10 +255,11 @@ __device__ __forceinline__ void tile_mac(const TileView<MESH_Q6_K> &V, const XFr
     }
 }
 
+// One workgroup's share of a launch.  bx: its index among the workgroups of its launch part (the whole launch, or one side of
+// a pair launch); by: its work item (expert launches).
 template <int TYPE, int NU, int SEGS, bool GROUPED>
-__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
-                                                                 int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
-                                                                 const SkinnyKernelArgs a) {
+__device__ __forceinline__ void skinny_workgroup(int bx, int by, const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+                                                 int p_ks, unsigned p_begins, unsigned p_split, const SkinnyKernelArgs &a) {
     // (leading scalar arguments: preloaded into SGPRs, see gemv.hip.  p_begins = first tile-row of matrix 1 | of matrix 2
     // << 16; p_split = tile-rows per workgroup | workgroups with one more << 16, computed on the host: no division and
     // no grid-size load stand before the first weight load)
@@ -268,12 +269,12 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
     if (GROUPED) {
         // item count and item are fetched together (the item buffer holds max_items entries, so the read is in bounds even
         // for a workgroup past the count): one memory round trip before the first weight load instead of two
-        const int32_t *it = a.items + (size_t)blockIdx.y * SK_ITEM_INTS;
+        const int32_t *it = a.items + (size_t)by * SK_ITEM_INTS;
         const int n_live = ldg<int>(a.n_items);
         const int2 head = ldg<int2>(reinterpret_cast<const int2 *>(it));
         const int slot_l = (int)(threadIdx.x & 15);
         const int p_mine = ldg<int>(it + 2 + slot_l), p_first = ldg<int>(it + 2);
-        if ((int)blockIdx.y >= n_live) return;
+        if (by >= n_live) return;
         const size_t eoff = (size_t)head.x * a.expert_stride;
         p_w0 += eoff; p_w1 += eoff; p_w2 += eoff;
         it_n = head.y;
@@ -294,8 +295,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
     const int m = lane & 15, g = lane >> 4;
     const int KS = p_ks, LK = __builtin_ctz((unsigned)KS), RS = SK_WAVES >> LK;      // KS is a power of two
     const int ks = wave & (KS - 1), rs = wave >> LK;
-    (void)p_rows;
-    const int sq = (int)(p_split & 0xFFFFu), sr = (int)(p_split >> 16), bx = blockIdx.x;
+    const int sq = (int)(p_split & 0xFFFFu), sr = (int)(p_split >> 16);
     const int tr0 = bx * sq + (bx < sr ? bx : sr);
     const int rows_here = sq + (bx < sr ? 1 : 0);
     const int n_i = rs < RS ? (nsb - ks + KS - 1) >> LK : 0;        // super-blocks of this wave (ks < KS <= nsb)
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
         const int t = o % SK_NT, r = (o / SK_NT) % 16, j = o / (SK_NT * 16);
         if (t >= (GROUPED ? it_n : a.T)) continue;
         // output row of column t: the token itself, or the pair the item lists for this slot
-        const size_t orow = GROUPED ? (size_t)a.items[(size_t)blockIdx.y * SK_ITEM_INTS + 2 + t] : (size_t)t;
+        const size_t orow = GROUPED ? (size_t)a.items[(size_t)by * SK_ITEM_INTS + 2 + t] : (size_t)t;
         const int tr = tr0 + j;
         int mi = 0;
         if (NU == 1) mi = (tr >= a.tile_begin[1] ? 1 : 0) + (tr >= a.tile_begin[2] ? 1 : 0);
@@ -441,6 +441,25 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *
 }
 
 template <int TYPE, int NU, int SEGS, bool GROUPED>
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, const uint8_t *p_w2, int p_K,
+                                                                 int p_ks, int p_rows, unsigned p_begins, unsigned p_split,
+                                                                 const SkinnyKernelArgs a) {
+    (void)p_rows;
+    skinny_workgroup<TYPE, NU, SEGS, GROUPED>((int)blockIdx.x, (int)blockIdx.y, p_xq, p_w0, p_w1, p_w2, p_K, p_ks, p_begins, p_split, a);
+}
+
+// Two launches over the same activations as one: the first grid_a workgroups run a q4_K launch, the others a q6_K launch (the q
+// and k projections of a layer next to a q6_K v projection).  Same arithmetic per workgroup as the separate launches.
+template <int SEGS_A, int SEGS_B>
+__global__ __launch_bounds__(SK_THREADS) void gemm_skinny_pair_kernel(const uint8_t *p_xq, const uint8_t *p_w0, const uint8_t *p_w1, int p_K, int p_ks_a,
+                                                                      int p_ks_b, int grid_a, unsigned p_begins, unsigned p_split_a, unsigned p_split_b,
+                                                                      const uint8_t *p_wb, const SkinnyKernelArgs a, const SkinnyKernelArgs b) {
+    const int bx = (int)blockIdx.x;
+    if (bx < grid_a) skinny_workgroup<MESH_Q4_K, 1, SEGS_A, false>(bx, 0, p_xq, p_w0, p_w1, p_w1, p_K, p_ks_a, p_begins, p_split_a, a);
+    else skinny_workgroup<MESH_Q6_K, 1, SEGS_B, false>(bx - grid_a, 0, p_xq, p_wb, p_wb, p_wb, p_K, p_ks_b, 0xFFFFFFFFu, p_split_b, b);
+}
+
+template <int TYPE, int NU, int SEGS, bool GROUPED>
 static int launch_skinny(const SkinnyKernelArgs &ka, const uint8_t *xq, int grid, int grid_y, size_t smem, hipStream_t stream) {
     static bool attr_set = false;
     if (!attr_set) {
@@ -479,13 +498,20 @@ static int skinny_n_cu() {
 
 size_t q16_block_bytes(int K) { return (size_t)K * 32 + 2 * (size_t)(K / 32) * 16 * sizeof(float); }
 
-// all matrices of `a` are tiled K-quants of one type
-static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
+// What a launch over the matrices of `a` (tiled K-quants of one type) needs, before the token block is chosen
+struct SkinnyLaunch {
+    SkinnyKernelArgs ka;
+    int type, NU, KS, grid, segs;
+    size_t smem;
+};
+static int skinny_prepare(const SkinnyArgs &a, SkinnyLaunch &L) {
     const int type = a.mat[0].type;
     const int nsb = a.K / QK_K, NU = a.epi == EPI_SWIGLU ? 2 : 1;
+    L.type = type; L.NU = NU;
     const int tile_bytes = type == MESH_Q4_K ? Q4K_TILE_BYTES : Q6K_TILE_BYTES;
     const size_t row_stride = (size_t)nsb * tile_bytes;
-    SkinnyKernelArgs ka{};
+    SkinnyKernelArgs &ka = L.ka;
+    ka = SkinnyKernelArgs{};
     int total_rows = 0;
     for (int i = 0; i < a.n_mat; ++i) {
         const int begin = (NU == 2 && i == 1) ? 0 : total_rows;     // gate and up share tile-row indices
@@ -528,30 +554,85 @@ static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
     }
     const int RS = SK_WAVES / KS;
     ka.ks = KS;
-    const int grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
-    const int rows_max = (total_rows + grid - 1) / grid;
-    const int segs = ((rows_max + RS - 1) / RS) * NU;   // per wave
-    if (segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d segments per wave", segs);
+    L.KS = KS;
+    L.grid = (total_rows + rows_per_wg - 1) / rows_per_wg;
+    const int rows_max = (total_rows + L.grid - 1) / L.grid;
+    L.segs = ((rows_max + RS - 1) / RS) * NU;           // per wave
+    if (L.segs > SK_SEGS_MAX) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d segments per wave", L.segs);
     if (total_rows > 0xFFFF) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %d tile-rows in one launch", total_rows);
     const int lds_tile = ((type == MESH_Q4_K ? LDS_TILE_Q4 : LDS_TILE_Q6) + 255) / 256 * 256;
-    const size_t smem = (size_t)SK_WAVES * (lds_tile + 2 * 512) + sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
-    if (smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %zu bytes of LDS needed", smem);
-    if (grouped) {
+    L.smem = (size_t)SK_WAVES * (lds_tile + 2 * 512) + sizeof(float) * (size_t)KS * rows_max * NU * 16 * SK_NT;
+    if (L.smem > SK_LDS_LIMIT) return fail(MESH_ERR_UNSUPPORTED, "gemm_skinny: %zu bytes of LDS needed", L.smem);
+    return MESH_OK;
+}
+// the kernel arguments for token block t / 16 of the call
+static SkinnyKernelArgs skinny_block(const SkinnyArgs &a, const SkinnyLaunch &L, int t) {
+    SkinnyKernelArgs kb = L.ka;
+    kb.T = std::min(SK_NT, a.T - t);
+    if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
+    kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
+    for (int i = 0; i < a.n_mat; ++i)
+        if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
+    return kb;
+}
+
+// all matrices of `a` are tiled K-quants of one type
+static int skinny_one_type(const SkinnyArgs &a, hipStream_t stream) {
+    SkinnyLaunch L;
+    int rc = skinny_prepare(a, L);
+    if (rc != MESH_OK) return rc;
+    const int type = L.type, NU = L.NU, segs = L.segs, grid = L.grid;
+    const size_t smem = L.smem;
+    if (a.items) {
+        SkinnyKernelArgs ka = L.ka;
         ka.T = SK_NT;
         if (type == MESH_Q4_K) return NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, ka, a.xq, grid, a.max_items, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, ka, a.xq, grid, a.max_items, smem, stream);
         return NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, ka, a.xq, grid, a.max_items, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, ka, a.xq, grid, a.max_items, smem, stream);
     }
     for (int t = 0; t < a.T; t += SK_NT) {
-        SkinnyKernelArgs kb = ka;
-        kb.T = std::min(SK_NT, a.T - t);
-        if (kb.rope.pos) { kb.rope.pos += t; kb.rope.seq += t; }
+        const SkinnyKernelArgs kb = skinny_block(a, L, t);
         const uint8_t *xq = a.xq + (size_t)(t / SK_NT) * q16_block_bytes(a.K);
-        kb.residual = a.residual ? a.residual + (size_t)t * a.ldres : nullptr;
-        for (int i = 0; i < a.n_mat; ++i)
-            if (kb.y[i]) kb.y[i] = a.mat[i].y + (size_t)t * a.mat[i].ldy;
-        int rc;
         if (type == MESH_Q4_K) rc = NU == 2 ? launch_skinny_segs<MESH_Q4_K, 2>(segs, kb, xq, grid, 1, smem, stream) : launch_skinny_segs<MESH_Q4_K, 1>(segs, kb, xq, grid, 1, smem, stream);
         else rc = NU == 2 ? launch_skinny_segs<MESH_Q6_K, 2>(segs, kb, xq, grid, 1, smem, stream) : launch_skinny_segs<MESH_Q6_K, 1>(segs, kb, xq, grid, 1, smem, stream);
+        if (rc != MESH_OK) return rc;
+    }
+    return MESH_OK;
+}
+
+template <int SEGS_A, int SEGS_B>
+static int launch_pair(const SkinnyKernelArgs &ka, const SkinnyKernelArgs &kb, const uint8_t *xq, int grid_a, int grid_b, size_t smem, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        MESH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_skinny_pair_kernel<SEGS_A, SEGS_B>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)SK_LDS_LIMIT));
+        attr_set = true;
+    }
+    MESH_LAUNCH((gemm_skinny_pair_kernel<SEGS_A, SEGS_B>), dim3((unsigned)(grid_a + grid_b)), dim3(SK_THREADS), smem, stream, xq, ka.wbase[0],
+                ka.wbase[1] ? ka.wbase[1] : ka.wbase[0], ka.K, ka.ks, kb.ks, grid_a, (unsigned)ka.tile_begin[1] | ((unsigned)ka.tile_begin[2] << 16),
+                (unsigned)(ka.tile_begin[3] / grid_a) | ((unsigned)(ka.tile_begin[3] % grid_a) << 16),
+                (unsigned)(kb.tile_begin[3] / grid_b) | ((unsigned)(kb.tile_begin[3] % grid_b) << 16), kb.wbase[0], ka, kb);
+    MESH_LAUNCH_CHECK();
+    return MESH_OK;
+}
+
+// `qa`: one or two q4_K matrices, `qb`: one q6_K matrix, same activations, plain-store epilogues (with or without RoPE): one
+// launch whose first workgroups are qa's and whose last are qb's.  MESH_ERR_UNSUPPORTED when the shapes do not fit (the
+// caller then launches them one after the other).
+static int skinny_pair(const SkinnyArgs &qa, const SkinnyArgs &qb, hipStream_t stream) {
+    SkinnyLaunch A, B;
+    int rc = skinny_prepare(qa, A);
+    if (rc != MESH_OK) return rc;
+    if ((rc = skinny_prepare(qb, B)) != MESH_OK) return rc;
+    if (B.segs > 2) return MESH_ERR_UNSUPPORTED;
+    const size_t smem = std::max(A.smem, B.smem);
+    const int sa = A.segs <= 1 ? 1 : A.segs <= 2 ? 2 : 4;
+    for (int t = 0; t < qa.T; t += SK_NT) {
+        const SkinnyKernelArgs ka = skinny_block(qa, A, t), kb = skinny_block(qb, B, t);
+        const uint8_t *xq = qa.xq + (size_t)(t / SK_NT) * q16_block_bytes(qa.K);
+        if (B.segs <= 1) rc = sa == 1 ? launch_pair<1, 1>(ka, kb, xq, A.grid, B.grid, smem, stream) : sa == 2 ? launch_pair<2, 1>(ka, kb, xq, A.grid, B.grid, smem, stream)
+                                                                                                            : launch_pair<4, 1>(ka, kb, xq, A.grid, B.grid, smem, stream);
+        else rc = sa == 1 ? launch_pair<1, 2>(ka, kb, xq, A.grid, B.grid, smem, stream) : sa == 2 ? launch_pair<2, 2>(ka, kb, xq, A.grid, B.grid, smem, stream)
+                                                                                                  : launch_pair<4, 2>(ka, kb, xq, A.grid, B.grid, smem, stream);
         if (rc != MESH_OK) return rc;
     }
     return MESH_OK;
@@ -908,7 +989,20 @@ int gemm_skinny(const SkinnyArgs &a, hipStream_t stream) {
     bool same = true;
     for (int i = 1; i < a.n_mat; ++i) same = same && a.mat[i].type == a.mat[0].type;
     if (same) return skinny_one_type(a, stream);
-    // mixed types (q/k in q4_K, v in q6_K): one launch per run of equal type
+    // mixed types (q/k in q4_K, v in q6_K): q4_K matrices followed by one q6_K matrix share a launch ...
+    if (a.pair_launch && !a.items && a.epi == EPI_STORE && a.mat[a.n_mat - 1].type == MESH_Q6_K) {
+        bool lead_q4 = true;
+        for (int k2 = 0; k2 + 1 < a.n_mat; ++k2) lead_q4 = lead_q4 && a.mat[k2].type == MESH_Q4_K;
+        if (lead_q4) {
+            SkinnyArgs qa = a, qb = a;
+            qa.n_mat = a.n_mat - 1;
+            qb.n_mat = 1;
+            qb.mat[0] = a.mat[a.n_mat - 1]; qb.kind[0] = a.kind[a.n_mat - 1];
+            const int rc = skinny_pair(qa, qb, stream);
+            if (rc != MESH_ERR_UNSUPPORTED) return rc;
+        }
+    }
+    // ... anything else: one launch per run of equal type
     int i = 0;
     while (i < a.n_mat) {
         int j = i + 1;

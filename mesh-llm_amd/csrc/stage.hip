@@ -651,6 +651,7 @@ static int run_layer_prefill(mesh_session *s, const LayerWeights &L, size_t il, 
         qa.mat[1] = mat_of(L.wk, s->k, KD, &L.bk);
         qa.mat[2] = mat_of(L.wv, s->v, KD, &L.bv);
         qa.xq = s->xq; qa.K = E; qa.T = T;
+        qa.pair_launch = s->tune.skinny_pair != 0;
         if (s->tune.gemv_rope && hp.rope_mode == ROPE_MODE_NORM && st->k_type == MESH_F16 && st->v_type == MESH_F16 && !L.q_norm.present() &&
             !L.k_norm.present() && hp.head_dim % 2 == 0 && hp.n_rot % 2 == 0) {
             qa.rope.pos = s->d_pos; qa.rope.seq = s->d_seq; qa.rope.inv_freq = st->rope_inv_freq;

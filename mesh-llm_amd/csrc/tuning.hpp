@@ -25,7 +25,7 @@ struct Tuning {
     int xq_handover = 1;           // the gate/up mat-vec leaves the FFN vector quantised for the down projection
     int skinny_f16 = 1;            // calls of skinny_min_tokens..gemm_min_tokens-1 tokens on the f16 matrix cores (0: integer, 16-bit activations)
     int skinny_norm_fused = 1;     // f16 skinny GEMM: the RMS norms ride in the launches around them (0: a norm launch of their own)
-    int skinny_pair = 1;           // f16 skinny GEMM: q4_K q/k and a q6_K v projection as one launch (0: one launch per type)
+    int skinny_pair = 1;           // skinny GEMMs: q4_K q/k and a q6_K v projection as one launch (0: one launch per type)
     int skinny_f16_wide = 1;       // batches of gemm_min_tokens..32 decode steps stay on the f16 skinny GEMM, 32 columns per pass (0: large-tile GEMM)
     int gemm_fused = 1;            // q/k/v and gate/up of a prefill call as one GEMM launch each
     int gemm_xdirect = 1;          // the prefill GEMM reads k8-major activations directly (0: row-major staged through LDS)

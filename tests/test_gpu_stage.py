@@ -527,6 +527,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=512, n_seq=16, n_batch=16)
     ses, ses4 = st.session(), st.session()
     ses_two = st.session(skinny_pair=0)        # q/k (q4_K) and v (q6_K) as two launches instead of one: the same bits
+    int_one, int_two = st.session(skinny_f16=0), st.session(skinny_f16=0, skinny_pair=0)      # the same for the integer kernel
     orc = StageOracle(cfg, tensors, 3, 5, 512, n_seq_max=16)
     rng = np.random.Generator(np.random.PCG64(12))
     n_past = 300
@@ -534,7 +535,7 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         for s in range(16):
             k = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
             v = (rng.standard_normal((n_past, 8, 128)) * 0.5).astype(np.float16).view(np.uint16)
-            for x_ in (ses, ses4, ses_two):
+            for x_ in (ses, ses4, ses_two, int_one, int_two):
                 x_.kv_write(il, s, 0, k, v)
             orc.k[il - 3, s, :, :n_past] = k.transpose(1, 0, 2)
             orc.v[il - 3, s, :, :n_past] = v.transpose(1, 0, 2)
@@ -552,12 +553,17 @@ def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
         assert rel_l2(got, alt) <= 3e-3, T
         two = ses_two.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
         assert np.array_equal(got, two), T
+        if T >= 5:                          # (the integer kernel takes batches from five tokens on)
+            i1 = int_one.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
+            i2 = int_two.decode(x, pos, seq=seqs).view(np.float32).reshape(T, 4096)
+            assert np.array_equal(i1, i2), T
+            assert rel_l2(i1, ref) <= 5e-4, T
         for q, p_ in ((seqs[0], pos[0]), (seqs[-1], pos[-1])):
             for il in (3, 4):
                 ka, va = ses.kv_read(il, q, p_, 1)
                 kb, vb = ses_two.kv_read(il, q, p_, 1)
                 assert np.array_equal(ka, kb) and np.array_equal(va, vb)
-    ses.close(); ses4.close(); ses_two.close(); st.close()
+    ses.close(); ses4.close(); ses_two.close(); int_one.close(); int_two.close(); st.close()
 
 
 def test_wide_decode_batch_takes_large_tile_gemm(tmp_path):
