@@ -4,9 +4,9 @@ GPU stage's output hidden state and the CPU oracle's on identical seeded weights
   C3  Llama-3-8B-shaped stage, ALL 16 layers (0-15 of 32), 4096-token KV context filled to depth 4095: decode at batch
       1, 4 and 16 (mat-vec kernels, skinny MFMA GEMM, matrix-core decode attention); a 2048-token prefill through two
       real-shape layers and a 256-token prefill through all 16 (large-tile MFMA GEMM, chunk attention).
-  C4  Qwen2.5-32B-shaped layers (hidden 5120, 40 / 8 heads, FFN 27648, q/k/v bias): decode batch 24 and 32 (large-tile
-      GEMM with K split over workgroups), a 320-token prefill (chunk attention with 5 query heads per KV head), over
-      f16 and over q8_0 / q4_0 caches.
+  C4  Qwen2.5-32B-shaped layers (hidden 5120, 40 / 8 heads, FFN 27648, q/k/v bias): decode batch 24 and 32 (f16 skinny
+      GEMM with two blocks of 16 activation columns per pass), a 320-token prefill (large-tile GEMM, chunk attention with
+      5 query heads per KV head), over f16 and over q8_0 / q4_0 caches; decode at KV depth 8191 of 8192 on all cache tiers.
   C5  Qwen3-30B-A3B-shaped 64-expert shard layer, router logits ~ N(0,1) + Zipf(1.1) expert bias, batch 16 on top of a
       filled KV cache.
 Every test prints the figure it measured.  The oracle's projections of prefill-sized calls go through numpy's float64
