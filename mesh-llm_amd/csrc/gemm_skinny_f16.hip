@@ -222,7 +222,7 @@ __device__ __forceinline__ void skinny_workgroup(int bx, const _Float16 *p_x, co
     const int p_begin1 = (int)(p_begins & 0xFFFFu), p_begin2 = (int)(p_begins >> 16);
     // (leading scalar arguments: preloaded into SGPRs, see gemv.hip)
     extern __shared__ __align__(16) uint8_t smem[];
-    float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 cols]
+    float *red = reinterpret_cast<float *>(smem);         // [KS][rows_here][NU][16 rows][16 NC columns]
     constexpr int TB = TileRegs<TYPE>::BYTES;
     constexpr int SK_DEPTH = TYPE == MESH_Q4_K ? SK_DEPTH_Q4 : SK_DEPTH_Q6;
     const int K = p_K, nsb = K / QK_K;
@@ -270,59 +270,57 @@ __device__ __forceinline__ void skinny_workgroup(int bx, const _Float16 *p_x, co
         const bool ok = f < total && seg_valid(seg);
         dst.load(tile_ptr(ok ? f / SEGS : n_i - 1, ok ? seg : 0), lane);
     };
-    {
-        // Activation fragments: 8 KB per super-block, column block and wave.  Only ONE super-block is held (32 registers per
-        // column block) and every fragment is fetched again, for the next super-block, right behind the last MFMAs that read
-        // it: one tile's time ahead of its use, enough for a hit in L2.  (Two whole super-blocks in registers, fetched a
-        // super-block ahead, cost 32 more registers per column block and measured 6% slower at 16 columns.)  A tile that
-        // is not computed (past the end, invalid segment) issues the same loads in the same order, so that the compiler's
-        // count of loads in flight is the same along both paths.
-        BFrags<TYPE> Bw[NC];
-        auto frag_koff = [](int t) { return (TYPE == MESH_Q4_K ? 32 * (t >> 2) + 8 * (t & 3) : 32 * (t >> 1) + 8 * (t & 1)) * 16; };
-        auto b_base = [&](int sb, int c) { return p_x + (size_t)c * SK_NT * K + (size_t)sb * (QK_K * 16) + lane_off; };
-        auto step = [&](const TileRegs<TYPE> &loaded, f4_t (&acc)[NC], bool valid, bool refill, int next_sb) {
-            const _Float16 *nb[NC];
+    // Activation fragments: 8 KB per super-block, column block and wave.  Only ONE super-block is held (32 registers per
+    // column block) and every fragment is fetched again, for the next super-block, right behind the last MFMAs that read
+    // it: one tile's time ahead of its use, enough for a hit in L2.  (Two whole super-blocks in registers, fetched a
+    // super-block ahead, cost 32 more registers per column block and measured 6% slower at 16 columns.)  A tile that
+    // is not computed (past the end, invalid segment) issues the same loads in the same order, so that the compiler's
+    // count of loads in flight is the same along both paths.
+    BFrags<TYPE> Bw[NC];
+    auto frag_koff = [](int t) { return (TYPE == MESH_Q4_K ? 32 * (t >> 2) + 8 * (t & 3) : 32 * (t >> 1) + 8 * (t & 1)) * 16; };
+    auto b_base = [&](int sb, int c) { return p_x + (size_t)c * SK_NT * K + (size_t)sb * (QK_K * 16) + lane_off; };
+    auto step = [&](const TileRegs<TYPE> &loaded, f4_t (&acc)[NC], bool valid, bool refill, int next_sb) {
+        const _Float16 *nb[NC];
 #pragma unroll
-            for (int c = 0; c < NC; ++c) nb[c] = b_base(next_sb, c);
-            if (valid) {
-                TileRegs<TYPE> tile = loaded;
-                to_mfma_lanes(tile, src_lane4);
-                TileFrags<TYPE> F;
-                F.prepare(tile, g);
+        for (int c = 0; c < NC; ++c) nb[c] = b_base(next_sb, c);
+        if (valid) {
+            TileRegs<TYPE> tile = loaded;
+            to_mfma_lanes(tile, src_lane4);
+            TileFrags<TYPE> F;
+            F.prepare(tile, g);
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const h8_t af = F.frag(t);
+            for (int t = 0; t < 8; ++t) {
+                const h8_t af = F.frag(t);
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(h8_t, Bw[c].b[t]), acc[c], 0, 0, 0);
-                    if (refill) {
-#pragma unroll
-                        for (int c = 0; c < NC; ++c) Bw[c].b[t] = ldg<uint4>(nb[c] + frag_koff(t));
-                    }
-                }
-            } else if (refill) {
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
+                for (int c = 0; c < NC; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(h8_t, Bw[c].b[t]), acc[c], 0, 0, 0);
+                if (refill) {
 #pragma unroll
                     for (int c = 0; c < NC; ++c) Bw[c].b[t] = ldg<uint4>(nb[c] + frag_koff(t));
-            }
-        };
-        if (total > 0) {
-#pragma unroll
-            for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
-#pragma unroll
-            for (int c = 0; c < NC; ++c) Bw[c].load(p_x + (size_t)c * SK_NT * K, lane_off, ks);
-            constexpr int RB = SEGS % SK_DEPTH == 0 ? 1 : SK_DEPTH;      // rounds per unrolled block: ring slots static inside it
-            constexpr int UB = RB * SEGS;
-            static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
-            for (int blk = 0; blk * RB < n_i; ++blk) {
-#pragma unroll
-                for (int q = 0; q < UB; ++q) {
-                    const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
-                    const int ii = blk * RB + r, f = ii * SEGS + seg;
-                    step(ring[slot], D[seg], ii < n_i && seg_valid(seg), seg == SEGS - 1, ks + KS * (ii + 1 < n_i ? ii + 1 : n_i - 1));
-                    load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
-                    __builtin_amdgcn_sched_barrier(0);
                 }
+            }
+        } else if (refill) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) Bw[c].b[t] = ldg<uint4>(nb[c] + frag_koff(t));
+        }
+    };
+    if (total > 0) {
+#pragma unroll
+        for (int f = 0; f < SK_DEPTH; ++f) load_tile(ring[f], f, f % SEGS);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) Bw[c].load(p_x + (size_t)c * SK_NT * K, lane_off, ks);
+        constexpr int RB = SEGS % SK_DEPTH == 0 ? 1 : SK_DEPTH;      // rounds per unrolled block: ring slots static inside it
+        constexpr int UB = RB * SEGS;
+        static_assert(UB % SK_DEPTH == 0, "ring slots must be static inside a block");
+        for (int blk = 0; blk * RB < n_i; ++blk) {
+#pragma unroll
+            for (int q = 0; q < UB; ++q) {
+                const int r = q / SEGS, seg = q % SEGS, slot = q % SK_DEPTH;
+                const int ii = blk * RB + r, f = ii * SEGS + seg;
+                step(ring[slot], D[seg], ii < n_i && seg_valid(seg), seg == SEGS - 1, ks + KS * (ii + 1 < n_i ? ii + 1 : n_i - 1));
+                load_tile(ring[slot], f + SK_DEPTH, (q + SK_DEPTH) % SEGS);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
