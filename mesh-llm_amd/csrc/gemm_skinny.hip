@@ -871,9 +871,71 @@ __global__ __launch_bounds__(256) void to_k8_kernel(const float *__restrict__ x,
     }
 }
 
+// The same for prefill-sized calls, one workgroup of 1024 threads per 8 tokens: thread (token = tid % 8, group lane = tid / 8)
+// keeps NG groups of 8 consecutive elements of its token's row in registers (one read of the row), the squares are added per
+// token over the workgroup, and 8 neighbouring threads write one contiguous 128-byte run of the block -- the per-token
+// kernel above writes 16 bytes every 256.  Rows of 1024 * NG elements.  The sum of squares is taken in another order than in
+// to_k8_kernel, so the scale can differ from that kernel's in its last bit.
+constexpr int K8B_THREADS = 1024, K8B_WAVES = K8B_THREADS / 64, K8B_TOK = 8, K8B_LANES = K8B_THREADS / K8B_TOK;
+template <int NG>
+__global__ __launch_bounds__(K8B_THREADS) void to_k8_block_kernel(const float *__restrict__ x, const float *__restrict__ w, float eps, int T,
+                                                                  _Float16 *__restrict__ y, unsigned *sat) {
+    constexpr int n = 8 * K8B_LANES * NG;
+    __shared__ float s_ss[K8B_WAVES][K8B_TOK];
+    const int tid = threadIdx.x, tl = tid % K8B_TOK, gl = tid / K8B_TOK, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x * K8B_TOK + tl;
+    const bool live = t < T;
+    const float *xt = x + (size_t)(live ? t : 0) * n;
+    float4 v[NG][2];
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+        const int i = 8 * (gl + K8B_LANES * j);
+        v[j][0] = live ? *reinterpret_cast<const float4 *>(xt + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[j][1] = live ? *reinterpret_cast<const float4 *>(xt + i + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NG; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) ss += (v[j][h].x * v[j][h].x + v[j][h].y * v[j][h].y) + (v[j][h].z * v[j][h].z + v[j][h].w * v[j][h].w);
+    // the eight lanes of a wave that hold the same token, then the waves in order
+    ss += __shfl_xor(ss, 8);
+    ss += __shfl_xor(ss, 16);
+    ss += __shfl_xor(ss, 32);
+    if (lane < K8B_TOK) s_ss[wave][lane] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int k = 0; k < K8B_WAVES; ++k) tot += s_ss[k][tl];
+    const float sc = 1.0f / sqrtf(tot / (float)n + eps);
+    _Float16 *yb = y + (size_t)(t / 16) * 16 * n + (size_t)(t % 16) * 8;        // element (t, k) at yb + (k / 8) * 128 + k % 8
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+        const int i = 8 * (gl + K8B_LANES * j);
+        const float4 g0 = *reinterpret_cast<const float4 *>(w + i), g1 = *reinterpret_cast<const float4 *>(w + i + 4);
+        const float4 v0 = v[j][0], v1 = v[j][1];
+        // (slots past the last token hold zeros: v is zero there)
+        *reinterpret_cast<uint4 *>(yb + (size_t)(i >> 3) * 128) =
+            make_uint4(sk_pack_h2(sat, v0.x * sc * g0.x, v0.y * sc * g0.y), sk_pack_h2(sat, v0.z * sc * g0.z, v0.w * sc * g0.w),
+                       sk_pack_h2(sat, v1.x * sc * g1.x, v1.y * sc * g1.y), sk_pack_h2(sat, v1.z * sc * g1.z, v1.w * sc * g1.w));
+    }
+}
+constexpr int K8B_MIN_TOKENS = 64;       // below: the per-token kernel (decode batches keep its bits)
+
 int rmsnorm_f16_k8(const float *x, const float *w, float eps, int T, int n, _Float16 *y, hipStream_t stream, unsigned *sat) {
     if (T <= 0) return MESH_OK;
     if (n % 8) return fail(MESH_ERR_INVALID, "rmsnorm_f16_k8: row length %d not a multiple of 8", n);
+    if (w && T >= K8B_MIN_TOKENS && n % (8 * K8B_LANES) == 0) {
+        // (the grid covers the padded batch: slots past the last token of the last block of 16 are written as zeros)
+        const dim3 grid((unsigned)((T + 15) / 16 * 16 / K8B_TOK)), block(K8B_THREADS);
+        switch (n / (8 * K8B_LANES)) {
+            case 2: MESH_LAUNCH(to_k8_block_kernel<2>, grid, block, 0, stream, x, w, eps, T, y, sat); MESH_LAUNCH_CHECK(); return MESH_OK;
+            case 4: MESH_LAUNCH(to_k8_block_kernel<4>, grid, block, 0, stream, x, w, eps, T, y, sat); MESH_LAUNCH_CHECK(); return MESH_OK;
+            case 5: MESH_LAUNCH(to_k8_block_kernel<5>, grid, block, 0, stream, x, w, eps, T, y, sat); MESH_LAUNCH_CHECK(); return MESH_OK;
+            case 8: MESH_LAUNCH(to_k8_block_kernel<8>, grid, block, 0, stream, x, w, eps, T, y, sat); MESH_LAUNCH_CHECK(); return MESH_OK;
+            default: break;     // other row lengths: the per-token kernel
+        }
+    }
     MESH_LAUNCH(to_k8_kernel, dim3((unsigned)((T + 15) / 16 * 16)), dim3(256), 0, stream, x, w, eps, T, n, y, sat);
     MESH_LAUNCH_CHECK();
     return MESH_OK;
