@@ -473,6 +473,7 @@ int session_new(mesh_stage *st, mesh_session **out) {
     s->d_seq = s->d_pos + B;
     s->d_tok = s->d_seq + B;
     MESH_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->h_meta), META_SLOTS * 3 * B * sizeof(int32_t), hipHostMallocDefault));
+    memset(s->h_meta, 0, META_SLOTS * 3 * B * sizeof(int32_t));
     // staging for packed in/out of the host-pointer entry point: f32 rows of n_embd in; the same or logits rows out
     // (logits of at most LOGITS_TOKENS_MAX tokens per call: a row of a 152k vocabulary is 0.6 MB)
     s->io_stage_bytes = B * (size_t)hp.n_embd * sizeof(float);
@@ -1233,8 +1234,9 @@ int stage_decode_dev(mesh_session *s, const mesh_batch *b, const void *d_in, int
     if (s->meta_counter && s->meta_counter % META_SLOTS == 0) MESH_HIP_TRY(hipStreamSynchronize(stream));   // ring wraps: older copies are done
     int32_t *slot = s->h_meta + (size_t)(s->meta_counter++ % META_SLOTS) * 3 * B;
     for (int i = 0; i < T; ++i) { slot[i] = b->pos[i]; slot[B + i] = b->seq_id ? b->seq_id[i] : 0; }
-    MESH_HIP_TRY(hipMemcpyAsync(s->d_pos, slot, T * sizeof(int32_t), hipMemcpyHostToDevice, stream));
-    MESH_HIP_TRY(hipMemcpyAsync(s->d_seq, slot + B, T * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+    // (one copy for both: the slot and the device buffer have the same layout, positions at 0 and sequence ids at B; a copy is
+    // a launch of its own on the stream, and the entries between T and B are never read)
+    MESH_HIP_TRY(hipMemcpyAsync(s->d_pos, slot, (B + T) * sizeof(int32_t), hipMemcpyHostToDevice, stream));
 
     if (tokens_in) {
         // embedding rows: one dequantize per token (ids are read on the host side by the caller's contract)
