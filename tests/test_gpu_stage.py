@@ -520,8 +520,8 @@ def test_prefill_chunks_of_a_model_with_one_query_head_per_kv_head(tmp_path):
 
 
 def test_batched_decode_skinny_gemm_matches_oracle_and_gemv_path(tmp_path):
-    """Decode batches of 4..16 tokens run their projections on the matrix cores (gemm_skinny.hip).  Real-shape layers
-    (one with q6_K attn_v / ffn_down, so q/k/v split into two launches), 16 sequences at KV depth 300, full and ragged
+    """Decode batches of 4..16 tokens run their projections on the matrix cores (gemm_skinny_f16.hip, gemm_skinny.hip).  Real-shape layers
+    (one with q6_K attn_v / ffn_down, so q/k/v mix two weight types: one pair launch, or two launches), 16 sequences at KV depth 300, full and ragged
     batches; against the oracle and against the same steps fed three at a time through the mat-vec kernel."""
     name = "llama3-8b"
     m, cfg, tensors, st = _open(tmp_path, name, [3, 4], 3, 5, n_ctx=512, n_seq=16, n_batch=16)
